@@ -1,0 +1,144 @@
+/*
+ * C ABI of libneuzip_hip.so: the MI355X (gfx950) NeuZip bf16 codec.
+ *
+ * This is the drop-in boundary for the reference's pybind11 extension
+ * `neuzip._cuda` (cuda/neuzip.cu:19-38): every entry point below names the
+ * reference method it stands in for.  Plain pointers and sizes only; device
+ * pointers are HIP device addresses, `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  All kernels are enqueued on the
+ * caller's stream; nothing here creates a private stream (the reference's
+ * private `estream`, cuda/high_level.cu:47, is not synchronised with the
+ * producer of its input and is not reproduced).
+ *
+ * Every function returns NZ_OK or a negative NZ_ERR_* code; a message for the
+ * last failure on the calling thread is available from nz_last_error().
+ *
+ * Dense bf16 pointers must be 16-byte aligned.
+ */
+#ifndef NEUZIP_HIP_H
+#define NEUZIP_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define NZ_OK 0
+#define NZ_ERR_ARG -1       /* bad argument / unsupported geometry           */
+#define NZ_ERR_DTYPE -2     /* "Unsupported data type", high_level.cu:160    */
+#define NZ_ERR_NOT_FOUND -3 /* "Data not found", high_level.cu:225           */
+#define NZ_ERR_HIP -4       /* a HIP runtime call failed                     */
+#define NZ_ERR_CAPACITY -5  /* output buffer too small                       */
+#define NZ_ERR_CORRUPT -6   /* compressed buffer failed validation           */
+#define NZ_ERR_ALIGN -7     /* dense pointer not 16-byte aligned             */
+#define NZ_ERR_ALGO -8      /* "Unsupported algorithm", high_level.cu:67     */
+
+/* dtype codes (only bf16 is implemented; the reference's fp16/fp32 branches,
+   high_level.cu:144-161, truncate the mantissa and are out of scope) */
+#define NZ_DTYPE_BF16 0
+#define NZ_DTYPE_F16 1
+#define NZ_DTYPE_F32 2
+
+/* algorithm codes: cuda/algorithms.cuh:8. Only ANS exists here. */
+#define NZ_ALGO_ANS 0
+
+#define NZ_DEFAULT_CHUNK 65536u   /* cuda/neuzip.cu:31 */
+#define NZ_DEFAULT_LANE_SYMS 1024u /* one wavefront per 64 KiB chunk */
+
+typedef struct nz_manager nz_manager;
+
+int nz_abi_version(void);
+const char* nz_last_error(void);
+
+/* ---- sizes ------------------------------------------------------------ */
+
+/* Packed sign+mantissa bytes for n elements at `precision` kept mantissa
+   bits: (n * (precision + 1) + 7) / 8, cuda/high_level.cu:81-83. */
+uint64_t nz_packed_bytes(uint64_t n, int precision);
+
+/* Capacity that always holds the entropy-coded exponent container of n
+   elements (stands in for nvcomp's max_compressed_buffer_size,
+   cuda/high_level.cu:106-108).  0 for an unsupported geometry. */
+uint64_t nz_exp_bound_bytes(uint64_t n, uint32_t chunk_size, uint32_t lane_syms);
+
+/* Device scratch needed by nz_encode for n elements. */
+uint64_t nz_encode_workspace_bytes(uint64_t n, uint32_t chunk_size, uint32_t lane_syms);
+
+/* ---- stateless kernels ------------------------------------------------ */
+
+/* Manager::split, cuda/high_level.cu:265-321: unpacked exponent byte and
+   sign|mantissa byte per element, precision forced to 7 (:289). */
+int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fractions,
+             void* stream);
+
+/* Manager::_write_to_cache, cuda/high_level.cu:76-130: split, then entropy
+   code the exponents.  `dev_packed` receives nz_packed_bytes() bytes,
+   `dev_comp` (capacity comp_cap >= nz_exp_bound_bytes) the container.
+   `dev_total` (device uint64) receives the container size, `dev_status`
+   (device uint32, OR-ed into) is non-zero on overflow.  If `host_total` is
+   not NULL the call synchronises the stream and returns the size and status
+   on the host (the reference's get_compressed_output_size sync, :114-115). */
+int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
+              uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
+              void* dev_workspace, uint64_t workspace_bytes, uint64_t* dev_total,
+              uint32_t* dev_status, uint64_t* host_total, void* stream);
+
+/* Manager::_decompress_and_merge, cuda/high_level.cu:169-206: entropy decode
+   and merge in one kernel.  `dev_status` (device uint32, may be NULL) is
+   OR-ed with a non-zero value when the container fails validation; with
+   `check` != 0 the call synchronises and returns NZ_ERR_CORRUPT in that
+   case.  chunk_size / lane_syms must be the ones used to encode. */
+int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed, uint64_t n,
+              int precision, uint32_t chunk_size, uint32_t lane_syms, void* dev_bf16_out,
+              uint32_t* dev_status, int check, void* stream);
+
+/* ---- handle store: template struct Manager, cuda/high_level.cu:26-322 -- */
+
+/* Manager(algorithm, chunk_size) for the class Manager_f{precision}_n{normalizer_size}
+   (cuda/neuzip.cu:19-38, neuzip/binding.py:69-70).  precision in {0,1,3,7};
+   normalizer_size must be 0 (block normalizers are not implemented);
+   lane_syms 0 selects NZ_DEFAULT_LANE_SYMS clipped to the chunk. */
+int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_t chunk_size,
+                      uint32_t lane_syms, nz_manager** out);
+void nz_manager_destroy(nz_manager* m);
+
+/* Manager::write(name, tensor), cuda/high_level.cu:132-162.  Replaces an
+   existing entry of the same name (:137-140).  Synchronises the stream once
+   to learn the compressed size (as the reference does, :114-115). */
+int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint64_t n,
+                     int dtype, void* stream);
+
+/* Manager::read(name), cuda/high_level.cu:223-250, into caller-owned memory of
+   at least `cap_elems` elements.  Asynchronous on `stream` (the reference
+   blocks the host here, :203; callers that need that call hipStreamSynchronize). */
+int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap_elems,
+                    void* stream);
+
+/* meta_cache lookup, cuda/high_level.cu:42-43,228-230. */
+int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype);
+
+/* Manager::size(name), cuda/high_level.cu:208-221: bytes held for the entry
+   (entropy-coded exponents + packed sign/mantissa); 0 if unknown. */
+uint64_t nz_manager_size(nz_manager* m, const char* name);
+
+/* Bytes of the exponent container alone / of the packed stream alone. */
+uint64_t nz_manager_exp_bytes(nz_manager* m, const char* name);
+uint64_t nz_manager_packed_bytes(nz_manager* m, const char* name);
+
+/* Raw device pointers of an entry (valid until it is rewritten or erased). */
+int nz_manager_buffers(nz_manager* m, const char* name, const void** dev_comp,
+                       uint64_t* comp_bytes, const void** dev_packed, uint64_t* packed_bytes);
+
+/* compress_cache.erase(name), cuda/high_level.cu:137-140. */
+int nz_manager_erase(nz_manager* m, const char* name);
+
+/* Synchronise `stream` and report NZ_ERR_CORRUPT if any read since the last
+   check saw a container that failed validation. */
+int nz_manager_check(nz_manager* m, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,220 @@
+"""Python façade of the codec: ``Manager`` and ``Algorithm``.
+
+Same surface as the reference's neuzip/binding.py:23-115 (constructor
+arguments, method names, handle strings, return shapes); the backend is the
+C ABI of libneuzip_hip.so instead of the pybind11 classes
+``neuzip._cuda.Manager_f{precision}_n{normalizer_size}``.
+"""
+from __future__ import annotations
+
+import ctypes
+import enum
+from typing import Optional
+
+import torch
+
+from neuzip_amd import _lib
+from neuzip_amd.utils import _convert
+
+_lib.load()  # hard failure when the extension is not built (reference: binding.py:15-20)
+
+
+class Algorithm(enum.Enum):
+    # neuzip/binding.py:23-27.  Only ANS has a native implementation here.
+    ans = 0
+    gdeflate = "gdeflate"
+    zstd = "zstd"
+    dummy = "dummy"
+
+
+_VALID_NORMALIZERS = (0, 1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024)  # cuda/neuzip.cu:47-105
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class _HipBackend:
+    """Backend object with the method set of the reference's C++ Manager
+    (cuda/neuzip.cu:28-37): read / write / size / linear / linear_without_bias / split."""
+
+    def __init__(self, precision: int, normalizer_size: int, chunk_size: int, lane_symbols: int):
+        self._L = _lib.load()
+        self._h = ctypes.c_void_p()
+        rc = self._L.nz_manager_create(_lib.ALGO_ANS, precision, normalizer_size, chunk_size,
+                                       lane_symbols, ctypes.byref(self._h))
+        _lib.raise_for(rc)
+        self._device = torch.device("cuda", torch.cuda.current_device())
+
+    def close(self):
+        if getattr(self, "_h", None) is not None and self._h:
+            self._L.nz_manager_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @staticmethod
+    def _dtype_code(t: torch.Tensor) -> int:
+        if t.dtype == torch.bfloat16:
+            return _lib.DTYPE_BF16
+        # cuda/high_level.cu:159-161
+        raise RuntimeError("Unsupported data type")
+
+    def write(self, handle: str, tensor: torch.Tensor) -> None:
+        if not tensor.is_cuda:  # cuda/high_level.cu:133-135
+            tensor = tensor.to(self._device)
+        code = self._dtype_code(tensor)
+        flat = tensor.detach().contiguous().view(-1)
+        if flat.data_ptr() % 16:
+            flat = flat.clone()
+        rc = self._L.nz_manager_write(self._h, handle.encode(), flat.data_ptr(), flat.numel(), code,
+                                      _stream_ptr(flat.device))
+        _lib.raise_for(rc)
+
+    def read(self, handle: str) -> torch.Tensor:
+        n = ctypes.c_uint64()
+        dt = ctypes.c_int()
+        _lib.raise_for(self._L.nz_manager_meta(self._h, handle.encode(), ctypes.byref(n), ctypes.byref(dt)))
+        out = torch.empty(n.value, dtype=torch.bfloat16, device=self._device)
+        rc = self._L.nz_manager_read(self._h, handle.encode(), out.data_ptr(), n.value,
+                                     _stream_ptr(self._device))
+        _lib.raise_for(rc)
+        return out
+
+    def size(self, handle: str) -> int:
+        return int(self._L.nz_manager_size(self._h, handle.encode()))
+
+    def exp_bytes(self, handle: str) -> int:
+        return int(self._L.nz_manager_exp_bytes(self._h, handle.encode()))
+
+    def packed_bytes(self, handle: str) -> int:
+        return int(self._L.nz_manager_packed_bytes(self._h, handle.encode()))
+
+    def check(self) -> None:
+        _lib.raise_for(self._L.nz_manager_check(self._h, _stream_ptr(self._device)))
+
+    def linear(self, handle: str, inputs: torch.Tensor, shape, bias: torch.Tensor) -> torch.Tensor:
+        # cuda/high_level.cu:252-257: addmm(bias, input, W^T) on a 2-D input
+        weight = self.read(handle).view(shape)
+        return torch.addmm(bias, inputs, weight.t())
+
+    def linear_without_bias(self, handle: str, inputs: torch.Tensor, shape) -> torch.Tensor:
+        # cuda/high_level.cu:259-263
+        weight = self.read(handle).view(shape)
+        return torch.matmul(inputs, weight.t())
+
+    def split(self, tensor: torch.Tensor):
+        if not tensor.is_cuda:  # cuda/high_level.cu:302-304
+            tensor = tensor.to(self._device)
+        self._dtype_code(tensor)
+        flat = tensor.detach().contiguous().view(-1)
+        if flat.data_ptr() % 16:
+            flat = flat.clone()
+        n = flat.numel()
+        exps = torch.empty(n, dtype=torch.uint8, device=flat.device)
+        fracs = torch.empty(n, dtype=torch.uint8, device=flat.device)
+        rc = self._L.nz_split(flat.data_ptr(), n, exps.data_ptr(), fracs.data_ptr(), _stream_ptr(flat.device))
+        _lib.raise_for(rc)
+        return [exps, fracs]
+
+
+class _DenseBackend:
+    """Uncompressed pass-through selected by ``Algorithm.dummy``
+    (the reference's DummyBackend, neuzip/binding.py:35-52)."""
+
+    def __init__(self):
+        self._store = {}
+
+    def write(self, handle: str, tensor: torch.Tensor) -> None:
+        self._store[handle] = tensor.cuda()
+
+    def read(self, handle: str) -> torch.Tensor:
+        return self._store[handle]
+
+    def size(self, handle: str) -> int:
+        t = self._store[handle]
+        return t.numel() * t.element_size()
+
+    def linear(self, handle: str, inputs: torch.Tensor, shape, bias=None) -> torch.Tensor:
+        with torch.no_grad():
+            return torch.nn.functional.linear(inputs, self.read(handle).reshape(shape), bias)
+
+    linear_without_bias = linear
+
+
+class Manager:
+    """Handle-keyed store of compressed tensors (neuzip/binding.py:55-115).
+
+    ``write`` returns the handle (auto-numbered ``"0"``, ``"1"``, ... when none
+    is given), ``read`` hands back a fresh dense tensor of the original shape,
+    ``linear`` computes ``x @ W^T (+ b)`` against the stored weight and
+    ``convert`` swaps the Linear layers of a model in place.
+    """
+
+    def __init__(
+        self,
+        algorithm: Algorithm = Algorithm.ans,
+        precision: int = 7,
+        normalizer_size=None,
+        chunk_size=2**16,
+        lane_symbols: int = 0,
+    ) -> None:
+        """``lane_symbols`` (extension; 0 = library default) is the number of
+        exponents each of the 64 rANS lanes of a wavefront codes per segment:
+        smaller values expose more wavefronts per chunk at the price of 32 bits
+        of coder state per lane and segment."""
+        normalizer_size = 0 if normalizer_size is None else normalizer_size
+        self.meta_dict = {}  # handle -> original shape
+        if algorithm == Algorithm.dummy:
+            self._be = _DenseBackend()
+            return
+        if algorithm != Algorithm.ans:
+            # the reference builds an nvcomp manager for these (cuda/high_level.cu:52-65);
+            # nvcomp does not exist on this platform
+            raise RuntimeError("Unsupported algorithm")
+        if precision not in (0, 1, 3, 7) or normalizer_size not in _VALID_NORMALIZERS:
+            # the reference resolves a class by name and fails the same way (binding.py:69-70)
+            raise AttributeError(
+                f"module 'neuzip._cuda' has no attribute 'Manager_f{precision}_n{normalizer_size}'"
+            )
+        if normalizer_size != 0:
+            raise NotImplementedError("block normalizers (normalizer_size > 0) are not implemented")
+        self._be = _HipBackend(precision, normalizer_size, chunk_size, lane_symbols)
+
+    # -- store ---------------------------------------------------------------
+    def write(self, tensor: torch.Tensor, handle: Optional[str] = None) -> str:
+        key = str(len(self.meta_dict)) if handle is None else handle
+        self.meta_dict[key] = tensor.shape
+        self._be.write(key, tensor)  # note the argument order of the backend
+        return key
+
+    def read(self, handle: str) -> torch.Tensor:
+        shape = self.meta_dict[handle]  # KeyError for an unknown handle, as in the reference
+        flat = self._be.read(handle)
+        return flat.requires_grad_(False).reshape(shape)
+
+    def size(self, handle: str) -> int:
+        return self._be.size(handle)
+
+    def linear(self, handle: str, inputs: torch.Tensor, bias=None) -> torch.Tensor:
+        shape = self.meta_dict[handle]
+        if bias is None:
+            return self._be.linear_without_bias(handle, inputs, shape)
+        return self._be.linear(handle, inputs, shape, bias)
+
+    # -- helpers -------------------------------------------------------------
+    def convert(self, module: torch.nn.Module) -> torch.nn.Module:
+        return _convert(self, module)
+
+    def split(self, tensor: torch.Tensor):
+        exp, frac = self._be.split(tensor)
+        return exp.reshape(tensor.shape), frac.reshape(tensor.shape)
+
+    def __del__(self):
+        be = self.__dict__.get("_be")
+        if be is not None and hasattr(be, "close"):
+            be.close()

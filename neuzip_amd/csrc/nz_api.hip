@@ -1,0 +1,483 @@
+// Host side of libneuzip_hip.so: the C ABI declared in include/neuzip_hip.h.
+//
+// Stands in for the reference's `template struct Manager`
+// (cuda/high_level.cu:26-322) and its pybind11 surface (cuda/neuzip.cu:19-38).
+// No torch types, no private streams: every kernel goes to the caller's stream.
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+#include <string>
+#include <unordered_map>
+
+#include "../../include/neuzip_hip.h"
+#include "nz_kernels.hip"
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const std::string& msg) {
+  g_err = msg;
+  return code;
+}
+
+#define NZ_HIP(call)                                                                  \
+  do {                                                                                \
+    hipError_t e_ = (call);                                                           \
+    if (e_ != hipSuccess)                                                             \
+      return fail(NZ_ERR_HIP, std::string(#call) + ": " + hipGetErrorString(e_));     \
+  } while (0)
+
+inline uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+bool precision_ok(int p) { return p == 7 || p == 3 || p == 1 || p == 0; }
+
+// Device scratch of one encode call.
+struct EncLayout {
+  uint64_t exps, enc_tab, tab_ser, info, slots, states, seg_words, seg_units, hdr, total, status, bytes;
+};
+
+EncLayout enc_layout(const NzGeom& g) {
+  EncLayout L;
+  uint64_t o = 0;
+  auto take = [&](uint64_t b) {
+    uint64_t at = o;
+    o = align_up(o + b, 256);
+    return at;
+  };
+  L.exps = take(g.n + 16);
+  L.enc_tab = take(g.n_chunks * 256 * 4);
+  L.tab_ser = take(g.n_chunks * NZ_TABLE_MAX_BYTES);
+  L.info = take(g.n_chunks * sizeof(NzChunkInfo));
+  L.slots = take(g.n_segs * (uint64_t)g.seg_syms);  // seg_syms/2 words of 2 bytes
+  L.states = take(g.n_segs * NZ_LANES * 4);
+  L.seg_words = take(g.n_segs * 4);
+  L.seg_units = take((g.n_segs + 1) * 4);
+  L.hdr = take(g.rec_off);
+  L.total = take(8);
+  L.status = take(4);
+  L.bytes = o;
+  return L;
+}
+
+template <int S>
+void launch_split_hist(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws,
+                       const EncLayout& L, hipStream_t st) {
+  hipLaunchKernelGGL(nz_split_hist_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(256), 0, st,
+                     (const uint16_t*)in, g.n, g.chunk_syms, packed, ws + L.exps,
+                     (uint32_t*)(ws + L.enc_tab), ws + L.tab_ser, (NzChunkInfo*)(ws + L.info));
+}
+
+// Phase 1: everything up to the directory.  Header + directory land in `hdr`
+// (g.rec_off bytes), the container size in *d_total.
+int encode_phase1(const NzGeom& g, int precision, const void* in, uint8_t* packed, uint8_t* ws,
+                  const EncLayout& L, uint8_t* hdr, uint64_t cap, uint64_t* d_total,
+                  uint32_t* d_status, hipStream_t st) {
+  if (g.n_chunks > 0) {
+    switch (precision) {
+      case 7: launch_split_hist<7>(g, in, packed, ws, L, st); break;
+      case 3: launch_split_hist<3>(g, in, packed, ws, L, st); break;
+      case 1: launch_split_hist<1>(g, in, packed, ws, L, st); break;
+      default: launch_split_hist<0>(g, in, packed, ws, L, st); break;
+    }
+    hipLaunchKernelGGL(nz_rans_encode_kernel, dim3((uint32_t)g.n_chunks), dim3(64 * g.spc), 0, st,
+                       ws + L.exps, g.n, g.chunk_syms, g.lane_syms, g.spc,
+                       (const uint32_t*)(ws + L.enc_tab), (const NzChunkInfo*)(ws + L.info),
+                       (uint16_t*)(ws + L.slots), (uint32_t*)(ws + L.states),
+                       (uint32_t*)(ws + L.seg_words));
+    hipLaunchKernelGGL(nz_chunk_finalize_kernel, dim3((uint32_t)((g.n_chunks + 255) / 256)),
+                       dim3(256), 0, st, g.n, g.chunk_syms, g.seg_syms, g.spc, g.n_chunks,
+                       (NzChunkInfo*)(ws + L.info), (const uint32_t*)(ws + L.seg_words),
+                       (uint32_t*)(ws + L.seg_units));
+  }
+  hipLaunchKernelGGL(nz_scan_kernel, dim3(1), dim3(1024), 0, st,
+                     (const uint32_t*)(ws + L.seg_units), g, hdr, cap, d_total, d_status);
+  NZ_HIP(hipGetLastError());
+  return NZ_OK;
+}
+
+// Phase 2: place the records behind a header/directory already at `comp`.
+int encode_phase2(const NzGeom& g, uint8_t* ws, const EncLayout& L, const uint32_t* dir,
+                  uint8_t* comp, uint64_t cap, hipStream_t st) {
+  if (g.n_segs > 0) {
+    hipLaunchKernelGGL(nz_compact_kernel, dim3((uint32_t)g.n_segs), dim3(256), 0, st,
+                       ws + L.exps, g, (const NzChunkInfo*)(ws + L.info), ws + L.tab_ser,
+                       (const uint16_t*)(ws + L.slots), (const uint32_t*)(ws + L.states),
+                       (const uint32_t*)(ws + L.seg_words), dir, comp, cap);
+    NZ_HIP(hipGetLastError());
+  }
+  return NZ_OK;
+}
+
+template <int S>
+void launch_decode(const NzGeom& g, const void* comp, uint64_t comp_bytes, const void* packed,
+                   void* out, uint32_t* d_status, hipStream_t st) {
+  const size_t lds = (NZ_M + g.spc * NZ_RING_DWORDS + 384) * 4;
+  hipLaunchKernelGGL(nz_decode_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(64 * g.spc), lds, st,
+                     (const uint8_t*)comp, comp_bytes, (const uint8_t*)packed, (uint16_t*)out, g,
+                     d_status);
+}
+
+int decode_launch(const NzGeom& g, int precision, const void* comp, uint64_t comp_bytes,
+                  const void* packed, void* out, uint32_t* d_status, hipStream_t st) {
+  if (g.n_chunks == 0) return NZ_OK;
+  switch (precision) {
+    case 7: launch_decode<7>(g, comp, comp_bytes, packed, out, d_status, st); break;
+    case 3: launch_decode<3>(g, comp, comp_bytes, packed, out, d_status, st); break;
+    case 1: launch_decode<1>(g, comp, comp_bytes, packed, out, d_status, st); break;
+    default: launch_decode<0>(g, comp, comp_bytes, packed, out, d_status, st); break;
+  }
+  NZ_HIP(hipGetLastError());
+  return NZ_OK;
+}
+
+int make_geom(NzGeom* g, uint64_t n, uint32_t chunk, uint32_t lane_syms) {
+  if (nz_geom_make(g, n, chunk, lane_syms))
+    return fail(NZ_ERR_ARG,
+                "unsupported geometry: lane_syms must be a multiple of 8 and chunk_size a "
+                "multiple of 64*lane_syms holding 1..8 segments");
+  if (g->n_chunks > 0x7FFFFFFFull) return fail(NZ_ERR_ARG, "tensor too large");
+  return NZ_OK;
+}
+
+struct Entry {
+  void* comp = nullptr;
+  uint64_t comp_bytes = 0, comp_cap = 0;
+  void* packed = nullptr;
+  uint64_t packed_bytes = 0, packed_cap = 0;
+  uint64_t n = 0;
+  int dtype = NZ_DTYPE_BF16;
+};
+
+}  // namespace
+
+struct nz_manager {
+  int precision;
+  uint32_t chunk_syms, lane_syms;
+  std::unordered_map<std::string, Entry> entries;  // compress_cache + meta_cache
+  std::mutex mu;
+  void* ws = nullptr;
+  uint64_t ws_bytes = 0;
+  uint32_t* d_status = nullptr;
+  uint64_t* h_pin = nullptr;  // pinned: [0] total, [1] status
+};
+
+extern "C" {
+
+int nz_abi_version(void) { return 1; }
+
+const char* nz_last_error(void) { return g_err.c_str(); }
+
+uint64_t nz_packed_bytes(uint64_t n, int precision) { return nz_packed_bytes_of(n, precision); }
+
+uint64_t nz_exp_bound_bytes(uint64_t n, uint32_t chunk_size, uint32_t lane_syms) {
+  NzGeom g;
+  if (nz_geom_make(&g, n, chunk_size, lane_syms)) return 0;
+  return nz_geom_bound(&g);
+}
+
+uint64_t nz_encode_workspace_bytes(uint64_t n, uint32_t chunk_size, uint32_t lane_syms) {
+  NzGeom g;
+  if (nz_geom_make(&g, n, chunk_size, lane_syms)) return 0;
+  return enc_layout(g).bytes;
+}
+
+int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fractions,
+             void* stream) {
+  if (n == 0) return NZ_OK;
+  if (!dev_bf16 || !dev_exponents || !dev_fractions) return fail(NZ_ERR_ARG, "null pointer");
+  if (((uintptr_t)dev_bf16 & 15) || ((uintptr_t)dev_exponents & 7) || ((uintptr_t)dev_fractions & 7))
+    return fail(NZ_ERR_ALIGN, "nz_split: pointers must be 16-byte (input) / 8-byte (outputs) aligned");
+  const uint64_t blocks = (n + 2047) / 2048;
+  if (blocks > 0x7FFFFFFFull) return fail(NZ_ERR_ARG, "tensor too large");
+  hipLaunchKernelGGL(nz_split_unpacked_kernel, dim3((uint32_t)blocks), dim3(256), 0,
+                     (hipStream_t)stream, (const uint16_t*)dev_bf16, n, (uint8_t*)dev_exponents,
+                     (uint8_t*)dev_fractions);
+  NZ_HIP(hipGetLastError());
+  return NZ_OK;
+}
+
+int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
+              uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
+              void* dev_workspace, uint64_t workspace_bytes, uint64_t* dev_total,
+              uint32_t* dev_status, uint64_t* host_total, void* stream) {
+  if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
+  NzGeom g;
+  if (int rc = make_geom(&g, n, chunk_size, lane_syms)) return rc;
+  if (!dev_comp || !dev_workspace || !dev_total || !dev_status || (n && (!dev_bf16 || !dev_packed)))
+    return fail(NZ_ERR_ARG, "null pointer");
+  if ((uintptr_t)dev_bf16 & 15) return fail(NZ_ERR_ALIGN, "dense input must be 16-byte aligned");
+  if (((uintptr_t)dev_packed & 7) || ((uintptr_t)dev_comp & 15) || ((uintptr_t)dev_workspace & 255))
+    return fail(NZ_ERR_ALIGN, "packed/comp/workspace buffers must be 8/16/256-byte aligned");
+  const EncLayout L = enc_layout(g);
+  if (workspace_bytes < L.bytes) return fail(NZ_ERR_CAPACITY, "workspace too small");
+  if (comp_cap < nz_geom_bound(&g)) return fail(NZ_ERR_CAPACITY, "dev_comp smaller than nz_exp_bound_bytes");
+  hipStream_t st = (hipStream_t)stream;
+  uint8_t* ws = (uint8_t*)dev_workspace;
+  if (int rc = encode_phase1(g, precision, dev_bf16, (uint8_t*)dev_packed, ws, L, (uint8_t*)dev_comp,
+                             comp_cap, dev_total, dev_status, st))
+    return rc;
+  if (int rc = encode_phase2(g, ws, L, (const uint32_t*)((uint8_t*)dev_comp + g.dir_off),
+                             (uint8_t*)dev_comp, comp_cap, st))
+    return rc;
+  if (host_total) {
+    uint32_t hs = 0;
+    NZ_HIP(hipMemcpyAsync(host_total, dev_total, 8, hipMemcpyDeviceToHost, st));
+    NZ_HIP(hipMemcpyAsync(&hs, dev_status, 4, hipMemcpyDeviceToHost, st));
+    NZ_HIP(hipStreamSynchronize(st));
+    if (hs & 1u) return fail(NZ_ERR_CAPACITY, "encoded container exceeds the output capacity");
+  }
+  return NZ_OK;
+}
+
+int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed, uint64_t n,
+              int precision, uint32_t chunk_size, uint32_t lane_syms, void* dev_bf16_out,
+              uint32_t* dev_status, int check, void* stream) {
+  if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
+  NzGeom g;
+  if (int rc = make_geom(&g, n, chunk_size, lane_syms)) return rc;
+  if (n == 0) return NZ_OK;
+  if (!dev_comp || !dev_packed || !dev_bf16_out) return fail(NZ_ERR_ARG, "null pointer");
+  if ((uintptr_t)dev_bf16_out & 15) return fail(NZ_ERR_ALIGN, "dense output must be 16-byte aligned");
+  if (((uintptr_t)dev_comp & 15) || ((uintptr_t)dev_packed & 7))
+    return fail(NZ_ERR_ALIGN, "comp/packed buffers must be 16/8-byte aligned");
+  if (check && !dev_status) return fail(NZ_ERR_ARG, "check requires dev_status");
+  if (comp_bytes < g.rec_off) return fail(NZ_ERR_CORRUPT, "container shorter than its directory");
+  hipStream_t st = (hipStream_t)stream;
+  if (int rc = decode_launch(g, precision, dev_comp, comp_bytes, dev_packed, dev_bf16_out, dev_status, st))
+    return rc;
+  if (check) {
+    uint32_t hs = 0;
+    NZ_HIP(hipMemcpyAsync(&hs, dev_status, 4, hipMemcpyDeviceToHost, st));
+    NZ_HIP(hipStreamSynchronize(st));
+    if (hs) return fail(NZ_ERR_CORRUPT, "compressed container failed validation (status " + std::to_string(hs) + ")");
+  }
+  return NZ_OK;
+}
+
+// ---------------------------------------------------------------------------
+// handle store
+// ---------------------------------------------------------------------------
+
+int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_t chunk_size,
+                      uint32_t lane_syms, nz_manager** out) {
+  if (!out) return fail(NZ_ERR_ARG, "null out pointer");
+  if (algorithm != NZ_ALGO_ANS) return fail(NZ_ERR_ALGO, "Unsupported algorithm");
+  if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
+  if (normalizer_size != 0) return fail(NZ_ERR_ARG, "block normalizers are not implemented (normalizer_size must be 0)");
+  if (lane_syms == 0) {
+    lane_syms = NZ_DEFAULT_LANE_SYMS;
+    while (lane_syms > 8 && (uint64_t)lane_syms * NZ_LANES > chunk_size) lane_syms /= 2;
+    while ((uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size) lane_syms *= 2;
+  }
+  NzGeom g;
+  if (int rc = make_geom(&g, 0, chunk_size, lane_syms)) return rc;
+  nz_manager* m = new nz_manager();
+  m->precision = precision;
+  m->chunk_syms = chunk_size;
+  m->lane_syms = lane_syms;
+  hipError_t e = hipMalloc((void**)&m->d_status, 256);
+  if (e == hipSuccess) e = hipMemset(m->d_status, 0, 256);
+  if (e == hipSuccess) e = hipHostMalloc((void**)&m->h_pin, 64, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    if (m->d_status) (void)hipFree(m->d_status);
+    delete m;
+    return fail(NZ_ERR_HIP, std::string("nz_manager_create: ") + hipGetErrorString(e));
+  }
+  *out = m;
+  return NZ_OK;
+}
+
+void nz_manager_destroy(nz_manager* m) {
+  if (!m) return;
+  for (auto& kv : m->entries) {
+    if (kv.second.comp) (void)hipFree(kv.second.comp);
+    if (kv.second.packed) (void)hipFree(kv.second.packed);
+  }
+  if (m->ws) (void)hipFree(m->ws);
+  if (m->d_status) (void)hipFree(m->d_status);
+  if (m->h_pin) (void)hipHostFree(m->h_pin);
+  delete m;
+}
+
+int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint64_t n, int dtype,
+                     void* stream) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  if (dtype != NZ_DTYPE_BF16) return fail(NZ_ERR_DTYPE, "Unsupported data type");
+  if (n && !dev_data) return fail(NZ_ERR_ARG, "null data pointer");
+  if ((uintptr_t)dev_data & 15) return fail(NZ_ERR_ALIGN, "dense input must be 16-byte aligned");
+  NzGeom g;
+  if (int rc = make_geom(&g, n, m->chunk_syms, m->lane_syms)) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  std::lock_guard<std::mutex> lock(m->mu);
+
+  const EncLayout L = enc_layout(g);
+  if (m->ws_bytes < L.bytes) {
+    // the previous scratch may still be in use by kernels on the stream
+    NZ_HIP(hipStreamSynchronize(st));
+    if (m->ws) NZ_HIP(hipFree(m->ws));
+    m->ws = nullptr;
+    m->ws_bytes = 0;
+    NZ_HIP(hipMalloc(&m->ws, L.bytes));
+    m->ws_bytes = L.bytes;
+  }
+  uint8_t* ws = (uint8_t*)m->ws;
+
+  // cuda/high_level.cu:137-140: an existing entry is replaced.  Its buffers are
+  // reused when large enough, which also avoids a device-wide hipFree stall.
+  Entry old;
+  auto it = m->entries.find(name);
+  if (it != m->entries.end()) {
+    old = it->second;
+    m->entries.erase(it);
+  }
+  Entry ent;
+  ent.n = n;
+  ent.dtype = dtype;
+  ent.packed_bytes = nz_packed_bytes_of(n, m->precision);
+  auto release = [&](Entry& e) {
+    if (e.comp) (void)hipFree(e.comp);
+    if (e.packed) (void)hipFree(e.packed);
+    e.comp = e.packed = nullptr;
+  };
+  if (old.packed && old.packed_cap >= ent.packed_bytes && old.packed_cap <= ent.packed_bytes + 4096) {
+    ent.packed = old.packed;
+    ent.packed_cap = old.packed_cap;
+    old.packed = nullptr;
+  } else {
+    ent.packed_cap = ent.packed_bytes ? ent.packed_bytes : 8;
+    hipError_t e = hipMalloc(&ent.packed, ent.packed_cap);
+    if (e != hipSuccess) {
+      release(old);
+      return fail(NZ_ERR_HIP, std::string("hipMalloc(packed): ") + hipGetErrorString(e));
+    }
+  }
+
+  uint64_t* d_total = (uint64_t*)(ws + L.total);
+  uint32_t* d_estat = (uint32_t*)(ws + L.status);
+  hipError_t e = hipMemsetAsync(d_estat, 0, 4, st);
+  int rc = e == hipSuccess ? NZ_OK : fail(NZ_ERR_HIP, hipGetErrorString(e));
+  if (rc == NZ_OK)
+    rc = encode_phase1(g, m->precision, dev_data, (uint8_t*)ent.packed, ws, L, ws + L.hdr,
+                       ~0ull, d_total, d_estat, st);
+  if (rc == NZ_OK) {
+    e = hipMemcpyAsync(m->h_pin, d_total, 8, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);  // the one host sync of a write
+    if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("size readback: ") + hipGetErrorString(e));
+  }
+  if (rc == NZ_OK) {
+    ent.comp_bytes = m->h_pin[0];
+    if (old.comp && old.comp_cap >= ent.comp_bytes && old.comp_cap <= ent.comp_bytes + ent.comp_bytes / 16 + 4096) {
+      ent.comp = old.comp;
+      ent.comp_cap = old.comp_cap;
+      old.comp = nullptr;
+    } else {
+      ent.comp_cap = ent.comp_bytes;
+      e = hipMalloc(&ent.comp, ent.comp_cap);
+      if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("hipMalloc(comp): ") + hipGetErrorString(e));
+    }
+  }
+  if (rc == NZ_OK) {
+    e = hipMemcpyAsync(ent.comp, ws + L.hdr, g.rec_off, hipMemcpyDeviceToDevice, st);
+    if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("header copy: ") + hipGetErrorString(e));
+  }
+  if (rc == NZ_OK)
+    rc = encode_phase2(g, ws, L, (const uint32_t*)(ws + L.hdr + g.dir_off), (uint8_t*)ent.comp,
+                       ent.comp_cap, st);
+  release(old);
+  if (rc != NZ_OK) {
+    release(ent);
+    return rc;
+  }
+  m->entries.emplace(name, ent);
+  return NZ_OK;
+}
+
+int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap_elems,
+                    void* stream) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  const Entry& ent = it->second;
+  if (cap_elems < ent.n) return fail(NZ_ERR_CAPACITY, "output smaller than the stored tensor");
+  if (ent.n == 0) return NZ_OK;
+  if (!dev_out) return fail(NZ_ERR_ARG, "null output pointer");
+  if ((uintptr_t)dev_out & 15) return fail(NZ_ERR_ALIGN, "dense output must be 16-byte aligned");
+  NzGeom g;
+  if (int rc = make_geom(&g, ent.n, m->chunk_syms, m->lane_syms)) return rc;
+  return decode_launch(g, m->precision, ent.comp, ent.comp_bytes, ent.packed, dev_out, m->d_status,
+                       (hipStream_t)stream);
+}
+
+int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  if (numel) *numel = it->second.n;
+  if (dtype) *dtype = it->second.dtype;
+  return NZ_OK;
+}
+
+uint64_t nz_manager_size(nz_manager* m, const char* name) {
+  if (!m || !name) return 0;
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  if (it == m->entries.end()) return 0;  // cuda/high_level.cu:209-211
+  return it->second.comp_bytes + it->second.packed_bytes;
+}
+
+uint64_t nz_manager_exp_bytes(nz_manager* m, const char* name) {
+  if (!m || !name) return 0;
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  return it == m->entries.end() ? 0 : it->second.comp_bytes;
+}
+
+uint64_t nz_manager_packed_bytes(nz_manager* m, const char* name) {
+  if (!m || !name) return 0;
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  return it == m->entries.end() ? 0 : it->second.packed_bytes;
+}
+
+int nz_manager_buffers(nz_manager* m, const char* name, const void** dev_comp, uint64_t* comp_bytes,
+                       const void** dev_packed, uint64_t* packed_bytes) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  if (dev_comp) *dev_comp = it->second.comp;
+  if (comp_bytes) *comp_bytes = it->second.comp_bytes;
+  if (dev_packed) *dev_packed = it->second.packed;
+  if (packed_bytes) *packed_bytes = it->second.packed_bytes;
+  return NZ_OK;
+}
+
+int nz_manager_erase(nz_manager* m, const char* name) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  // kernels reading these buffers may still be in flight
+  NZ_HIP(hipDeviceSynchronize());
+  if (it->second.comp) (void)hipFree(it->second.comp);
+  if (it->second.packed) (void)hipFree(it->second.packed);
+  m->entries.erase(it);
+  return NZ_OK;
+}
+
+int nz_manager_check(nz_manager* m, void* stream) {
+  if (!m) return fail(NZ_ERR_ARG, "null manager");
+  hipStream_t st = (hipStream_t)stream;
+  std::lock_guard<std::mutex> lock(m->mu);
+  NZ_HIP(hipMemcpyAsync(&m->h_pin[1], m->d_status, 4, hipMemcpyDeviceToHost, st));
+  NZ_HIP(hipMemsetAsync(m->d_status, 0, 4, st));
+  NZ_HIP(hipStreamSynchronize(st));
+  const uint32_t hs = (uint32_t)m->h_pin[1];
+  if (hs) return fail(NZ_ERR_CORRUPT, "a read saw a container that failed validation (status " + std::to_string(hs) + ")");
+  return NZ_OK;
+}
+
+}  // extern "C"

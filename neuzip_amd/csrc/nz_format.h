@@ -1,0 +1,93 @@
+// Container geometry shared by the host API and the gfx950 kernels.
+//
+// The exponent stream of one tensor (N bytes, one per bf16 element) is stored
+// as
+//
+//   header (64 B) | directory ((n_segs + 1) x u32) | segment records
+//
+// * chunk   = `chunk_syms` consecutive exponents that share one 12-bit
+//             frequency table (the reference hands nvcomp the same unit:
+//             chunk_size = 65536, cuda/neuzip.cu:31).
+// * segment = 64 * `lane_syms` consecutive exponents decoded by ONE wavefront:
+//             64 interleaved rANS states, lane l owning the 8-symbol groups
+//             (g * 64 + l) * 8 + j.  A chunk holds 1..8 segments.
+// * directory entry k = offset of segment k's record in 4-byte units from
+//             `rec_off`; entry n_segs = end of the last record.
+// * record  = [table, first segment of a chunk only] [64 x u32 final encoder
+//             states] [u16 renormalisation words, front-to-back in decode
+//             order] padded to 4 bytes; or, for a chunk whose coded form
+//             would not be smaller, [0xFF 0 0 0, first segment only] raw
+//             exponent bytes padded to 4.
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#define NZ_MAGIC 0x315A4E41u
+#define NZ_FORMAT_VERSION 1u
+#define NZ_PROB_BITS 12
+#define NZ_M (1u << NZ_PROB_BITS)
+#define NZ_L (1u << 16)
+#define NZ_LANES 64
+#define NZ_GROUP 8
+#define NZ_GROUP_SYMS 512
+#define NZ_HEADER_BYTES 64
+#define NZ_MODE_RAW 0xFF
+#define NZ_MODE_BITMAP 0x00
+#define NZ_MAX_RUNS 15
+#define NZ_TABLE_MAX_BYTES 424 /* 1 + 32 + 384 rounded up to a multiple of 8 */
+#define NZ_MAX_SEGS_PER_CHUNK 8
+
+struct NzGeom {
+  uint64_t n;
+  uint32_t chunk_syms;
+  uint32_t lane_syms;
+  uint32_t seg_syms;
+  uint32_t spc;  // segments per chunk
+  uint64_t n_chunks;
+  uint64_t n_segs;
+  uint64_t dir_off;
+  uint64_t rec_off;
+};
+
+// Device-side per-chunk record produced by the split/histogram kernel.
+struct NzChunkInfo {
+  uint32_t tab_len;  // serialized table bytes (multiple of 4)
+  uint32_t pad_sym;  // most frequent symbol: stands in for elements past the end
+  uint32_t raw;      // 1 when the chunk is stored raw
+  uint32_t reserved;
+};
+
+static inline int nz_geom_check(uint32_t chunk_syms, uint32_t lane_syms) {
+  if (lane_syms < NZ_GROUP || (lane_syms % NZ_GROUP) != 0 || lane_syms > (1u << 16)) return -1;
+  uint64_t seg = (uint64_t)lane_syms * NZ_LANES;
+  if (chunk_syms == 0 || (chunk_syms % seg) != 0) return -1;
+  uint64_t spc = chunk_syms / seg;
+  if (spc < 1 || spc > NZ_MAX_SEGS_PER_CHUNK) return -1;
+  if (chunk_syms > (1u << 24)) return -1;
+  return 0;
+}
+
+static inline int nz_geom_make(NzGeom* g, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms) {
+  if (nz_geom_check(chunk_syms, lane_syms)) return -1;
+  g->n = n;
+  g->chunk_syms = chunk_syms;
+  g->lane_syms = lane_syms;
+  g->seg_syms = lane_syms * NZ_LANES;
+  g->spc = chunk_syms / g->seg_syms;
+  g->n_chunks = (n + chunk_syms - 1) / chunk_syms;
+  g->n_segs = (n + g->seg_syms - 1) / g->seg_syms;
+  if (g->n_segs >= 0xFFFFFFFEull) return -1;
+  g->dir_off = NZ_HEADER_BYTES;
+  g->rec_off = (NZ_HEADER_BYTES + 4 * (g->n_segs + 1) + 15) & ~(uint64_t)15;
+  return 0;
+}
+
+// Upper bound of the container size: no chunk is ever stored larger than raw.
+static inline uint64_t nz_geom_bound(const NzGeom* g) {
+  return g->rec_off + g->n + 4 * g->n_segs + 4 * g->n_chunks;
+}
+
+static inline uint64_t nz_packed_bytes_of(uint64_t n, int s) {
+  return (n * (uint64_t)(s + 1) + 7) / 8;  // cuda/high_level.cu:81-83
+}

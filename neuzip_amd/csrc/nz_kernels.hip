@@ -1,0 +1,768 @@
+// gfx950 (CDNA4, wave64) kernels of the NeuZip bf16 codec.
+//
+//   nz_split_unpacked_kernel   Manager::split            cuda/high_level.cu:265-321
+//   nz_split_hist_kernel       kernel_aligned_split      cuda/kernels.cuh:62-156
+//                              + per-chunk exponent histogram, 12-bit frequency
+//                              table and its serialized form
+//   nz_rans_encode_kernel      nvcomp ANS compress       cuda/high_level.cu:103-115
+//   nz_chunk_finalize_kernel   \ exact-size compaction    cuda/high_level.cu:117-124
+//   nz_scan_kernel              > (done on the device, no host round trip
+//   nz_compact_kernel          /  between the kernels)
+//   nz_decode_kernel           nvcomp ANS decompress + kernel_aligned_merge fused:
+//                              cuda/high_level.cu:184-201, cuda/kernels.cuh:167-217
+//
+// The whole path is byte/integer work bound by HBM traffic; there is no dense
+// contraction, hence no MFMA.  One wavefront decodes one segment with 64
+// interleaved rANS states; the exponent never exists in HBM on the decode side.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "nz_format.h"
+
+#define NZ_RING_WORDS 2048u  // per-wave LDS ring of renormalisation words
+#define NZ_RING_DWORDS (NZ_RING_WORDS / 2)
+
+// ----------------------------------------------------------------------------
+// element-wise split / merge arithmetic
+// ----------------------------------------------------------------------------
+
+// Exponent byte and (sign | kept mantissa) field of one bf16 value.  This is the
+// closed form of cuda/kernels.cuh:122-137,153-155: round the 15-bit magnitude
+// half-up to S kept mantissa bits, the carry running into the exponent and the
+// exponent byte wrapping 255 -> 0 exactly like the reference's uint8 store.
+template <int S>
+__device__ __forceinline__ void nz_split_one(uint32_t v, uint32_t& exp, uint32_t& repr) {
+  if constexpr (S == 7) {
+    exp = (v >> 7) & 0xFFu;
+    repr = ((v >> 8) & 0x80u) | (v & 0x7Fu);
+  } else {
+    uint32_t a = ((v & 0x7FFFu) + (1u << (6 - S))) & 0x7FFFu;
+    exp = a >> 7;
+    repr = ((v >> 15) << S) | ((a >> (7 - S)) & ((1u << S) - 1u));
+  }
+}
+
+// Position of element j (0..7) of an 8-element group inside the group's S+1
+// packed bytes, MSB first (cuda/kernels.cuh:86-89): bit offset inside the
+// little-endian integer that holds those bytes.
+template <int S>
+__device__ __forceinline__ constexpr uint32_t nz_field_shift(int j) {
+  return 8u * ((uint32_t)(j * (S + 1)) >> 3) + (7u - S - ((uint32_t)(j * (S + 1)) & 7u));
+}
+
+// cuda/kernels.cuh:197-206 for a non-NaN result (the float multiply by +-1.0f of
+// :213-216 only moves the sign bit into place).
+template <int S>
+__device__ __forceinline__ uint32_t nz_merge_one(uint32_t exp, uint32_t repr) {
+  uint32_t frac = (repr & ((1u << S) - 1u)) << (7 - S);
+  uint32_t sign = (repr >> S) & 1u;
+  return (sign << 15) | (exp << 7) | frac;
+}
+
+__device__ __forceinline__ uint32_t nz_lane_id() {
+  return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+
+__device__ __forceinline__ uint32_t nz_rank_below(uint64_t mask) {
+  return __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32),
+                                   __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+}
+
+__device__ __forceinline__ uint32_t nz_get12(const uint8_t* p, uint32_t i) {
+  uint32_t bit = 12u * i;
+  const uint8_t* q = p + (bit >> 3);
+  uint32_t w = (uint32_t)q[0] | ((uint32_t)q[1] << 8);
+  return (w >> (bit & 4u)) & 0xFFFu;
+}
+
+// ----------------------------------------------------------------------------
+// Manager::split: unpacked exponent and sign|mantissa bytes, precision 7 always
+// (cuda/high_level.cu:289-296 forces f_bits_save = 7).
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void nz_split_unpacked_kernel(const uint16_t* __restrict__ in,
+                                                                uint64_t n,
+                                                                uint8_t* __restrict__ exps,
+                                                                uint8_t* __restrict__ fracs) {
+  uint64_t i0 = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (i0 >= n) return;
+  if (i0 + 8 <= n) {
+    uint4 v = *reinterpret_cast<const uint4*>(in + i0);
+    uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    uint64_t e = 0, f = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      uint32_t h = (w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu, ex, rp;
+      nz_split_one<7>(h, ex, rp);
+      e |= (uint64_t)ex << (8 * j);
+      f |= (uint64_t)rp << (8 * j);
+    }
+    *reinterpret_cast<uint64_t*>(exps + i0) = e;
+    *reinterpret_cast<uint64_t*>(fracs + i0) = f;
+  } else {
+    for (uint64_t i = i0; i < n; ++i) {
+      uint32_t ex, rp;
+      nz_split_one<7>(in[i], ex, rp);
+      exps[i] = (uint8_t)ex;
+      fracs[i] = (uint8_t)rp;
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------
+// split + histogram + table: one workgroup per chunk
+// ----------------------------------------------------------------------------
+
+__device__ __forceinline__ uint32_t nz_block_sum_256(uint32_t v, uint32_t* red) {
+  // 256 threads = 4 waves
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+
+__device__ __forceinline__ uint32_t nz_block_max_256(uint32_t v, uint32_t* red) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    uint32_t t = __shfl_xor(v, o, 64);
+    v = t > v ? t : v;
+  }
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  uint32_t a = red[0] > red[1] ? red[0] : red[1];
+  uint32_t b = red[2] > red[3] ? red[2] : red[3];
+  return a > b ? a : b;
+}
+
+template <int S>
+__global__ __launch_bounds__(256) void nz_split_hist_kernel(
+    const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms,
+    uint8_t* __restrict__ packed, uint8_t* __restrict__ exps, uint32_t* __restrict__ enc_tab,
+    uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info) {
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t freq_s[256];
+  __shared__ uint32_t red[4];
+  __shared__ uint32_t scan_s[4];
+
+  const uint32_t tid = threadIdx.x;
+  const uint64_t c = blockIdx.x;
+  const uint64_t base = c * chunk_syms;
+  const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
+
+  hist[tid] = 0;
+  __syncthreads();
+
+  for (uint32_t i = tid * 8; i < cn; i += 256 * 8) {
+    const uint64_t gi = base + i;
+    uint32_t ex[8], rp[8];
+    const uint32_t rem = cn - i;
+    if (rem >= 8) {
+      uint4 v = *reinterpret_cast<const uint4*>(in + gi);
+      uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) nz_split_one<S>((w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu, ex[j], rp[j]);
+      uint64_t e = 0, f = 0;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        e |= (uint64_t)ex[j] << (8 * j);
+        f |= (uint64_t)rp[j] << nz_field_shift<S>(j);
+      }
+      *reinterpret_cast<uint64_t*>(exps + gi) = e;
+      uint8_t* pp = packed + (gi * (S + 1)) / 8;
+      if constexpr (S == 7) *reinterpret_cast<uint64_t*>(pp) = f;
+      else if constexpr (S == 3) *reinterpret_cast<uint32_t*>(pp) = (uint32_t)f;
+      else if constexpr (S == 1) *reinterpret_cast<uint16_t*>(pp) = (uint16_t)f;
+      else *pp = (uint8_t)f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) atomicAdd(&hist[ex[j]], 1u);
+    } else {
+      // last elements of the tensor: missing ones contribute zero bits
+      // (cuda/kernels.cuh:92), and only ceil(rem*(S+1)/8) packed bytes exist.
+      uint64_t f = 0;
+      for (uint32_t j = 0; j < rem; ++j) {
+        nz_split_one<S>(in[gi + j], ex[0], rp[0]);
+        exps[gi + j] = (uint8_t)ex[0];
+        uint32_t bit = j * (S + 1);
+        f |= (uint64_t)rp[0] << (8u * (bit >> 3) + (7u - S - (bit & 7u)));
+        atomicAdd(&hist[ex[0]], 1u);
+      }
+      uint8_t* pp = packed + (gi * (S + 1)) / 8;
+      uint32_t nb = (rem * (S + 1) + 7) / 8;
+      for (uint32_t b = 0; b < nb; ++b) pp[b] = (uint8_t)(f >> (8 * b));
+    }
+  }
+  __syncthreads();
+
+  // ---- quantise the histogram to 12-bit frequencies (sum exactly 4096) ----
+  const uint32_t cnt = hist[tid];
+  const uint32_t live = cnt > 0;
+  const uint32_t k = nz_block_sum_256(live, red);
+  uint32_t f = live ? 1u + (uint32_t)(((uint64_t)cnt * (NZ_M - k)) / cn) : 0u;
+  const uint32_t sum = nz_block_sum_256(f, red);
+  // most frequent symbol, lowest index on ties (cnt <= 2^24 fits above the index byte)
+  const uint32_t key = nz_block_max_256((cnt << 8) | (255u - tid), red);
+  const uint32_t imax = 255u - (key & 0xFFu);
+  if (tid == imax) f += NZ_M - sum;
+  if (k == 1) f = (tid == imax) ? (NZ_M - 1) : ((tid == (imax ^ 1u)) ? 1u : 0u);
+  freq_s[tid] = f;
+
+  // exclusive prefix sum over the 256 symbols
+  uint32_t incl = f;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    uint32_t t = __shfl_up(incl, o, 64);
+    if ((tid & 63) >= (uint32_t)o) incl += t;
+  }
+  if ((tid & 63) == 63) scan_s[tid >> 6] = incl;
+  __syncthreads();
+  uint32_t woff = 0;
+  for (uint32_t w = 0; w < (tid >> 6); ++w) woff += scan_s[w];
+  const uint32_t cum = woff + incl - f;
+  enc_tab[c * 256 + tid] = (f << 16) | cum;
+
+  // ---- serialise the table (one thread; <= 256 short iterations) ----
+  if (tid == 0) {
+    uint8_t* out = tab_ser + c * NZ_TABLE_MAX_BYTES;
+    uint32_t runs = 0, kk = 0;
+    for (int i = 0; i < 256; ++i) {
+      if (freq_s[i]) {
+        ++kk;
+        if (i == 0 || !freq_s[i - 1]) ++runs;
+      }
+    }
+    uint32_t head;
+    if (runs >= 1 && runs <= NZ_MAX_RUNS) {
+      out[0] = (uint8_t)runs;
+      uint32_t r = 0;
+      int i = 0;
+      while (i < 256) {
+        if (freq_s[i]) {
+          int j = i;
+          while (j < 256 && freq_s[j]) ++j;
+          out[1 + 2 * r] = (uint8_t)i;
+          out[2 + 2 * r] = (uint8_t)(j - i - 1);
+          ++r;
+          i = j;
+        } else {
+          ++i;
+        }
+      }
+      head = 1 + 2 * runs;
+    } else {
+      out[0] = NZ_MODE_BITMAP;
+      for (int b = 0; b < 32; ++b) {
+        uint32_t m = 0;
+        for (int q = 0; q < 8; ++q) m |= (freq_s[8 * b + q] ? 1u : 0u) << q;
+        out[1 + b] = (uint8_t)m;
+      }
+      head = 33;
+    }
+    // 12-bit fields, two per three bytes
+    uint32_t j = 0, hold = 0;
+    uint8_t* fp = out + head;
+    for (int i = 0; i < 256; ++i) {
+      uint32_t fv = freq_s[i];
+      if (!fv) continue;
+      if ((j & 1) == 0) {
+        hold = fv;
+      } else {
+        uint32_t b0 = 3 * (j >> 1);
+        fp[b0] = (uint8_t)(hold & 0xFF);
+        fp[b0 + 1] = (uint8_t)((hold >> 8) | ((fv & 0xF) << 4));
+        fp[b0 + 2] = (uint8_t)(fv >> 4);
+      }
+      ++j;
+    }
+    if (j & 1) {
+      uint32_t b0 = 3 * (j >> 1);
+      fp[b0] = (uint8_t)(hold & 0xFF);
+      fp[b0 + 1] = (uint8_t)(hold >> 8);
+    }
+    uint32_t bytes = head + (12 * kk + 7) / 8;
+    uint32_t padded = (bytes + 3) & ~3u;
+    for (uint32_t b = bytes; b < padded; ++b) out[b] = 0;
+    NzChunkInfo ci;
+    ci.tab_len = padded;
+    ci.pad_sym = imax;
+    ci.raw = 0;
+    ci.reserved = 0;
+    info[c] = ci;
+  }
+}
+
+// ----------------------------------------------------------------------------
+// rANS encode: one workgroup per chunk, one wavefront per segment
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_kernel(
+    const uint8_t* __restrict__ exps, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
+    uint32_t spc, const uint32_t* __restrict__ enc_tab, const NzChunkInfo* __restrict__ info,
+    uint16_t* __restrict__ slots, uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words) {
+  __shared__ uint32_t tab[256];
+  const uint64_t c = blockIdx.x;
+  for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) tab[i] = enc_tab[c * 256 + i];
+  __syncthreads();
+
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t seg_syms = lane_syms * NZ_LANES;
+  const uint64_t seg = c * spc + wave;
+  const uint64_t seg_base = seg * seg_syms;
+  if (seg_base >= n) return;
+  const uint32_t seg_n = (uint32_t)((n - seg_base) < seg_syms ? (n - seg_base) : seg_syms);
+  const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
+  const uint32_t cap_words = seg_syms / 2;
+  const uint32_t pad = info[c].pad_sym;
+  uint16_t* slot = slots + seg * cap_words;
+  const uint8_t* src = exps + seg_base;
+
+  uint32_t x = NZ_L;
+  uint32_t pos = cap_words;
+  bool overflow = false;
+  for (uint32_t g = ngroups; g-- > 0 && !overflow;) {
+    const uint32_t idx0 = (g * NZ_LANES + lane) * NZ_GROUP;
+    uint64_t sy;
+    if (idx0 + 8 <= seg_n) {
+      sy = *reinterpret_cast<const uint64_t*>(src + idx0);
+    } else {
+      sy = 0;
+      for (int j = 0; j < 8; ++j) {
+        uint32_t b = (idx0 + j < seg_n) ? src[idx0 + j] : pad;
+        sy |= (uint64_t)b << (8 * j);
+      }
+    }
+#pragma unroll
+    for (int j = 7; j >= 0; --j) {
+      const uint32_t sym = (uint32_t)(sy >> (8 * j)) & 0xFFu;
+      const uint32_t e = tab[sym];
+      const uint32_t f = e >> 16, cum = e & 0xFFFFu;
+      const bool need = x >= (f << 20);
+      const uint64_t m = __ballot(need);
+      const uint32_t cnt = (uint32_t)__popcll(m);
+      if (cnt > pos) {
+        overflow = true;
+        break;
+      }
+      pos -= cnt;
+      if (need) {
+        slot[pos + nz_rank_below(m)] = (uint16_t)(x & 0xFFFFu);
+        x >>= 16;
+      }
+      const uint32_t q = x / f;
+      x = (q << NZ_PROB_BITS) + (x - q * f) + cum;
+    }
+  }
+  states[seg * NZ_LANES + lane] = x;
+  if (lane == 0) seg_words[seg] = overflow ? 0xFFFFFFFFu : (cap_words - pos);
+}
+
+// ----------------------------------------------------------------------------
+// per chunk: coded or raw, and the record size of each of its segments
+// ----------------------------------------------------------------------------
+__global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32_t seg_syms,
+                                         uint32_t spc, uint64_t n_chunks,
+                                         NzChunkInfo* __restrict__ info,
+                                         const uint32_t* __restrict__ seg_words,
+                                         uint32_t* __restrict__ seg_units) {
+  const uint64_t c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= n_chunks) return;
+  const uint64_t base = c * chunk_syms;
+  const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
+  const uint32_t nseg = (cn + seg_syms - 1) / seg_syms;
+  const uint32_t tab_len = info[c].tab_len;
+  uint64_t rans_total = tab_len, raw_total = 4;
+  bool overflow = false;
+  for (uint32_t k = 0; k < nseg; ++k) {
+    const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
+    const uint32_t w = seg_words[c * spc + k];
+    if (w == 0xFFFFFFFFu) overflow = true;
+    else rans_total += 256 + 2 * (uint64_t)((w + 1) & ~1u);
+    raw_total += (sn + 3) & ~3u;
+  }
+  const bool raw = overflow || rans_total >= raw_total;
+  info[c].raw = raw ? 1u : 0u;
+  for (uint32_t k = 0; k < nseg; ++k) {
+    const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
+    const uint32_t w = seg_words[c * spc + k];
+    uint32_t bytes;
+    if (raw) bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u);
+    else bytes = (k == 0 ? tab_len : 0u) + 256u + 2u * ((w + 1) & ~1u);
+    seg_units[c * spc + k] = bytes / 4;
+  }
+}
+
+// ----------------------------------------------------------------------------
+// exclusive scan of the record sizes -> directory, header, total size
+// (single workgroup; a tensor has at most a few hundred thousand segments)
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(1024) void nz_scan_kernel(const uint32_t* __restrict__ seg_units,
+                                                       NzGeom g, uint8_t* __restrict__ comp,
+                                                       uint64_t cap, uint64_t* __restrict__ d_total,
+                                                       uint32_t* __restrict__ d_status) {
+  // `comp` only needs room for the header and directory (g.rec_off bytes); the
+  // records are placed by nz_compact_kernel, possibly in another buffer.
+  __shared__ uint64_t wsum[16];
+  __shared__ uint64_t carry_s;
+  uint32_t* dir = reinterpret_cast<uint32_t*>(comp + g.dir_off);
+  const uint32_t tid = threadIdx.x;
+  if (tid == 0) carry_s = 0;
+  __syncthreads();
+  for (uint64_t start = 0; start < g.n_segs; start += 1024) {
+    const uint64_t i = start + tid;
+    const uint64_t v = i < g.n_segs ? seg_units[i] : 0;
+    uint64_t incl = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      uint64_t t = __shfl_up(incl, o, 64);
+      if ((tid & 63) >= (uint32_t)o) incl += t;
+    }
+    if ((tid & 63) == 63) wsum[tid >> 6] = incl;
+    __syncthreads();
+    uint64_t woff = carry_s;
+    for (uint32_t w = 0; w < (tid >> 6); ++w) woff += wsum[w];
+    if (i < g.n_segs) dir[i] = (uint32_t)(woff + incl - v);
+    __syncthreads();
+    if (tid == 1023) carry_s = woff + incl;
+    __syncthreads();
+  }
+  if (tid == 0) {
+    const uint64_t units = carry_s;
+    dir[g.n_segs] = (uint32_t)units;
+    // zero the alignment gap between directory and records
+    for (uint64_t b = g.dir_off + 4 * (g.n_segs + 1); b < g.rec_off; ++b) comp[b] = 0;
+    const uint64_t total = g.rec_off + 4 * units;
+    uint32_t* h = reinterpret_cast<uint32_t*>(comp);
+    h[0] = NZ_MAGIC;
+    h[1] = NZ_FORMAT_VERSION;
+    h[2] = (uint32_t)(g.n & 0xFFFFFFFFu);
+    h[3] = (uint32_t)(g.n >> 32);
+    h[4] = g.chunk_syms;
+    h[5] = g.lane_syms;
+    h[6] = (uint32_t)g.n_chunks;
+    h[7] = (uint32_t)g.n_segs;
+    h[8] = (uint32_t)g.dir_off;
+    h[9] = (uint32_t)g.rec_off;
+    h[10] = (uint32_t)(total & 0xFFFFFFFFu);
+    h[11] = (uint32_t)(total >> 32);
+    h[12] = h[13] = h[14] = h[15] = 0;
+    *d_total = total;
+    if (total > cap || units > 0xFFFFFFFFull) atomicOr(d_status, 1u);
+  }
+}
+
+// ----------------------------------------------------------------------------
+// move every segment record to its final place: one workgroup per segment
+// ----------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void nz_compact_kernel(
+    const uint8_t* __restrict__ exps, NzGeom g, const NzChunkInfo* __restrict__ info,
+    const uint8_t* __restrict__ tab_ser, const uint16_t* __restrict__ slots,
+    const uint32_t* __restrict__ states, const uint32_t* __restrict__ seg_words,
+    const uint32_t* __restrict__ dir, uint8_t* __restrict__ comp, uint64_t cap) {
+  const uint64_t seg = blockIdx.x;
+  const uint64_t c = seg / g.spc;
+  const uint32_t k = (uint32_t)(seg - c * g.spc);
+  const uint64_t o0 = dir[seg], o1 = dir[seg + 1];
+  if (g.rec_off + 4 * o1 > cap) return;  // flagged by the scan kernel
+  uint8_t* dst = comp + g.rec_off + 4 * o0;
+  const uint64_t seg_base = seg * g.seg_syms;
+  const uint32_t sn = (uint32_t)((g.n - seg_base) < g.seg_syms ? (g.n - seg_base) : g.seg_syms);
+  const NzChunkInfo ci = info[c];
+  const uint32_t tid = threadIdx.x;
+  if (ci.raw) {
+    uint32_t off = 0;
+    if (k == 0) {
+      if (tid < 4) dst[tid] = tid == 0 ? NZ_MODE_RAW : 0;
+      off = 4;
+    }
+    const uint32_t padded = (sn + 3) & ~3u;
+    for (uint32_t i = tid; i < padded; i += 256) dst[off + i] = i < sn ? exps[seg_base + i] : 0;
+    return;
+  }
+  uint32_t off = 0;
+  if (k == 0) {
+    const uint8_t* t = tab_ser + c * NZ_TABLE_MAX_BYTES;
+    for (uint32_t i = tid; i < ci.tab_len; i += 256) dst[i] = t[i];
+    off = ci.tab_len;
+  }
+  uint32_t* sdst = reinterpret_cast<uint32_t*>(dst + off);
+  if (tid < 64) sdst[tid] = states[seg * NZ_LANES + tid];
+  const uint32_t w = seg_words[seg];
+  const uint32_t cap_words = g.seg_syms / 2;
+  const uint16_t* src = slots + seg * cap_words + (cap_words - w);
+  uint16_t* wdst = reinterpret_cast<uint16_t*>(dst + off + 256);
+  for (uint32_t i = tid; i < w; i += 256) wdst[i] = src[i];
+  if ((w & 1) && tid == 0) wdst[w] = 0;
+}
+
+// ----------------------------------------------------------------------------
+// fused rANS decode + merge: one workgroup per chunk, one wavefront per segment
+// ----------------------------------------------------------------------------
+//
+// LDS: 4096-entry slot table (freq << 20 | (slot - cum) << 8 | symbol), then a
+// 4 KiB ring of renormalisation words per wavefront, then table-parse scratch.
+// A rANS step per lane: one table read, one multiply-add, and when the state
+// falls below 2^16 a 16-bit word taken at (words consumed so far by the wave +
+// rank of the lane among the lanes that need one).
+
+template <int S>
+__device__ __forceinline__ void nz_store_group(uint16_t* __restrict__ out, uint64_t sm,
+                                               const uint32_t (&ex)[8]) {
+  uint32_t o[4];
+#pragma unroll
+  for (int j = 0; j < 8; j += 2) {
+    uint32_t r0 = (uint32_t)(sm >> nz_field_shift<S>(j)) & ((2u << S) - 1u);
+    uint32_t r1 = (uint32_t)(sm >> nz_field_shift<S>(j + 1)) & ((2u << S) - 1u);
+    o[j >> 1] = nz_merge_one<S>(ex[j], r0) | (nz_merge_one<S>(ex[j + 1], r1) << 16);
+  }
+  *reinterpret_cast<uint4*>(out) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+template <int S>
+__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
+    const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
+    uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status) {
+  extern __shared__ uint32_t lds[];
+  uint32_t* lut = lds;                                   // 4096 dwords
+  uint32_t* rings = lds + NZ_M;                          // spc * 1024 dwords
+  uint32_t* scratch = rings + g.spc * NZ_RING_DWORDS;    // 106 + 257 dwords
+  uint8_t* tb = reinterpret_cast<uint8_t*>(scratch);     // table bytes (424)
+  uint32_t* cum = scratch + NZ_TABLE_MAX_BYTES / 4;      // 257 entries
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t wave = tid >> 6;
+  const uint32_t lane = tid & 63;
+  const uint64_t c = blockIdx.x;
+  const uint64_t seg0 = c * g.spc;
+  const uint64_t chunk_base = c * g.chunk_syms;
+  const uint32_t cn =
+      (uint32_t)((g.n - chunk_base) < g.chunk_syms ? (g.n - chunk_base) : g.chunk_syms);
+  const uint32_t nseg = (cn + g.seg_syms - 1) / g.seg_syms;
+  const uint32_t* dir = reinterpret_cast<const uint32_t*>(comp + g.dir_off);
+
+  // record of the chunk's first segment starts with the table
+  const uint64_t f0 = dir[seg0], f1 = dir[seg0 + 1];
+  if (f1 < f0 || g.rec_off + 4 * f1 > comp_bytes || f1 == f0) {
+    if (tid == 0) atomicOr(d_status, 2u);
+    return;
+  }
+  const uint8_t* rec0 = comp + g.rec_off + 4 * f0;
+  const uint32_t rec0_bytes = (uint32_t)(4 * (f1 - f0));
+  // stage up to 424 table bytes
+  for (uint32_t i = tid; i < NZ_TABLE_MAX_BYTES / 4; i += blockDim.x)
+    scratch[i] = (4 * i < rec0_bytes) ? reinterpret_cast<const uint32_t*>(rec0)[i] : 0u;
+  __syncthreads();
+  const uint32_t mode = tb[0];
+  uint32_t tab_len = 4;
+
+  if (mode != NZ_MODE_RAW) {
+    if (mode > NZ_MAX_RUNS) {
+      if (tid == 0) atomicOr(d_status, 2u);
+      return;
+    }
+    uint32_t head, kk = 0;
+    if (mode == NZ_MODE_BITMAP) {
+      head = 33;
+      for (int b = 0; b < 32; ++b) kk += __popc((uint32_t)tb[1 + b]);
+    } else {
+      head = 1 + 2 * mode;
+      for (uint32_t r = 0; r < mode; ++r) kk += (uint32_t)tb[2 + 2 * r] + 1u;
+    }
+    if (kk > 256) kk = 256;  // corrupt input: stay inside the staged bytes
+    tab_len = (head + (12 * kk + 7) / 8 + 3) & ~3u;
+    __syncthreads();  // everyone has read tb before cum (which follows it) is written
+    // frequency of every symbol -> cum[sym + 1] temporarily
+    for (uint32_t sym = tid; sym < 256; sym += blockDim.x) {
+      uint32_t live = 0, rank = 0;
+      if (mode == NZ_MODE_BITMAP) {
+        live = (tb[1 + (sym >> 3)] >> (sym & 7)) & 1u;
+        for (uint32_t b = 0; b < (sym >> 3); ++b) rank += __popc((uint32_t)tb[1 + b]);
+        rank += __popc((uint32_t)tb[1 + (sym >> 3)] & ((1u << (sym & 7)) - 1u));
+      } else {
+        uint32_t acc = 0;
+        for (uint32_t r = 0; r < mode; ++r) {
+          const uint32_t st = tb[1 + 2 * r], ln = (uint32_t)tb[2 + 2 * r] + 1u;
+          if (sym >= st && sym < st + ln) {
+            live = 1;
+            rank = acc + sym - st;
+          }
+          acc += ln;
+        }
+      }
+      if (rank > 255) rank = 255;
+      cum[sym + 1] = live ? nz_get12(tb + head, rank) : 0u;
+    }
+    __syncthreads();
+    // inclusive scan by wavefront 0, four symbols per lane
+    if (wave == 0) {
+      uint32_t a0 = cum[4 * lane + 1], a1 = cum[4 * lane + 2], a2 = cum[4 * lane + 3],
+               a3 = cum[4 * lane + 4];
+      uint32_t tot = a0 + a1 + a2 + a3, incl = tot;
+#pragma unroll
+      for (int o = 1; o < 64; o <<= 1) {
+        uint32_t t = __shfl_up(incl, o, 64);
+        if (lane >= (uint32_t)o) incl += t;
+      }
+      uint32_t ex = incl - tot;
+      cum[4 * lane + 1] = ex + a0;
+      cum[4 * lane + 2] = ex + a0 + a1;
+      cum[4 * lane + 3] = ex + a0 + a1 + a2;
+      cum[4 * lane + 4] = incl;
+      if (lane == 0) cum[0] = 0;
+    }
+    __syncthreads();
+    if (cum[256] != NZ_M) {
+      if (tid == 0) atomicOr(d_status, 2u);
+      return;
+    }
+    // slot table: binary search of the owning symbol
+    for (uint32_t slot = tid; slot < NZ_M; slot += blockDim.x) {
+      uint32_t lo = 0, hi = 256;  // cum[lo] <= slot < cum[hi]
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        uint32_t mid = (lo + hi) >> 1;
+        if (cum[mid] <= slot) lo = mid; else hi = mid;
+      }
+      const uint32_t cl = cum[lo];
+      const uint32_t f = cum[lo + 1] - cl;
+      lut[slot] = (f << 20) | ((slot - cl) << 8) | lo;
+    }
+  }
+  __syncthreads();
+
+  if (wave >= nseg) return;
+  const uint64_t seg = seg0 + wave;
+  const uint64_t seg_base = seg * g.seg_syms;
+  const uint32_t seg_n = (uint32_t)((g.n - seg_base) < g.seg_syms ? (g.n - seg_base) : g.seg_syms);
+  const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
+  uint64_t o0 = dir[seg], o1 = dir[seg + 1];
+  if (o1 < o0 || g.rec_off + 4 * o1 > comp_bytes) {
+    if (lane == 0) atomicOr(d_status, 2u);
+    return;
+  }
+  uint64_t rec_start = g.rec_off + 4 * o0;
+  uint64_t rec_bytes = 4 * (o1 - o0);
+  if (wave == 0) {
+    if (rec_bytes < tab_len) {
+      if (lane == 0) atomicOr(d_status, 2u);
+      return;
+    }
+    rec_start += tab_len;
+    rec_bytes -= tab_len;
+  }
+  const uint8_t* pk = packed + (seg_base * (S + 1)) / 8;
+  uint16_t* dst = out + seg_base;
+
+  if (mode == NZ_MODE_RAW) {
+    if (rec_bytes < seg_n) {
+      if (lane == 0) atomicOr(d_status, 2u);
+      return;
+    }
+    const uint8_t* raw = comp + rec_start;
+    for (uint32_t gq = 0; gq < ngroups; ++gq) {
+      const uint32_t idx0 = (gq * NZ_LANES + lane) * NZ_GROUP;
+      if (idx0 >= seg_n) continue;
+      const uint32_t rem = seg_n - idx0;
+      if (rem >= 8) {
+        uint64_t sy = (uint64_t)reinterpret_cast<const uint32_t*>(raw + idx0)[0] |
+                      ((uint64_t)reinterpret_cast<const uint32_t*>(raw + idx0)[1] << 32);
+        uint64_t sm;
+        const uint8_t* pp = pk + (idx0 * (S + 1)) / 8;
+        if constexpr (S == 7) sm = *reinterpret_cast<const uint64_t*>(pp);
+        else if constexpr (S == 3) sm = *reinterpret_cast<const uint32_t*>(pp);
+        else if constexpr (S == 1) sm = *reinterpret_cast<const uint16_t*>(pp);
+        else sm = *pp;
+        uint32_t ex[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ex[j] = (uint32_t)(sy >> (8 * j)) & 0xFFu;
+        nz_store_group<S>(dst + idx0, sm, ex);
+      } else {
+        for (uint32_t j = 0; j < rem; ++j) {
+          const uint32_t bit = (idx0 + j) * (S + 1);
+          const uint32_t rp = ((uint32_t)pk[bit >> 3] >> (7u - S - (bit & 7u))) & ((2u << S) - 1u);
+          dst[idx0 + j] = (uint16_t)nz_merge_one<S>(raw[idx0 + j], rp);
+        }
+      }
+    }
+    return;
+  }
+
+  if (rec_bytes < 256) {
+    if (lane == 0) atomicOr(d_status, 2u);
+    return;
+  }
+  uint32_t x = reinterpret_cast<const uint32_t*>(comp + rec_start)[lane];
+  const uint32_t* cw = reinterpret_cast<const uint32_t*>(comp + rec_start + 256);
+  const uint32_t ndw = (uint32_t)((rec_bytes - 256) / 4);
+  uint32_t* ring32 = rings + wave * NZ_RING_DWORDS;
+  const uint16_t* ring = reinterpret_cast<const uint16_t*>(ring32);
+
+  // initial fill: 768 dwords = 1536 words
+#pragma unroll
+  for (uint32_t q = 0; q < 12; ++q) {
+    const uint32_t d = lane + 64 * q;
+    ring32[d] = d < ndw ? cw[d] : 0u;
+  }
+  uint32_t filled = 768;  // dwords staged so far
+  uint32_t base = 0;      // words consumed so far
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+
+  for (uint32_t gq = 0; gq < ngroups; ++gq) {
+    const uint32_t idx0 = (gq * NZ_LANES + lane) * NZ_GROUP;
+    // keep at least 512 words ahead of the read position: a group consumes at
+    // most 8 * 64 words, the ring holds 2048.
+    const bool refill = (2 * filled - base) <= 1536u;
+    uint32_t r[4];
+    if (refill) {
+#pragma unroll
+      for (uint32_t q = 0; q < 4; ++q) {
+        const uint32_t d = filled + lane + 64 * q;
+        r[q] = d < ndw ? cw[d] : 0u;
+      }
+    }
+    const bool full = idx0 + 8 <= seg_n;
+    uint64_t sm = 0;
+    if (full) {
+      const uint8_t* pp = pk + (idx0 * (S + 1)) / 8;
+      if constexpr (S == 7) sm = *reinterpret_cast<const uint64_t*>(pp);
+      else if constexpr (S == 3) sm = *reinterpret_cast<const uint32_t*>(pp);
+      else if constexpr (S == 1) sm = *reinterpret_cast<const uint16_t*>(pp);
+      else sm = *pp;
+    }
+    uint32_t ex[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t e = lut[x & (NZ_M - 1)];
+      x = (e >> 20) * (x >> NZ_PROB_BITS) + ((e >> 8) & 0xFFFu);
+      ex[j] = e & 0xFFu;
+      const bool need = x < NZ_L;
+      const uint64_t m = __ballot(need);
+      const uint32_t w = ring[(base + nz_rank_below(m)) & (NZ_RING_WORDS - 1)];
+      if (need) x = (x << 16) | w;
+      base += (uint32_t)__popcll(m);
+    }
+    if (full) {
+      nz_store_group<S>(dst + idx0, sm, ex);
+    } else if (idx0 < seg_n) {
+      const uint32_t rem = seg_n - idx0;
+      for (uint32_t j = 0; j < rem; ++j) {
+        const uint64_t bit = (uint64_t)(idx0 + j) * (S + 1);
+        const uint32_t rp = ((uint32_t)pk[bit >> 3] >> (7u - S - (uint32_t)(bit & 7u))) & ((2u << S) - 1u);
+        dst[idx0 + j] = (uint16_t)nz_merge_one<S>(ex[j], rp);
+      }
+    }
+    if (refill) {
+#pragma unroll
+      for (uint32_t q = 0; q < 4; ++q) ring32[(filled + lane + 64 * q) & (NZ_RING_DWORDS - 1)] = r[q];
+      filled += 256;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+  // every lane must be back at the encoder's start state and the wave must
+  // not have read past its record
+  const bool bad = (x != NZ_L) || (base > 2 * ndw);
+  if (__ballot(bad) != 0 && lane == 0) atomicOr(d_status, 4u);
+}
+

@@ -1,0 +1,4 @@
+from neuzip_amd.nn.linear import Linear
+from neuzip_amd.nn.module import Parameter
+
+__all__ = ["Parameter", "Linear"]

@@ -1,0 +1,179 @@
+"""HIP path vs CPU oracle through the C ABI (needs an MI355X)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import bf16_bits_normal, chunk_entropy_bytes, closed_form_recon, stress_bits
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def _lib():
+    from neuzip_amd import _lib
+
+    return _lib.load(), _lib
+
+
+def _to_dev(bits: np.ndarray):
+    return torch.from_numpy(bits.view(np.int16).copy()).cuda()
+
+
+def gpu_encode(bits, s, chunk=65536, lane=1024):
+    L, m = _lib()
+    n = bits.size
+    d_in = _to_dev(bits) if n else torch.empty(0, dtype=torch.int16, device="cuda")
+    cap = L.nz_exp_bound_bytes(n, chunk, lane)
+    assert cap > 0
+    ws_bytes = L.nz_encode_workspace_bytes(n, chunk, lane)
+    comp = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+    packed = torch.zeros(max(8, L.nz_packed_bytes(n, s)), dtype=torch.uint8, device="cuda")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    aux = torch.zeros(4, dtype=torch.int64, device="cuda")
+    total = ctypes.c_uint64(0)
+    st = torch.cuda.current_stream().cuda_stream
+    rc = L.nz_encode(d_in.data_ptr(), n, s, chunk, lane, packed.data_ptr(), comp.data_ptr(), cap,
+                     ws.data_ptr(), ws_bytes, aux.data_ptr(), aux.data_ptr() + 8, ctypes.byref(total), st)
+    assert rc == 0, m.last_error()
+    torch.cuda.synchronize()
+    return comp[: total.value].clone(), packed[: L.nz_packed_bytes(n, s)].clone()
+
+
+def gpu_decode(comp, packed, n, s, chunk=65536, lane=1024, check=True):
+    L, m = _lib()
+    out = torch.zeros(max(n, 8), dtype=torch.int16, device="cuda")
+    status = torch.zeros(2, dtype=torch.int32, device="cuda")
+    if packed.numel() < 8:
+        packed = torch.cat([packed, torch.zeros(8, dtype=torch.uint8, device="cuda")])
+    st = torch.cuda.current_stream().cuda_stream
+    rc = L.nz_decode(comp.data_ptr(), comp.numel(), packed.data_ptr(), n, s, chunk, lane,
+                     out.data_ptr(), status.data_ptr(), 1 if check else 0, st)
+    torch.cuda.synchronize()
+    return rc, out[:n].cpu().numpy().view(np.uint16)
+
+
+SIZES = [0, 1, 7, 8, 9, 511, 512, 513, 4095, 65535, 65536, 65537, 200_000, 1_000_003]
+
+
+@pytest.mark.parametrize("s", [7, 3, 1, 0])
+@pytest.mark.parametrize("n", SIZES)
+def test_roundtrip_matches_oracle(oracle, n, s):
+    bits = bf16_bits_normal(n, seed=n + s)
+    print(f"case n={n} s={s}", flush=True)
+    comp, packed = gpu_encode(bits, s)
+    # container and packed stream are byte-identical to the oracle's
+    o_comp, o_packed = oracle.compress_bf16(bits, s, 65536, 1024)
+    assert np.array_equal(packed.cpu().numpy(), o_packed)
+    assert np.array_equal(comp.cpu().numpy(), o_comp)
+    rc, out = gpu_decode(comp, packed, n, s)
+    assert rc == 0
+    assert np.array_equal(out, oracle.reconstruct(bits, s))
+    assert np.array_equal(out, closed_form_recon(bits, s))
+
+
+@pytest.mark.parametrize("lane,chunk", [(128, 65536), (256, 65536), (512, 65536), (1024, 65536),
+                                        (8, 512), (64, 4096), (2048, 1 << 20)])
+def test_geometries(oracle, lane, chunk):
+    n = 3 * chunk + 1234 if chunk <= 65536 else chunk + 777
+    bits = bf16_bits_normal(n, seed=lane)
+    print(f"case lane={lane} chunk={chunk} n={n}", flush=True)
+    comp, packed = gpu_encode(bits, 7, chunk, lane)
+    o_comp, _ = oracle.compress_bf16(bits, 7, chunk, lane)
+    assert np.array_equal(comp.cpu().numpy(), o_comp)
+    rc, out = gpu_decode(comp, packed, n, 7, chunk, lane)
+    assert rc == 0 and np.array_equal(out, bits)
+
+
+def test_all_bit_patterns(oracle):
+    allv = np.arange(65536, dtype=np.uint16)
+    bits = np.tile(allv, 3)
+    for s in (7, 3, 1, 0):
+        print(f"case all patterns s={s}", flush=True)
+        comp, packed = gpu_encode(bits, s)
+        rc, out = gpu_decode(comp, packed, bits.size, s)
+        assert rc == 0
+        assert np.array_equal(out, closed_form_recon(bits, s))
+        assert np.array_equal(out, oracle.reconstruct(bits, s))
+
+
+def test_cross_cpu_gpu(oracle):
+    n = 300_000
+    bits = stress_bits(300, 1000, seed=5)
+    for s in (7, 3):
+        print(f"case cross s={s}", flush=True)
+        o_comp, o_packed = oracle.compress_bf16(bits, s, 65536, 512)
+        rc, out = gpu_decode(torch.from_numpy(o_comp).cuda(), torch.from_numpy(o_packed).cuda(), n, s, 65536, 512)
+        assert rc == 0 and np.array_equal(out, oracle.reconstruct(bits, s))
+        comp, packed = gpu_encode(bits, s, 65536, 512)
+        rc2, out2 = oracle.decompress_bf16(comp.cpu().numpy(), packed.cpu().numpy(), n, s)
+        assert rc2 == 0 and np.array_equal(out2, oracle.reconstruct(bits, s))
+
+
+def test_incompressible_goes_raw(oracle):
+    rng = np.random.default_rng(3)
+    n = 150_000
+    bits = rng.integers(0, 65536, n).astype(np.uint16)
+    print("case raw", flush=True)
+    comp, packed = gpu_encode(bits, 7)
+    o_comp, _ = oracle.compress_bf16(bits, 7, 65536, 1024)
+    assert np.array_equal(comp.cpu().numpy(), o_comp)
+    L, _m = _lib()
+    assert comp.numel() <= L.nz_exp_bound_bytes(n, 65536, 1024)
+    rc, out = gpu_decode(comp, packed, n, 7)
+    assert rc == 0 and np.array_equal(out, bits)
+
+
+def test_constant_and_two_symbol(oracle):
+    for name, bits in (("zeros", np.zeros(70_000, np.uint16)),
+                       ("const", np.full(70_000, 0x3C00, np.uint16)),
+                       ("two", np.where(np.arange(70_000) % 97 == 0, 0x3C00, 0x0080).astype(np.uint16))):
+        print(f"case {name}", flush=True)
+        comp, packed = gpu_encode(bits, 7)
+        o_comp, _ = oracle.compress_bf16(bits, 7, 65536, 1024)
+        assert np.array_equal(comp.cpu().numpy(), o_comp)
+        rc, out = gpu_decode(comp, packed, bits.size, 7)
+        assert rc == 0 and np.array_equal(out, bits)
+
+
+def test_corrupt_container_is_reported(oracle):
+    n = 100_000
+    bits = bf16_bits_normal(n, seed=11)
+    comp, packed = gpu_encode(bits, 7)
+    bad = comp.clone()
+    bad[bad.numel() // 2] ^= 0x5A  # flip bits inside the word stream
+    print("case corrupt words", flush=True)
+    rc, _ = gpu_decode(bad, packed, n, 7)
+    assert rc == -6
+    bad = comp.clone()
+    bad[64:72] = 0xFF  # directory entries out of range
+    print("case corrupt directory", flush=True)
+    rc, _ = gpu_decode(bad, packed, n, 7)
+    assert rc == -6
+
+
+def test_ratio_close_to_entropy(oracle):
+    n = 4096 * 4096
+    bits = bf16_bits_normal(n, seed=0)
+    exps = ((bits >> 7) & 0xFF).astype(np.uint8)
+    bound = chunk_entropy_bytes(exps)
+    comp, _ = gpu_encode(bits, 7)
+    overhead = comp.numel() / bound - 1.0
+    print(f"container {comp.numel()} B, entropy bound {bound:.0f} B, overhead {100 * overhead:.3f}%", flush=True)
+    assert overhead < 0.0125
+
+
+def test_split_api(oracle):
+    L, m = _lib()
+    for n in (0, 5, 2048, 100_001):
+        bits = bf16_bits_normal(n, seed=n)
+        d = _to_dev(bits) if n else torch.empty(0, dtype=torch.int16, device="cuda")
+        e = torch.zeros(max(n, 8), dtype=torch.uint8, device="cuda")
+        f = torch.zeros(max(n, 8), dtype=torch.uint8, device="cuda")
+        rc = L.nz_split(d.data_ptr(), n, e.data_ptr(), f.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, m.last_error()
+        torch.cuda.synchronize()
+        oe, of = oracle.split(bits, 7)
+        assert np.array_equal(e[:n].cpu().numpy(), oe)
+        assert np.array_equal(f[:n].cpu().numpy(), of)
