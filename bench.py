@@ -60,7 +60,8 @@ class Codec:
             raise SystemExit("unsupported chunk_size / lane_symbols combination")
         self.cap = cap
         self.comp = torch.empty(cap, dtype=torch.uint8, device="cuda")
-        self.packed_bytes = int(L.nz_packed_bytes(n, precision))
+        self.packed_bytes = int(L.nz_packed_stored_bytes(n, precision, lane))
+        self.packed_ref_bytes = int(L.nz_packed_bytes(n, precision))
         self.packed = torch.empty(max(8, self.packed_bytes), dtype=torch.uint8, device="cuda")
         self.ws_bytes = int(L.nz_encode_workspace_bytes(n, chunk, lane))
         self.ws = torch.empty(self.ws_bytes, dtype=torch.uint8, device="cuda")
@@ -148,6 +149,8 @@ def main():
         rec = ((a & 0x8000) | (((mag + (1 << (6 - s))) & 0x7FFF) & (0x7FFF ^ ((1 << (7 - s)) - 1)))).astype(np.uint16)
         bit_exact = bool(np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), rec))
 
+    headline_out = out.view(torch.int16).cpu().numpy().view(np.uint16).copy()
+
     # ---- the timed region: K decode launches ----
     wall, mean_launch, med_launch = time_launches(torch, lambda: codec.decode(out), args.steps, args.warmup)
     ms_per_step = wall / args.steps * 1e3
@@ -193,7 +196,7 @@ def main():
             "compressed_exponent_bytes": codec.total,
             "packed_sign_mantissa_bytes": codec.packed_bytes,
             "stored_over_dense": round((codec.total + codec.packed_bytes) / dense_bytes, 5),
-            "exponent_bytes_over_entropy_bound": round(codec.total / bound, 5),
+            "exponent_bytes_over_entropy_bound": round((codec.total + codec.packed_bytes - codec.packed_ref_bytes) / bound, 5),
         },
         "roofline": {
             "bound": "hbm",
@@ -247,7 +250,7 @@ def main():
                 raise RuntimeError("oracle failed to decode the GPU container")
             if time.perf_counter() - t_budget > 30:
                 break
-        cpu_ok = bool(np.array_equal(rec, out.view(torch.int16).cpu().numpy().view(np.uint16)))
+        cpu_ok = bool(np.array_equal(rec, headline_out))
         result["cpu_baseline"] = {
             "value": round(dense_bytes / statistics.median(times) / 1e9, 3),
             "unit": "GB/s",

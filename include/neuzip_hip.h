@@ -45,7 +45,7 @@ extern "C" {
 #define NZ_ALGO_ANS 0
 
 #define NZ_DEFAULT_CHUNK 65536u   /* cuda/neuzip.cu:31 */
-#define NZ_DEFAULT_LANE_SYMS 1024u /* one wavefront per 64 KiB chunk */
+#define NZ_DEFAULT_LANE_SYMS 512u /* two wavefronts per 64 KiB chunk */
 
 typedef struct nz_manager nz_manager;
 
@@ -57,6 +57,12 @@ const char* nz_last_error(void);
 /* Packed sign+mantissa bytes for n elements at `precision` kept mantissa
    bits: (n * (precision + 1) + 7) / 8, cuda/high_level.cu:81-83. */
 uint64_t nz_packed_bytes(uint64_t n, int precision);
+
+/* Bytes actually stored for the packed stream: the last 128 bytes of every
+   full segment (64 * lane_syms elements) travel inside the entropy coder's
+   start states instead (16 bits per rANS lane), so each full segment stores
+   128 bytes fewer than the reference layout. */
+uint64_t nz_packed_stored_bytes(uint64_t n, int precision, uint32_t lane_syms);
 
 /* Capacity that always holds the entropy-coded exponent container of n
    elements (stands in for nvcomp's max_compressed_buffer_size,
@@ -74,7 +80,7 @@ int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fr
              void* stream);
 
 /* Manager::_write_to_cache, cuda/high_level.cu:76-130: split, then entropy
-   code the exponents.  `dev_packed` receives nz_packed_bytes() bytes,
+   code the exponents.  `dev_packed` receives nz_packed_stored_bytes() bytes,
    `dev_comp` (capacity comp_cap >= nz_exp_bound_bytes) the container.
    `dev_total` (device uint64) receives the container size, `dev_status`
    (device uint32, OR-ed into) is non-zero on overflow.  If `host_total` is

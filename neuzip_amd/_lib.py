@@ -18,10 +18,10 @@ ERR_ARG, ERR_DTYPE, ERR_NOT_FOUND, ERR_HIP, ERR_CAPACITY, ERR_CORRUPT, ERR_ALIGN
 DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 ALGO_ANS = 0
 DEFAULT_CHUNK = 65536
-DEFAULT_LANE_SYMS = 1024
+DEFAULT_LANE_SYMS = 512
 
 EXPORTS = [
-    "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_exp_bound_bytes",
+    "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",
     "nz_encode_workspace_bytes", "nz_split", "nz_encode", "nz_decode",
     "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_read",
     "nz_manager_meta", "nz_manager_size", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
@@ -49,6 +49,8 @@ def load() -> ctypes.CDLL:
     L.nz_last_error.argtypes = []
     L.nz_packed_bytes.restype = u64
     L.nz_packed_bytes.argtypes = [u64, i32]
+    L.nz_packed_stored_bytes.restype = u64
+    L.nz_packed_stored_bytes.argtypes = [u64, i32, u32]
     L.nz_exp_bound_bytes.restype = u64
     L.nz_exp_bound_bytes.argtypes = [u64, u32, u32]
     L.nz_encode_workspace_bytes.restype = u64

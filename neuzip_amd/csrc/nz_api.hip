@@ -34,7 +34,7 @@ bool precision_ok(int p) { return p == 7 || p == 3 || p == 1 || p == 0; }
 
 // Device scratch of one encode call.
 struct EncLayout {
-  uint64_t exps, enc_tab, tab_ser, info, slots, states, seg_words, seg_units, hdr, total, status, bytes;
+  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_units, hdr, total, status, bytes;
 };
 
 EncLayout enc_layout(const NzGeom& g) {
@@ -49,6 +49,7 @@ EncLayout enc_layout(const NzGeom& g) {
   L.enc_tab = take(g.n_chunks * 256 * 4);
   L.tab_ser = take(g.n_chunks * NZ_TABLE_MAX_BYTES);
   L.info = take(g.n_chunks * sizeof(NzChunkInfo));
+  L.carry = take(g.n_segs * NZ_CARRY_BYTES);
   L.slots = take(g.n_segs * (uint64_t)g.seg_syms);  // seg_syms/2 words of 2 bytes
   L.states = take(g.n_segs * NZ_LANES * 4);
   L.seg_words = take(g.n_segs * 4);
@@ -64,8 +65,9 @@ template <int S>
 void launch_split_hist(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws,
                        const EncLayout& L, hipStream_t st) {
   hipLaunchKernelGGL(nz_split_hist_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(256), 0, st,
-                     (const uint16_t*)in, g.n, g.chunk_syms, packed, ws + L.exps,
-                     (uint32_t*)(ws + L.enc_tab), ws + L.tab_ser, (NzChunkInfo*)(ws + L.info));
+                     (const uint16_t*)in, g.n, g.chunk_syms, g.seg_syms, packed, ws + L.carry,
+                     ws + L.exps, (uint32_t*)(ws + L.enc_tab), ws + L.tab_ser,
+                     (NzChunkInfo*)(ws + L.info));
 }
 
 // Phase 1: everything up to the directory.  Header + directory land in `hdr`
@@ -83,7 +85,8 @@ int encode_phase1(const NzGeom& g, int precision, const void* in, uint8_t* packe
     hipLaunchKernelGGL(nz_rans_encode_kernel, dim3((uint32_t)g.n_chunks), dim3(64 * g.spc), 0, st,
                        ws + L.exps, g.n, g.chunk_syms, g.lane_syms, g.spc,
                        (const uint32_t*)(ws + L.enc_tab), (const NzChunkInfo*)(ws + L.info),
-                       (uint16_t*)(ws + L.slots), (uint32_t*)(ws + L.states),
+                       (const uint16_t*)(ws + L.carry), (uint16_t*)(ws + L.slots),
+                       (uint32_t*)(ws + L.states),
                        (uint32_t*)(ws + L.seg_words));
     hipLaunchKernelGGL(nz_chunk_finalize_kernel, dim3((uint32_t)((g.n_chunks + 255) / 256)),
                        dim3(256), 0, st, g.n, g.chunk_syms, g.seg_syms, g.spc, g.n_chunks,
@@ -102,7 +105,8 @@ int encode_phase2(const NzGeom& g, uint8_t* ws, const EncLayout& L, const uint32
   if (g.n_segs > 0) {
     hipLaunchKernelGGL(nz_compact_kernel, dim3((uint32_t)g.n_segs), dim3(256), 0, st,
                        ws + L.exps, g, (const NzChunkInfo*)(ws + L.info), ws + L.tab_ser,
-                       (const uint16_t*)(ws + L.slots), (const uint32_t*)(ws + L.states),
+                       ws + L.carry, (const uint16_t*)(ws + L.slots),
+                       (const uint32_t*)(ws + L.states),
                        (const uint32_t*)(ws + L.seg_words), dir, comp, cap);
     NZ_HIP(hipGetLastError());
   }
@@ -164,11 +168,16 @@ struct nz_manager {
 
 extern "C" {
 
-int nz_abi_version(void) { return 1; }
+int nz_abi_version(void) { return 2; }
 
 const char* nz_last_error(void) { return g_err.c_str(); }
 
 uint64_t nz_packed_bytes(uint64_t n, int precision) { return nz_packed_bytes_of(n, precision); }
+
+uint64_t nz_packed_stored_bytes(uint64_t n, int precision, uint32_t lane_syms) {
+  if (lane_syms < 16) return 0;
+  return nz_packed_stored_bytes_of(n, precision, lane_syms);
+}
 
 uint64_t nz_exp_bound_bytes(uint64_t n, uint32_t chunk_size, uint32_t lane_syms) {
   NzGeom g;
@@ -334,7 +343,7 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   Entry ent;
   ent.n = n;
   ent.dtype = dtype;
-  ent.packed_bytes = nz_packed_bytes_of(n, m->precision);
+  ent.packed_bytes = nz_packed_stored_bytes_of(n, m->precision, m->lane_syms);
   auto release = [&](Entry& e) {
     if (e.comp) (void)hipFree(e.comp);
     if (e.packed) (void)hipFree(e.packed);

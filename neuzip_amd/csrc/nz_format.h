@@ -17,14 +17,21 @@
 //             states] [u16 renormalisation words, front-to-back in decode
 //             order] padded to 4 bytes; or, for a chunk whose coded form
 //             would not be smaller, [0xFF 0 0 0, first segment only] raw
-//             exponent bytes padded to 4.
+//             exponent bytes padded to 4 [+ 64 x u16 carried bits if full].
+// * carry   = the encoder of a FULL segment starts lane l in state
+//             2^16 | c_l instead of 2^16, where c_l are bytes 2l, 2l+1 of the
+//             last 128 bytes of the segment's packed sign|mantissa stream.
+//             Those 128 bytes are not stored in the packed stream (every full
+//             segment stores NZ_CARRY_BYTES fewer); the decoder finds them in
+//             the low halves of its final states.  This returns 16 of the
+//             ~24 bits that flushing a 32-bit rANS state costs per lane.
 #pragma once
 
 #include <stddef.h>
 #include <stdint.h>
 
 #define NZ_MAGIC 0x315A4E41u
-#define NZ_FORMAT_VERSION 1u
+#define NZ_FORMAT_VERSION 2u
 #define NZ_PROB_BITS 12
 #define NZ_M (1u << NZ_PROB_BITS)
 #define NZ_L (1u << 16)
@@ -37,6 +44,7 @@
 #define NZ_MAX_RUNS 15
 #define NZ_TABLE_MAX_BYTES 424 /* 1 + 32 + 384 rounded up to a multiple of 8 */
 #define NZ_MAX_SEGS_PER_CHUNK 8
+#define NZ_CARRY_BYTES 128 /* 64 lanes x 16 bits */
 
 struct NzGeom {
   uint64_t n;
@@ -59,7 +67,7 @@ struct NzChunkInfo {
 };
 
 static inline int nz_geom_check(uint32_t chunk_syms, uint32_t lane_syms) {
-  if (lane_syms < NZ_GROUP || (lane_syms % NZ_GROUP) != 0 || lane_syms > (1u << 16)) return -1;
+  if (lane_syms < 16 || (lane_syms % NZ_GROUP) != 0 || lane_syms > (1u << 16)) return -1;
   uint64_t seg = (uint64_t)lane_syms * NZ_LANES;
   if (chunk_syms == 0 || (chunk_syms % seg) != 0) return -1;
   uint64_t spc = chunk_syms / seg;
@@ -85,9 +93,15 @@ static inline int nz_geom_make(NzGeom* g, uint64_t n, uint32_t chunk_syms, uint3
 
 // Upper bound of the container size: no chunk is ever stored larger than raw.
 static inline uint64_t nz_geom_bound(const NzGeom* g) {
-  return g->rec_off + g->n + 4 * g->n_segs + 4 * g->n_chunks;
+  return g->rec_off + g->n + (4 + NZ_CARRY_BYTES) * g->n_segs + 4 * g->n_chunks;
 }
 
 static inline uint64_t nz_packed_bytes_of(uint64_t n, int s) {
   return (n * (uint64_t)(s + 1) + 7) / 8;  // cuda/high_level.cu:81-83
+}
+
+// Bytes actually stored for the packed stream: the reference size minus the
+// carried bytes of every full segment.
+static inline uint64_t nz_packed_stored_bytes_of(uint64_t n, int s, uint32_t lane_syms) {
+  return nz_packed_bytes_of(n, s) - (uint64_t)NZ_CARRY_BYTES * (n / ((uint64_t)lane_syms * NZ_LANES));
 }

@@ -138,9 +138,9 @@ __device__ __forceinline__ uint32_t nz_block_max_256(uint32_t v, uint32_t* red) 
 
 template <int S>
 __global__ __launch_bounds__(256) void nz_split_hist_kernel(
-    const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms,
-    uint8_t* __restrict__ packed, uint8_t* __restrict__ exps, uint32_t* __restrict__ enc_tab,
-    uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info) {
+    const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms,
+    uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
+    uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info) {
   __shared__ uint32_t hist[256];
   __shared__ uint32_t freq_s[256];
   __shared__ uint32_t red[4];
@@ -154,8 +154,21 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
   hist[tid] = 0;
   __syncthreads();
 
+  // Packed bytes go to the stored layout: segment k starts at k * keep, and the
+  // last NZ_CARRY_BYTES of a full segment go to carry[k] instead (they ride in
+  // the rANS start states).
+  const uint32_t seg_p = seg_syms / 8 * (S + 1);
+  const uint32_t keep = seg_p - NZ_CARRY_BYTES;
+  const uint64_t seg0 = base / seg_syms;
+
   for (uint32_t i = tid * 8; i < cn; i += 256 * 8) {
     const uint64_t gi = base + i;
+    const uint32_t sk = i / seg_syms;                    // segment inside the chunk
+    const uint32_t sb = (i - sk * seg_syms) / 8 * (S + 1);  // byte inside the segment
+    const uint64_t seg = seg0 + sk;
+    const bool seg_full = (seg + 1) * seg_syms <= n;
+    uint8_t* pp = (seg_full && sb >= keep) ? carry + seg * NZ_CARRY_BYTES + (sb - keep)
+                                           : packed + seg * keep + sb;
     uint32_t ex[8], rp[8];
     const uint32_t rem = cn - i;
     if (rem >= 8) {
@@ -170,7 +183,6 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
         f |= (uint64_t)rp[j] << nz_field_shift<S>(j);
       }
       *reinterpret_cast<uint64_t*>(exps + gi) = e;
-      uint8_t* pp = packed + (gi * (S + 1)) / 8;
       if constexpr (S == 7) *reinterpret_cast<uint64_t*>(pp) = f;
       else if constexpr (S == 3) *reinterpret_cast<uint32_t*>(pp) = (uint32_t)f;
       else if constexpr (S == 1) *reinterpret_cast<uint16_t*>(pp) = (uint16_t)f;
@@ -188,7 +200,6 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
         f |= (uint64_t)rp[0] << (8u * (bit >> 3) + (7u - S - (bit & 7u)));
         atomicAdd(&hist[ex[0]], 1u);
       }
-      uint8_t* pp = packed + (gi * (S + 1)) / 8;
       uint32_t nb = (rem * (S + 1) + 7) / 8;
       for (uint32_t b = 0; b < nb; ++b) pp[b] = (uint8_t)(f >> (8 * b));
     }
@@ -298,7 +309,8 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_kernel(
     const uint8_t* __restrict__ exps, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
     uint32_t spc, const uint32_t* __restrict__ enc_tab, const NzChunkInfo* __restrict__ info,
-    uint16_t* __restrict__ slots, uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words) {
+    const uint16_t* __restrict__ carry, uint16_t* __restrict__ slots,
+    uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words) {
   __shared__ uint32_t tab[256];
   const uint64_t c = blockIdx.x;
   for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) tab[i] = enc_tab[c * 256 + i];
@@ -317,7 +329,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
   uint16_t* slot = slots + seg * cap_words;
   const uint8_t* src = exps + seg_base;
 
-  uint32_t x = NZ_L;
+  // a full segment starts from 2^16 | 16 carried bits of the packed stream
+  uint32_t x = NZ_L | (seg_n == seg_syms ? (uint32_t)carry[seg * NZ_LANES + lane] : 0u);
   uint32_t pos = cap_words;
   bool overflow = false;
   for (uint32_t g = ngroups; g-- > 0 && !overflow;) {
@@ -378,7 +391,7 @@ __global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32
     const uint32_t w = seg_words[c * spc + k];
     if (w == 0xFFFFFFFFu) overflow = true;
     else rans_total += 256 + 2 * (uint64_t)((w + 1) & ~1u);
-    raw_total += (sn + 3) & ~3u;
+    raw_total += ((sn + 3) & ~3u) + (sn == seg_syms ? NZ_CARRY_BYTES : 0u);
   }
   const bool raw = overflow || rans_total >= raw_total;
   info[c].raw = raw ? 1u : 0u;
@@ -386,7 +399,7 @@ __global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
     const uint32_t w = seg_words[c * spc + k];
     uint32_t bytes;
-    if (raw) bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u);
+    if (raw) bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u) + (sn == seg_syms ? NZ_CARRY_BYTES : 0u);
     else bytes = (k == 0 ? tab_len : 0u) + 256u + 2u * ((w + 1) & ~1u);
     seg_units[c * spc + k] = bytes / 4;
   }
@@ -456,9 +469,10 @@ __global__ __launch_bounds__(1024) void nz_scan_kernel(const uint32_t* __restric
 // ----------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void nz_compact_kernel(
     const uint8_t* __restrict__ exps, NzGeom g, const NzChunkInfo* __restrict__ info,
-    const uint8_t* __restrict__ tab_ser, const uint16_t* __restrict__ slots,
-    const uint32_t* __restrict__ states, const uint32_t* __restrict__ seg_words,
-    const uint32_t* __restrict__ dir, uint8_t* __restrict__ comp, uint64_t cap) {
+    const uint8_t* __restrict__ tab_ser, const uint8_t* __restrict__ carry,
+    const uint16_t* __restrict__ slots, const uint32_t* __restrict__ states,
+    const uint32_t* __restrict__ seg_words, const uint32_t* __restrict__ dir,
+    uint8_t* __restrict__ comp, uint64_t cap) {
   const uint64_t seg = blockIdx.x;
   const uint64_t c = seg / g.spc;
   const uint32_t k = (uint32_t)(seg - c * g.spc);
@@ -477,6 +491,7 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
     }
     const uint32_t padded = (sn + 3) & ~3u;
     for (uint32_t i = tid; i < padded; i += 256) dst[off + i] = i < sn ? exps[seg_base + i] : 0;
+    if (sn == g.seg_syms && tid < NZ_CARRY_BYTES) dst[off + padded + tid] = carry[seg * NZ_CARRY_BYTES + tid];
     return;
   }
   uint32_t off = 0;
@@ -505,6 +520,15 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
 // falls below 2^16 a 16-bit word taken at (words consumed so far by the wave +
 // rank of the lane among the lanes that need one).
 
+// S+1 packed bytes of one 8-element group, as a little-endian integer
+template <int S>
+__device__ __forceinline__ uint64_t nz_load_sm(const uint8_t* p) {
+  if constexpr (S == 7) return *reinterpret_cast<const uint64_t*>(p);
+  else if constexpr (S == 3) return *reinterpret_cast<const uint32_t*>(p);
+  else if constexpr (S == 1) return *reinterpret_cast<const uint16_t*>(p);
+  else return *p;
+}
+
 template <int S>
 __device__ __forceinline__ void nz_store_group(uint16_t* __restrict__ out, uint64_t sm,
                                                const uint32_t (&ex)[8]) {
@@ -517,6 +541,68 @@ __device__ __forceinline__ void nz_store_group(uint16_t* __restrict__ out, uint6
   }
   *reinterpret_cast<uint4*>(out) = make_uint4(o[0], o[1], o[2], o[3]);
 }
+
+// Decoder state of one wavefront.
+struct NzWaveDec {
+  const uint32_t* lut;
+  uint32_t* ring32;
+  const uint32_t* cw;  // renormalisation words of the record, as dwords
+  uint32_t ndw;        // dwords available in the record
+  uint32_t lane;
+  uint32_t x;          // this lane's rANS state
+  uint32_t base;       // words consumed by the wave
+  uint32_t filled;     // dwords staged into the ring
+
+  __device__ __forceinline__ void start(uint32_t x0) {
+    x = x0;
+    // 768 dwords = 1536 words ahead
+#pragma unroll
+    for (uint32_t q = 0; q < 12; ++q) {
+      const uint32_t d = lane + 64 * q;
+      ring32[d] = d < ndw ? cw[d] : 0u;
+    }
+    filled = 768;
+    base = 0;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+
+  // Decode the next 8 symbols of every lane.  A group consumes at most
+  // 8 * 64 words; the ring (2048 words) is topped up by 512 words whenever
+  // fewer than 1536 + 512 are staged, so 512 are always ahead of `base`.
+  __device__ __forceinline__ void group(uint32_t (&ex)[8]) {
+    const bool refill = (2 * filled - base) <= 1536u;
+    uint32_t r[4];
+    if (refill) {
+#pragma unroll
+      for (uint32_t q = 0; q < 4; ++q) {
+        const uint32_t d = filled + lane + 64 * q;
+        r[q] = d < ndw ? cw[d] : 0u;
+      }
+    }
+    const uint16_t* ring = reinterpret_cast<const uint16_t*>(ring32);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t e = lut[x & (NZ_M - 1)];
+      x = (e >> 20) * (x >> NZ_PROB_BITS) + ((e >> 8) & 0xFFFu);
+      ex[j] = e & 0xFFu;
+      const bool need = x < NZ_L;
+      const uint64_t m = __ballot(need);
+      const uint32_t at = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                                    __builtin_amdgcn_mbcnt_lo((uint32_t)m, base));
+      const uint32_t w = ring[at & (NZ_RING_WORDS - 1)];
+      if (need) x = (x << 16) | w;
+      base += (uint32_t)__popcll(m);
+    }
+    if (refill) {
+#pragma unroll
+      for (uint32_t q = 0; q < 4; ++q) ring32[(filled + lane + 64 * q) & (NZ_RING_DWORDS - 1)] = r[q];
+      filled += 256;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+};
 
 template <int S>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
@@ -542,7 +628,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
 
   // record of the chunk's first segment starts with the table
   const uint64_t f0 = dir[seg0], f1 = dir[seg0 + 1];
-  if (f1 < f0 || g.rec_off + 4 * f1 > comp_bytes || f1 == f0) {
+  if (f1 <= f0 || g.rec_off + 4 * f1 > comp_bytes) {
     if (tid == 0) atomicOr(d_status, 2u);
     return;
   }
@@ -570,8 +656,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     }
     if (kk > 256) kk = 256;  // corrupt input: stay inside the staged bytes
     tab_len = (head + (12 * kk + 7) / 8 + 3) & ~3u;
-    __syncthreads();  // everyone has read tb before cum (which follows it) is written
-    // frequency of every symbol -> cum[sym + 1] temporarily
+    // frequency of every symbol -> cum[sym + 1] for now
     for (uint32_t sym = tid; sym < 256; sym += blockDim.x) {
       uint32_t live = 0, rank = 0;
       if (mode == NZ_MODE_BITMAP) {
@@ -650,28 +735,31 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     rec_start += tab_len;
     rec_bytes -= tab_len;
   }
-  const uint8_t* pk = packed + (seg_base * (S + 1)) / 8;
+  // stored packed layout: every full segment keeps seg_p - 128 bytes, its last
+  // 128 bytes ride in the coder states (or behind the symbols of a raw record)
+  const bool carry = seg_n == g.seg_syms;
+  const uint32_t seg_p = g.seg_syms / 8 * (S + 1);
+  const uint32_t keep = seg_p - NZ_CARRY_BYTES;
+  const uint8_t* pk = packed + seg * keep;
   uint16_t* dst = out + seg_base;
 
   if (mode == NZ_MODE_RAW) {
-    if (rec_bytes < seg_n) {
+    const uint32_t padded = (seg_n + 3) & ~3u;
+    if (rec_bytes < padded + (carry ? NZ_CARRY_BYTES : 0u)) {
       if (lane == 0) atomicOr(d_status, 2u);
       return;
     }
     const uint8_t* raw = comp + rec_start;
+    const uint8_t* tailp = raw + padded;
     for (uint32_t gq = 0; gq < ngroups; ++gq) {
       const uint32_t idx0 = (gq * NZ_LANES + lane) * NZ_GROUP;
       if (idx0 >= seg_n) continue;
       const uint32_t rem = seg_n - idx0;
+      const uint32_t b = idx0 / 8 * (S + 1);
       if (rem >= 8) {
         uint64_t sy = (uint64_t)reinterpret_cast<const uint32_t*>(raw + idx0)[0] |
                       ((uint64_t)reinterpret_cast<const uint32_t*>(raw + idx0)[1] << 32);
-        uint64_t sm;
-        const uint8_t* pp = pk + (idx0 * (S + 1)) / 8;
-        if constexpr (S == 7) sm = *reinterpret_cast<const uint64_t*>(pp);
-        else if constexpr (S == 3) sm = *reinterpret_cast<const uint32_t*>(pp);
-        else if constexpr (S == 1) sm = *reinterpret_cast<const uint16_t*>(pp);
-        else sm = *pp;
+        const uint64_t sm = (carry && b >= keep) ? nz_load_sm<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
         uint32_t ex[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) ex[j] = (uint32_t)(sy >> (8 * j)) & 0xFFu;
@@ -691,78 +779,59 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     if (lane == 0) atomicOr(d_status, 2u);
     return;
   }
-  uint32_t x = reinterpret_cast<const uint32_t*>(comp + rec_start)[lane];
-  const uint32_t* cw = reinterpret_cast<const uint32_t*>(comp + rec_start + 256);
-  const uint32_t ndw = (uint32_t)((rec_bytes - 256) / 4);
-  uint32_t* ring32 = rings + wave * NZ_RING_DWORDS;
-  const uint16_t* ring = reinterpret_cast<const uint16_t*>(ring32);
+  NzWaveDec w;
+  w.lut = lut;
+  w.ring32 = rings + wave * NZ_RING_DWORDS;
+  w.cw = reinterpret_cast<const uint32_t*>(comp + rec_start + 256);
+  w.ndw = (uint32_t)((rec_bytes - 256) / 4);
+  w.lane = lane;
+  w.start(reinterpret_cast<const uint32_t*>(comp + rec_start)[lane]);
 
-  // initial fill: 768 dwords = 1536 words
-#pragma unroll
-  for (uint32_t q = 0; q < 12; ++q) {
-    const uint32_t d = lane + 64 * q;
-    ring32[d] = d < ndw ? cw[d] : 0u;
-  }
-  uint32_t filled = 768;  // dwords staged so far
-  uint32_t base = 0;      // words consumed so far
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-
-  for (uint32_t gq = 0; gq < ngroups; ++gq) {
+  // groups whose packed bytes are (partly) carried are merged after the loop
+  const uint32_t tailg = carry ? (S == 0 ? 2u : 1u) : 0u;
+  const uint32_t body = ngroups - tailg;
+  for (uint32_t gq = 0; gq < body; ++gq) {
     const uint32_t idx0 = (gq * NZ_LANES + lane) * NZ_GROUP;
-    // keep at least 512 words ahead of the read position: a group consumes at
-    // most 8 * 64 words, the ring holds 2048.
-    const bool refill = (2 * filled - base) <= 1536u;
-    uint32_t r[4];
-    if (refill) {
-#pragma unroll
-      for (uint32_t q = 0; q < 4; ++q) {
-        const uint32_t d = filled + lane + 64 * q;
-        r[q] = d < ndw ? cw[d] : 0u;
-      }
-    }
     const bool full = idx0 + 8 <= seg_n;
     uint64_t sm = 0;
-    if (full) {
-      const uint8_t* pp = pk + (idx0 * (S + 1)) / 8;
-      if constexpr (S == 7) sm = *reinterpret_cast<const uint64_t*>(pp);
-      else if constexpr (S == 3) sm = *reinterpret_cast<const uint32_t*>(pp);
-      else if constexpr (S == 1) sm = *reinterpret_cast<const uint16_t*>(pp);
-      else sm = *pp;
-    }
+    if (full) sm = nz_load_sm<S>(pk + idx0 / 8 * (S + 1));
     uint32_t ex[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const uint32_t e = lut[x & (NZ_M - 1)];
-      x = (e >> 20) * (x >> NZ_PROB_BITS) + ((e >> 8) & 0xFFFu);
-      ex[j] = e & 0xFFu;
-      const bool need = x < NZ_L;
-      const uint64_t m = __ballot(need);
-      const uint32_t w = ring[(base + nz_rank_below(m)) & (NZ_RING_WORDS - 1)];
-      if (need) x = (x << 16) | w;
-      base += (uint32_t)__popcll(m);
-    }
+    w.group(ex);
     if (full) {
       nz_store_group<S>(dst + idx0, sm, ex);
     } else if (idx0 < seg_n) {
       const uint32_t rem = seg_n - idx0;
       for (uint32_t j = 0; j < rem; ++j) {
-        const uint64_t bit = (uint64_t)(idx0 + j) * (S + 1);
-        const uint32_t rp = ((uint32_t)pk[bit >> 3] >> (7u - S - (uint32_t)(bit & 7u))) & ((2u << S) - 1u);
+        const uint32_t bit = (idx0 + j) * (S + 1);
+        const uint32_t rp = ((uint32_t)pk[bit >> 3] >> (7u - S - (bit & 7u))) & ((2u << S) - 1u);
         dst[idx0 + j] = (uint16_t)nz_merge_one<S>(ex[j], rp);
       }
     }
-    if (refill) {
+  }
+  uint32_t ext[2][8];
 #pragma unroll
-      for (uint32_t q = 0; q < 4; ++q) ring32[(filled + lane + 64 * q) & (NZ_RING_DWORDS - 1)] = r[q];
-      filled += 256;
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+  for (uint32_t t = 0; t < 2; ++t)
+    if (t < tailg) w.group(ext[t]);
+
+  // every lane must be back at the encoder's start state (2^16 | carried bits)
+  // and the wave must not have read past its record
+  const bool bad = (carry ? (w.x >> 16) != 1u : w.x != NZ_L) || (w.base > 2 * w.ndw);
+  if (__ballot(bad) != 0 && lane == 0) atomicOr(d_status, 4u);
+
+  if (carry) {
+    // the ring is dead now: park the 128 carried bytes at its start
+    reinterpret_cast<uint16_t*>(w.ring32)[lane] = (uint16_t)(w.x & 0xFFFFu);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const uint8_t* tailp = reinterpret_cast<const uint8_t*>(w.ring32);
+#pragma unroll
+    for (uint32_t t = 0; t < 2; ++t) {
+      if (t < tailg) {
+        const uint32_t idx0 = ((body + t) * NZ_LANES + lane) * NZ_GROUP;
+        const uint32_t b = idx0 / 8 * (S + 1);
+        const uint64_t sm = b >= keep ? nz_load_sm<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
+        nz_store_group<S>(dst + idx0, sm, ext[t]);
+      }
     }
   }
-  // every lane must be back at the encoder's start state and the wave must
-  // not have read past its record
-  const bool bad = (x != NZ_L) || (base > 2 * ndw);
-  if (__ballot(bad) != 0 && lane == 0) atomicOr(d_status, 4u);
 }
-

@@ -283,7 +283,7 @@ typedef struct {
 } geom_t;
 
 int nzo_check_geometry(uint32_t chunk_syms, uint32_t lane_syms) {
-  if (lane_syms < NZO_GROUP || lane_syms % NZO_GROUP) return NZO_ERR_ARG;
+  if (lane_syms < 16 || lane_syms % NZO_GROUP) return NZO_ERR_ARG;
   if (lane_syms > (1u << 16)) return NZO_ERR_ARG;
   uint64_t seg = (uint64_t)lane_syms * NZO_LANES;
   if (chunk_syms == 0 || chunk_syms % seg) return NZO_ERR_ARG;
@@ -310,15 +310,16 @@ static int make_geom(geom_t* g, uint64_t n, uint32_t chunk_syms, uint32_t lane_s
 
 /* worst-case bytes of one segment record holding seg_n symbols */
 static size_t seg_rec_cap(const geom_t* g) {
-  /* table (<= 420) + states (256) + words (<= seg_syms bytes) ; RAW: 4 + seg_syms */
+  /* table (<= 420) + states (256) + words (<= seg_syms bytes) ; RAW: 4 + seg_syms + 128 */
   return 420 + 256 + (size_t)g->seg_syms + 8;
 }
 
 size_t nzo_exp_bound(uint64_t n, uint32_t chunk_syms, uint32_t lane_syms) {
   geom_t g;
   if (make_geom(&g, n, chunk_syms, lane_syms)) return 0;
-  /* a chunk is never stored larger than its RAW form: 4 + pad4(seg_n) per segment */
-  return g.rec_off + (size_t)n + 4 * (size_t)g.n_segs + 4 * (size_t)g.n_chunks;
+  /* a chunk is never stored larger than its RAW form: 4 per chunk, and per
+     segment pad4(seg_n) symbols + 128 carried bytes */
+  return g.rec_off + (size_t)n + (4 + 2 * NZO_LANES) * (size_t)g.n_segs + 4 * (size_t)g.n_chunks;
 }
 
 static void put32(uint8_t* p, uint32_t v) {
@@ -344,10 +345,11 @@ static uint32_t get16(const uint8_t* p) { return (uint32_t)p[0] | ((uint32_t)p[1
    so that the decoder reads them front to back.  Returns the number of words,
    or -1 when more than cap_words would be needed (segment stored RAW). */
 static int64_t encode_segment(const uint8_t* syms, uint32_t seg_n, int pad_sym,
-                              const uint16_t* freq, const uint16_t* cum, uint16_t* words,
-                              uint32_t cap_words, uint32_t states[NZO_LANES]) {
+                              const uint16_t* freq, const uint16_t* cum, const uint16_t* seeds,
+                              uint16_t* words, uint32_t cap_words, uint32_t states[NZO_LANES]) {
   uint32_t x[NZO_LANES];
-  for (int l = 0; l < NZO_LANES; ++l) x[l] = NZO_L;
+  /* the encoder's start state carries 16 payload bits per lane (see header) */
+  for (int l = 0; l < NZO_LANES; ++l) x[l] = NZO_L | (seeds ? seeds[l] : 0u);
   uint32_t ngroups = (seg_n + NZO_GROUP_SYMS - 1) / NZO_GROUP_SYMS;
   uint32_t pos = cap_words;
   for (uint32_t g = ngroups; g-- > 0;) {
@@ -382,7 +384,7 @@ static int64_t encode_segment(const uint8_t* syms, uint32_t seg_n, int pad_sym,
 }
 
 static int decode_segment(const uint8_t* rec, size_t rec_bytes, uint32_t seg_n,
-                          const uint32_t* lut, uint8_t* out) {
+                          const uint32_t* lut, uint8_t* out, uint16_t* seeds) {
   if (rec_bytes < 256) return NZO_ERR_CORRUPT;
   uint32_t x[NZO_LANES];
   for (int l = 0; l < NZO_LANES; ++l) {
@@ -408,8 +410,12 @@ static int decode_segment(const uint8_t* rec, size_t rec_bytes, uint32_t seg_n,
     }
   }
   if (base > nwords) return NZO_ERR_CORRUPT;
-  for (int l = 0; l < NZO_LANES; ++l)
-    if (x[l] != NZO_L) return NZO_ERR_CORRUPT;
+  for (int l = 0; l < NZO_LANES; ++l) {
+    /* back at the encoder's start state: 2^16 | payload (payload 0 when nothing is carried) */
+    if ((x[l] >> 16) != 1u) return NZO_ERR_CORRUPT;
+    if (seeds) seeds[l] = (uint16_t)(x[l] & 0xFFFFu);
+    else if (x[l] != NZO_L) return NZO_ERR_CORRUPT;
+  }
   return NZO_OK;
 }
 
@@ -420,13 +426,14 @@ static int decode_segment(const uint8_t* rec, size_t rec_bytes, uint32_t seg_n,
 typedef struct {
   const geom_t* g;
   const uint8_t* syms;
+  const uint16_t* seeds; /* 64 per full segment, or NULL */
   uint8_t* scratch;      /* n_segs * seg_rec_cap */
   uint32_t* seg_bytes;   /* n_segs */
   uint64_t c0, c1;       /* chunk range */
 } enc_job_t;
 
-static void encode_chunk(const geom_t* g, const uint8_t* syms, uint64_t c, uint8_t* scratch,
-                         uint32_t* seg_bytes) {
+static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint16_t* seeds, uint64_t c,
+                         uint8_t* scratch, uint32_t* seg_bytes) {
   uint64_t base = c * g->chunk_syms;
   uint64_t cn64 = g->n - base < g->chunk_syms ? g->n - base : g->chunk_syms;
   uint32_t cn = (uint32_t)cn64;
@@ -458,7 +465,9 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, uint64_t c, uint8
     }
     uint32_t states[NZO_LANES];
     uint16_t* words = (uint16_t*)malloc((size_t)g->seg_syms + 8);
-    int64_t nw = encode_segment(cs + (size_t)k * g->seg_syms, sn, pad, freq, cum, words,
+    /* only full segments carry payload in their start states */
+    const uint16_t* sd = (seeds && sn == g->seg_syms) ? seeds + (seg0 + k) * NZO_LANES : NULL;
+    int64_t nw = encode_segment(cs + (size_t)k * g->seg_syms, sn, pad, freq, cum, sd, words,
                                 g->seg_syms / 2, states);
     if (nw < 0) {
       overflow = 1;
@@ -475,7 +484,7 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, uint64_t c, uint8
     free(words);
     seg_bytes[seg0 + k] = (uint32_t)off;
     rans_total += off - (k == 0 ? tbytes : 0);
-    raw_total += ((size_t)sn + 3) & ~(size_t)3;
+    raw_total += (((size_t)sn + 3) & ~(size_t)3) + (sn == g->seg_syms ? 2 * NZO_LANES : 0);
   }
   if (overflow || rans_total >= raw_total) {
     for (uint32_t k = 0; k < nseg; ++k) {
@@ -490,14 +499,21 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, uint64_t c, uint8
       memcpy(rec + off, cs + (size_t)k * g->seg_syms, sn);
       size_t padded = ((size_t)sn + 3) & ~(size_t)3;
       memset(rec + off + sn, 0, padded - sn);
-      seg_bytes[seg0 + k] = (uint32_t)(off + padded);
+      off += padded;
+      if (sn == g->seg_syms) { /* a raw full segment still has to hold its 64 x 16 carried bits */
+        for (int l = 0; l < NZO_LANES; ++l)
+          put16(rec + off + 2 * l, seeds ? seeds[(seg0 + k) * NZO_LANES + l] : 0u);
+        off += 2 * NZO_LANES;
+      }
+      seg_bytes[seg0 + k] = (uint32_t)off;
     }
   }
 }
 
 static void* enc_worker(void* arg) {
   enc_job_t* j = (enc_job_t*)arg;
-  for (uint64_t c = j->c0; c < j->c1; ++c) encode_chunk(j->g, j->syms, c, j->scratch, j->seg_bytes);
+  for (uint64_t c = j->c0; c < j->c1; ++c)
+    encode_chunk(j->g, j->syms, j->seeds, c, j->scratch, j->seg_bytes);
   return NULL;
 }
 
@@ -518,7 +534,7 @@ static void write_header(uint8_t* out, const geom_t* g, uint64_t total) {
 }
 
 int64_t nzo_exp_encode(const uint8_t* syms, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
-                       uint8_t* out, size_t cap, int threads) {
+                       const uint16_t* seeds, uint8_t* out, size_t cap, int threads) {
   geom_t g;
   if (make_geom(&g, n, chunk_syms, lane_syms)) return NZO_ERR_ARG;
   if (cap < g.rec_off) return NZO_ERR_CAP;
@@ -537,6 +553,7 @@ int64_t nzo_exp_encode(const uint8_t* syms, uint64_t n, uint32_t chunk_syms, uin
   for (int t = 0; t < threads; ++t) {
     jobs[t].g = &g;
     jobs[t].syms = syms;
+    jobs[t].seeds = seeds;
     jobs[t].scratch = scratch;
     jobs[t].seg_bytes = seg_bytes;
     jobs[t].c0 = g.n_chunks * (uint64_t)t / (uint64_t)threads;
@@ -594,12 +611,13 @@ typedef struct {
   const uint8_t* comp;
   size_t comp_bytes;
   uint8_t* out;
+  uint16_t* seeds; /* 64 per full segment, or NULL */
   uint64_t c0, c1;
   int status;
 } dec_job_t;
 
 static int decode_chunk(const geom_t* g, const uint8_t* comp, size_t comp_bytes, uint64_t c,
-                        uint8_t* out) {
+                        uint8_t* out, uint16_t* seeds) {
   uint64_t base = c * g->chunk_syms;
   uint32_t cn = (uint32_t)(g->n - base < g->chunk_syms ? g->n - base : g->chunk_syms);
   uint32_t nseg = (cn + g->seg_syms - 1) / g->seg_syms;
@@ -629,11 +647,16 @@ static int decode_chunk(const geom_t* g, const uint8_t* comp, size_t comp_bytes,
         rbytes -= used;
       }
     }
+    uint16_t tmp[NZO_LANES];
+    uint16_t* sd = sn == g->seg_syms ? (seeds ? seeds + (seg0 + k) * NZO_LANES : tmp) : NULL;
     if (raw) {
-      if (rbytes < sn) return NZO_ERR_CORRUPT;
+      size_t padded = ((size_t)sn + 3) & ~(size_t)3;
+      if (rbytes < padded + (sd ? 2 * NZO_LANES : 0)) return NZO_ERR_CORRUPT;
       memcpy(dst, rec, sn);
+      if (sd)
+        for (int l = 0; l < NZO_LANES; ++l) sd[l] = (uint16_t)get16(rec + padded + 2 * l);
     } else {
-      int r = decode_segment(rec, rbytes, sn, lut, dst);
+      int r = decode_segment(rec, rbytes, sn, lut, dst, sd);
       if (r) return r;
     }
   }
@@ -644,7 +667,7 @@ static void* dec_worker(void* arg) {
   dec_job_t* j = (dec_job_t*)arg;
   j->status = NZO_OK;
   for (uint64_t c = j->c0; c < j->c1; ++c) {
-    int r = decode_chunk(j->g, j->comp, j->comp_bytes, c, j->out);
+    int r = decode_chunk(j->g, j->comp, j->comp_bytes, c, j->out, j->seeds);
     if (r) {
       j->status = r;
       break;
@@ -654,7 +677,7 @@ static void* dec_worker(void* arg) {
 }
 
 int nzo_exp_decode(const uint8_t* comp, size_t comp_bytes, uint64_t n, uint8_t* syms_out,
-                   int threads) {
+                   uint16_t* seeds_out, int threads) {
   if (comp_bytes < NZO_HEADER_BYTES) return NZO_ERR_CORRUPT;
   if (get32(comp) != NZO_MAGIC || get32(comp + 4) != NZO_VERSION) return NZO_ERR_CORRUPT;
   uint64_t hn = (uint64_t)get32(comp + 8) | ((uint64_t)get32(comp + 12) << 32);
@@ -678,6 +701,7 @@ int nzo_exp_decode(const uint8_t* comp, size_t comp_bytes, uint64_t n, uint8_t* 
     jobs[t].comp = comp;
     jobs[t].comp_bytes = (size_t)total;
     jobs[t].out = syms_out;
+    jobs[t].seeds = seeds_out;
     jobs[t].c0 = g.n_chunks * (uint64_t)t / (uint64_t)threads;
     jobs[t].c1 = g.n_chunks * (uint64_t)(t + 1) / (uint64_t)threads;
     if (threads == 1)
@@ -748,25 +772,73 @@ static void run_sm(void* (*fn)(void*), const uint16_t* data, uint16_t* out, uint
   free(jobs);
 }
 
+/* Stored layout of the packed sign|mantissa stream: the reference layout
+   (byte idx*(s+1)/8, MSB first) with the last 128 bytes of every FULL segment
+   taken out; those 64 x 16 bits ride in the start states of the segment's 64
+   rANS lanes (lane l carries bytes 2l and 2l+1, little endian). */
+size_t nzo_packed_stored_bytes(uint64_t n, int s, uint32_t lane_syms) {
+  uint64_t seg = (uint64_t)lane_syms * NZO_LANES;
+  return nzo_packed_bytes(n, s) - 2 * NZO_LANES * (size_t)(n / seg);
+}
+
 int64_t nzo_compress_bf16(const uint16_t* data, uint64_t n, int s, uint32_t chunk_syms,
                           uint32_t lane_syms, uint8_t* fractions, uint8_t* comp, size_t cap,
                           int threads) {
   if (!(s == 7 || s == 3 || s == 1 || s == 0)) return NZO_ERR_ARG;
+  if (nzo_check_geometry(chunk_syms, lane_syms)) return NZO_ERR_ARG;
   uint8_t* exps = (uint8_t*)malloc((size_t)n + 1);
-  if (!exps) return NZO_ERR_CAP;
-  run_sm(split_worker, data, NULL, exps, fractions, n, s, threads);
-  int64_t r = nzo_exp_encode(exps, n, chunk_syms, lane_syms, comp, cap, threads);
+  uint8_t* full = (uint8_t*)malloc(nzo_packed_bytes(n, s) + 1);
+  uint64_t seg = (uint64_t)lane_syms * NZO_LANES, nfull = n / seg;
+  uint16_t* seeds = (uint16_t*)malloc((size_t)(nfull + 1) * NZO_LANES * 2);
+  if (!exps || !full || !seeds) {
+    free(exps);
+    free(full);
+    free(seeds);
+    return NZO_ERR_CAP;
+  }
+  run_sm(split_worker, data, NULL, exps, full, n, s, threads);
+  size_t seg_p = (size_t)(seg * (uint64_t)(s + 1) / 8), keep = seg_p - 2 * NZO_LANES;
+  for (uint64_t k = 0; k < nfull; ++k) {
+    memcpy(fractions + k * keep, full + k * seg_p, keep);
+    for (int l = 0; l < NZO_LANES; ++l)
+      seeds[k * NZO_LANES + l] = (uint16_t)get16(full + k * seg_p + keep + 2 * l);
+  }
+  memcpy(fractions + nfull * keep, full + nfull * seg_p, nzo_packed_bytes(n, s) - nfull * seg_p);
+  int64_t r = nzo_exp_encode(exps, n, chunk_syms, lane_syms, seeds, comp, cap, threads);
   free(exps);
+  free(full);
+  free(seeds);
   return r;
 }
 
 int nzo_decompress_bf16(const uint8_t* comp, size_t comp_bytes, const uint8_t* fractions,
                         uint64_t n, int s, uint16_t* data, int threads) {
   if (!(s == 7 || s == 3 || s == 1 || s == 0)) return NZO_ERR_ARG;
+  if (comp_bytes < NZO_HEADER_BYTES) return NZO_ERR_CORRUPT;
+  uint32_t lane_syms = get32(comp + 20);
+  if (nzo_check_geometry(get32(comp + 16), lane_syms)) return NZO_ERR_CORRUPT;
+  uint64_t seg = (uint64_t)lane_syms * NZO_LANES, nfull = n / seg;
   uint8_t* exps = (uint8_t*)malloc((size_t)n + 1);
-  if (!exps) return NZO_ERR_CAP;
-  int r = nzo_exp_decode(comp, comp_bytes, n, exps, threads);
-  if (r == NZO_OK) run_sm(merge_worker, NULL, data, exps, (uint8_t*)fractions, n, s, threads);
+  uint8_t* full = (uint8_t*)malloc(nzo_packed_bytes(n, s) + 1);
+  uint16_t* seeds = (uint16_t*)malloc((size_t)(nfull + 1) * NZO_LANES * 2);
+  if (!exps || !full || !seeds) {
+    free(exps);
+    free(full);
+    free(seeds);
+    return NZO_ERR_CAP;
+  }
+  int r = nzo_exp_decode(comp, comp_bytes, n, exps, seeds, threads);
+  if (r == NZO_OK) {
+    size_t seg_p = (size_t)(seg * (uint64_t)(s + 1) / 8), keep = seg_p - 2 * NZO_LANES;
+    for (uint64_t k = 0; k < nfull; ++k) {
+      memcpy(full + k * seg_p, fractions + k * keep, keep);
+      for (int l = 0; l < NZO_LANES; ++l) put16(full + k * seg_p + keep + 2 * l, seeds[k * NZO_LANES + l]);
+    }
+    memcpy(full + nfull * seg_p, fractions + nfull * keep, nzo_packed_bytes(n, s) - nfull * seg_p);
+    run_sm(merge_worker, NULL, data, exps, full, n, s, threads);
+  }
   free(exps);
+  free(full);
+  free(seeds);
   return r;
 }

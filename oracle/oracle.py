@@ -59,10 +59,12 @@ def lib() -> ctypes.CDLL:
         L.nzo_exp_bound.restype = ctypes.c_size_t
         L.nzo_exp_bound.argtypes = [ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32]
         L.nzo_exp_encode.restype = ctypes.c_int64
-        L.nzo_exp_encode.argtypes = [u8p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32, u8p,
+        L.nzo_exp_encode.argtypes = [u8p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32, u16p, u8p,
                                      ctypes.c_size_t, ctypes.c_int]
         L.nzo_exp_decode.restype = ctypes.c_int
-        L.nzo_exp_decode.argtypes = [u8p, ctypes.c_size_t, ctypes.c_uint64, u8p, ctypes.c_int]
+        L.nzo_exp_decode.argtypes = [u8p, ctypes.c_size_t, ctypes.c_uint64, u8p, u16p, ctypes.c_int]
+        L.nzo_packed_stored_bytes.restype = ctypes.c_size_t
+        L.nzo_packed_stored_bytes.argtypes = [ctypes.c_uint64, ctypes.c_int, ctypes.c_uint32]
         L.nzo_compress_bf16.restype = ctypes.c_int64
         L.nzo_compress_bf16.argtypes = [u16p, ctypes.c_uint64, ctypes.c_int, ctypes.c_uint32,
                                         ctypes.c_uint32, u8p, u8p, ctypes.c_size_t, ctypes.c_int]
@@ -153,24 +155,42 @@ def exp_bound(n: int, chunk_syms: int, lane_syms: int) -> int:
     return int(lib().nzo_exp_bound(n, chunk_syms, lane_syms))
 
 
-def exp_encode(syms: np.ndarray, chunk_syms: int = 65536, lane_syms: int = 512, threads: int = 1) -> np.ndarray:
+def packed_stored_bytes(n: int, s: int, lane_syms: int) -> int:
+    return int(lib().nzo_packed_stored_bytes(n, s, lane_syms))
+
+
+def exp_encode(syms: np.ndarray, chunk_syms: int = 65536, lane_syms: int = 512, threads: int = 1,
+               seeds: np.ndarray | None = None) -> np.ndarray:
+    """Entropy-code a byte stream; `seeds` (uint16, 64 per full segment) is the
+    payload carried in the coder's start states."""
     syms = _u8(syms)
     cap = exp_bound(syms.size, chunk_syms, lane_syms)
     if cap == 0:
         raise ValueError("unsupported geometry")
     out = np.zeros(cap, np.uint8)
-    r = lib().nzo_exp_encode(_p(syms, ctypes.c_uint8), syms.size, chunk_syms, lane_syms,
+    sp = None
+    if seeds is not None:
+        seeds = np.ascontiguousarray(seeds, dtype=np.uint16).reshape(-1)
+        assert seeds.size >= 64 * (syms.size // (64 * lane_syms))
+        sp = _p(seeds, ctypes.c_uint16)
+    r = lib().nzo_exp_encode(_p(syms, ctypes.c_uint8), syms.size, chunk_syms, lane_syms, sp,
                              _p(out, ctypes.c_uint8), cap, threads)
     if r < 0:
         raise RuntimeError(f"nzo_exp_encode failed: {r}")
     return out[:r].copy()
 
 
-def exp_decode(comp: np.ndarray, n: int, threads: int = 1):
+def exp_decode(comp: np.ndarray, n: int, threads: int = 1, lane_syms: int | None = None):
+    """Returns (rc, symbols) or, with lane_syms given, (rc, symbols, seeds)."""
     comp = _u8(comp)
     out = np.zeros(n, np.uint8)
-    rc = lib().nzo_exp_decode(_p(comp, ctypes.c_uint8), comp.size, n, _p(out, ctypes.c_uint8), threads)
-    return int(rc), out
+    if lane_syms is None:
+        rc = lib().nzo_exp_decode(_p(comp, ctypes.c_uint8), comp.size, n, _p(out, ctypes.c_uint8), None, threads)
+        return int(rc), out
+    seeds = np.zeros(64 * (n // (64 * lane_syms)) + 64, np.uint16)
+    rc = lib().nzo_exp_decode(_p(comp, ctypes.c_uint8), comp.size, n, _p(out, ctypes.c_uint8),
+                              _p(seeds, ctypes.c_uint16), threads)
+    return int(rc), out, seeds[: 64 * (n // (64 * lane_syms))]
 
 
 def compress_bf16(bits: np.ndarray, s: int, chunk_syms: int = 65536, lane_syms: int = 512, threads: int = 1):
@@ -180,7 +200,7 @@ def compress_bf16(bits: np.ndarray, s: int, chunk_syms: int = 65536, lane_syms: 
     if cap == 0:
         raise ValueError("unsupported geometry")
     comp = np.zeros(cap, np.uint8)
-    frac = np.zeros(packed_bytes(n, s), np.uint8)
+    frac = np.zeros(packed_stored_bytes(n, s, lane_syms), np.uint8)
     r = lib().nzo_compress_bf16(_p(bits, ctypes.c_uint16), n, s, chunk_syms, lane_syms,
                                 _p(frac, ctypes.c_uint8), _p(comp, ctypes.c_uint8), cap, threads)
     if r < 0:
