@@ -11,7 +11,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libneuzip_hip.so")
+# NEUZIP_HIP_LIB points at an alternative build of the library (development aid)
+LIB_PATH = os.environ.get("NEUZIP_HIP_LIB") or os.path.join(_HERE, "libneuzip_hip.so")
 
 OK = 0
 ERR_ARG, ERR_DTYPE, ERR_NOT_FOUND, ERR_HIP, ERR_CAPACITY, ERR_CORRUPT, ERR_ALIGN, ERR_ALGO = range(-1, -9, -1)

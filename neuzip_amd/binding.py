@@ -98,9 +98,13 @@ class _HipBackend:
         _lib.raise_for(self._L.nz_manager_check(self._h, _stream_ptr(self._device)))
 
     def linear(self, handle: str, inputs: torch.Tensor, shape, bias: torch.Tensor) -> torch.Tensor:
-        # cuda/high_level.cu:252-257: addmm(bias, input, W^T) on a 2-D input
+        # cuda/high_level.cu:252-257: addmm(bias, input, W^T).  The reference only
+        # accepts a 2-D input here; inputs with leading batch dimensions take
+        # the equivalent F.linear route.
         weight = self.read(handle).view(shape)
-        return torch.addmm(bias, inputs, weight.t())
+        if inputs.dim() == 2:
+            return torch.addmm(bias, inputs, weight.t())
+        return torch.nn.functional.linear(inputs, weight, bias)
 
     def linear_without_bias(self, handle: str, inputs: torch.Tensor, shape) -> torch.Tensor:
         # cuda/high_level.cu:259-263

@@ -590,8 +590,11 @@ struct NzWaveDec {
       const uint64_t m = __ballot(need);
       const uint32_t at = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
                                                     __builtin_amdgcn_mbcnt_lo((uint32_t)m, base));
-      const uint32_t w = ring[at & (NZ_RING_WORDS - 1)];
-      if (need) x = (x << 16) | w;
+      uint32_t w = ring[at & (NZ_RING_WORDS - 1)];
+      // keep the word read unconditional: the step stays straight-line code
+      // instead of an exec-mask branch around the LDS read
+      asm volatile("" : "+v"(w));
+      x = need ? ((x << 16) | w) : x;
       base += (uint32_t)__popcll(m);
     }
     if (refill) {
@@ -700,17 +703,26 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
       if (tid == 0) atomicOr(d_status, 2u);
       return;
     }
-    // slot table: binary search of the owning symbol
-    for (uint32_t slot = tid; slot < NZ_M; slot += blockDim.x) {
-      uint32_t lo = 0, hi = 256;  // cum[lo] <= slot < cum[hi]
+    // slot table: the lanes of a wave hold (cum, freq) of four symbols each; the
+    // live symbols are walked with ballot/readlane and every thread of the
+    // workgroup fills a stride of the symbol's slot range.
+    {
+      uint32_t cv[5];
 #pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        uint32_t mid = (lo + hi) >> 1;
-        if (cum[mid] <= slot) lo = mid; else hi = mid;
+      for (int j = 0; j < 5; ++j) cv[j] = cum[4 * lane + j];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t fj = cv[j + 1] - cv[j];
+        uint64_t live = __ballot(fj != 0);
+        while (live) {
+          const int l = __builtin_ctzll(live);
+          live &= live - 1;
+          const uint32_t f = __builtin_amdgcn_readlane(fj, l);
+          const uint32_t cb = __builtin_amdgcn_readlane(cv[j], l);
+          const uint32_t ebase = (f << 20) | (uint32_t)(4 * l + j);
+          for (uint32_t i = tid; i < f; i += blockDim.x) lut[cb + i] = ebase | (i << 8);
+        }
       }
-      const uint32_t cl = cum[lo];
-      const uint32_t f = cum[lo + 1] - cl;
-      lut[slot] = (f << 20) | ((slot - cl) << 8) | lo;
     }
   }
   __syncthreads();

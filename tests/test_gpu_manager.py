@@ -1,0 +1,216 @@
+"""GPU: the Manager / nn / ops surface on the native backend, against the
+oracle's reconstruction and plain torch layers (neuzip/binding.py:55-111,
+neuzip/nn/linear.py, neuzip/ops/linear.py, neuzip/__init__.py:25-35)."""
+from functools import partial
+
+import numpy as np
+import pytest
+
+from conftest import bf16_bits_normal, closed_form_recon
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def bits_of(t):
+    return t.detach().contiguous().view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1)
+
+
+def from_bits(bits, shape, device="cuda"):
+    return torch.from_numpy(bits.view(np.int16).copy()).view(torch.bfloat16).reshape(shape).to(device)
+
+
+@pytest.mark.parametrize("precision", (7, 3, 1, 0))
+def test_write_read_size(oracle, precision):
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=precision)
+    shapes = [(4096, 1024), (3, 5, 7), (1,), (513, 129), (0,)]
+    handles = []
+    for i, shp in enumerate(shapes):
+        n = int(np.prod(shp))
+        w = from_bits(bf16_bits_normal(n, seed=i + precision), shp)
+        h = mgr.write(w)
+        handles.append(h)
+        assert h == str(i)  # auto handles are "0", "1", ... (binding.py:75-76)
+        out = mgr.read(h)
+        assert out.shape == torch.Size(shp) and out.dtype == torch.bfloat16 and not out.requires_grad
+        assert np.array_equal(bits_of(out), oracle.reconstruct(bits_of(w), precision))
+        o_comp, o_packed = oracle.compress_bf16(bits_of(w), precision, 65536, 512)
+        assert mgr.size(h) == o_comp.size + o_packed.size  # exponents + packed bytes held
+        assert mgr._be.packed_bytes(h) == o_packed.size
+    assert mgr.size("nope") == 0  # cuda/high_level.cu:209-211
+    with pytest.raises(KeyError):
+        mgr.read("nope")
+    with pytest.raises(RuntimeError, match="Data not found"):
+        mgr._be.read("nope")
+    mgr._be.check()
+
+
+def test_overwrite_same_handle_and_named_handles(oracle):
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager()
+    a = from_bits(bf16_bits_normal(70_000, 1), (70_000,))
+    b = from_bits(bf16_bits_normal(10_000, 2), (100, 100))
+    assert mgr.write(a, "w") == "w"
+    assert mgr.write(b, "w") == "w"  # erase + insert (cuda/high_level.cu:137-142)
+    assert torch.equal(mgr.read("w"), b)
+    assert mgr.write(a) == "1"  # len(meta_dict) == 1
+    assert torch.equal(mgr.read("1"), a)
+    for _ in range(3):  # rewrite in place with fresh values, as the update hook does
+        a = a * 1.01
+        mgr.write(a, "1")
+        assert torch.equal(mgr.read("1"), a)
+
+
+def test_dtype_and_device_handling():
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager()
+    with pytest.raises(RuntimeError, match="Unsupported data type"):
+        mgr.write(torch.zeros(8, dtype=torch.float32, device="cuda"))
+    with pytest.raises(RuntimeError, match="Unsupported data type"):
+        mgr.write(torch.zeros(8, dtype=torch.float16, device="cuda"))
+    cpu = torch.randn(33, 77).to(torch.bfloat16)
+    h = mgr.write(cpu)  # host tensors are moved to the GPU (cuda/high_level.cu:133-135)
+    out = mgr.read(h)
+    assert out.is_cuda and torch.equal(out.cpu(), cpu)
+    # non-contiguous and oddly offset views
+    base = torch.randn(64, 64, device="cuda").to(torch.bfloat16)
+    h2 = mgr.write(base.t())
+    assert torch.equal(mgr.read(h2), base.t())
+    flat = torch.randn(1001, device="cuda").to(torch.bfloat16)
+    h3 = mgr.write(flat[1:])
+    assert torch.equal(mgr.read(h3), flat[1:])
+
+
+def test_split_api(oracle):
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=3)  # split always uses 7 kept bits (cuda/high_level.cu:289)
+    w = from_bits(bf16_bits_normal(3 * 1000, 5), (3, 1000))
+    e, f = mgr.split(w)
+    assert e.shape == w.shape and f.shape == w.shape and e.dtype == torch.uint8 and f.dtype == torch.uint8
+    oe, of = oracle.split(bits_of(w), 7)
+    assert np.array_equal(e.cpu().numpy().reshape(-1), oe)
+    assert np.array_equal(f.cpu().numpy().reshape(-1), of)
+
+
+@pytest.mark.parametrize("precision", (7, 3))
+@pytest.mark.parametrize("bias", (True, False))
+def test_linear_forward_backward(oracle, precision, bias):
+    import neuzip_amd
+
+    torch.manual_seed(0)
+    mgr = neuzip_amd.Manager(precision=precision)
+    dense = torch.nn.Linear(256, 384, bias=bias).to(torch.bfloat16)
+    dense.weight.data.normal_(0, 0.02)
+    w_rec = from_bits(oracle.reconstruct(bits_of(dense.weight.data), precision), (384, 256))
+    model = torch.nn.Sequential(dense)
+    mgr.convert(model)
+    model = model.cuda()
+    lin = model[0]
+    assert isinstance(lin, neuzip_amd.nn.Linear) and lin.weight.numel() == 0
+    assert torch.equal(lin.weight(), w_rec)
+    for shape in ((7, 256), (2, 5, 256)):
+        x = torch.randn(*shape, device="cuda", dtype=torch.bfloat16)
+        x1, x2 = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+        y1 = lin(x1)
+        y2 = torch.nn.functional.linear(x2, w_rec, lin.bias)
+        assert torch.equal(y1, y2)
+        g = torch.randn_like(y1)
+        lin.weight._gradient = None
+        y1.backward(g)
+        wr = w_rec.clone().requires_grad_(True)
+        torch.nn.functional.linear(x2, wr, lin.bias).backward(g)
+        assert torch.equal(x1.grad, x2.grad)
+        assert torch.allclose(lin.weight._gradient.float(), wr.grad.float(), rtol=1e-2, atol=1e-2)
+        assert lin.weight.grad.numel() == 0
+
+
+def _toy(seed):
+    torch.manual_seed(seed)
+    m = torch.nn.Sequential(torch.nn.Linear(64, 128), torch.nn.GELU(), torch.nn.Linear(128, 64, bias=False)).to(torch.bfloat16)
+    for p in m.parameters():
+        p.data.normal_(0, 0.02)
+    return m
+
+
+class _Sched:
+    def get_last_lr(self):
+        return [0.05]
+
+
+def test_lossless_training_matches_dense_bit_for_bit():
+    """Reference idiom (examples/training/train_clm.py:641-653): SGD applied from
+    post-accumulate hooks; with 7 kept bits the compressed run must equal the
+    dense bf16 run exactly, step after step."""
+    import neuzip_amd
+
+    dense = _toy(3).cuda()
+    comp = _toy(3)
+    mgr = neuzip_amd.Manager(precision=7)
+    mgr.convert(comp)
+    comp = comp.cuda()
+    sched = _Sched()
+    for p in dense.parameters():
+        p.register_post_accumulate_grad_hook(partial(neuzip_amd.lomo_hook, sched))
+    for p in comp.parameters():
+        hook = neuzip_amd.compressed_lomo_hook if isinstance(p, neuzip_amd.nn.Parameter) else neuzip_amd.lomo_hook
+        p.register_post_accumulate_grad_hook(partial(hook, sched))
+    torch.manual_seed(7)
+    for step in range(5):
+        x = torch.randn(16, 64, device="cuda", dtype=torch.bfloat16)
+        l1 = dense(x).float().pow(2).mean()
+        l2 = comp(x).float().pow(2).mean()
+        assert torch.equal(l1, l2), step
+        l1.backward()
+        l2.backward()
+        assert torch.equal(comp[0].weight(), dense[0].weight.data), step
+        assert torch.equal(comp[2].weight(), dense[2].weight.data), step
+        assert torch.equal(comp[0].bias.data, dense[0].bias.data)
+    mgr._be.check()
+
+
+def test_lossy_update_equals_reconstruction_of_update(oracle):
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=3)
+    lin = torch.nn.Linear(96, 80, bias=False).to(torch.bfloat16)
+    lin.weight.data.normal_(0, 0.02)
+    m = torch.nn.Sequential(lin)
+    mgr.convert(m)
+    m = m.cuda()
+    p = m[0].weight
+    w0 = p()
+    p._gradient = torch.randn(80, 96, device="cuda", dtype=torch.bfloat16)
+    want = w0.clone().add_(p._gradient, alpha=-0.05)
+    neuzip_amd.compressed_lomo_hook(_Sched(), p)
+    got = p()
+    assert np.array_equal(bits_of(got), closed_form_recon(bits_of(want), 3))
+
+
+def test_side_stream_write_and_read():
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        w = (torch.randn(2048, 512, device="cuda") * 0.02).to(torch.bfloat16)  # produced on `side`
+        h = mgr.write(w)  # codec kernels are ordered behind the producer on the same stream
+        out = mgr.read(h)
+        assert torch.equal(out, w)
+    side.synchronize()
+
+
+def test_dummy_backend():
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(algorithm=neuzip_amd.Algorithm.dummy)
+    w = torch.randn(4, 8).to(torch.bfloat16)
+    h = mgr.write(w)
+    assert mgr.size(h) == 64 and torch.equal(mgr.read(h).cpu(), w)
+    x = torch.randn(3, 8, device="cuda", dtype=torch.bfloat16)
+    assert torch.equal(mgr.linear(h, x), torch.nn.functional.linear(x, w.cuda()))

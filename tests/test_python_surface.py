@@ -1,0 +1,187 @@
+"""CPU: the Python surface (module conversion, Parameter, CompressedLinear,
+update hooks) against torch reference semantics, with a dense stand-in for the
+native manager so that no GPU is needed.  Mirrors neuzip/utils.py:57-68,
+neuzip/nn/*.py, neuzip/ops/linear.py and neuzip/__init__.py:16-35."""
+import numpy as np
+import pytest
+
+torch = pytest.importorskip("torch")
+
+import neuzip_amd
+from neuzip_amd.nn import Linear, Parameter
+from neuzip_amd.utils import _convert
+
+
+class FakeManager:
+    """CPU manager with the oracle's reconstruction as storage semantics."""
+
+    def __init__(self, oracle, precision=7):
+        self.o, self.s = oracle, precision
+        self.meta_dict, self.store, self.writes = {}, {}, []
+
+    def write(self, tensor, handle=None):
+        key = str(len(self.meta_dict)) if handle is None else handle
+        self.meta_dict[key] = tensor.shape
+        bits = tensor.detach().contiguous().view(torch.int16).numpy().view(np.uint16).reshape(-1)
+        rec = self.o.reconstruct(bits, self.s)
+        self.store[key] = torch.from_numpy(rec.view(np.int16).copy()).view(torch.bfloat16)
+        self.writes.append(key)
+        return key
+
+    def read(self, handle):
+        return self.store[handle].clone().reshape(self.meta_dict[handle])
+
+    def size(self, handle):
+        return self.store[handle].numel()
+
+    def linear(self, handle, inputs, bias=None):
+        return torch.nn.functional.linear(inputs, self.read(handle), bias)
+
+    def convert(self, module):
+        return _convert(self, module)
+
+
+class Block(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.attn = torch.nn.Sequential(torch.nn.Linear(8, 8), torch.nn.ReLU(), torch.nn.Linear(8, 8, bias=False))
+        self.norm = torch.nn.LayerNorm(8)
+
+
+class Toy(torch.nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.embed = torch.nn.Embedding(11, 8)
+        self.layers = torch.nn.ModuleList([Block(), Block()])
+        self.lm_head = torch.nn.Linear(8, 11, bias=False)
+        self.my_lm_head_proj = torch.nn.Linear(8, 8)
+
+
+def test_convert_structure(oracle):
+    model = Toy().to(torch.bfloat16)
+    mgr = FakeManager(oracle)
+    out = mgr.convert(model)
+    assert out is model
+    # every nn.Linear outside names containing "lm_head" is swapped; embeddings are not
+    assert isinstance(model.lm_head, torch.nn.Linear)
+    assert isinstance(model.my_lm_head_proj, torch.nn.Linear)
+    assert isinstance(model.embed, torch.nn.Embedding)
+    converted = [m for m in model.modules() if isinstance(m, Linear)]
+    assert len(converted) == 4
+    assert sorted(mgr.meta_dict) == ["0", "1", "2", "3"]  # handles are str(len(meta_dict))
+    for m in converted:
+        assert isinstance(m.weight, Parameter) and m.weight is m._p
+        assert m.weight.numel() == 0 and m.weight.dtype == torch.bfloat16
+        assert m.weight._shape == (m.out_features, m.in_features)
+        assert repr(m).startswith("Linear(! in_features=")
+    assert model.layers[0].attn[2].bias is None and model.layers[0].attn[0].bias is not None
+
+
+def test_conv1d_is_recognised(oracle):
+    Conv1D = pytest.importorskip("transformers.pytorch_utils").Conv1D
+    from neuzip_amd.utils import _convertible_types
+
+    assert Conv1D in _convertible_types() and torch.nn.Linear in _convertible_types()
+
+
+@pytest.mark.parametrize("precision", (7, 3))
+def test_forward_backward_match_dense_linear(oracle, precision):
+    torch.manual_seed(0)
+    dense = torch.nn.Linear(16, 12).to(torch.bfloat16)
+    dense.weight.data.normal_(0, 0.02)
+    mgr = FakeManager(oracle, precision)
+    comp = Linear(mgr, dense)
+    w_rec = mgr.read("0")
+    ref = torch.nn.Linear(16, 12).to(torch.bfloat16)
+    ref.weight.data.copy_(w_rec)
+    ref.bias.data.copy_(dense.bias.data)
+
+    x = torch.randn(3, 5, 16, dtype=torch.bfloat16)
+    x1, x2 = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    y1, y2 = comp(x1), ref(x2)
+    assert torch.equal(y1, y2)
+    g = torch.randn_like(y1)
+    y1.backward(g)
+    y2.backward(g)
+    assert torch.equal(x1.grad, x2.grad)
+    assert torch.equal(comp.bias.grad, ref.bias.grad)
+    # weight gradient accumulates on _gradient, autograd only sees a zero-size dummy
+    assert torch.equal(comp.weight._gradient, ref.weight.grad)
+    assert comp.weight.grad is not None and comp.weight.grad.numel() == 0
+    y1b = comp(x1)
+    y1b.backward(g)
+    assert torch.equal(comp.weight._gradient, 2 * ref.weight.grad)
+
+
+def test_autocast_cast_and_grad_dtype(oracle):
+    dense = torch.nn.Linear(8, 4, bias=False).to(torch.bfloat16)
+    comp = Linear(FakeManager(oracle), dense)
+    x = torch.randn(2, 8, dtype=torch.float32, requires_grad=True)
+    with torch.autocast("cuda", dtype=torch.bfloat16, enabled=True):
+        if not torch.is_autocast_enabled():
+            pytest.skip("autocast flag cannot be enabled without a GPU build")
+        y = comp(x)
+    assert y.dtype == torch.bfloat16
+    y.float().sum().backward()
+    assert x.grad.dtype == torch.float32  # cast back to the caller's dtype (ops/linear.py:34)
+
+
+class _Sched:
+    def __init__(self, lr):
+        self.lr = lr
+
+    def get_last_lr(self):
+        return [self.lr]
+
+
+def test_compressed_lomo_hook(oracle):
+    torch.manual_seed(1)
+    dense = torch.nn.Linear(8, 8, bias=False).to(torch.bfloat16)
+    mgr = FakeManager(oracle, 7)
+    comp = Linear(mgr, dense)
+    p = comp.weight
+    w0 = mgr.read(p._handle)
+    neuzip_amd.compressed_lomo_hook(_Sched(0.5), p)  # no gradient yet: nothing happens
+    assert mgr.writes == ["0"]
+    p._gradient = torch.ones(8, 8, dtype=torch.bfloat16)
+    neuzip_amd.compressed_lomo_hook(_Sched(0.5), p)
+    assert mgr.writes == ["0", "0"]  # rewritten under the same handle
+    assert p._gradient is None and p.grad is None
+    assert torch.equal(mgr.read(p._handle), w0 - 0.5)
+
+
+def test_post_accumulate_hook_fires(oracle):
+    torch.manual_seed(2)
+    dense = torch.nn.Linear(8, 8).to(torch.bfloat16)
+    mgr = FakeManager(oracle, 7)
+    comp = Linear(mgr, dense)
+    w0 = mgr.read("0")
+    from functools import partial
+
+    comp.weight.register_post_accumulate_grad_hook(partial(neuzip_amd.compressed_lomo_hook, _Sched(0.25)))
+    x = torch.randn(4, 8, dtype=torch.bfloat16)
+    comp(x).float().sum().backward()
+    gw = torch.mm(torch.ones(4, 8, dtype=torch.bfloat16).t(), x)
+    assert torch.equal(mgr.read("0"), w0 - 0.25 * gw)
+    assert comp.weight._gradient is None
+
+
+def test_lomo_hook_dense():
+    p = torch.nn.Parameter(torch.ones(3))
+    neuzip_amd.lomo_hook(_Sched(0.1), p)  # no grad: no-op
+    p.grad = torch.full((3,), 2.0)
+    neuzip_amd.lomo_hook(_Sched(0.1), p)
+    assert torch.allclose(p.data, torch.full((3,), 0.8)) and p.grad is None
+
+
+def test_manager_argument_errors():
+    A = neuzip_amd.Algorithm
+    assert {m.name for m in A} == {"ans", "gdeflate", "zstd", "dummy"}  # neuzip/binding.py:23-27
+    with pytest.raises(AttributeError, match="Manager_f5_n0"):
+        neuzip_amd.Manager(precision=5)
+    with pytest.raises(AttributeError, match="Manager_f7_n3"):
+        neuzip_amd.Manager(normalizer_size=3)
+    with pytest.raises(RuntimeError, match="Unsupported algorithm"):
+        neuzip_amd.Manager(algorithm=A.zstd)
+    with pytest.raises(NotImplementedError):
+        neuzip_amd.Manager(normalizer_size=32)
