@@ -46,6 +46,8 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--cpu-threads", type=int, default=0, help="0 = all host cores given to this process")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run five plain 256 MiB device copies (to scale FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
 
 
@@ -124,6 +126,16 @@ def main():
     if not torch.cuda.is_available():
         print("no GPU visible", file=sys.stderr)
         return 2
+
+    if args.calibrate_copy:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "5 device copies", "bytes_read_per_copy": 256 << 20,
+                          "bytes_written_per_copy": 256 << 20}))
+        return 0
 
     n = args.rows * args.cols
     lane = args.lane_symbols or lib_mod.DEFAULT_LANE_SYMS
