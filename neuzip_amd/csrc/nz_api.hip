@@ -116,7 +116,7 @@ int encode_phase2(const NzGeom& g, uint8_t* ws, const EncLayout& L, const uint32
 template <int S>
 void launch_decode(const NzGeom& g, const void* comp, uint64_t comp_bytes, const void* packed,
                    void* out, uint32_t* d_status, hipStream_t st) {
-  const size_t lds = (NZ_M + g.spc * NZ_RING_DWORDS + 384) * 4;
+  const size_t lds = (2 * NZ_M + g.spc * NZ_RING_ALLOC_DWORDS) * 4;
   hipLaunchKernelGGL(nz_decode_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(64 * g.spc), lds, st,
                      (const uint8_t*)comp, comp_bytes, (const uint8_t*)packed, (uint16_t*)out, g,
                      d_status);

@@ -514,11 +514,18 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
 // fused rANS decode + merge: one workgroup per chunk, one wavefront per segment
 // ----------------------------------------------------------------------------
 //
-// LDS: 4096-entry slot table (freq << 20 | (slot - cum) << 8 | symbol), then a
-// 4 KiB ring of renormalisation words per wavefront, then table-parse scratch.
+// LDS: a 4096-entry slot table of 8-byte entries
+//          lo = freq | symbol << 24      hi = slot - cum[symbol]
+//      (so that one v_mad_u32_u24 of lo's low 24 bits gives the next state and
+//      the symbol is a whole byte for v_perm_b32) and a ring of 2048
+//      renormalisation words per wavefront; the table-parse scratch aliases the
+//      rings (it is dead before the first ring is filled).  Two wavefronts per
+//      chunk need exactly 40 KiB, so four workgroups share the 160 KiB of a CU.
 // A rANS step per lane: one table read, one multiply-add, and when the state
 // falls below 2^16 a 16-bit word taken at (words consumed so far by the wave +
 // rank of the lane among the lanes that need one).
+
+#define NZ_RING_ALLOC_DWORDS NZ_RING_DWORDS
 
 // S+1 packed bytes of one 8-element group, as a little-endian integer
 template <int S>
@@ -529,80 +536,120 @@ __device__ __forceinline__ uint64_t nz_load_sm(const uint8_t* p) {
   else return *p;
 }
 
+// Merge 8 exponents (byte 3 of ew[j]) with the group's packed bytes and store
+// 8 bf16 values with one 16-byte store.
 template <int S>
 __device__ __forceinline__ void nz_store_group(uint16_t* __restrict__ out, uint64_t sm,
-                                               const uint32_t (&ex)[8]) {
+                                               const uint32_t (&ew)[8]) {
   uint32_t o[4];
+  if constexpr (S == 7) {
+    // out16 = sign << 15 | exp << 7 | mant, byte b = sign << 7 | mant.  Per pair:
+    //   t = exponents at bits 7..14 and 23..30 (two v_perm bytes, one shift)
+    //   u = bytes [b0 b0 b1 b1]: sign lands on bit 15 / 31, mantissa on 0..6 / 16..22
+    //   out = bitfield insert of t's exponent bits into u
+    const uint32_t lo = (uint32_t)sm, hi = (uint32_t)(sm >> 32);
 #pragma unroll
-  for (int j = 0; j < 8; j += 2) {
-    uint32_t r0 = (uint32_t)(sm >> nz_field_shift<S>(j)) & ((2u << S) - 1u);
-    uint32_t r1 = (uint32_t)(sm >> nz_field_shift<S>(j + 1)) & ((2u << S) - 1u);
-    o[j >> 1] = nz_merge_one<S>(ex[j], r0) | (nz_merge_one<S>(ex[j + 1], r1) << 16);
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t q = __builtin_amdgcn_perm(ew[2 * k + 1], ew[2 * k], 0x0c070c03u);
+      const uint32_t t = q << 7;
+      const uint32_t w = k < 2 ? lo : hi;
+      const uint32_t u = __builtin_amdgcn_perm(0u, w, (k & 1) ? 0x03030202u : 0x01010000u);
+      o[k] = (t & 0x7F807F80u) | (u & ~0x7F807F80u);
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      uint32_t r0 = (uint32_t)(sm >> nz_field_shift<S>(j)) & ((2u << S) - 1u);
+      uint32_t r1 = (uint32_t)(sm >> nz_field_shift<S>(j + 1)) & ((2u << S) - 1u);
+      o[j >> 1] = nz_merge_one<S>(ew[j] >> 24, r0) | (nz_merge_one<S>(ew[j + 1] >> 24, r1) << 16);
+    }
   }
   *reinterpret_cast<uint4*>(out) = make_uint4(o[0], o[1], o[2], o[3]);
 }
 
 // Decoder state of one wavefront.
 struct NzWaveDec {
-  const uint32_t* lut;
+  const uint2* lut;
   uint32_t* ring32;
-  const uint32_t* cw;  // renormalisation words of the record, as dwords
-  uint32_t ndw;        // dwords available in the record
+  const uint32_t* rec;  // the record as dwords: 64 states, then the renormalisation words
+  uint32_t last;        // index of the last dword of the record (>= 63)
   uint32_t lane;
   uint32_t x;          // this lane's rANS state
   uint32_t base;       // words consumed by the wave
   uint32_t filled;     // dwords staged into the ring
 
-  __device__ __forceinline__ void start(uint32_t x0) {
-    x = x0;
+  __device__ __forceinline__ void ring_put(uint32_t d, uint32_t v) {
+    ring32[d & (NZ_RING_DWORDS - 1)] = v;
+  }
+
+  // Word dword d of the record; indices past the end are clamped to the last
+  // dword so that every load is unconditional and in bounds (a valid stream
+  // never consumes those words).
+  __device__ __forceinline__ uint32_t word_dword(uint32_t d) const {
+    const uint32_t i = 64u + d;
+    return rec[i < last ? i : last];
+  }
+
+  __device__ __forceinline__ void start() {
+    x = rec[lane];
     // 768 dwords = 1536 words ahead
+    uint32_t v[12];
 #pragma unroll
-    for (uint32_t q = 0; q < 12; ++q) {
-      const uint32_t d = lane + 64 * q;
-      ring32[d] = d < ndw ? cw[d] : 0u;
-    }
+    for (uint32_t q = 0; q < 12; ++q) v[q] = word_dword(lane + 64 * q);
+#pragma unroll
+    for (uint32_t q = 0; q < 12; ++q) ring_put(lane + 64 * q, v[q]);
     filled = 768;
     base = 0;
+    pend = false;
+#pragma unroll
+    for (uint32_t q = 0; q < 4; ++q) r[q] = 0;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
 
-  // Decode the next 8 symbols of every lane.  A group consumes at most
-  // 8 * 64 words; the ring (2048 words) is topped up by 512 words whenever
-  // fewer than 1536 + 512 are staged, so 512 are always ahead of `base`.
-  __device__ __forceinline__ void group(uint32_t (&ex)[8]) {
-    const bool refill = (2 * filled - base) <= 1536u;
-    uint32_t r[4];
-    if (refill) {
+  // Decode the next 8 symbols of every lane into byte 3 of ew[0..7].
+  //
+  // Ring upkeep is software-pipelined over two groups so that no load is
+  // waited for in the group that issued it: at the start of a group the 512
+  // words fetched during the previous group are committed to the ring if that
+  // fetch was wanted (`pend`), then the next 512 words are fetched into
+  // registers unconditionally (clamped addresses, mostly cache hits) and marked
+  // wanted when no more than 1024 words are staged ahead.  A group consumes at
+  // most 8 * 64 = 512 words, so at least 512 words are ahead of `base` at every
+  // group start and the window [base, filled) never exceeds 1536 of the 2048
+  // ring words.
+  uint32_t r[4];
+  bool pend;
+
+  __device__ __forceinline__ void group(uint32_t (&ew)[8]) {
+    if (pend) {
 #pragma unroll
-      for (uint32_t q = 0; q < 4; ++q) {
-        const uint32_t d = filled + lane + 64 * q;
-        r[q] = d < ndw ? cw[d] : 0u;
-      }
-    }
-    const uint16_t* ring = reinterpret_cast<const uint16_t*>(ring32);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const uint32_t e = lut[x & (NZ_M - 1)];
-      x = (e >> 20) * (x >> NZ_PROB_BITS) + ((e >> 8) & 0xFFFu);
-      ex[j] = e & 0xFFu;
-      const bool need = x < NZ_L;
-      const uint64_t m = __ballot(need);
-      const uint32_t at = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
-                                                    __builtin_amdgcn_mbcnt_lo((uint32_t)m, base));
-      uint32_t w = ring[at & (NZ_RING_WORDS - 1)];
-      // keep the word read unconditional: the step stays straight-line code
-      // instead of an exec-mask branch around the LDS read
-      asm volatile("" : "+v"(w));
-      x = need ? ((x << 16) | w) : x;
-      base += (uint32_t)__popcll(m);
-    }
-    if (refill) {
-#pragma unroll
-      for (uint32_t q = 0; q < 4; ++q) ring32[(filled + lane + 64 * q) & (NZ_RING_DWORDS - 1)] = r[q];
+      for (uint32_t q = 0; q < 4; ++q) ring_put(filled + lane + 64 * q, r[q]);
       filled += 256;
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
+    }
+    pend = (2 * filled - base) <= 1024u;
+#pragma unroll
+    for (uint32_t q = 0; q < 4; ++q) r[q] = word_dword(filled + lane + 64 * q);
+    const uint16_t* ring = reinterpret_cast<const uint16_t*>(ring32);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint2 e = lut[x & (NZ_M - 1)];
+      x = __umul24(e.x, x >> NZ_PROB_BITS) + e.y;
+      ew[j] = e.x;
+      const bool need = x < NZ_L;
+      const uint64_t m = __ballot(need);
+      const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                                      __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+      uint32_t w = ring[(base + rank) & (NZ_RING_WORDS - 1)];
+      // keep the word read unconditional: straight-line code, no exec-mask branch
+      asm volatile("" : "+v"(w));
+      // renormalise: x = x << 16 | w, as one byte permute whose selector was
+      // chosen while the word was in flight
+      const uint32_t sel = need ? 0x05040100u : 0x07060504u;
+      x = __builtin_amdgcn_perm(x, w, sel);
+      base += (uint32_t)__popcll(m);
     }
   }
 };
@@ -612,14 +659,14 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
     uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status) {
   extern __shared__ uint32_t lds[];
-  uint32_t* lut = lds;                                   // 4096 dwords
-  uint32_t* rings = lds + NZ_M;                          // spc * 1024 dwords
-  uint32_t* scratch = rings + g.spc * NZ_RING_DWORDS;    // 106 + 257 dwords
-  uint8_t* tb = reinterpret_cast<uint8_t*>(scratch);     // table bytes (424)
-  uint32_t* cum = scratch + NZ_TABLE_MAX_BYTES / 4;      // 257 entries
+  uint2* lut = reinterpret_cast<uint2*>(lds);                   // 4096 x 8 bytes
+  uint32_t* rings = lds + 2 * NZ_M;                             // spc rings
+  uint32_t* scratch = rings;                                    // 106 + 257 dwords, dead before the rings fill
+  uint8_t* tb = reinterpret_cast<uint8_t*>(scratch);            // table bytes (424)
+  uint32_t* cum = scratch + NZ_TABLE_MAX_BYTES / 4;             // 257 entries
 
   const uint32_t tid = threadIdx.x;
-  const uint32_t wave = tid >> 6;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keep it scalar
   const uint32_t lane = tid & 63;
   const uint64_t c = blockIdx.x;
   const uint64_t seg0 = c * g.spc;
@@ -719,8 +766,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
           live &= live - 1;
           const uint32_t f = __builtin_amdgcn_readlane(fj, l);
           const uint32_t cb = __builtin_amdgcn_readlane(cv[j], l);
-          const uint32_t ebase = (f << 20) | (uint32_t)(4 * l + j);
-          for (uint32_t i = tid; i < f; i += blockDim.x) lut[cb + i] = ebase | (i << 8);
+          const uint32_t elo = f | ((uint32_t)(4 * l + j) << 24);
+          for (uint32_t i = tid; i < f; i += blockDim.x) lut[cb + i] = make_uint2(elo, i);
         }
       }
     }
@@ -772,10 +819,10 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
         uint64_t sy = (uint64_t)reinterpret_cast<const uint32_t*>(raw + idx0)[0] |
                       ((uint64_t)reinterpret_cast<const uint32_t*>(raw + idx0)[1] << 32);
         const uint64_t sm = (carry && b >= keep) ? nz_load_sm<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
-        uint32_t ex[8];
+        uint32_t ew[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ex[j] = (uint32_t)(sy >> (8 * j)) & 0xFFu;
-        nz_store_group<S>(dst + idx0, sm, ex);
+        for (int j = 0; j < 8; ++j) ew[j] = (uint32_t)((sy >> (8 * j)) & 0xFFu) << 24;
+        nz_store_group<S>(dst + idx0, sm, ew);
       } else {
         for (uint32_t j = 0; j < rem; ++j) {
           const uint32_t bit = (idx0 + j) * (S + 1);
@@ -793,30 +840,43 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
   }
   NzWaveDec w;
   w.lut = lut;
-  w.ring32 = rings + wave * NZ_RING_DWORDS;
-  w.cw = reinterpret_cast<const uint32_t*>(comp + rec_start + 256);
-  w.ndw = (uint32_t)((rec_bytes - 256) / 4);
+  w.ring32 = rings + wave * NZ_RING_ALLOC_DWORDS;
+  w.rec = reinterpret_cast<const uint32_t*>(comp + rec_start);
+  w.last = (uint32_t)(rec_bytes / 4) - 1u;
   w.lane = lane;
-  w.start(reinterpret_cast<const uint32_t*>(comp + rec_start)[lane]);
+  w.start();
 
   // groups whose packed bytes are (partly) carried are merged after the loop
   const uint32_t tailg = carry ? (S == 0 ? 2u : 1u) : 0u;
   const uint32_t body = ngroups - tailg;
-  for (uint32_t gq = 0; gq < body; ++gq) {
-    const uint32_t idx0 = (gq * NZ_LANES + lane) * NZ_GROUP;
-    const bool full = idx0 + 8 <= seg_n;
-    uint64_t sm = 0;
-    if (full) sm = nz_load_sm<S>(pk + idx0 / 8 * (S + 1));
-    uint32_t ex[8];
-    w.group(ex);
-    if (full) {
-      nz_store_group<S>(dst + idx0, sm, ex);
-    } else if (idx0 < seg_n) {
-      const uint32_t rem = seg_n - idx0;
+  // Groups in which every lane has 8 elements run without any predicate; the
+  // packed bytes are fetched one group ahead of their use (the address of the
+  // fetch past the last group is clamped, its value unused).
+  const uint32_t whole = seg_n / NZ_GROUP_SYMS < body ? seg_n / NZ_GROUP_SYMS : body;
+  const uint32_t lane_off = lane * (S + 1);
+  const uint32_t last_off = whole ? (whole - 1) * NZ_LANES * (S + 1) + lane_off : 0u;
+  uint64_t sm_next = whole ? nz_load_sm<S>(pk + lane_off) : 0;
+  for (uint32_t gq = 0; gq < whole; ++gq) {
+    const uint64_t sm = sm_next;
+    const uint32_t noff = (gq + 1) * NZ_LANES * (S + 1) + lane_off;
+    sm_next = nz_load_sm<S>(pk + (noff < last_off ? noff : last_off));
+    uint32_t ew[8];
+    w.group(ew);
+    nz_store_group<S>(dst + (gq * NZ_LANES + lane) * NZ_GROUP, sm, ew);
+  }
+  if (whole < body) {  // the ragged last group of the tensor
+    const uint32_t idx0 = (whole * NZ_LANES + lane) * NZ_GROUP;
+    uint32_t ew[8];
+    w.group(ew);
+    if (idx0 < seg_n) {
+      const uint32_t rem = seg_n - idx0 < 8 ? seg_n - idx0 : 8;
       for (uint32_t j = 0; j < rem; ++j) {
         const uint32_t bit = (idx0 + j) * (S + 1);
         const uint32_t rp = ((uint32_t)pk[bit >> 3] >> (7u - S - (bit & 7u))) & ((2u << S) - 1u);
-        dst[idx0 + j] = (uint16_t)nz_merge_one<S>(ex[j], rp);
+        uint32_t sym = 0;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) sym = (uint32_t)q == j ? (ew[q] >> 24) : sym;
+        dst[idx0 + j] = (uint16_t)nz_merge_one<S>(sym, rp);
       }
     }
   }
@@ -827,7 +887,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
 
   // every lane must be back at the encoder's start state (2^16 | carried bits)
   // and the wave must not have read past its record
-  const bool bad = (carry ? (w.x >> 16) != 1u : w.x != NZ_L) || (w.base > 2 * w.ndw);
+  const bool bad = (carry ? (w.x >> 16) != 1u : w.x != NZ_L) || (w.base > 2 * (w.last - 63u));
   if (__ballot(bad) != 0 && lane == 0) atomicOr(d_status, 4u);
 
   if (carry) {
