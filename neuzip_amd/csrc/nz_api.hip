@@ -54,7 +54,7 @@ EncLayout enc_layout(const NzGeom& g) {
   L.states = take(g.n_segs * NZ_LANES * 4);
   L.seg_words = take(g.n_segs * 4);
   L.seg_units = take((g.n_segs + 1) * 4);
-  L.hdr = take(g.rec_off);
+  L.hdr = take(g.rec_off + NZ_TAIL_PAD);
   L.total = take(8);
   L.status = take(4);
   L.bytes = o;
@@ -251,7 +251,7 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
   if (((uintptr_t)dev_comp & 15) || ((uintptr_t)dev_packed & 7))
     return fail(NZ_ERR_ALIGN, "comp/packed buffers must be 16/8-byte aligned");
   if (check && !dev_status) return fail(NZ_ERR_ARG, "check requires dev_status");
-  if (comp_bytes < g.rec_off) return fail(NZ_ERR_CORRUPT, "container shorter than its directory");
+  if (comp_bytes < g.rec_off + NZ_TAIL_PAD) return fail(NZ_ERR_CORRUPT, "container shorter than its directory");
   hipStream_t st = (hipStream_t)stream;
   if (int rc = decode_launch(g, precision, dev_comp, comp_bytes, dev_packed, dev_bf16_out, dev_status, st))
     return rc;
@@ -387,7 +387,8 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
     }
   }
   if (rc == NZ_OK) {
-    e = hipMemcpyAsync(ent.comp, ws + L.hdr, g.rec_off, hipMemcpyDeviceToDevice, st);
+    e = hipMemcpyAsync(ent.comp, ws + L.hdr, g.rec_off + (g.n_segs ? 0 : NZ_TAIL_PAD),
+                       hipMemcpyDeviceToDevice, st);
     if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("header copy: ") + hipGetErrorString(e));
   }
   if (rc == NZ_OK)

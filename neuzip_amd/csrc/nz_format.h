@@ -3,7 +3,7 @@
 // The exponent stream of one tensor (N bytes, one per bf16 element) is stored
 // as
 //
-//   header (64 B) | directory ((n_segs + 1) x u32) | segment records
+//   header (64 B) | directory ((n_segs + 1) x u32) | segment records | 16 zero bytes
 //
 // * chunk   = `chunk_syms` consecutive exponents that share one 12-bit
 //             frequency table (the reference hands nvcomp the same unit:
@@ -45,6 +45,7 @@
 #define NZ_TABLE_MAX_BYTES 424 /* 1 + 32 + 384 rounded up to a multiple of 8 */
 #define NZ_MAX_SEGS_PER_CHUNK 8
 #define NZ_CARRY_BYTES 128 /* 64 lanes x 16 bits */
+#define NZ_TAIL_PAD 16     /* zero bytes after the last record: 16-byte loads stay inside */
 
 struct NzGeom {
   uint64_t n;
@@ -93,7 +94,7 @@ static inline int nz_geom_make(NzGeom* g, uint64_t n, uint32_t chunk_syms, uint3
 
 // Upper bound of the container size: no chunk is ever stored larger than raw.
 static inline uint64_t nz_geom_bound(const NzGeom* g) {
-  return g->rec_off + g->n + (4 + NZ_CARRY_BYTES) * g->n_segs + 4 * g->n_chunks;
+  return g->rec_off + g->n + (4 + NZ_CARRY_BYTES) * g->n_segs + 4 * g->n_chunks + NZ_TAIL_PAD;
 }
 
 static inline uint64_t nz_packed_bytes_of(uint64_t n, int s) {

@@ -444,7 +444,9 @@ __global__ __launch_bounds__(1024) void nz_scan_kernel(const uint32_t* __restric
     dir[g.n_segs] = (uint32_t)units;
     // zero the alignment gap between directory and records
     for (uint64_t b = g.dir_off + 4 * (g.n_segs + 1); b < g.rec_off; ++b) comp[b] = 0;
-    const uint64_t total = g.rec_off + 4 * units;
+    const uint64_t total = g.rec_off + 4 * units + NZ_TAIL_PAD;
+    if (g.n_segs == 0)  // otherwise the last segment's compaction writes the closing zeros
+      for (uint32_t b = 0; b < NZ_TAIL_PAD; ++b) comp[g.rec_off + b] = 0;
     uint32_t* h = reinterpret_cast<uint32_t*>(comp);
     h[0] = NZ_MAGIC;
     h[1] = NZ_FORMAT_VERSION;
@@ -477,8 +479,10 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
   const uint64_t c = seg / g.spc;
   const uint32_t k = (uint32_t)(seg - c * g.spc);
   const uint64_t o0 = dir[seg], o1 = dir[seg + 1];
-  if (g.rec_off + 4 * o1 > cap) return;  // flagged by the scan kernel
+  if (g.rec_off + 4 * o1 + NZ_TAIL_PAD > cap) return;  // flagged by the scan kernel
   uint8_t* dst = comp + g.rec_off + 4 * o0;
+  if (seg + 1 == g.n_segs && threadIdx.x >= 256 - NZ_TAIL_PAD)  // closing zeros
+    comp[g.rec_off + 4 * o1 + (threadIdx.x - (256 - NZ_TAIL_PAD))] = 0;
   const uint64_t seg_base = seg * g.seg_syms;
   const uint32_t sn = (uint32_t)((g.n - seg_base) < g.seg_syms ? (g.n - seg_base) : g.seg_syms);
   const NzChunkInfo ci = info[c];
@@ -570,39 +574,44 @@ __device__ __forceinline__ void nz_store_group(uint16_t* __restrict__ out, uint6
 // Decoder state of one wavefront.
 struct NzWaveDec {
   const uint2* lut;
-  uint32_t* ring32;
-  const uint32_t* rec;  // the record as dwords: 64 states, then the renormalisation words
-  uint32_t last;        // index of the last dword of the record (>= 63)
+  uint32_t* ring32;       // 1024 dwords = 2048 words
+  const uint8_t* words;   // first renormalisation word of the record (uniform)
+  const uint8_t* last16;  // last 16-byte block that may be loaded: container end - 16 (uniform)
+  uint32_t nwords;        // words the record holds
   uint32_t lane;
-  uint32_t x;          // this lane's rANS state
-  uint32_t base;       // words consumed by the wave
-  uint32_t filled;     // dwords staged into the ring
+  uint32_t x;             // this lane's rANS state
+  uint32_t base;          // words consumed by the wave
+  uint32_t filled;        // dwords staged into the ring (multiple of 256)
+  uint4 r;                // 8 words fetched during the previous group
+  bool pend;              // ... and whether they are to be committed
 
-  __device__ __forceinline__ void ring_put(uint32_t d, uint32_t v) {
-    ring32[d & (NZ_RING_DWORDS - 1)] = v;
+  // 16 bytes of the word stream at dword index d (multiple of 4 per lane).
+  // Addresses are clamped to the container's closing padding, so every load is
+  // unconditional and in bounds; words past the record are never consumed by
+  // a valid stream.
+  __device__ __forceinline__ uint4 fetch(uint32_t d) const {
+    const uint8_t* p = words + 4ull * d;
+    p = p < last16 ? p : last16;
+    const uint32_t* q = reinterpret_cast<const uint32_t*>(p);
+    return make_uint4(q[0], q[1], q[2], q[3]);
   }
 
-  // Word dword d of the record; indices past the end are clamped to the last
-  // dword so that every load is unconditional and in bounds (a valid stream
-  // never consumes those words).
-  __device__ __forceinline__ uint32_t word_dword(uint32_t d) const {
-    const uint32_t i = 64u + d;
-    return rec[i < last ? i : last];
+  __device__ __forceinline__ void commit(uint32_t d, const uint4& v) {
+    *reinterpret_cast<uint4*>(ring32 + (d & (NZ_RING_DWORDS - 1))) = v;
   }
 
-  __device__ __forceinline__ void start() {
-    x = rec[lane];
+  __device__ __forceinline__ void start(uint32_t x0) {
+    x = x0;
     // 768 dwords = 1536 words ahead
-    uint32_t v[12];
+    uint4 v[3];
 #pragma unroll
-    for (uint32_t q = 0; q < 12; ++q) v[q] = word_dword(lane + 64 * q);
+    for (uint32_t q = 0; q < 3; ++q) v[q] = fetch(256 * q + 4 * lane);
 #pragma unroll
-    for (uint32_t q = 0; q < 12; ++q) ring_put(lane + 64 * q, v[q]);
+    for (uint32_t q = 0; q < 3; ++q) commit(256 * q + 4 * lane, v[q]);
     filled = 768;
     base = 0;
     pend = false;
-#pragma unroll
-    for (uint32_t q = 0; q < 4; ++q) r[q] = 0;
+    r = make_uint4(0, 0, 0, 0);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
@@ -618,21 +627,21 @@ struct NzWaveDec {
   // most 8 * 64 = 512 words, so at least 512 words are ahead of `base` at every
   // group start and the window [base, filled) never exceeds 1536 of the 2048
   // ring words.
-  uint32_t r[4];
-  bool pend;
-
   __device__ __forceinline__ void group(uint32_t (&ew)[8]) {
     if (pend) {
-#pragma unroll
-      for (uint32_t q = 0; q < 4; ++q) ring_put(filled + lane + 64 * q, r[q]);
+      commit(filled + 4 * lane, r);
       filled += 256;
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
     }
     pend = (2 * filled - base) <= 1024u;
-#pragma unroll
-    for (uint32_t q = 0; q < 4; ++q) r[q] = word_dword(filled + lane + 64 * q);
-    const uint16_t* ring = reinterpret_cast<const uint16_t*>(ring32);
+    r = fetch(filled + 4 * lane);
+    // LDS byte address of the ring (4 KiB aligned inside the workgroup's LDS)
+    typedef __attribute__((address_space(3))) uint32_t lds_u32;
+    typedef __attribute__((address_space(3))) const uint16_t lds_cu16;
+    const uint32_t ring_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((lds_u32*)ring32));
+    uint32_t wmask = 2 * NZ_RING_WORDS - 2;  // kept in a VGPR: v_and_or_b32 takes one scalar operand
+    asm volatile("" : "+v"(wmask));
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const uint2 e = lut[x & (NZ_M - 1)];
@@ -642,7 +651,10 @@ struct NzWaveDec {
       const uint64_t m = __ballot(need);
       const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
                                                       __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-      uint32_t w = ring[(base + rank) & (NZ_RING_WORDS - 1)];
+      // word (base + rank) mod 2048 of the ring: add-shift, then bitfield insert
+      uint32_t at;
+      asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(at) : "v"((rank + base) << 1), "v"(wmask), "s"(ring_addr));
+      uint32_t w = *(lds_cu16*)(uintptr_t)at;
       // keep the word read unconditional: straight-line code, no exec-mask branch
       asm volatile("" : "+v"(w));
       // renormalise: x = x << 16 | w, as one byte permute whose selector was
@@ -838,13 +850,17 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     if (lane == 0) atomicOr(d_status, 2u);
     return;
   }
+  // the record position is the same for all lanes: keep it in scalar registers
+  const uint64_t rs = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(rec_start >> 32)) << 32) |
+                      __builtin_amdgcn_readfirstlane((uint32_t)rec_start);
   NzWaveDec w;
   w.lut = lut;
   w.ring32 = rings + wave * NZ_RING_ALLOC_DWORDS;
-  w.rec = reinterpret_cast<const uint32_t*>(comp + rec_start);
-  w.last = (uint32_t)(rec_bytes / 4) - 1u;
+  w.words = comp + rs + 256;
+  w.last16 = comp + comp_bytes - NZ_TAIL_PAD;
+  w.nwords = __builtin_amdgcn_readfirstlane((uint32_t)((rec_bytes - 256) / 2));
   w.lane = lane;
-  w.start();
+  w.start(reinterpret_cast<const uint32_t*>(comp + rs)[lane]);
 
   // groups whose packed bytes are (partly) carried are merged after the loop
   const uint32_t tailg = carry ? (S == 0 ? 2u : 1u) : 0u;
@@ -862,7 +878,12 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     sm_next = nz_load_sm<S>(pk + (noff < last_off ? noff : last_off));
     uint32_t ew[8];
     w.group(ew);
-    nz_store_group<S>(dst + (gq * NZ_LANES + lane) * NZ_GROUP, sm, ew);
+    // the merge starts only here: its wait for the packed bytes (fetched a group
+    // ago) must not be hoisted in front of the rANS steps, where it would also
+    // wait for the previous group's store
+    uint32_t sml = (uint32_t)sm, smh = (uint32_t)(sm >> 32);
+    asm volatile("" : "+v"(sml), "+v"(smh), "+v"(ew[7]));
+    nz_store_group<S>(dst + (gq * NZ_LANES + lane) * NZ_GROUP, ((uint64_t)smh << 32) | sml, ew);
   }
   if (whole < body) {  // the ragged last group of the tensor
     const uint32_t idx0 = (whole * NZ_LANES + lane) * NZ_GROUP;
@@ -887,7 +908,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
 
   // every lane must be back at the encoder's start state (2^16 | carried bits)
   // and the wave must not have read past its record
-  const bool bad = (carry ? (w.x >> 16) != 1u : w.x != NZ_L) || (w.base > 2 * (w.last - 63u));
+  const bool bad = (carry ? (w.x >> 16) != 1u : w.x != NZ_L) || (w.base > w.nwords);
   if (__ballot(bad) != 0 && lane == 0) atomicOr(d_status, 4u);
 
   if (carry) {

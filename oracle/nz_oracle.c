@@ -319,7 +319,8 @@ size_t nzo_exp_bound(uint64_t n, uint32_t chunk_syms, uint32_t lane_syms) {
   if (make_geom(&g, n, chunk_syms, lane_syms)) return 0;
   /* a chunk is never stored larger than its RAW form: 4 per chunk, and per
      segment pad4(seg_n) symbols + 128 carried bytes */
-  return g.rec_off + (size_t)n + (4 + 2 * NZO_LANES) * (size_t)g.n_segs + 4 * (size_t)g.n_chunks;
+  return g.rec_off + (size_t)n + (4 + 2 * NZO_LANES) * (size_t)g.n_segs + 4 * (size_t)g.n_chunks +
+         NZO_TAIL_PAD;
 }
 
 static void put32(uint8_t* p, uint32_t v) {
@@ -587,7 +588,14 @@ int64_t nzo_exp_encode(const uint8_t* syms, uint64_t n, uint32_t chunk_syms, uin
   }
   put32(out + g.dir_off + 4 * g.n_segs, (uint32_t)units);
   {
-    uint64_t total = g.rec_off + 4 * units;
+    /* 16 zero bytes close the container so that 16-byte loads of the last
+       words never leave it */
+    uint64_t total = g.rec_off + 4 * units + NZO_TAIL_PAD;
+    if (total > cap) {
+      ret = NZO_ERR_CAP;
+      goto done;
+    }
+    memset(out + g.rec_off + 4 * units, 0, NZO_TAIL_PAD);
     write_header(out, &g, total);
     ret = (int64_t)total;
   }
@@ -689,7 +697,7 @@ int nzo_exp_decode(const uint8_t* comp, size_t comp_bytes, uint64_t n, uint8_t* 
     return NZO_ERR_CORRUPT;
   uint64_t total = (uint64_t)get32(comp + 40) | ((uint64_t)get32(comp + 44) << 32);
   if (total > comp_bytes || total < g.rec_off) return NZO_ERR_CORRUPT;
-  if (g.rec_off + 4 * (uint64_t)get32(comp + g.dir_off + 4 * g.n_segs) != total)
+  if (g.rec_off + 4 * (uint64_t)get32(comp + g.dir_off + 4 * g.n_segs) + NZO_TAIL_PAD != total)
     return NZO_ERR_CORRUPT;
   if (threads < 1) threads = 1;
   if ((uint64_t)threads > g.n_chunks) threads = g.n_chunks ? (int)g.n_chunks : 1;
@@ -699,7 +707,7 @@ int nzo_exp_decode(const uint8_t* comp, size_t comp_bytes, uint64_t n, uint8_t* 
   for (int t = 0; t < threads; ++t) {
     jobs[t].g = &g;
     jobs[t].comp = comp;
-    jobs[t].comp_bytes = (size_t)total;
+    jobs[t].comp_bytes = (size_t)total - NZO_TAIL_PAD;
     jobs[t].out = syms_out;
     jobs[t].seeds = seeds_out;
     jobs[t].c0 = g.n_chunks * (uint64_t)t / (uint64_t)threads;

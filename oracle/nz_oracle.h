@@ -50,6 +50,7 @@ extern "C" {
 #define NZO_MODE_RAW 0xFF
 #define NZO_MODE_BITMAP 0x00
 #define NZO_MAX_RUNS 15
+#define NZO_TAIL_PAD 16
 
 /* ---- split / merge ---- */
 size_t nzo_packed_bytes(uint64_t n, int s);
