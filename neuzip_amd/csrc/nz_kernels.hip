@@ -19,6 +19,8 @@
 
 #include "nz_format.h"
 
+#define NZ_HIST_COPIES 8u
+#define NZ_HIST_STRIDE 257u
 #define NZ_RING_WORDS 2048u  // per-wave LDS ring of renormalisation words
 #define NZ_RING_DWORDS (NZ_RING_WORDS / 2)
 
@@ -141,7 +143,11 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
     const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms,
     uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
     uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info) {
-  __shared__ uint32_t hist[256];
+  // 8 histogram copies (one per lane & 7) at a stride of 257 words: exponents of
+  // weights cluster on a few values, so a single copy would serialise most of
+  // a wavefront's atomics on one address; the odd stride keeps the copies of a
+  // bin in different banks
+  __shared__ uint32_t hist[NZ_HIST_COPIES * NZ_HIST_STRIDE];
   __shared__ uint32_t freq_s[256];
   __shared__ uint32_t red[4];
   __shared__ uint32_t scan_s[4];
@@ -151,8 +157,9 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
   const uint64_t base = c * chunk_syms;
   const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
 
-  hist[tid] = 0;
+  for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += 256) hist[i] = 0;
   __syncthreads();
+  uint32_t* myhist = hist + (tid & (NZ_HIST_COPIES - 1)) * NZ_HIST_STRIDE;
 
   // Packed bytes go to the stored layout: segment k starts at k * keep, and the
   // last NZ_CARRY_BYTES of a full segment go to carry[k] instead (they ride in
@@ -188,7 +195,7 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
       else if constexpr (S == 1) *reinterpret_cast<uint16_t*>(pp) = (uint16_t)f;
       else *pp = (uint8_t)f;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) atomicAdd(&hist[ex[j]], 1u);
+      for (int j = 0; j < 8; ++j) atomicAdd(&myhist[ex[j]], 1u);
     } else {
       // last elements of the tensor: missing ones contribute zero bits
       // (cuda/kernels.cuh:92), and only ceil(rem*(S+1)/8) packed bytes exist.
@@ -198,7 +205,7 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
         exps[gi + j] = (uint8_t)ex[0];
         uint32_t bit = j * (S + 1);
         f |= (uint64_t)rp[0] << (8u * (bit >> 3) + (7u - S - (bit & 7u)));
-        atomicAdd(&hist[ex[0]], 1u);
+        atomicAdd(&myhist[ex[0]], 1u);
       }
       uint32_t nb = (rem * (S + 1) + 7) / 8;
       for (uint32_t b = 0; b < nb; ++b) pp[b] = (uint8_t)(f >> (8 * b));
@@ -207,7 +214,9 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
   __syncthreads();
 
   // ---- quantise the histogram to 12-bit frequencies (sum exactly 4096) ----
-  const uint32_t cnt = hist[tid];
+  uint32_t cnt = 0;
+#pragma unroll
+  for (uint32_t k = 0; k < NZ_HIST_COPIES; ++k) cnt += hist[k * NZ_HIST_STRIDE + tid];
   const uint32_t live = cnt > 0;
   const uint32_t k = nz_block_sum_256(live, red);
   uint32_t f = live ? 1u + (uint32_t)(((uint64_t)cnt * (NZ_M - k)) / cn) : 0u;
@@ -362,8 +371,13 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
         slot[pos + nz_rank_below(m)] = (uint16_t)(x & 0xFFFFu);
         x >>= 16;
       }
-      const uint32_t q = x / f;
-      x = (q << NZ_PROB_BITS) + (x - q * f) + cum;
+      // x < f << 20 here, so the quotient fits 20 bits and a float reciprocal
+      // estimate is off by at most one: fix it up exactly
+      uint32_t q = (uint32_t)(__uint2float_rz(x) * __frcp_rn(__uint2float_rz(f)));
+      uint32_t rem = x - q * f;
+      if ((int32_t)rem < 0) { --q; rem += f; }
+      if (rem >= f) { ++q; rem -= f; }
+      x = (q << NZ_PROB_BITS) + rem + cum;
     }
   }
   states[seg * NZ_LANES + lane] = x;
