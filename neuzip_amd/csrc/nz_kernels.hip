@@ -320,9 +320,14 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
     uint32_t spc, const uint32_t* __restrict__ enc_tab, const NzChunkInfo* __restrict__ info,
     const uint16_t* __restrict__ carry, uint16_t* __restrict__ slots,
     uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words) {
-  __shared__ uint32_t tab[256];
+  // per symbol: x = freq << 16 | cum, y = bits of 1.0f / freq
+  __shared__ uint2 tab[256];
   const uint64_t c = blockIdx.x;
-  for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) tab[i] = enc_tab[c * 256 + i];
+  for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) {
+    const uint32_t fc = enc_tab[c * 256 + i];
+    const uint32_t f = fc >> 16;
+    tab[i] = make_uint2(fc, __float_as_uint(f ? 1.0f / (float)f : 0.0f));
+  }
   __syncthreads();
 
   const uint32_t wave = threadIdx.x >> 6;
@@ -357,8 +362,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
 #pragma unroll
     for (int j = 7; j >= 0; --j) {
       const uint32_t sym = (uint32_t)(sy >> (8 * j)) & 0xFFu;
-      const uint32_t e = tab[sym];
-      const uint32_t f = e >> 16, cum = e & 0xFFFFu;
+      const uint2 e = tab[sym];
+      const uint32_t f = e.x >> 16, cum = e.x & 0xFFFFu;
       const bool need = x >= (f << 20);
       const uint64_t m = __ballot(need);
       const uint32_t cnt = (uint32_t)__popcll(m);
@@ -371,13 +376,16 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
         slot[pos + nz_rank_below(m)] = (uint16_t)(x & 0xFFFFu);
         x >>= 16;
       }
-      // x < f << 20 here, so the quotient fits 20 bits and a float reciprocal
-      // estimate is off by at most one: fix it up exactly
-      uint32_t q = (uint32_t)(__uint2float_rz(x) * __frcp_rn(__uint2float_rz(f)));
-      uint32_t rem = x - q * f;
-      if ((int32_t)rem < 0) { --q; rem += f; }
-      if (rem >= f) { ++q; rem -= f; }
-      x = (q << NZ_PROB_BITS) + rem + cum;
+      // x < f << 20 here, so the quotient is below 2^20 and the float estimate
+      // x * (1/f) (three roundings of 2^-24 each) is off by less than one:
+      // truncate, then correct by the sign of the remainder.  With the exact
+      // quotient q the new state is (q << 12) + (x - q f) + cum
+      //                            = x + q (4096 - f) + cum.
+      uint32_t q = (uint32_t)((float)x * __uint_as_float(e.y));
+      const int32_t rem = (int32_t)(x - __umul24(q, f));
+      q += (rem >= (int32_t)f) ? 1u : 0u;
+      q -= (rem < 0) ? 1u : 0u;
+      x = __umul24(q, NZ_M - f) + (x + cum);
     }
   }
   states[seg * NZ_LANES + lane] = x;
