@@ -41,11 +41,20 @@ def parse_args():
     ap.add_argument("--cols", type=int, default=4096)
     ap.add_argument("--precision", type=int, default=7, choices=[7, 3, 1, 0])
     ap.add_argument("--chunk-size", type=int, default=65536)
-    ap.add_argument("--lane-symbols", type=int, default=0, help="0 = library default")
+    ap.add_argument("--lane-symbols", type=int, default=0, help="0 = library default; -1 = per-tensor (model workloads)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--cpu-threads", type=int, default=0, help="0 = all host cores given to this process")
+    ap.add_argument("--workload", default="tensor", choices=["tensor", "llama8b", "gpt2m"],
+                    help="tensor: decode of one 16384x4096 weight (the headline metric); llama8b: 512-token "
+                         "prompt + greedy decode on a Llama-3-8B-shaped model with compressed weights; "
+                         "gpt2m: training steps on a GPT-2-medium-shaped model with compressed weights")
+    ap.add_argument("--layers", type=int, default=0, help="override the layer count of the model workloads")
+    ap.add_argument("--prompt-len", type=int, default=512)
+    ap.add_argument("--decode-steps", type=int, default=128)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--seq-len", type=int, default=1024)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run five plain 256 MiB device copies (to scale FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
@@ -111,6 +120,176 @@ def time_launches(torch, fn, steps, warmup):
     return wall, statistics.fmean(per), statistics.median(per)
 
 
+def _timed(torch, fn):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = fn()
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0, out
+
+
+def run_llama8b(args, torch):
+    """BASELINE config 3: all Linear weights stored lossless-compressed, batch 1,
+    512-token prompt + 128 greedy steps, against the same model with dense weights."""
+    import neuzip_amd
+    from bench_models import LlamaShaped
+
+    layers = args.layers or 32
+    torch.manual_seed(args.seed)
+    with torch.device("cuda"):
+        torch.set_default_dtype(torch.bfloat16)
+        model = LlamaShaped(layers=layers)
+        torch.set_default_dtype(torch.float32)
+    model.eval()
+    prompt = torch.randint(0, 128256, (1, args.prompt_len), device="cuda")
+    steps = args.decode_steps
+
+    def gen():
+        return model.generate(prompt, steps)
+
+    def prefill():
+        with torch.no_grad():
+            return model.forward(prompt, 0, [[None, None] for _ in model.layers])
+
+    res = {}
+    _timed(torch, lambda: model.generate(prompt, 4))  # warm-up
+    res["dense_prefill_s"], _ = _timed(torch, prefill)
+    res["dense_total_s"], dense_tokens = _timed(torch, gen)
+    dense_param_bytes = sum(p.numel() * p.element_size() for p in model.parameters())
+
+    mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size,
+                             lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
+    t_conv, _ = _timed(torch, lambda: mgr.convert(model))
+    torch.cuda.empty_cache()
+    comp_bytes = sum(mgr.size(h) for h in mgr.meta_dict)
+    comp_dense_bytes = sum(2 * int(np.prod(shp)) for shp in mgr.meta_dict.values())
+
+    _timed(torch, lambda: model.generate(prompt, 4))
+    res["compressed_prefill_s"], _ = _timed(torch, prefill)
+    res["compressed_total_s"], comp_tokens = _timed(torch, gen)
+    with neuzip_amd.DecompressAhead(mgr, model):
+        _timed(torch, lambda: model.generate(prompt, 4))
+        res["ahead_prefill_s"], _ = _timed(torch, prefill)
+        res["ahead_total_s"], ahead_tokens = _timed(torch, gen)
+    mgr._be.check()
+    same = bool(torch.equal(dense_tokens, comp_tokens) and torch.equal(dense_tokens, ahead_tokens))
+    best = min(res["compressed_total_s"], res["ahead_total_s"])
+    out = {
+        "metric": "llama8b_shape_compressed_decode_tok_s",
+        "value": round(steps / best, 2),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": 4,
+        "ms_per_step": round(best / steps * 1e3, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": f"Llama-3-8B-shaped random-init decoder, {layers} layers, batch 1, {args.prompt_len}-token "
+                        f"prompt + {steps} greedy steps, Linear weights compressed (precision {args.precision})",
+            "tokens_identical_to_dense": same,
+            "dense_tok_s": round(steps / res["dense_total_s"], 2),
+            "compressed_tok_s_no_ahead": round(steps / res["compressed_total_s"], 2),
+            "compressed_tok_s_decompress_ahead": round(steps / res["ahead_total_s"], 2),
+            "latency_ratio_vs_dense_total": round(best / res["dense_total_s"], 3),
+            "latency_ratio_vs_dense_prefill": round(min(res["compressed_prefill_s"], res["ahead_prefill_s"]) / res["dense_prefill_s"], 3),
+            "seconds": {k: round(v, 4) for k, v in res.items()},
+            "convert_s": round(t_conv, 3),
+            "compressed_weight_bytes": comp_bytes,
+            "dense_bytes_of_compressed_weights": comp_dense_bytes,
+            "stored_over_dense": round(comp_bytes / comp_dense_bytes, 5),
+            "dense_model_bytes": dense_param_bytes,
+        },
+    }
+    print(json.dumps(out))
+    return 0
+
+
+def run_gpt2m(args, torch):
+    """BASELINE config 4: GPT-2-medium-shaped model, weights kept compressed and
+    re-compressed after every AdamW step; reports the codec share of the step."""
+    import neuzip_amd
+    from bench_models import CompressedAdamW, GPT2Shaped
+
+    layers = args.layers or 24
+    torch.manual_seed(args.seed)
+    with torch.device("cuda"):
+        torch.set_default_dtype(torch.bfloat16)
+        model = GPT2Shaped(layers=layers, ctx=args.seq_len)
+        torch.set_default_dtype(torch.float32)
+    mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size,
+                             lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
+    mgr.convert(model)
+    comp_params = [p for p in model.parameters() if isinstance(p, neuzip_amd.nn.Parameter)]
+    rest = [p for p in model.parameters() if not isinstance(p, neuzip_amd.nn.Parameter)]
+    opt_c = CompressedAdamW(comp_params, lr=1e-4)
+    opt_d = torch.optim.AdamW(rest, lr=1e-4)
+
+    # time every codec call with events on the stream it runs on
+    be = mgr._be
+    spans = []
+    raw_read, raw_write = be.read, be.write
+
+    def timed(fn, kind):
+        def wrapper(*a, **k):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            r = fn(*a, **k)
+            e1.record()
+            spans.append((kind, e0, e1))
+            return r
+        return wrapper
+
+    be.read, be.write = timed(raw_read, "decode"), timed(raw_write, "encode")
+
+    def step():
+        ids = torch.randint(0, 50257, (args.batch, args.seq_len), device="cuda")
+        logits = model(ids[:, :-1])
+        loss = torch.nn.functional.cross_entropy(logits.float().reshape(-1, logits.shape[-1]), ids[:, 1:].reshape(-1))
+        loss.backward()
+        opt_c.step()
+        opt_d.step()
+        opt_d.zero_grad(set_to_none=True)
+        return loss
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    spans.clear()
+    t0 = time.perf_counter()
+    losses = [step() for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dec = sum(a.elapsed_time(b) for k, a, b in spans if k == "decode") * 1e-3
+    enc = sum(a.elapsed_time(b) for k, a, b in spans if k == "encode") * 1e-3
+    n_dec = sum(1 for k, _, _ in spans if k == "decode")
+    n_enc = sum(1 for k, _, _ in spans if k == "encode")
+    mgr._be.check()
+    tokens = args.batch * (args.seq_len - 1) * args.steps
+    out = {
+        "metric": "gpt2m_shape_compressed_training_tok_s",
+        "value": round(tokens / wall, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": f"GPT-2-medium-shaped random-init model, {layers} layers, batch {args.batch} x seq {args.seq_len}, "
+                        f"bf16 weights compressed (precision {args.precision}), re-compressed after each AdamW step",
+            "codec_share_of_step": round((dec + enc) / wall, 4),
+            "decode_s_per_step": round(dec / args.steps, 5),
+            "encode_s_per_step": round(enc / args.steps, 5),
+            "decodes_per_step": n_dec / args.steps,
+            "encodes_per_step": n_enc / args.steps,
+            "compressed_tensors": len(comp_params),
+            "lane_symbols": "auto" if args.lane_symbols < 0 else (args.lane_symbols or 512),
+            "stored_over_dense": round(sum(mgr.size(p._handle) for p in comp_params) /
+                                       sum(2 * int(np.prod(p._shape)) for p in comp_params), 5),
+            "first_loss": round(float(losses[0]), 4),
+            "last_loss": round(float(losses[-1]), 4),
+        },
+    }
+    print(json.dumps(out))
+    return 0
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -136,6 +315,11 @@ def main():
         print(json.dumps({"calibration": "5 device copies", "bytes_read_per_copy": 256 << 20,
                           "bytes_written_per_copy": 256 << 20}))
         return 0
+
+    if args.workload == "llama8b":
+        return run_llama8b(args, torch)
+    if args.workload == "gpt2m":
+        return run_gpt2m(args, torch)
 
     n = args.rows * args.cols
     lane = args.lane_symbols or lib_mod.DEFAULT_LANE_SYMS

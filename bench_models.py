@@ -1,0 +1,193 @@
+"""Random-init decoder models of the shapes BASELINE.json names, for bench.py.
+
+Only shapes and layer types matter here (all weights are N(0, 0.02) from a
+seed, all inputs uniform random token ids): the benchmark measures the codec
+inside a realistic sequence of Linear layers, not model quality.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+
+
+def _init_linear(lin: torch.nn.Linear):
+    lin.weight.data.normal_(0.0, 0.02)
+    if lin.bias is not None:
+        lin.bias.data.zero_()
+
+
+class RMSNorm(torch.nn.Module):
+    def __init__(self, d, eps=1e-5):
+        super().__init__()
+        self.weight = torch.nn.Parameter(torch.ones(d))
+        self.eps = eps
+
+    def forward(self, x):
+        v = x.float()
+        v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + self.eps)
+        return (v * self.weight.float()).to(x.dtype)
+
+
+def _rope(x, pos, theta=500000.0):
+    # x: [B, H, T, D]; pos: [T]
+    d = x.shape[-1]
+    inv = 1.0 / (theta ** (torch.arange(0, d, 2, device=x.device, dtype=torch.float32) / d))
+    ang = pos.float()[:, None] * inv[None, :]
+    cos, sin = ang.cos()[None, None], ang.sin()[None, None]
+    x1, x2 = x.float()[..., 0::2], x.float()[..., 1::2]
+    out = torch.stack((x1 * cos - x2 * sin, x1 * sin + x2 * cos), dim=-1).flatten(-2)
+    return out.to(x.dtype)
+
+
+class LlamaBlock(torch.nn.Module):
+    def __init__(self, d, n_q, n_kv, ffn):
+        super().__init__()
+        self.n_q, self.n_kv, self.hd = n_q, n_kv, d // n_q
+        self.input_norm = RMSNorm(d)
+        self.q_proj = torch.nn.Linear(d, n_q * self.hd, bias=False)
+        self.k_proj = torch.nn.Linear(d, n_kv * self.hd, bias=False)
+        self.v_proj = torch.nn.Linear(d, n_kv * self.hd, bias=False)
+        self.o_proj = torch.nn.Linear(n_q * self.hd, d, bias=False)
+        self.post_norm = RMSNorm(d)
+        self.gate_proj = torch.nn.Linear(d, ffn, bias=False)
+        self.up_proj = torch.nn.Linear(d, ffn, bias=False)
+        self.down_proj = torch.nn.Linear(ffn, d, bias=False)
+        for m in (self.q_proj, self.k_proj, self.v_proj, self.o_proj, self.gate_proj, self.up_proj, self.down_proj):
+            _init_linear(m)
+
+    def forward(self, x, pos, cache):
+        B, T, _ = x.shape
+        h = self.input_norm(x)
+        q = self.q_proj(h).view(B, T, self.n_q, self.hd).transpose(1, 2)
+        k = self.k_proj(h).view(B, T, self.n_kv, self.hd).transpose(1, 2)
+        v = self.v_proj(h).view(B, T, self.n_kv, self.hd).transpose(1, 2)
+        q, k = _rope(q, pos), _rope(k, pos)
+        if cache is not None:
+            if cache[0] is not None:
+                k = torch.cat((cache[0], k), dim=2)
+                v = torch.cat((cache[1], v), dim=2)
+            cache[0], cache[1] = k, v
+        rep = self.n_q // self.n_kv
+        kk = k.repeat_interleave(rep, dim=1)
+        vv = v.repeat_interleave(rep, dim=1)
+        a = F.scaled_dot_product_attention(q, kk, vv, is_causal=(T > 1))
+        x = x + self.o_proj(a.transpose(1, 2).reshape(B, T, -1))
+        h = self.post_norm(x)
+        return x + self.down_proj(F.silu(self.gate_proj(h)) * self.up_proj(h))
+
+
+class LlamaShaped(torch.nn.Module):
+    """32 layers, d=4096, 32 q / 8 kv heads, FFN 14336, vocab 128256 by default."""
+
+    def __init__(self, layers=32, d=4096, n_q=32, n_kv=8, ffn=14336, vocab=128256):
+        super().__init__()
+        self.embed = torch.nn.Embedding(vocab, d)
+        self.embed.weight.data.normal_(0.0, 0.02)
+        self.layers = torch.nn.ModuleList([LlamaBlock(d, n_q, n_kv, ffn) for _ in range(layers)])
+        self.norm = RMSNorm(d)
+        self.lm_head = torch.nn.Linear(d, vocab, bias=False)  # left dense by convert()
+        _init_linear(self.lm_head)
+
+    def forward(self, ids, start, caches):
+        pos = torch.arange(start, start + ids.shape[1], device=ids.device)
+        x = self.embed(ids)
+        for blk, c in zip(self.layers, caches):
+            x = blk(x, pos, c)
+        return self.lm_head(self.norm(x[:, -1:]))
+
+    @torch.no_grad()
+    def generate(self, prompt, steps):
+        """Greedy decode: prefill the prompt, then `steps` single-token steps."""
+        caches = [[None, None] for _ in self.layers]
+        logits = self.forward(prompt, 0, caches)
+        tok = logits.argmax(-1)
+        out = [tok]
+        t = prompt.shape[1]
+        for _ in range(steps - 1):
+            logits = self.forward(tok, t, caches)
+            tok = logits.argmax(-1)
+            out.append(tok)
+            t += 1
+        return torch.cat(out, dim=1)
+
+
+class GPT2Block(torch.nn.Module):
+    def __init__(self, d, heads):
+        super().__init__()
+        self.heads = heads
+        self.ln1 = torch.nn.LayerNorm(d)
+        self.qkv = torch.nn.Linear(d, 3 * d)
+        self.proj = torch.nn.Linear(d, d)
+        self.ln2 = torch.nn.LayerNorm(d)
+        self.fc = torch.nn.Linear(d, 4 * d)
+        self.fc2 = torch.nn.Linear(4 * d, d)
+        for m in (self.qkv, self.proj, self.fc, self.fc2):
+            _init_linear(m)
+
+    def forward(self, x):
+        B, T, D = x.shape
+        q, k, v = self.qkv(self.ln1(x)).view(B, T, 3, self.heads, D // self.heads).permute(2, 0, 3, 1, 4)
+        a = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        x = x + self.proj(a.transpose(1, 2).reshape(B, T, D))
+        return x + self.fc2(F.gelu(self.fc(self.ln2(x))))
+
+
+class GPT2Shaped(torch.nn.Module):
+    """24 layers, d=1024, 16 heads, vocab 50257 by default (GPT-2 medium shape)."""
+
+    def __init__(self, layers=24, d=1024, heads=16, vocab=50257, ctx=1024):
+        super().__init__()
+        self.wte = torch.nn.Embedding(vocab, d)
+        self.wpe = torch.nn.Embedding(ctx, d)
+        self.wte.weight.data.normal_(0.0, 0.02)
+        self.wpe.weight.data.normal_(0.0, 0.02)
+        self.blocks = torch.nn.ModuleList([GPT2Block(d, heads) for _ in range(layers)])
+        self.ln_f = torch.nn.LayerNorm(d)
+        self.lm_head = torch.nn.Linear(d, vocab, bias=False)
+        _init_linear(self.lm_head)
+
+    def forward(self, ids):
+        T = ids.shape[1]
+        x = self.wte(ids) + self.wpe(torch.arange(T, device=ids.device))[None]
+        for b in self.blocks:
+            x = b(x)
+        return self.lm_head(self.ln_f(x))
+
+
+class CompressedAdamW:
+    """AdamW for compressed parameters: decompress, update, re-compress under the
+    same handle (the read -> update -> write idiom of neuzip/__init__.py:25-35
+    with Adam moments kept dense in fp32)."""
+
+    def __init__(self, params, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01):
+        self.params = list(params)
+        self.lr, self.b1, self.b2, self.eps, self.wd = lr, betas[0], betas[1], eps, weight_decay
+        self.state = {}
+        self.t = 0
+
+    @torch.no_grad()
+    def step(self):
+        self.t += 1
+        c1 = 1.0 - self.b1 ** self.t
+        c2 = 1.0 - self.b2 ** self.t
+        for p in self.params:
+            g = p._gradient
+            if g is None:
+                continue
+            st = self.state.get(p._handle)
+            if st is None:
+                st = (torch.zeros_like(g, dtype=torch.float32), torch.zeros_like(g, dtype=torch.float32))
+                self.state[p._handle] = st
+            m, v = st
+            gf = g.float()
+            m.mul_(self.b1).add_(gf, alpha=1 - self.b1)
+            v.mul_(self.b2).addcmul_(gf, gf, value=1 - self.b2)
+            w = p()  # decompress
+            wf = w.float()
+            wf.mul_(1 - self.lr * self.wd)
+            wf.addcdiv_(m, (v / c2).sqrt_().add_(self.eps), value=-self.lr / c1)
+            p._manager.write(wf.to(w.dtype), p._handle)  # re-compress
+            p._gradient = None
+            p.grad = None

@@ -46,6 +46,7 @@ extern "C" {
 
 #define NZ_DEFAULT_CHUNK 65536u   /* cuda/neuzip.cu:31 */
 #define NZ_DEFAULT_LANE_SYMS 512u /* two wavefronts per 64 KiB chunk */
+#define NZ_LANE_SYMS_AUTO 0xFFFFFFFFu /* nz_manager_create: choose per tensor */
 
 typedef struct nz_manager nz_manager;
 
@@ -105,7 +106,9 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
 /* Manager(algorithm, chunk_size) for the class Manager_f{precision}_n{normalizer_size}
    (cuda/neuzip.cu:19-38, neuzip/binding.py:69-70).  precision in {0,1,3,7};
    normalizer_size must be 0 (block normalizers are not implemented);
-   lane_syms 0 selects NZ_DEFAULT_LANE_SYMS clipped to the chunk. */
+   lane_syms 0 selects NZ_DEFAULT_LANE_SYMS clipped to the chunk;
+   NZ_LANE_SYMS_AUTO shortens the segments of tensors too small to fill the GPU
+   at the default (more wavefronts, ~8.5 bits of container per extra lane). */
 int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_t chunk_size,
                       uint32_t lane_syms, nz_manager** out);
 void nz_manager_destroy(nz_manager* m);

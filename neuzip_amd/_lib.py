@@ -20,6 +20,7 @@ DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 ALGO_ANS = 0
 DEFAULT_CHUNK = 65536
 DEFAULT_LANE_SYMS = 512
+LANE_SYMS_AUTO = 0xFFFFFFFF
 
 EXPORTS = [
     "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",

@@ -41,6 +41,8 @@ class _HipBackend:
     def __init__(self, precision: int, normalizer_size: int, chunk_size: int, lane_symbols: int):
         self._L = _lib.load()
         self._h = ctypes.c_void_p()
+        if lane_symbols == "auto":
+            lane_symbols = _lib.LANE_SYMS_AUTO
         rc = self._L.nz_manager_create(_lib.ALGO_ANS, precision, normalizer_size, chunk_size,
                                        lane_symbols, ctypes.byref(self._h))
         _lib.raise_for(rc)
@@ -82,6 +84,20 @@ class _HipBackend:
         out = torch.empty(n.value, dtype=torch.bfloat16, device=self._device)
         rc = self._L.nz_manager_read(self._h, handle.encode(), out.data_ptr(), n.value,
                                      _stream_ptr(self._device))
+        _lib.raise_for(rc)
+        return out
+
+    def numel(self, handle: str) -> int:
+        n = ctypes.c_uint64()
+        _lib.raise_for(self._L.nz_manager_meta(self._h, handle.encode(), ctypes.byref(n), None))
+        return int(n.value)
+
+    def read_into(self, handle: str, out: torch.Tensor) -> torch.Tensor:
+        """Decompress into caller-provided bf16 storage (no allocation), on the current stream."""
+        if out.dtype != torch.bfloat16 or not out.is_contiguous():
+            raise ValueError("read_into needs a contiguous bfloat16 tensor")
+        rc = self._L.nz_manager_read(self._h, handle.encode(), out.data_ptr(), out.numel(),
+                                     _stream_ptr(out.device))
         _lib.raise_for(rc)
         return out
 
@@ -167,10 +183,13 @@ class Manager:
         chunk_size=2**16,
         lane_symbols: int = 0,
     ) -> None:
-        """``lane_symbols`` (extension; 0 = library default) is the number of
+        """``lane_symbols`` (extension; 0 = library default of 512) is the number of
         exponents each of the 64 rANS lanes of a wavefront codes per segment:
-        smaller values expose more wavefronts per chunk at the price of 32 bits
-        of coder state per lane and segment."""
+        smaller values expose more wavefronts per chunk at the price of about
+        8.5 bits of container per lane and segment.  ``"auto"`` keeps the default
+        for large tensors and shortens the segments of small ones so that they
+        still fill the GPU (meant for training, where every weight is decoded
+        three times and encoded once per step)."""
         normalizer_size = 0 if normalizer_size is None else normalizer_size
         self.meta_dict = {}  # handle -> original shape
         if algorithm == Algorithm.dummy:

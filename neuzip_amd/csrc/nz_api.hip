@@ -151,6 +151,7 @@ struct Entry {
   uint64_t packed_bytes = 0, packed_cap = 0;
   uint64_t n = 0;
   int dtype = NZ_DTYPE_BF16;
+  uint32_t lane_syms = 0;  // geometry this entry was written with
 };
 
 }  // namespace
@@ -158,6 +159,7 @@ struct Entry {
 struct nz_manager {
   int precision;
   uint32_t chunk_syms, lane_syms;
+  bool auto_lanes = false;  // pick lane_syms per tensor so that small tensors still fill the GPU
   std::unordered_map<std::string, Entry> entries;  // compress_cache + meta_cache
   std::mutex mu;
   void* ws = nullptr;
@@ -274,7 +276,8 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   if (algorithm != NZ_ALGO_ANS) return fail(NZ_ERR_ALGO, "Unsupported algorithm");
   if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
   if (normalizer_size != 0) return fail(NZ_ERR_ARG, "block normalizers are not implemented (normalizer_size must be 0)");
-  if (lane_syms == 0) {
+  const bool auto_lanes = lane_syms == NZ_LANE_SYMS_AUTO;
+  if (lane_syms == 0 || auto_lanes) {
     lane_syms = NZ_DEFAULT_LANE_SYMS;
     while (lane_syms > 8 && (uint64_t)lane_syms * NZ_LANES > chunk_size) lane_syms /= 2;
     while ((uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size) lane_syms *= 2;
@@ -285,6 +288,7 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   m->precision = precision;
   m->chunk_syms = chunk_size;
   m->lane_syms = lane_syms;
+  m->auto_lanes = auto_lanes;
   hipError_t e = hipMalloc((void**)&m->d_status, 256);
   if (e == hipSuccess) e = hipMemset(m->d_status, 0, 256);
   if (e == hipSuccess) e = hipHostMalloc((void**)&m->h_pin, 64, hipHostMallocDefault);
@@ -315,8 +319,19 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   if (dtype != NZ_DTYPE_BF16) return fail(NZ_ERR_DTYPE, "Unsupported data type");
   if (n && !dev_data) return fail(NZ_ERR_ARG, "null data pointer");
   if ((uintptr_t)dev_data & 15) return fail(NZ_ERR_ALIGN, "dense input must be 16-byte aligned");
+  // Throughput of both codec directions is set by the number of wavefronts in
+  // flight (one per 64 * lane_syms elements).  In auto mode a tensor too small
+  // to give every SIMD two wavefronts at the default gets shorter segments,
+  // down to the 8 segments a chunk may hold, at ~8.5 bits per extra lane.
+  uint32_t lane_syms = m->lane_syms;
+  if (m->auto_lanes) {
+    while (lane_syms > 16 && (lane_syms / 2) % NZ_GROUP == 0 &&
+           (uint64_t)(lane_syms / 2) * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK >= m->chunk_syms &&
+           n / ((uint64_t)lane_syms * NZ_LANES) < 2048)
+      lane_syms /= 2;
+  }
   NzGeom g;
-  if (int rc = make_geom(&g, n, m->chunk_syms, m->lane_syms)) return rc;
+  if (int rc = make_geom(&g, n, m->chunk_syms, lane_syms)) return rc;
   hipStream_t st = (hipStream_t)stream;
   std::lock_guard<std::mutex> lock(m->mu);
 
@@ -343,7 +358,8 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   Entry ent;
   ent.n = n;
   ent.dtype = dtype;
-  ent.packed_bytes = nz_packed_stored_bytes_of(n, m->precision, m->lane_syms);
+  ent.lane_syms = lane_syms;
+  ent.packed_bytes = nz_packed_stored_bytes_of(n, m->precision, lane_syms);
   auto release = [&](Entry& e) {
     if (e.comp) (void)hipFree(e.comp);
     if (e.packed) (void)hipFree(e.packed);
@@ -381,7 +397,9 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
       ent.comp_cap = old.comp_cap;
       old.comp = nullptr;
     } else {
-      ent.comp_cap = ent.comp_bytes;
+      // a little headroom: the next write of this handle (an optimizer step
+      // later) is a few bytes longer or shorter and can reuse the buffer
+      ent.comp_cap = ent.comp_bytes + ent.comp_bytes / 64 + 1024;
       e = hipMalloc(&ent.comp, ent.comp_cap);
       if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("hipMalloc(comp): ") + hipGetErrorString(e));
     }
@@ -415,7 +433,7 @@ int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap
   if (!dev_out) return fail(NZ_ERR_ARG, "null output pointer");
   if ((uintptr_t)dev_out & 15) return fail(NZ_ERR_ALIGN, "dense output must be 16-byte aligned");
   NzGeom g;
-  if (int rc = make_geom(&g, ent.n, m->chunk_syms, m->lane_syms)) return rc;
+  if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
   return decode_launch(g, m->precision, ent.comp, ent.comp_bytes, ent.packed, dev_out, m->d_status,
                        (hipStream_t)stream);
 }
