@@ -64,7 +64,7 @@ EncLayout enc_layout(const NzGeom& g) {
 template <int S>
 void launch_split_hist(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws,
                        const EncLayout& L, hipStream_t st) {
-  hipLaunchKernelGGL(nz_split_hist_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(256), 0, st,
+  hipLaunchKernelGGL(nz_split_hist_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(NZ_SPLIT_THREADS), 0, st,
                      (const uint16_t*)in, g.n, g.chunk_syms, g.seg_syms, packed, ws + L.carry,
                      ws + L.exps, (uint32_t*)(ws + L.enc_tab), ws + L.tab_ser,
                      (NzChunkInfo*)(ws + L.info));

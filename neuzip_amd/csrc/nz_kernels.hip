@@ -114,17 +114,22 @@ __global__ __launch_bounds__(256) void nz_split_unpacked_kernel(const uint16_t* 
 // split + histogram + table: one workgroup per chunk
 // ----------------------------------------------------------------------------
 
-__device__ __forceinline__ uint32_t nz_block_sum_256(uint32_t v, uint32_t* red) {
-  // 256 threads = 4 waves
+#define NZ_SPLIT_THREADS 1024u
+#define NZ_SPLIT_WAVES (NZ_SPLIT_THREADS / 64u)
+
+__device__ __forceinline__ uint32_t nz_block_sum(uint32_t v, uint32_t* red) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
   __syncthreads();
-  return red[0] + red[1] + red[2] + red[3];
+  uint32_t t = 0;
+#pragma unroll
+  for (uint32_t w = 0; w < NZ_SPLIT_WAVES; ++w) t += red[w];
+  return t;
 }
 
-__device__ __forceinline__ uint32_t nz_block_max_256(uint32_t v, uint32_t* red) {
+__device__ __forceinline__ uint32_t nz_block_max(uint32_t v, uint32_t* red) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     uint32_t t = __shfl_xor(v, o, 64);
@@ -133,13 +138,14 @@ __device__ __forceinline__ uint32_t nz_block_max_256(uint32_t v, uint32_t* red) 
   __syncthreads();
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
   __syncthreads();
-  uint32_t a = red[0] > red[1] ? red[0] : red[1];
-  uint32_t b = red[2] > red[3] ? red[2] : red[3];
-  return a > b ? a : b;
+  uint32_t t = 0;
+#pragma unroll
+  for (uint32_t w = 0; w < NZ_SPLIT_WAVES; ++w) t = red[w] > t ? red[w] : t;
+  return t;
 }
 
 template <int S>
-__global__ __launch_bounds__(256) void nz_split_hist_kernel(
+__global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
     const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms,
     uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
     uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info) {
@@ -148,16 +154,17 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
   // a wavefront's atomics on one address; the odd stride keeps the copies of a
   // bin in different banks
   __shared__ uint32_t hist[NZ_HIST_COPIES * NZ_HIST_STRIDE];
-  __shared__ uint32_t freq_s[256];
-  __shared__ uint32_t red[4];
+  __shared__ uint32_t red[NZ_SPLIT_WAVES];
   __shared__ uint32_t scan_s[4];
+  __shared__ uint64_t mw[4];
+  __shared__ uint32_t cf[256];
 
   const uint32_t tid = threadIdx.x;
   const uint64_t c = blockIdx.x;
   const uint64_t base = c * chunk_syms;
   const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
 
-  for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += 256) hist[i] = 0;
+  for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += NZ_SPLIT_THREADS) hist[i] = 0;
   __syncthreads();
   uint32_t* myhist = hist + (tid & (NZ_HIST_COPIES - 1)) * NZ_HIST_STRIDE;
 
@@ -168,7 +175,7 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
   const uint32_t keep = seg_p - NZ_CARRY_BYTES;
   const uint64_t seg0 = base / seg_syms;
 
-  for (uint32_t i = tid * 8; i < cn; i += 256 * 8) {
+  for (uint32_t i = tid * 8; i < cn; i += NZ_SPLIT_THREADS * 8) {
     const uint64_t gi = base + i;
     const uint32_t sk = i / seg_syms;                    // segment inside the chunk
     const uint32_t sb = (i - sk * seg_syms) / 8 * (S + 1);  // byte inside the segment
@@ -214,19 +221,23 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
   __syncthreads();
 
   // ---- quantise the histogram to 12-bit frequencies (sum exactly 4096) ----
+  // threads 0..255 own one symbol each; the others take part in the reductions
+  // with neutral values
+  const bool own = tid < 256;
   uint32_t cnt = 0;
+  if (own) {
 #pragma unroll
-  for (uint32_t k = 0; k < NZ_HIST_COPIES; ++k) cnt += hist[k * NZ_HIST_STRIDE + tid];
+    for (uint32_t k = 0; k < NZ_HIST_COPIES; ++k) cnt += hist[k * NZ_HIST_STRIDE + tid];
+  }
   const uint32_t live = cnt > 0;
-  const uint32_t k = nz_block_sum_256(live, red);
+  const uint32_t k = nz_block_sum(live, red);
   uint32_t f = live ? 1u + (uint32_t)(((uint64_t)cnt * (NZ_M - k)) / cn) : 0u;
-  const uint32_t sum = nz_block_sum_256(f, red);
+  const uint32_t sum = nz_block_sum(f, red);
   // most frequent symbol, lowest index on ties (cnt <= 2^24 fits above the index byte)
-  const uint32_t key = nz_block_max_256((cnt << 8) | (255u - tid), red);
+  const uint32_t key = nz_block_max(own ? ((cnt << 8) | (255u - tid)) : 0u, red);
   const uint32_t imax = 255u - (key & 0xFFu);
   if (tid == imax) f += NZ_M - sum;
   if (k == 1) f = (tid == imax) ? (NZ_M - 1) : ((tid == (imax ^ 1u)) ? 1u : 0u);
-  freq_s[tid] = f;
 
   // exclusive prefix sum over the 256 symbols
   uint32_t incl = f;
@@ -235,73 +246,86 @@ __global__ __launch_bounds__(256) void nz_split_hist_kernel(
     uint32_t t = __shfl_up(incl, o, 64);
     if ((tid & 63) >= (uint32_t)o) incl += t;
   }
-  if ((tid & 63) == 63) scan_s[tid >> 6] = incl;
+  if (own && (tid & 63) == 63) scan_s[tid >> 6] = incl;
   __syncthreads();
-  uint32_t woff = 0;
-  for (uint32_t w = 0; w < (tid >> 6); ++w) woff += scan_s[w];
-  const uint32_t cum = woff + incl - f;
-  enc_tab[c * 256 + tid] = (f << 16) | cum;
+  if (own) {
+    uint32_t woff = 0;
+    for (uint32_t w = 0; w < (tid >> 6); ++w) woff += scan_s[w];
+    const uint32_t cum = woff + incl - f;
+    enc_tab[c * 256 + tid] = (f << 16) | cum;
+  }
 
-  // ---- serialise the table (one thread; <= 256 short iterations) ----
+  // ---- serialise the table, in parallel ----
+  // 256-bit live mask from the ballots of the four owning waves; the rank of a
+  // live symbol is the number of live symbols below it.
+  const uint64_t bal = __ballot(own && f != 0);
+  if (own && (tid & 63) == 0) mw[tid >> 6] = bal;
+  __syncthreads();
+  const uint64_t m0 = mw[0], m1 = mw[1], m2 = mw[2], m3 = mw[3];
+  const uint32_t kk = (uint32_t)(__popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3));
+  if (own && f != 0) {
+    const uint32_t w = tid >> 6;
+    const uint32_t below = (w > 0 ? (uint32_t)__popcll(m0) : 0u) + (w > 1 ? (uint32_t)__popcll(m1) : 0u) +
+                           (w > 2 ? (uint32_t)__popcll(m2) : 0u) +
+                           (uint32_t)__popcll(bal & ((1ull << (tid & 63)) - 1ull));
+    cf[below] = f;
+  }
+  // a run starts at a live symbol whose predecessor is not live
+  const uint64_t s0 = m0 & ~(m0 << 1);
+  const uint64_t s1 = m1 & ~((m1 << 1) | (m0 >> 63));
+  const uint64_t s2 = m2 & ~((m2 << 1) | (m1 >> 63));
+  const uint64_t s3 = m3 & ~((m3 << 1) | (m2 >> 63));
+  const uint32_t runs = (uint32_t)(__popcll(s0) + __popcll(s1) + __popcll(s2) + __popcll(s3));
+  const bool run_form = runs >= 1 && runs <= NZ_MAX_RUNS;
+  const uint32_t head = run_form ? 1u + 2u * runs : 33u;
+  uint8_t* out = tab_ser + c * NZ_TABLE_MAX_BYTES;
+  __syncthreads();
+  // 12-bit fields, two per three bytes
+  for (uint32_t pj = tid; 2 * pj < kk; pj += NZ_SPLIT_THREADS) {
+    const uint32_t a = cf[2 * pj];
+    const bool two = 2 * pj + 1 < kk;
+    const uint32_t b = two ? cf[2 * pj + 1] : 0u;
+    uint8_t* fp = out + head + 3 * pj;
+    fp[0] = (uint8_t)(a & 0xFF);
+    fp[1] = (uint8_t)((a >> 8) | ((b & 0xF) << 4));
+    if (two) fp[2] = (uint8_t)(b >> 4);
+  }
+  if (!run_form && tid < 32) {
+    const uint64_t mq = tid < 8 ? m0 : (tid < 16 ? m1 : (tid < 24 ? m2 : m3));
+    out[1 + tid] = (uint8_t)(mq >> (8 * (tid & 7)));
+  }
   if (tid == 0) {
-    uint8_t* out = tab_ser + c * NZ_TABLE_MAX_BYTES;
-    uint32_t runs = 0, kk = 0;
-    for (int i = 0; i < 256; ++i) {
-      if (freq_s[i]) {
-        ++kk;
-        if (i == 0 || !freq_s[i - 1]) ++runs;
-      }
-    }
-    uint32_t head;
-    if (runs >= 1 && runs <= NZ_MAX_RUNS) {
+    if (run_form) {
       out[0] = (uint8_t)runs;
+      const uint64_t mm[4] = {m0, m1, m2, m3};
+      const uint64_t ss[4] = {s0, s1, s2, s3};
       uint32_t r = 0;
-      int i = 0;
-      while (i < 256) {
-        if (freq_s[i]) {
-          int j = i;
-          while (j < 256 && freq_s[j]) ++j;
-          out[1 + 2 * r] = (uint8_t)i;
-          out[2 + 2 * r] = (uint8_t)(j - i - 1);
+      for (int w = 0; w < 4; ++w) {
+        uint64_t sm = ss[w];
+        while (sm) {
+          const uint32_t b = (uint32_t)__builtin_ctzll(sm);
+          sm &= sm - 1;
+          // first symbol at or after the start that is not live
+          uint32_t end = 256;
+          uint64_t dead = ~mm[w] & ~((b ? (1ull << b) : 1ull) - 1ull);
+          if (b == 0) dead = ~mm[w];
+          for (int v = w; v < 4; ++v) {
+            if (v > w) dead = ~mm[v];
+            if (dead) {
+              end = 64u * v + (uint32_t)__builtin_ctzll(dead);
+              break;
+            }
+          }
+          out[1 + 2 * r] = (uint8_t)(64u * w + b);
+          out[2 + 2 * r] = (uint8_t)(end - (64u * w + b) - 1u);
           ++r;
-          i = j;
-        } else {
-          ++i;
         }
       }
-      head = 1 + 2 * runs;
     } else {
       out[0] = NZ_MODE_BITMAP;
-      for (int b = 0; b < 32; ++b) {
-        uint32_t m = 0;
-        for (int q = 0; q < 8; ++q) m |= (freq_s[8 * b + q] ? 1u : 0u) << q;
-        out[1 + b] = (uint8_t)m;
-      }
-      head = 33;
     }
-    // 12-bit fields, two per three bytes
-    uint32_t j = 0, hold = 0;
-    uint8_t* fp = out + head;
-    for (int i = 0; i < 256; ++i) {
-      uint32_t fv = freq_s[i];
-      if (!fv) continue;
-      if ((j & 1) == 0) {
-        hold = fv;
-      } else {
-        uint32_t b0 = 3 * (j >> 1);
-        fp[b0] = (uint8_t)(hold & 0xFF);
-        fp[b0 + 1] = (uint8_t)((hold >> 8) | ((fv & 0xF) << 4));
-        fp[b0 + 2] = (uint8_t)(fv >> 4);
-      }
-      ++j;
-    }
-    if (j & 1) {
-      uint32_t b0 = 3 * (j >> 1);
-      fp[b0] = (uint8_t)(hold & 0xFF);
-      fp[b0 + 1] = (uint8_t)(hold >> 8);
-    }
-    uint32_t bytes = head + (12 * kk + 7) / 8;
-    uint32_t padded = (bytes + 3) & ~3u;
+    const uint32_t bytes = head + (12 * kk + 7) / 8;
+    const uint32_t padded = (bytes + 3) & ~3u;
     for (uint32_t b = bytes; b < padded; ++b) out[b] = 0;
     NzChunkInfo ci;
     ci.tab_len = padded;
