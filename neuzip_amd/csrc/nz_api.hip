@@ -50,7 +50,7 @@ EncLayout enc_layout(const NzGeom& g) {
   L.tab_ser = take(g.n_chunks * NZ_TABLE_MAX_BYTES);
   L.info = take(g.n_chunks * sizeof(NzChunkInfo));
   L.carry = take(g.n_segs * NZ_CARRY_BYTES);
-  L.slots = take(g.n_segs * (uint64_t)g.seg_syms);  // seg_syms/2 words of 2 bytes
+  L.slots = take(g.n_segs * 2 * (uint64_t)g.seg_syms);  // one 2-byte word per symbol: the worst case
   L.states = take(g.n_segs * NZ_LANES * 4);
   L.seg_words = take(g.n_segs * 4);
   L.seg_units = take((g.n_segs + 1) * 4);

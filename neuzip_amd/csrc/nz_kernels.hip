@@ -339,22 +339,30 @@ __global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
 // ----------------------------------------------------------------------------
 // rANS encode: one workgroup per chunk, one wavefront per segment
 // ----------------------------------------------------------------------------
+//
+// The 64 lanes run backwards over their symbols.  Per symbol: emit the low 16
+// state bits when the state is at or above freq << 20 (ranked into the word
+// slot back to front, so that the decoder reads front to back), then
+// x = (x / f) << 12 | (x % f) + cum.  A segment's slot holds one word per
+// symbol, the most any input can emit, so there is no overflow path; a chunk
+// that codes to more than its raw size is stored raw by the finalize kernel.
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_kernel(
     const uint8_t* __restrict__ exps, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
     uint32_t spc, const uint32_t* __restrict__ enc_tab, const NzChunkInfo* __restrict__ info,
     const uint16_t* __restrict__ carry, uint16_t* __restrict__ slots,
     uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words) {
-  // per symbol: x = freq << 16 | cum, y = bits of 1.0f / freq
-  __shared__ uint2 tab[256];
+  // per symbol: x = freq << 20 (renormalisation threshold), y = freq, z = cum,
+  // w = bits of 1.0f / freq
+  __shared__ uint4 tab[256];
   const uint64_t c = blockIdx.x;
   for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) {
     const uint32_t fc = enc_tab[c * 256 + i];
     const uint32_t f = fc >> 16;
-    tab[i] = make_uint2(fc, __float_as_uint(f ? 1.0f / (float)f : 0.0f));
+    tab[i] = make_uint4(f << 20, f, fc & 0xFFFFu, __float_as_uint(f ? 1.0f / (float)f : 0.0f));
   }
   __syncthreads();
 
-  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t seg_syms = lane_syms * NZ_LANES;
   const uint64_t seg = c * spc + wave;
@@ -362,7 +370,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
   if (seg_base >= n) return;
   const uint32_t seg_n = (uint32_t)((n - seg_base) < seg_syms ? (n - seg_base) : seg_syms);
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
-  const uint32_t cap_words = seg_syms / 2;
+  const uint32_t cap_words = seg_syms;
   const uint32_t pad = info[c].pad_sym;
   uint16_t* slot = slots + seg * cap_words;
   const uint8_t* src = exps + seg_base;
@@ -370,8 +378,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
   // a full segment starts from 2^16 | 16 carried bits of the packed stream
   uint32_t x = NZ_L | (seg_n == seg_syms ? (uint32_t)carry[seg * NZ_LANES + lane] : 0u);
   uint32_t pos = cap_words;
-  bool overflow = false;
-  for (uint32_t g = ngroups; g-- > 0 && !overflow;) {
+  for (uint32_t g = ngroups; g-- > 0;) {
     const uint32_t idx0 = (g * NZ_LANES + lane) * NZ_GROUP;
     uint64_t sy;
     if (idx0 + 8 <= seg_n) {
@@ -383,37 +390,32 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
         sy |= (uint64_t)b << (8 * j);
       }
     }
+    // the table entries do not depend on the state: fetch all eight up front
+    uint4 e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = tab[(uint32_t)(sy >> (8 * j)) & 0xFFu];
 #pragma unroll
     for (int j = 7; j >= 0; --j) {
-      const uint32_t sym = (uint32_t)(sy >> (8 * j)) & 0xFFu;
-      const uint2 e = tab[sym];
-      const uint32_t f = e.x >> 16, cum = e.x & 0xFFFFu;
-      const bool need = x >= (f << 20);
+      const uint32_t f = e[j].y;
+      const bool need = x >= e[j].x;
       const uint64_t m = __ballot(need);
-      const uint32_t cnt = (uint32_t)__popcll(m);
-      if (cnt > pos) {
-        overflow = true;
-        break;
-      }
-      pos -= cnt;
-      if (need) {
-        slot[pos + nz_rank_below(m)] = (uint16_t)(x & 0xFFFFu);
-        x >>= 16;
-      }
+      pos -= (uint32_t)__popcll(m);
+      if (need) slot[pos + nz_rank_below(m)] = (uint16_t)(x & 0xFFFFu);
+      x = need ? (x >> 16) : x;
       // x < f << 20 here, so the quotient is below 2^20 and the float estimate
       // x * (1/f) (three roundings of 2^-24 each) is off by less than one:
       // truncate, then correct by the sign of the remainder.  With the exact
       // quotient q the new state is (q << 12) + (x - q f) + cum
       //                            = x + q (4096 - f) + cum.
-      uint32_t q = (uint32_t)((float)x * __uint_as_float(e.y));
+      uint32_t q = (uint32_t)((float)x * __uint_as_float(e[j].w));
       const int32_t rem = (int32_t)(x - __umul24(q, f));
       q += (rem >= (int32_t)f) ? 1u : 0u;
       q -= (rem < 0) ? 1u : 0u;
-      x = __umul24(q, NZ_M - f) + (x + cum);
+      x = __umul24(q, NZ_M - f) + (x + e[j].z);
     }
   }
   states[seg * NZ_LANES + lane] = x;
-  if (lane == 0) seg_words[seg] = overflow ? 0xFFFFFFFFu : (cap_words - pos);
+  if (lane == 0) seg_words[seg] = cap_words - pos;
 }
 
 // ----------------------------------------------------------------------------
@@ -431,15 +433,13 @@ __global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32
   const uint32_t nseg = (cn + seg_syms - 1) / seg_syms;
   const uint32_t tab_len = info[c].tab_len;
   uint64_t rans_total = tab_len, raw_total = 4;
-  bool overflow = false;
   for (uint32_t k = 0; k < nseg; ++k) {
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
     const uint32_t w = seg_words[c * spc + k];
-    if (w == 0xFFFFFFFFu) overflow = true;
-    else rans_total += 256 + 2 * (uint64_t)((w + 1) & ~1u);
+    rans_total += 256 + 2 * (uint64_t)((w + 1) & ~1u);
     raw_total += ((sn + 3) & ~3u) + (sn == seg_syms ? NZ_CARRY_BYTES : 0u);
   }
-  const bool raw = overflow || rans_total >= raw_total;
+  const bool raw = rans_total >= raw_total;
   info[c].raw = raw ? 1u : 0u;
   for (uint32_t k = 0; k < nseg; ++k) {
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
@@ -553,7 +553,7 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
   uint32_t* sdst = reinterpret_cast<uint32_t*>(dst + off);
   if (tid < 64) sdst[tid] = states[seg * NZ_LANES + tid];
   const uint32_t w = seg_words[seg];
-  const uint32_t cap_words = g.seg_syms / 2;
+  const uint32_t cap_words = g.seg_syms;
   const uint16_t* src = slots + seg * cap_words + (cap_words - w);
   uint16_t* wdst = reinterpret_cast<uint16_t*>(dst + off + 256);
   for (uint32_t i = tid; i < w; i += 256) wdst[i] = src[i];

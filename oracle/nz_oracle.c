@@ -310,8 +310,8 @@ static int make_geom(geom_t* g, uint64_t n, uint32_t chunk_syms, uint32_t lane_s
 
 /* worst-case bytes of one segment record holding seg_n symbols */
 static size_t seg_rec_cap(const geom_t* g) {
-  /* table (<= 420) + states (256) + words (<= seg_syms bytes) ; RAW: 4 + seg_syms + 128 */
-  return 420 + 256 + (size_t)g->seg_syms + 8;
+  /* table (<= 420) + states (256) + words (at most one per symbol) ; RAW: 4 + seg_syms + 128 */
+  return 420 + 256 + 2 * (size_t)g->seg_syms + 8;
 }
 
 size_t nzo_exp_bound(uint64_t n, uint32_t chunk_syms, uint32_t lane_syms) {
@@ -465,11 +465,12 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint16_t* s
       off = tbytes;
     }
     uint32_t states[NZO_LANES];
-    uint16_t* words = (uint16_t*)malloc((size_t)g->seg_syms + 8);
+    uint16_t* words = (uint16_t*)malloc(2 * (size_t)g->seg_syms + 8);
     /* only full segments carry payload in their start states */
     const uint16_t* sd = (seeds && sn == g->seg_syms) ? seeds + (seg0 + k) * NZO_LANES : NULL;
+    /* one word per symbol is the most a segment can emit: no overflow */
     int64_t nw = encode_segment(cs + (size_t)k * g->seg_syms, sn, pad, freq, cum, sd, words,
-                                g->seg_syms / 2, states);
+                                g->seg_syms, states);
     if (nw < 0) {
       overflow = 1;
       nw = 0;
