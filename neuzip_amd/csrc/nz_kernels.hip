@@ -21,7 +21,7 @@
 
 #define NZ_HIST_COPIES 8u
 #define NZ_HIST_STRIDE 257u
-#define NZ_RING_WORDS 2048u  // per-wave LDS ring of renormalisation words
+#define NZ_RING_WORDS 1024u  // per-wave LDS ring of renormalisation words
 #define NZ_RING_DWORDS (NZ_RING_WORDS / 2)
 
 // ----------------------------------------------------------------------------
@@ -567,10 +567,11 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
 // LDS: a 4096-entry slot table of 8-byte entries
 //          lo = freq | symbol << 24      hi = slot - cum[symbol]
 //      (so that one v_mad_u32_u24 of lo's low 24 bits gives the next state and
-//      the symbol is a whole byte for v_perm_b32) and a ring of 2048
-//      renormalisation words per wavefront; the table-parse scratch aliases the
-//      rings (it is dead before the first ring is filled).  Two wavefronts per
-//      chunk need exactly 40 KiB, so four workgroups share the 160 KiB of a CU.
+//      the symbol is a whole byte for v_perm_b32) and a ring of 1024
+//      renormalisation words (2 KiB) per wavefront; the table-parse scratch
+//      aliases the rings (it is dead before the first ring is filled).  Up to
+//      four wavefronts per chunk need at most 40 KiB, so four workgroups share
+//      the 160 KiB of a CU.
 // A rANS step per lane: one table read, one multiply-add, and when the state
 // falls below 2^16 a 16-bit word taken at (words consumed so far by the wave +
 // rank of the lane among the lanes that need one).
@@ -628,8 +629,7 @@ struct NzWaveDec {
   uint32_t x;             // this lane's rANS state
   uint32_t base;          // words consumed by the wave
   uint32_t filled;        // dwords staged into the ring (multiple of 256)
-  uint4 r;                // 8 words fetched during the previous group
-  bool pend;              // ... and whether they are to be committed
+  uint4 r;                // 8 words per lane fetched during the previous group
 
   // 16 bytes of the word stream at dword index d (multiple of 4 per lane).
   // Addresses are clamped to the container's closing padding, so every load is
@@ -648,15 +648,14 @@ struct NzWaveDec {
 
   __device__ __forceinline__ void start(uint32_t x0) {
     x = x0;
-    // 768 dwords = 1536 words ahead
-    uint4 v[3];
+    // fill the whole ring: 512 dwords = 1024 words ahead
+    uint4 v[2];
 #pragma unroll
-    for (uint32_t q = 0; q < 3; ++q) v[q] = fetch(256 * q + 4 * lane);
+    for (uint32_t q = 0; q < 2; ++q) v[q] = fetch(256 * q + 4 * lane);
 #pragma unroll
-    for (uint32_t q = 0; q < 3; ++q) commit(256 * q + 4 * lane, v[q]);
-    filled = 768;
+    for (uint32_t q = 0; q < 2; ++q) commit(256 * q + 4 * lane, v[q]);
+    filled = 512;
     base = 0;
-    pend = false;
     r = make_uint4(0, 0, 0, 0);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -665,22 +664,20 @@ struct NzWaveDec {
   // Decode the next 8 symbols of every lane into byte 3 of ew[0..7].
   //
   // Ring upkeep is software-pipelined over two groups so that no load is
-  // waited for in the group that issued it: at the start of a group the 512
-  // words fetched during the previous group are committed to the ring if that
-  // fetch was wanted (`pend`), then the next 512 words are fetched into
-  // registers unconditionally (clamped addresses, mostly cache hits) and marked
-  // wanted when no more than 1024 words are staged ahead.  A group consumes at
-  // most 8 * 64 = 512 words, so at least 512 words are ahead of `base` at every
-  // group start and the window [base, filled) never exceeds 1536 of the 2048
+  // waited for in the group that issued it: every group fetches the 512 words
+  // that follow the staged ones into registers (clamped addresses, mostly
+  // cache hits); at the start of the next group they are committed to the
+  // ring if no more than 512 words are still ahead of `base`.  A group
+  // consumes at most 8 * 64 = 512 words, so at least 512 words are ahead at
+  // every group start and the window [base, filled) never exceeds the 1024
   // ring words.
   __device__ __forceinline__ void group(uint32_t (&ew)[8]) {
-    if (pend) {
+    if ((2 * filled - base) <= 512u) {
       commit(filled + 4 * lane, r);
       filled += 256;
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
     }
-    pend = (2 * filled - base) <= 1024u;
     r = fetch(filled + 4 * lane);
     // LDS byte address of the ring (4 KiB aligned inside the workgroup's LDS)
     typedef __attribute__((address_space(3))) uint32_t lds_u32;
