@@ -34,7 +34,7 @@ bool precision_ok(int p) { return p == 7 || p == 3 || p == 1 || p == 0; }
 
 // Device scratch of one encode call.
 struct EncLayout {
-  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_units, hdr, total, status, bytes;
+  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, hdr, total, status, bytes;
 };
 
 EncLayout enc_layout(const NzGeom& g) {
@@ -51,8 +51,9 @@ EncLayout enc_layout(const NzGeom& g) {
   L.info = take(g.n_chunks * sizeof(NzChunkInfo));
   L.carry = take(g.n_segs * NZ_CARRY_BYTES);
   L.slots = take(g.n_segs * 2 * (uint64_t)g.seg_syms);  // one 2-byte word per symbol: the worst case
-  L.states = take(g.n_segs * NZ_LANES * 4);
+  L.states = take(g.n_segs * NZ_STATE_MAX_BYTES);
   L.seg_words = take(g.n_segs * 4);
+  L.seg_sbytes = take(g.n_segs * 4);
   L.seg_units = take((g.n_segs + 1) * 4);
   L.hdr = take(g.rec_off + NZ_TAIL_PAD);
   L.total = take(8);
@@ -87,11 +88,11 @@ int encode_phase1(const NzGeom& g, int precision, const void* in, uint8_t* packe
                        (const uint32_t*)(ws + L.enc_tab), (const NzChunkInfo*)(ws + L.info),
                        (const uint16_t*)(ws + L.carry), (uint16_t*)(ws + L.slots),
                        (uint32_t*)(ws + L.states),
-                       (uint32_t*)(ws + L.seg_words));
+                       (uint32_t*)(ws + L.seg_words), (uint32_t*)(ws + L.seg_sbytes));
     hipLaunchKernelGGL(nz_chunk_finalize_kernel, dim3((uint32_t)((g.n_chunks + 255) / 256)),
                        dim3(256), 0, st, g.n, g.chunk_syms, g.seg_syms, g.spc, g.n_chunks,
                        (NzChunkInfo*)(ws + L.info), (const uint32_t*)(ws + L.seg_words),
-                       (uint32_t*)(ws + L.seg_units));
+                       (const uint32_t*)(ws + L.seg_sbytes), (uint32_t*)(ws + L.seg_units));
   }
   hipLaunchKernelGGL(nz_scan_kernel, dim3(1), dim3(1024), 0, st,
                      (const uint32_t*)(ws + L.seg_units), g, hdr, cap, d_total, d_status);
@@ -107,7 +108,8 @@ int encode_phase2(const NzGeom& g, uint8_t* ws, const EncLayout& L, const uint32
                        ws + L.exps, g, (const NzChunkInfo*)(ws + L.info), ws + L.tab_ser,
                        ws + L.carry, (const uint16_t*)(ws + L.slots),
                        (const uint32_t*)(ws + L.states),
-                       (const uint32_t*)(ws + L.seg_words), dir, comp, cap);
+                       (const uint32_t*)(ws + L.seg_words), (const uint32_t*)(ws + L.seg_sbytes), dir,
+                       comp, cap);
     NZ_HIP(hipGetLastError());
   }
   return NZ_OK;
@@ -170,7 +172,7 @@ struct nz_manager {
 
 extern "C" {
 
-int nz_abi_version(void) { return 2; }
+int nz_abi_version(void) { return 3; }
 
 const char* nz_last_error(void) { return g_err.c_str(); }
 

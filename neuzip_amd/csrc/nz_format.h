@@ -13,9 +13,12 @@
 //             (g * 64 + l) * 8 + j.  A chunk holds 1..8 segments.
 // * directory entry k = offset of segment k's record in 4-byte units from
 //             `rec_off`; entry n_segs = end of the last record.
-// * record  = [table, first segment of a chunk only] [64 x u32 final encoder
-//             states] [u16 renormalisation words, front-to-back in decode
-//             order] padded to 4 bytes; or, for a chunk whose coded form
+// * record  = [table, first segment of a chunk only] [final encoder states:
+//             64 two-bit length codes (lane l at bits 2l, 2l+1; code c = the
+//             state takes 5 + c nibbles) and the states as a little-endian
+//             nibble stream in lane order, padded to 4 bytes] [u16
+//             renormalisation words, front-to-back in decode order] padded to
+//             4 bytes; or, for a chunk whose coded form
 //             would not be smaller, [0xFF 0 0 0, first segment only] raw
 //             exponent bytes padded to 4 [+ 64 x u16 carried bits if full].
 // * carry   = the encoder of a FULL segment starts lane l in state
@@ -31,7 +34,7 @@
 #include <stdint.h>
 
 #define NZ_MAGIC 0x315A4E41u
-#define NZ_FORMAT_VERSION 2u
+#define NZ_FORMAT_VERSION 3u
 #define NZ_PROB_BITS 12
 #define NZ_M (1u << NZ_PROB_BITS)
 #define NZ_L (1u << 16)
@@ -45,6 +48,7 @@
 #define NZ_TABLE_MAX_BYTES 424 /* 1 + 32 + 384 rounded up to a multiple of 8 */
 #define NZ_MAX_SEGS_PER_CHUNK 8
 #define NZ_CARRY_BYTES 128 /* 64 lanes x 16 bits */
+#define NZ_STATE_MAX_BYTES 272 /* 16 bytes of length codes + 64 x 32 bits */
 #define NZ_TAIL_PAD 16     /* zero bytes after the last record: 16-byte loads stay inside */
 
 struct NzGeom {

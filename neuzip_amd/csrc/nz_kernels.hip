@@ -70,6 +70,16 @@ __device__ __forceinline__ uint32_t nz_rank_below(uint64_t mask) {
                                    __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
 }
 
+// inclusive prefix sum over the 64 lanes of a wavefront
+__device__ __forceinline__ uint32_t nz_wave_scan(uint32_t v, uint32_t lane) {
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const uint32_t t = __shfl_up(v, o, 64);
+    if (lane >= (uint32_t)o) v += t;
+  }
+  return v;
+}
+
 __device__ __forceinline__ uint32_t nz_get12(const uint8_t* p, uint32_t i) {
   uint32_t bit = 12u * i;
   const uint8_t* q = p + (bit >> 3);
@@ -350,7 +360,9 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
     const uint8_t* __restrict__ exps, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
     uint32_t spc, const uint32_t* __restrict__ enc_tab, const NzChunkInfo* __restrict__ info,
     const uint16_t* __restrict__ carry, uint16_t* __restrict__ slots,
-    uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words) {
+    uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words,
+    uint32_t* __restrict__ seg_state_bytes) {
+  __shared__ uint32_t sbuf[NZ_MAX_SEGS_PER_CHUNK][NZ_STATE_MAX_BYTES / 4];
   // per symbol: x = freq << 20 (renormalisation threshold), y = freq, z = cum,
   // w = bits of 1.0f / freq
   __shared__ uint4 tab[256];
@@ -414,8 +426,31 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
       x = __umul24(q, NZ_M - f) + (x + e[j].z);
     }
   }
-  states[seg * NZ_LANES + lane] = x;
-  if (lane == 0) seg_words[seg] = cap_words - pos;
+  // Final states, variable length: 64 two-bit codes (code c = 5 + c nibbles),
+  // then the states as a little-endian nibble stream in lane order.  A state
+  // is >= 2^16, so it takes 20..32 bits; a flat 32 would waste ~4 more per lane.
+  const uint32_t code = (x >> 20 ? 1u : 0u) + (x >> 24 ? 1u : 0u) + (x >> 28 ? 1u : 0u);
+  const uint32_t nn = 5u + code;
+  const uint32_t incl = nz_wave_scan(nn, lane);
+  const uint32_t at = incl - nn;  // nibble offset of this lane's field
+  const uint32_t total = __builtin_amdgcn_readlane(incl, 63);
+  const uint32_t sbytes = 16u + ((((total + 1u) >> 1) + 3u) & ~3u);
+  uint32_t* sb = sbuf[wave];
+  for (uint32_t i = lane; i < NZ_STATE_MAX_BYTES / 4; i += 64) sb[i] = 0;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  atomicOr(&sb[lane >> 4], code << (2 * (lane & 15)));
+  const uint64_t field = (uint64_t)x << (4 * (at & 7));
+  atomicOr(&sb[4 + (at >> 3)], (uint32_t)field);
+  if (field >> 32) atomicOr(&sb[5 + (at >> 3)], (uint32_t)(field >> 32));
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  uint32_t* sdst = states + seg * (NZ_STATE_MAX_BYTES / 4);
+  for (uint32_t i = lane; i < sbytes / 4; i += 64) sdst[i] = sb[i];
+  if (lane == 0) {
+    seg_words[seg] = cap_words - pos;
+    seg_state_bytes[seg] = sbytes;
+  }
 }
 
 // ----------------------------------------------------------------------------
@@ -425,6 +460,7 @@ __global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32
                                          uint32_t spc, uint64_t n_chunks,
                                          NzChunkInfo* __restrict__ info,
                                          const uint32_t* __restrict__ seg_words,
+                                         const uint32_t* __restrict__ seg_state_bytes,
                                          uint32_t* __restrict__ seg_units) {
   const uint64_t c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= n_chunks) return;
@@ -436,7 +472,7 @@ __global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32
   for (uint32_t k = 0; k < nseg; ++k) {
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
     const uint32_t w = seg_words[c * spc + k];
-    rans_total += 256 + 2 * (uint64_t)((w + 1) & ~1u);
+    rans_total += seg_state_bytes[c * spc + k] + 2 * (uint64_t)((w + 1) & ~1u);
     raw_total += ((sn + 3) & ~3u) + (sn == seg_syms ? NZ_CARRY_BYTES : 0u);
   }
   const bool raw = rans_total >= raw_total;
@@ -446,7 +482,7 @@ __global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32
     const uint32_t w = seg_words[c * spc + k];
     uint32_t bytes;
     if (raw) bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u) + (sn == seg_syms ? NZ_CARRY_BYTES : 0u);
-    else bytes = (k == 0 ? tab_len : 0u) + 256u + 2u * ((w + 1) & ~1u);
+    else bytes = (k == 0 ? tab_len : 0u) + seg_state_bytes[c * spc + k] + 2u * ((w + 1) & ~1u);
     seg_units[c * spc + k] = bytes / 4;
   }
 }
@@ -519,8 +555,8 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
     const uint8_t* __restrict__ exps, NzGeom g, const NzChunkInfo* __restrict__ info,
     const uint8_t* __restrict__ tab_ser, const uint8_t* __restrict__ carry,
     const uint16_t* __restrict__ slots, const uint32_t* __restrict__ states,
-    const uint32_t* __restrict__ seg_words, const uint32_t* __restrict__ dir,
-    uint8_t* __restrict__ comp, uint64_t cap) {
+    const uint32_t* __restrict__ seg_words, const uint32_t* __restrict__ seg_state_bytes,
+    const uint32_t* __restrict__ dir, uint8_t* __restrict__ comp, uint64_t cap) {
   const uint64_t seg = blockIdx.x;
   const uint64_t c = seg / g.spc;
   const uint32_t k = (uint32_t)(seg - c * g.spc);
@@ -551,11 +587,12 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
     off = ci.tab_len;
   }
   uint32_t* sdst = reinterpret_cast<uint32_t*>(dst + off);
-  if (tid < 64) sdst[tid] = states[seg * NZ_LANES + tid];
+  const uint32_t sbytes = seg_state_bytes[seg];
+  if (tid < sbytes / 4) sdst[tid] = states[seg * (NZ_STATE_MAX_BYTES / 4) + tid];
   const uint32_t w = seg_words[seg];
   const uint32_t cap_words = g.seg_syms;
   const uint16_t* src = slots + seg * cap_words + (cap_words - w);
-  uint16_t* wdst = reinterpret_cast<uint16_t*>(dst + off + 256);
+  uint16_t* wdst = reinterpret_cast<uint16_t*>(dst + off + sbytes);
   for (uint32_t i = tid; i < w; i += 256) wdst[i] = src[i];
   if ((w & 1) && tid == 0) wdst[w] = 0;
 }
@@ -889,21 +926,36 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     return;
   }
 
-  if (rec_bytes < 256) {
+  if (rec_bytes < 16) {
     if (lane == 0) atomicOr(d_status, 2u);
     return;
   }
   // the record position is the same for all lanes: keep it in scalar registers
   const uint64_t rs = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(rec_start >> 32)) << 32) |
                       __builtin_amdgcn_readfirstlane((uint32_t)rec_start);
+  // final encoder states: 64 two-bit length codes, then a nibble stream
+  const uint32_t* rec32 = reinterpret_cast<const uint32_t*>(comp + rs);
+  const uint32_t nn = 5u + ((rec32[lane >> 4] >> (2 * (lane & 15))) & 3u);
+  const uint32_t incl = nz_wave_scan(nn, lane);
+  const uint32_t at = incl - nn;
+  const uint32_t sbytes = 16u + ((((__builtin_amdgcn_readlane(incl, 63) + 1u) >> 1) + 3u) & ~3u);
+  if (rec_bytes < sbytes) {
+    if (lane == 0) atomicOr(d_status, 2u);
+    return;
+  }
+  // the 8 bytes read here may reach into the words or the next record; the
+  // container's closing padding keeps them in bounds
+  const uint32_t fb = 16u + (at >> 1);
+  const uint64_t win = (uint64_t)rec32[fb >> 2] | ((uint64_t)rec32[(fb >> 2) + 1] << 32);
+  const uint32_t x0 = (uint32_t)(win >> (8 * (fb & 3) + 4 * (at & 1))) & (0xFFFFFFFFu >> (32 - 4 * nn));
   NzWaveDec w;
   w.lut = lut;
   w.ring32 = rings + wave * NZ_RING_ALLOC_DWORDS;
-  w.words = comp + rs + 256;
+  w.words = comp + rs + sbytes;
   w.last16 = comp + comp_bytes - NZ_TAIL_PAD;
-  w.nwords = __builtin_amdgcn_readfirstlane((uint32_t)((rec_bytes - 256) / 2));
+  w.nwords = __builtin_amdgcn_readfirstlane((uint32_t)((rec_bytes - sbytes) / 2));
   w.lane = lane;
-  w.start(reinterpret_cast<const uint32_t*>(comp + rs)[lane]);
+  w.start(x0);
 
   // groups whose packed bytes are (partly) carried are merged after the loop
   const uint32_t tailg = carry ? (S == 0 ? 2u : 1u) : 0u;

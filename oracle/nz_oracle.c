@@ -310,8 +310,8 @@ static int make_geom(geom_t* g, uint64_t n, uint32_t chunk_syms, uint32_t lane_s
 
 /* worst-case bytes of one segment record holding seg_n symbols */
 static size_t seg_rec_cap(const geom_t* g) {
-  /* table (<= 420) + states (256) + words (at most one per symbol) ; RAW: 4 + seg_syms + 128 */
-  return 420 + 256 + 2 * (size_t)g->seg_syms + 8;
+  /* table (<= 420) + states (<= 272) + words (at most one per symbol) ; RAW: 4 + seg_syms + 128 */
+  return 420 + 272 + 2 * (size_t)g->seg_syms + 8;
 }
 
 size_t nzo_exp_bound(uint64_t n, uint32_t chunk_syms, uint32_t lane_syms) {
@@ -341,6 +341,49 @@ static uint32_t get16(const uint8_t* p) { return (uint32_t)p[0] | ((uint32_t)p[1
 /* ------------------------------------------------------------------------- */
 /* segment encode / decode: 64 lanes, lane l owns symbols (g*64+l)*8 + j     */
 /* ------------------------------------------------------------------------- */
+
+/* Final encoder states, variable length: 64 two-bit length codes (lane l at
+   bits 2l, 2l+1 of a 16-byte little-endian block; code c means the state is
+   stored in 5 + c nibbles), then the states as a little-endian nibble stream in
+   lane order, zero padded to a multiple of 4 bytes.  A state is >= 2^16, so it
+   needs 20..32 bits; storing only the nibbles in use saves about 4 bits per
+   lane over a flat 32. */
+static size_t pack_states(const uint32_t x[NZO_LANES], uint8_t* out) {
+  uint8_t nib[NZO_LANES * 8 + 8];
+  size_t t = 0;
+  memset(out, 0, 16);
+  for (int l = 0; l < NZO_LANES; ++l) {
+    uint32_t c = 0;
+    while (c < 3 && (x[l] >> (4 * (5 + c))) != 0) ++c;
+    out[(2 * l) >> 3] |= (uint8_t)(c << ((2 * l) & 7));
+    for (uint32_t k = 0; k < 5 + c; ++k) nib[t++] = (x[l] >> (4 * k)) & 0xF;
+  }
+  size_t bytes = ((t + 1) / 2 + 3) & ~(size_t)3;
+  memset(out + 16, 0, bytes);
+  for (size_t k = 0; k < t; ++k) out[16 + (k >> 1)] |= (uint8_t)(nib[k] << (4 * (k & 1)));
+  return 16 + bytes;
+}
+
+static int unpack_states(const uint8_t* rec, size_t avail, uint32_t x[NZO_LANES], size_t* used) {
+  if (avail < 16) return NZO_ERR_CORRUPT;
+  size_t t = 0;
+  uint32_t n[NZO_LANES];
+  for (int l = 0; l < NZO_LANES; ++l) {
+    n[l] = 5 + ((rec[(2 * l) >> 3] >> ((2 * l) & 7)) & 3);
+    t += n[l];
+  }
+  size_t bytes = ((t + 1) / 2 + 3) & ~(size_t)3;
+  if (avail < 16 + bytes) return NZO_ERR_CORRUPT;
+  size_t k = 0;
+  for (int l = 0; l < NZO_LANES; ++l) {
+    uint32_t v = 0;
+    for (uint32_t q = 0; q < n[l]; ++q, ++k)
+      v |= (uint32_t)((rec[16 + (k >> 1)] >> (4 * (k & 1))) & 0xF) << (4 * q);
+    x[l] = v;
+  }
+  *used = 16 + bytes;
+  return NZO_OK;
+}
 
 /* Encode one segment.  Words are produced back to front into words[cap_words]
    so that the decoder reads them front to back.  Returns the number of words,
@@ -386,14 +429,13 @@ static int64_t encode_segment(const uint8_t* syms, uint32_t seg_n, int pad_sym,
 
 static int decode_segment(const uint8_t* rec, size_t rec_bytes, uint32_t seg_n,
                           const uint32_t* lut, uint8_t* out, uint16_t* seeds) {
-  if (rec_bytes < 256) return NZO_ERR_CORRUPT;
   uint32_t x[NZO_LANES];
-  for (int l = 0; l < NZO_LANES; ++l) {
-    x[l] = get32(rec + 4 * l);
+  size_t sbytes;
+  if (unpack_states(rec, rec_bytes, x, &sbytes)) return NZO_ERR_CORRUPT;
+  for (int l = 0; l < NZO_LANES; ++l)
     if (x[l] < NZO_L) return NZO_ERR_CORRUPT;
-  }
-  const uint8_t* w = rec + 256;
-  size_t nwords = (rec_bytes - 256) / 2, base = 0;
+  const uint8_t* w = rec + sbytes;
+  size_t nwords = (rec_bytes - sbytes) / 2, base = 0;
   uint32_t ngroups = (seg_n + NZO_GROUP_SYMS - 1) / NZO_GROUP_SYMS;
   for (uint32_t g = 0; g < ngroups; ++g) {
     for (int j = 0; j < NZO_GROUP; ++j) {
@@ -475,8 +517,7 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint16_t* s
       overflow = 1;
       nw = 0;
     }
-    for (int l = 0; l < NZO_LANES; ++l) put32(rec + off + 4 * l, states[l]);
-    off += 256;
+    off += pack_states(states, rec + off);
     for (int64_t i = 0; i < nw; ++i) put16(rec + off + 2 * i, words[i]);
     off += 2 * (size_t)nw;
     if (nw & 1) {

@@ -39,7 +39,7 @@ extern "C" {
 
 /* ---- format constants (shared with the HIP implementation by value) ---- */
 #define NZO_MAGIC 0x315A4E41u /* "ANZ1" little endian */
-#define NZO_VERSION 2u
+#define NZO_VERSION 3u
 #define NZO_PROB_BITS 12
 #define NZO_M (1u << NZO_PROB_BITS)
 #define NZO_L (1u << 16)

@@ -50,7 +50,7 @@ def decode_container(comp: bytes, n: int):
     """-> (symbols uint8[n], carried uint16[64 * full_segments])."""
     comp = bytes(comp)
     magic, version = _u32(comp, 0), _u32(comp, 4)
-    assert magic == 0x315A4E41 and version == 2
+    assert magic == 0x315A4E41 and version == 3
     assert _u32(comp, 8) | (_u32(comp, 12) << 32) == n
     chunk, lane = _u32(comp, 16), _u32(comp, 20)
     seg = 64 * lane
@@ -77,8 +77,18 @@ def decode_container(comp: bytes, n: int):
         freq = table
         cum = np.concatenate([[0], np.cumsum(freq)])
         slot2sym = np.repeat(np.arange(256), freq)
-        x = list(struct.unpack_from("<64I", rec, 0))
-        words = np.frombuffer(rec[256:], "<u2")
+        # 64 two-bit length codes, then the states as little-endian nibbles
+        flags = int.from_bytes(rec[:16], "little")
+        lens = [5 + ((flags >> (2 * l)) & 3) for l in range(64)]
+        total = sum(lens)
+        sbytes = ((total + 1) // 2 + 3) & ~3
+        stream = int.from_bytes(rec[16:16 + sbytes], "little")
+        x, at = [], 0
+        for n_l in lens:
+            x.append((stream >> (4 * at)) & ((1 << (4 * n_l)) - 1))
+            at += n_l
+        assert all(v >= L for v in x)
+        words = np.frombuffer(rec[16 + sbytes:], "<u2")
         pos = 0
         groups = (sn + 511) // 512
         for g in range(groups):

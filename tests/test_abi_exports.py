@@ -24,7 +24,7 @@ def test_header_symbols_are_exported():
     for name in names:
         assert hasattr(L, name), f"{name} declared in include/neuzip_hip.h but not exported"
     assert sorted(_lib.EXPORTS) == names  # the ctypes binding covers the whole header
-    assert L.nz_abi_version() == 2
+    assert L.nz_abi_version() == 3
 
 
 def test_size_helpers_match_oracle(oracle):
