@@ -71,7 +71,7 @@ class Codec:
             raise SystemExit("unsupported chunk_size / lane_symbols combination")
         self.cap = cap
         self.comp = torch.empty(cap, dtype=torch.uint8, device="cuda")
-        self.packed_bytes = int(L.nz_packed_stored_bytes(n, precision, lane))
+        self.packed_bytes = int(L.nz_packed_stored_bytes(n, precision, chunk, lane))
         self.packed_ref_bytes = int(L.nz_packed_bytes(n, precision))
         self.packed = torch.empty(max(8, self.packed_bytes), dtype=torch.uint8, device="cuda")
         self.ws_bytes = int(L.nz_encode_workspace_bytes(n, chunk, lane))

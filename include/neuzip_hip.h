@@ -60,10 +60,11 @@ const char* nz_last_error(void);
 uint64_t nz_packed_bytes(uint64_t n, int precision);
 
 /* Bytes actually stored for the packed stream: the last 128 bytes of every
-   full segment (64 * lane_syms elements) travel inside the entropy coder's
-   start states instead (16 bits per rANS lane), so each full segment stores
-   128 bytes fewer than the reference layout. */
-uint64_t nz_packed_stored_bytes(uint64_t n, int precision, uint32_t lane_syms);
+   full segment (a chunk is cut into segments of 64 * lane_syms elements, the
+   last one shorter) travel inside the entropy coder's start states instead
+   (16 bits per rANS lane), so each full segment stores 128 bytes fewer than
+   the reference layout. */
+uint64_t nz_packed_stored_bytes(uint64_t n, int precision, uint32_t chunk_size, uint32_t lane_syms);
 
 /* Capacity that always holds the entropy-coded exponent container of n
    elements (stands in for nvcomp's max_compressed_buffer_size,

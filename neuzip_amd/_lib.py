@@ -52,7 +52,7 @@ def load() -> ctypes.CDLL:
     L.nz_packed_bytes.restype = u64
     L.nz_packed_bytes.argtypes = [u64, i32]
     L.nz_packed_stored_bytes.restype = u64
-    L.nz_packed_stored_bytes.argtypes = [u64, i32, u32]
+    L.nz_packed_stored_bytes.argtypes = [u64, i32, u32, u32]
     L.nz_exp_bound_bytes.restype = u64
     L.nz_exp_bound_bytes.argtypes = [u64, u32, u32]
     L.nz_encode_workspace_bytes.restype = u64

@@ -66,7 +66,7 @@ template <int S>
 void launch_split_hist(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws,
                        const EncLayout& L, hipStream_t st) {
   hipLaunchKernelGGL(nz_split_hist_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(NZ_SPLIT_THREADS), 0, st,
-                     (const uint16_t*)in, g.n, g.chunk_syms, g.seg_syms, packed, ws + L.carry,
+                     (const uint16_t*)in, g.n, g.chunk_syms, g.seg_syms, g.spc, packed, ws + L.carry,
                      ws + L.exps, (uint32_t*)(ws + L.enc_tab), ws + L.tab_ser,
                      (NzChunkInfo*)(ws + L.info));
 }
@@ -140,8 +140,8 @@ int decode_launch(const NzGeom& g, int precision, const void* comp, uint64_t com
 int make_geom(NzGeom* g, uint64_t n, uint32_t chunk, uint32_t lane_syms) {
   if (nz_geom_make(g, n, chunk, lane_syms))
     return fail(NZ_ERR_ARG,
-                "unsupported geometry: lane_syms must be a multiple of 8 and chunk_size a "
-                "multiple of 64*lane_syms holding 1..8 segments");
+                "unsupported geometry: lane_syms must be a multiple of 8 (>= 16), chunk_size a multiple "
+                "of 512 cut into 1..8 segments of 64*lane_syms, the last one at least 1024 long");
   if (g->n_chunks > 0x7FFFFFFFull) return fail(NZ_ERR_ARG, "tensor too large");
   return NZ_OK;
 }
@@ -172,15 +172,16 @@ struct nz_manager {
 
 extern "C" {
 
-int nz_abi_version(void) { return 3; }
+int nz_abi_version(void) { return 4; }
 
 const char* nz_last_error(void) { return g_err.c_str(); }
 
 uint64_t nz_packed_bytes(uint64_t n, int precision) { return nz_packed_bytes_of(n, precision); }
 
-uint64_t nz_packed_stored_bytes(uint64_t n, int precision, uint32_t lane_syms) {
-  if (lane_syms < 16) return 0;
-  return nz_packed_stored_bytes_of(n, precision, lane_syms);
+uint64_t nz_packed_stored_bytes(uint64_t n, int precision, uint32_t chunk_size, uint32_t lane_syms) {
+  NzGeom g;
+  if (nz_geom_make(&g, n, chunk_size, lane_syms)) return 0;
+  return nz_packed_stored_bytes_of(&g, precision);
 }
 
 uint64_t nz_exp_bound_bytes(uint64_t n, uint32_t chunk_size, uint32_t lane_syms) {
@@ -327,10 +328,9 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   // down to the 8 segments a chunk may hold, at ~8.5 bits per extra lane.
   uint32_t lane_syms = m->lane_syms;
   if (m->auto_lanes) {
-    while (lane_syms > 16 && (lane_syms / 2) % NZ_GROUP == 0 &&
-           (uint64_t)(lane_syms / 2) * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK >= m->chunk_syms &&
+    while (lane_syms > 16 && nz_geom_check(m->chunk_syms, (lane_syms / 2 + 7) & ~7u) == 0 &&
            n / ((uint64_t)lane_syms * NZ_LANES) < 2048)
-      lane_syms /= 2;
+      lane_syms = (lane_syms / 2 + 7) & ~7u;
   }
   NzGeom g;
   if (int rc = make_geom(&g, n, m->chunk_syms, lane_syms)) return rc;
@@ -361,7 +361,7 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   ent.n = n;
   ent.dtype = dtype;
   ent.lane_syms = lane_syms;
-  ent.packed_bytes = nz_packed_stored_bytes_of(n, m->precision, lane_syms);
+  ent.packed_bytes = nz_packed_stored_bytes_of(&g, m->precision);
   auto release = [&](Entry& e) {
     if (e.comp) (void)hipFree(e.comp);
     if (e.packed) (void)hipFree(e.packed);

@@ -10,7 +10,9 @@
 //             chunk_size = 65536, cuda/neuzip.cu:31).
 // * segment = 64 * `lane_syms` consecutive exponents decoded by ONE wavefront:
 //             64 interleaved rANS states, lane l owning the 8-symbol groups
-//             (g * 64 + l) * 8 + j.  A chunk holds 1..8 segments.
+//             (g * 64 + l) * 8 + j.  A chunk is cut into spc = 1..8 segments,
+//             the last one holding what remains of the chunk (>= 1024
+//             symbols); segment c * spc + k is the k-th segment of chunk c.
 // * directory entry k = offset of segment k's record in 4-byte units from
 //             `rec_off`; entry n_segs = end of the last record.
 // * record  = [table, first segment of a chunk only] [final encoder states:
@@ -33,8 +35,14 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#ifdef __HIPCC__
+#define NZ_HD __host__ __device__
+#else
+#define NZ_HD
+#endif
+
 #define NZ_MAGIC 0x315A4E41u
-#define NZ_FORMAT_VERSION 3u
+#define NZ_FORMAT_VERSION 4u
 #define NZ_PROB_BITS 12
 #define NZ_M (1u << NZ_PROB_BITS)
 #define NZ_L (1u << 16)
@@ -74,10 +82,10 @@ struct NzChunkInfo {
 static inline int nz_geom_check(uint32_t chunk_syms, uint32_t lane_syms) {
   if (lane_syms < 16 || (lane_syms % NZ_GROUP) != 0 || lane_syms > (1u << 16)) return -1;
   uint64_t seg = (uint64_t)lane_syms * NZ_LANES;
-  if (chunk_syms == 0 || (chunk_syms % seg) != 0) return -1;
-  uint64_t spc = chunk_syms / seg;
+  if (chunk_syms == 0 || (chunk_syms % NZ_GROUP_SYMS) != 0 || chunk_syms > (1u << 24)) return -1;
+  uint64_t spc = (chunk_syms + seg - 1) / seg;
   if (spc < 1 || spc > NZ_MAX_SEGS_PER_CHUNK) return -1;
-  if (chunk_syms > (1u << 24)) return -1;
+  if (chunk_syms - (spc - 1) * seg < 1024) return -1;  // the last segment must be able to carry 128 bytes
   return 0;
 }
 
@@ -87,9 +95,9 @@ static inline int nz_geom_make(NzGeom* g, uint64_t n, uint32_t chunk_syms, uint3
   g->chunk_syms = chunk_syms;
   g->lane_syms = lane_syms;
   g->seg_syms = lane_syms * NZ_LANES;
-  g->spc = chunk_syms / g->seg_syms;
+  g->spc = (chunk_syms + g->seg_syms - 1) / g->seg_syms;
   g->n_chunks = (n + chunk_syms - 1) / chunk_syms;
-  g->n_segs = (n + g->seg_syms - 1) / g->seg_syms;
+  g->n_segs = (n / chunk_syms) * g->spc + ((n % chunk_syms) + g->seg_syms - 1) / g->seg_syms;
   if (g->n_segs >= 0xFFFFFFFEull) return -1;
   g->dir_off = NZ_HEADER_BYTES;
   g->rec_off = (NZ_HEADER_BYTES + 4 * (g->n_segs + 1) + 15) & ~(uint64_t)15;
@@ -105,8 +113,20 @@ static inline uint64_t nz_packed_bytes_of(uint64_t n, int s) {
   return (n * (uint64_t)(s + 1) + 7) / 8;  // cuda/high_level.cu:81-83
 }
 
+// Symbols segment k of a chunk holds when the tensor does not end inside it.
+NZ_HD static inline uint32_t nz_seg_nominal(uint32_t chunk_syms, uint32_t seg_syms, uint32_t spc, uint32_t k) {
+  return k + 1 < spc ? seg_syms : chunk_syms - (spc - 1) * seg_syms;
+}
+
+// Segments the tensor does not end inside ("full": they carry 128 packed bytes).
+static inline uint64_t nz_full_segments(const NzGeom* g) {
+  uint64_t rem = g->n % g->chunk_syms, fs = rem / g->seg_syms;
+  if (fs > g->spc - 1) fs = g->spc - 1;
+  return (g->n / g->chunk_syms) * g->spc + fs;
+}
+
 // Bytes actually stored for the packed stream: the reference size minus the
 // carried bytes of every full segment.
-static inline uint64_t nz_packed_stored_bytes_of(uint64_t n, int s, uint32_t lane_syms) {
-  return nz_packed_bytes_of(n, s) - (uint64_t)NZ_CARRY_BYTES * (n / ((uint64_t)lane_syms * NZ_LANES));
+static inline uint64_t nz_packed_stored_bytes_of(const NzGeom* g, int s) {
+  return nz_packed_bytes_of(g->n, s) - (uint64_t)NZ_CARRY_BYTES * nz_full_segments(g);
 }

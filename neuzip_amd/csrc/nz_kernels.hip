@@ -156,7 +156,7 @@ __device__ __forceinline__ uint32_t nz_block_max(uint32_t v, uint32_t* red) {
 
 template <int S>
 __global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
-    const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms,
+    const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms, uint32_t spc,
     uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
     uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info) {
   // 8 histogram copies (one per lane & 7) at a stride of 257 words: exponents of
@@ -181,18 +181,20 @@ __global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
   // Packed bytes go to the stored layout: segment k starts at k * keep, and the
   // last NZ_CARRY_BYTES of a full segment go to carry[k] instead (they ride in
   // the rANS start states).
-  const uint32_t seg_p = seg_syms / 8 * (S + 1);
-  const uint32_t keep = seg_p - NZ_CARRY_BYTES;
-  const uint64_t seg0 = base / seg_syms;
+  const uint32_t seg_keep = seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES;     // of a segment of nominal length
+  const uint64_t chunk_keep = (uint64_t)chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * spc;
+  const uint64_t seg0 = c * spc;
 
   for (uint32_t i = tid * 8; i < cn; i += NZ_SPLIT_THREADS * 8) {
     const uint64_t gi = base + i;
     const uint32_t sk = i / seg_syms;                    // segment inside the chunk
     const uint32_t sb = (i - sk * seg_syms) / 8 * (S + 1);  // byte inside the segment
     const uint64_t seg = seg0 + sk;
-    const bool seg_full = (seg + 1) * seg_syms <= n;
+    const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, sk);
+    const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
+    const bool seg_full = base + (uint64_t)sk * seg_syms + nom <= n;
     uint8_t* pp = (seg_full && sb >= keep) ? carry + seg * NZ_CARRY_BYTES + (sb - keep)
-                                           : packed + seg * keep + sb;
+                                           : packed + c * chunk_keep + (uint64_t)sk * seg_keep + sb;
     uint32_t ex[8], rp[8];
     const uint32_t rem = cn - i;
     if (rem >= 8) {
@@ -378,9 +380,10 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t seg_syms = lane_syms * NZ_LANES;
   const uint64_t seg = c * spc + wave;
-  const uint64_t seg_base = seg * seg_syms;
+  const uint64_t seg_base = c * chunk_syms + (uint64_t)wave * seg_syms;
   if (seg_base >= n) return;
-  const uint32_t seg_n = (uint32_t)((n - seg_base) < seg_syms ? (n - seg_base) : seg_syms);
+  const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, wave);
+  const uint32_t seg_n = (uint32_t)((n - seg_base) < nom ? (n - seg_base) : nom);
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
   const uint32_t cap_words = seg_syms;
   const uint32_t pad = info[c].pad_sym;
@@ -388,7 +391,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
   const uint8_t* src = exps + seg_base;
 
   // a full segment starts from 2^16 | 16 carried bits of the packed stream
-  uint32_t x = NZ_L | (seg_n == seg_syms ? (uint32_t)carry[seg * NZ_LANES + lane] : 0u);
+  uint32_t x = NZ_L | (seg_n == nom ? (uint32_t)carry[seg * NZ_LANES + lane] : 0u);
   uint32_t pos = cap_words;
   for (uint32_t g = ngroups; g-- > 0;) {
     const uint32_t idx0 = (g * NZ_LANES + lane) * NZ_GROUP;
@@ -473,7 +476,7 @@ __global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
     const uint32_t w = seg_words[c * spc + k];
     rans_total += seg_state_bytes[c * spc + k] + 2 * (uint64_t)((w + 1) & ~1u);
-    raw_total += ((sn + 3) & ~3u) + (sn == seg_syms ? NZ_CARRY_BYTES : 0u);
+    raw_total += ((sn + 3) & ~3u) + (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
   }
   const bool raw = rans_total >= raw_total;
   info[c].raw = raw ? 1u : 0u;
@@ -481,7 +484,9 @@ __global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
     const uint32_t w = seg_words[c * spc + k];
     uint32_t bytes;
-    if (raw) bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u) + (sn == seg_syms ? NZ_CARRY_BYTES : 0u);
+    if (raw)
+      bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u) +
+              (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
     else bytes = (k == 0 ? tab_len : 0u) + seg_state_bytes[c * spc + k] + 2u * ((w + 1) & ~1u);
     seg_units[c * spc + k] = bytes / 4;
   }
@@ -565,8 +570,9 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
   uint8_t* dst = comp + g.rec_off + 4 * o0;
   if (seg + 1 == g.n_segs && threadIdx.x >= 256 - NZ_TAIL_PAD)  // closing zeros
     comp[g.rec_off + 4 * o1 + (threadIdx.x - (256 - NZ_TAIL_PAD))] = 0;
-  const uint64_t seg_base = seg * g.seg_syms;
-  const uint32_t sn = (uint32_t)((g.n - seg_base) < g.seg_syms ? (g.n - seg_base) : g.seg_syms);
+  const uint64_t seg_base = c * g.chunk_syms + (uint64_t)k * g.seg_syms;
+  const uint32_t nom = nz_seg_nominal(g.chunk_syms, g.seg_syms, g.spc, k);
+  const uint32_t sn = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
   const NzChunkInfo ci = info[c];
   const uint32_t tid = threadIdx.x;
   if (ci.raw) {
@@ -577,7 +583,7 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
     }
     const uint32_t padded = (sn + 3) & ~3u;
     for (uint32_t i = tid; i < padded; i += 256) dst[off + i] = i < sn ? exps[seg_base + i] : 0;
-    if (sn == g.seg_syms && tid < NZ_CARRY_BYTES) dst[off + padded + tid] = carry[seg * NZ_CARRY_BYTES + tid];
+    if (sn == nom && tid < NZ_CARRY_BYTES) dst[off + padded + tid] = carry[seg * NZ_CARRY_BYTES + tid];
     return;
   }
   uint32_t off = 0;
@@ -868,8 +874,9 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
 
   if (wave >= nseg) return;
   const uint64_t seg = seg0 + wave;
-  const uint64_t seg_base = seg * g.seg_syms;
-  const uint32_t seg_n = (uint32_t)((g.n - seg_base) < g.seg_syms ? (g.n - seg_base) : g.seg_syms);
+  const uint64_t seg_base = chunk_base + (uint64_t)wave * g.seg_syms;
+  const uint32_t nom = nz_seg_nominal(g.chunk_syms, g.seg_syms, g.spc, wave);
+  const uint32_t seg_n = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
   uint64_t o0 = dir[seg], o1 = dir[seg + 1];
   if (o1 < o0 || g.rec_off + 4 * o1 > comp_bytes) {
@@ -888,10 +895,10 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
   }
   // stored packed layout: every full segment keeps seg_p - 128 bytes, its last
   // 128 bytes ride in the coder states (or behind the symbols of a raw record)
-  const bool carry = seg_n == g.seg_syms;
-  const uint32_t seg_p = g.seg_syms / 8 * (S + 1);
-  const uint32_t keep = seg_p - NZ_CARRY_BYTES;
-  const uint8_t* pk = packed + seg * keep;
+  const bool carry = seg_n == nom;
+  const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
+  const uint64_t chunk_keep = (uint64_t)g.chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * g.spc;
+  const uint8_t* pk = packed + c * chunk_keep + (uint64_t)wave * (g.seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES);
   uint16_t* dst = out + seg_base;
 
   if (mode == NZ_MODE_RAW) {

@@ -286,10 +286,12 @@ int nzo_check_geometry(uint32_t chunk_syms, uint32_t lane_syms) {
   if (lane_syms < 16 || lane_syms % NZO_GROUP) return NZO_ERR_ARG;
   if (lane_syms > (1u << 16)) return NZO_ERR_ARG;
   uint64_t seg = (uint64_t)lane_syms * NZO_LANES;
-  if (chunk_syms == 0 || chunk_syms % seg) return NZO_ERR_ARG;
-  uint64_t spc = chunk_syms / seg;
+  if (chunk_syms == 0 || chunk_syms % NZO_GROUP_SYMS || chunk_syms > (1u << 24)) return NZO_ERR_ARG;
+  /* a chunk is cut into spc segments of 64 * lane_syms symbols, the last one
+     holding what remains (at least 1024 symbols, so that it can carry 128 bytes) */
+  uint64_t spc = (chunk_syms + seg - 1) / seg;
   if (spc < 1 || spc > 8) return NZO_ERR_ARG;
-  if (chunk_syms > (1u << 24)) return NZO_ERR_ARG;
+  if (chunk_syms - (spc - 1) * seg < 1024) return NZO_ERR_ARG;
   return NZO_OK;
 }
 
@@ -299,13 +301,19 @@ static int make_geom(geom_t* g, uint64_t n, uint32_t chunk_syms, uint32_t lane_s
   g->chunk_syms = chunk_syms;
   g->lane_syms = lane_syms;
   g->seg_syms = lane_syms * NZO_LANES;
-  g->spc = chunk_syms / g->seg_syms;
+  g->spc = (chunk_syms + g->seg_syms - 1) / g->seg_syms;
   g->n_chunks = (n + chunk_syms - 1) / chunk_syms;
-  g->n_segs = (n + g->seg_syms - 1) / g->seg_syms;
+  /* segment c * spc + k is the k-th segment of chunk c; a ragged last chunk has fewer */
+  g->n_segs = (n / chunk_syms) * g->spc + ((n % chunk_syms) + g->seg_syms - 1) / g->seg_syms;
   if (g->n_segs >= 0xFFFFFFFEull) return NZO_ERR_ARG;
   g->dir_off = NZO_HEADER_BYTES;
   g->rec_off = (NZO_HEADER_BYTES + 4 * (size_t)(g->n_segs + 1) + 15) & ~(size_t)15;
   return NZO_OK;
+}
+
+/* symbols segment k of a chunk holds when the tensor does not end inside it */
+static uint32_t seg_nominal(const geom_t* g, uint32_t k) {
+  return k + 1 < g->spc ? g->seg_syms : g->chunk_syms - (g->spc - 1) * g->seg_syms;
 }
 
 /* worst-case bytes of one segment record holding seg_n symbols */
@@ -509,7 +517,7 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint16_t* s
     uint32_t states[NZO_LANES];
     uint16_t* words = (uint16_t*)malloc(2 * (size_t)g->seg_syms + 8);
     /* only full segments carry payload in their start states */
-    const uint16_t* sd = (seeds && sn == g->seg_syms) ? seeds + (seg0 + k) * NZO_LANES : NULL;
+    const uint16_t* sd = (seeds && sn == seg_nominal(g, k)) ? seeds + (seg0 + k) * NZO_LANES : NULL;
     /* one word per symbol is the most a segment can emit: no overflow */
     int64_t nw = encode_segment(cs + (size_t)k * g->seg_syms, sn, pad, freq, cum, sd, words,
                                 g->seg_syms, states);
@@ -527,7 +535,7 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint16_t* s
     free(words);
     seg_bytes[seg0 + k] = (uint32_t)off;
     rans_total += off - (k == 0 ? tbytes : 0);
-    raw_total += (((size_t)sn + 3) & ~(size_t)3) + (sn == g->seg_syms ? 2 * NZO_LANES : 0);
+    raw_total += (((size_t)sn + 3) & ~(size_t)3) + (sn == seg_nominal(g, k) ? 2 * NZO_LANES : 0);
   }
   if (overflow || rans_total >= raw_total) {
     for (uint32_t k = 0; k < nseg; ++k) {
@@ -543,7 +551,7 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint16_t* s
       size_t padded = ((size_t)sn + 3) & ~(size_t)3;
       memset(rec + off + sn, 0, padded - sn);
       off += padded;
-      if (sn == g->seg_syms) { /* a raw full segment still has to hold its 64 x 16 carried bits */
+      if (sn == seg_nominal(g, k)) { /* a raw full segment still has to hold its 64 x 16 carried bits */
         for (int l = 0; l < NZO_LANES; ++l)
           put16(rec + off + 2 * l, seeds ? seeds[(seg0 + k) * NZO_LANES + l] : 0u);
         off += 2 * NZO_LANES;
@@ -698,7 +706,7 @@ static int decode_chunk(const geom_t* g, const uint8_t* comp, size_t comp_bytes,
       }
     }
     uint16_t tmp[NZO_LANES];
-    uint16_t* sd = sn == g->seg_syms ? (seeds ? seeds + (seg0 + k) * NZO_LANES : tmp) : NULL;
+    uint16_t* sd = sn == seg_nominal(g, k) ? (seeds ? seeds + (seg0 + k) * NZO_LANES : tmp) : NULL;
     if (raw) {
       size_t padded = ((size_t)sn + 3) & ~(size_t)3;
       if (rbytes < padded + (sd ? 2 * NZO_LANES : 0)) return NZO_ERR_CORRUPT;
@@ -825,21 +833,58 @@ static void run_sm(void* (*fn)(void*), const uint16_t* data, uint16_t* out, uint
 /* Stored layout of the packed sign|mantissa stream: the reference layout
    (byte idx*(s+1)/8, MSB first) with the last 128 bytes of every FULL segment
    taken out; those 64 x 16 bits ride in the start states of the segment's 64
-   rANS lanes (lane l carries bytes 2l and 2l+1, little endian). */
-size_t nzo_packed_stored_bytes(uint64_t n, int s, uint32_t lane_syms) {
-  uint64_t seg = (uint64_t)lane_syms * NZO_LANES;
-  return nzo_packed_bytes(n, s) - 2 * NZO_LANES * (size_t)(n / seg);
+   rANS lanes (lane l carries bytes 2l and 2l+1, little endian).  A segment is
+   full when the tensor does not end inside it. */
+static uint64_t full_segments(const geom_t* g) {
+  uint64_t rem = g->n % g->chunk_syms, fs = rem / g->seg_syms;
+  if (fs > g->spc - 1) fs = g->spc - 1;
+  return (g->n / g->chunk_syms) * g->spc + fs;
+}
+
+size_t nzo_packed_stored_bytes(uint64_t n, int s, uint32_t chunk_syms, uint32_t lane_syms) {
+  geom_t g;
+  if (make_geom(&g, n, chunk_syms, lane_syms)) return 0;
+  return nzo_packed_bytes(n, s) - 2 * NZO_LANES * (size_t)full_segments(&g);
+}
+
+/* move the packed bytes between the reference layout (`full`) and the stored
+   layout + per-segment carried bytes */
+static void carry_layout(const geom_t* g, int s, uint8_t* full, uint8_t* stored, uint16_t* seeds,
+                         int to_stored) {
+  size_t total = nzo_packed_bytes(g->n, s), src = 0, dst = 0;
+  for (uint64_t c = 0; c < g->n_chunks; ++c) {
+    uint64_t base = c * g->chunk_syms;
+    uint32_t cn = (uint32_t)(g->n - base < g->chunk_syms ? g->n - base : g->chunk_syms);
+    uint32_t nseg = (cn + g->seg_syms - 1) / g->seg_syms;
+    for (uint32_t k = 0; k < nseg; ++k) {
+      uint32_t sn = cn - k * g->seg_syms < g->seg_syms ? cn - k * g->seg_syms : g->seg_syms;
+      int is_full = sn == seg_nominal(g, k);
+      size_t bytes = is_full ? (size_t)sn * (size_t)(s + 1) / 8 : total - src;
+      size_t keep = is_full ? bytes - 2 * NZO_LANES : bytes;
+      if (to_stored) memcpy(stored + dst, full + src, keep);
+      else memcpy(full + src, stored + dst, keep);
+      if (is_full) {
+        uint16_t* sd = seeds + (c * g->spc + k) * NZO_LANES;
+        for (int l = 0; l < NZO_LANES; ++l) {
+          if (to_stored) sd[l] = (uint16_t)get16(full + src + keep + 2 * l);
+          else put16(full + src + keep + 2 * l, sd[l]);
+        }
+      }
+      src += bytes;
+      dst += keep;
+    }
+  }
 }
 
 int64_t nzo_compress_bf16(const uint16_t* data, uint64_t n, int s, uint32_t chunk_syms,
                           uint32_t lane_syms, uint8_t* fractions, uint8_t* comp, size_t cap,
                           int threads) {
   if (!(s == 7 || s == 3 || s == 1 || s == 0)) return NZO_ERR_ARG;
-  if (nzo_check_geometry(chunk_syms, lane_syms)) return NZO_ERR_ARG;
+  geom_t g;
+  if (make_geom(&g, n, chunk_syms, lane_syms)) return NZO_ERR_ARG;
   uint8_t* exps = (uint8_t*)malloc((size_t)n + 1);
   uint8_t* full = (uint8_t*)malloc(nzo_packed_bytes(n, s) + 1);
-  uint64_t seg = (uint64_t)lane_syms * NZO_LANES, nfull = n / seg;
-  uint16_t* seeds = (uint16_t*)malloc((size_t)(nfull + 1) * NZO_LANES * 2);
+  uint16_t* seeds = (uint16_t*)calloc((size_t)(g.n_segs + 1) * NZO_LANES, 2);
   if (!exps || !full || !seeds) {
     free(exps);
     free(full);
@@ -847,13 +892,7 @@ int64_t nzo_compress_bf16(const uint16_t* data, uint64_t n, int s, uint32_t chun
     return NZO_ERR_CAP;
   }
   run_sm(split_worker, data, NULL, exps, full, n, s, threads);
-  size_t seg_p = (size_t)(seg * (uint64_t)(s + 1) / 8), keep = seg_p - 2 * NZO_LANES;
-  for (uint64_t k = 0; k < nfull; ++k) {
-    memcpy(fractions + k * keep, full + k * seg_p, keep);
-    for (int l = 0; l < NZO_LANES; ++l)
-      seeds[k * NZO_LANES + l] = (uint16_t)get16(full + k * seg_p + keep + 2 * l);
-  }
-  memcpy(fractions + nfull * keep, full + nfull * seg_p, nzo_packed_bytes(n, s) - nfull * seg_p);
+  carry_layout(&g, s, full, fractions, seeds, 1);
   int64_t r = nzo_exp_encode(exps, n, chunk_syms, lane_syms, seeds, comp, cap, threads);
   free(exps);
   free(full);
@@ -865,12 +904,11 @@ int nzo_decompress_bf16(const uint8_t* comp, size_t comp_bytes, const uint8_t* f
                         uint64_t n, int s, uint16_t* data, int threads) {
   if (!(s == 7 || s == 3 || s == 1 || s == 0)) return NZO_ERR_ARG;
   if (comp_bytes < NZO_HEADER_BYTES) return NZO_ERR_CORRUPT;
-  uint32_t lane_syms = get32(comp + 20);
-  if (nzo_check_geometry(get32(comp + 16), lane_syms)) return NZO_ERR_CORRUPT;
-  uint64_t seg = (uint64_t)lane_syms * NZO_LANES, nfull = n / seg;
+  geom_t g;
+  if (make_geom(&g, n, get32(comp + 16), get32(comp + 20))) return NZO_ERR_CORRUPT;
   uint8_t* exps = (uint8_t*)malloc((size_t)n + 1);
   uint8_t* full = (uint8_t*)malloc(nzo_packed_bytes(n, s) + 1);
-  uint16_t* seeds = (uint16_t*)malloc((size_t)(nfull + 1) * NZO_LANES * 2);
+  uint16_t* seeds = (uint16_t*)calloc((size_t)(g.n_segs + 1) * NZO_LANES, 2);
   if (!exps || !full || !seeds) {
     free(exps);
     free(full);
@@ -879,12 +917,7 @@ int nzo_decompress_bf16(const uint8_t* comp, size_t comp_bytes, const uint8_t* f
   }
   int r = nzo_exp_decode(comp, comp_bytes, n, exps, seeds, threads);
   if (r == NZO_OK) {
-    size_t seg_p = (size_t)(seg * (uint64_t)(s + 1) / 8), keep = seg_p - 2 * NZO_LANES;
-    for (uint64_t k = 0; k < nfull; ++k) {
-      memcpy(full + k * seg_p, fractions + k * keep, keep);
-      for (int l = 0; l < NZO_LANES; ++l) put16(full + k * seg_p + keep + 2 * l, seeds[k * NZO_LANES + l]);
-    }
-    memcpy(full + nfull * seg_p, fractions + nfull * keep, nzo_packed_bytes(n, s) - nfull * seg_p);
+    carry_layout(&g, s, full, (uint8_t*)fractions, seeds, 0);
     run_sm(merge_worker, NULL, data, exps, full, n, s, threads);
   }
   free(exps);

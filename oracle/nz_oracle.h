@@ -39,7 +39,7 @@ extern "C" {
 
 /* ---- format constants (shared with the HIP implementation by value) ---- */
 #define NZO_MAGIC 0x315A4E41u /* "ANZ1" little endian */
-#define NZO_VERSION 3u
+#define NZO_VERSION 4u
 #define NZO_PROB_BITS 12
 #define NZO_M (1u << NZO_PROB_BITS)
 #define NZO_L (1u << 16)
@@ -54,7 +54,7 @@ extern "C" {
 
 /* ---- split / merge ---- */
 size_t nzo_packed_bytes(uint64_t n, int s);
-size_t nzo_packed_stored_bytes(uint64_t n, int s, uint32_t lane_syms);
+size_t nzo_packed_stored_bytes(uint64_t n, int s, uint32_t chunk_syms, uint32_t lane_syms);
 void nzo_split_bf16(const uint16_t* data, uint64_t n, int s, uint8_t* exponents, uint8_t* fractions);
 void nzo_merge_bf16(const uint8_t* exponents, const uint8_t* fractions, uint64_t n, int s, uint16_t* data);
 /* literal float path of kernels.cuh:208-216 (NaN canonicalised to 0x7FC0, host c10 rule) */
@@ -70,8 +70,9 @@ int nzo_table_parse(const uint8_t* in, size_t avail, uint16_t freq[256], size_t*
 /* ---- exponent container ---- */
 int nzo_check_geometry(uint32_t chunk_syms, uint32_t lane_syms);
 size_t nzo_exp_bound(uint64_t n, uint32_t chunk_syms, uint32_t lane_syms);
-/* seeds: 64 x u16 per FULL segment (segment k at seeds + 64*k), the payload
-   carried in the rANS start states; NULL = all zero / ignored. */
+/* seeds: 64 x u16 per segment (segment c*spc + k at seeds + 64*(c*spc + k); only
+   full segments use theirs), the payload carried in the rANS start states;
+   NULL = all zero / ignored. */
 int64_t nzo_exp_encode(const uint8_t* syms, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
                        const uint16_t* seeds, uint8_t* out, size_t cap, int threads);
 int nzo_exp_decode(const uint8_t* comp, size_t comp_bytes, uint64_t n, uint8_t* syms_out,

@@ -64,7 +64,7 @@ def lib() -> ctypes.CDLL:
         L.nzo_exp_decode.restype = ctypes.c_int
         L.nzo_exp_decode.argtypes = [u8p, ctypes.c_size_t, ctypes.c_uint64, u8p, u16p, ctypes.c_int]
         L.nzo_packed_stored_bytes.restype = ctypes.c_size_t
-        L.nzo_packed_stored_bytes.argtypes = [ctypes.c_uint64, ctypes.c_int, ctypes.c_uint32]
+        L.nzo_packed_stored_bytes.argtypes = [ctypes.c_uint64, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32]
         L.nzo_compress_bf16.restype = ctypes.c_int64
         L.nzo_compress_bf16.argtypes = [u16p, ctypes.c_uint64, ctypes.c_int, ctypes.c_uint32,
                                         ctypes.c_uint32, u8p, u8p, ctypes.c_size_t, ctypes.c_int]
@@ -155,8 +155,15 @@ def exp_bound(n: int, chunk_syms: int, lane_syms: int) -> int:
     return int(lib().nzo_exp_bound(n, chunk_syms, lane_syms))
 
 
-def packed_stored_bytes(n: int, s: int, lane_syms: int) -> int:
-    return int(lib().nzo_packed_stored_bytes(n, s, lane_syms))
+def packed_stored_bytes(n: int, s: int, lane_syms: int, chunk_syms: int = 65536) -> int:
+    return int(lib().nzo_packed_stored_bytes(n, s, chunk_syms, lane_syms))
+
+
+def segment_count(n: int, chunk_syms: int, lane_syms: int) -> int:
+    """Segments of the container: chunk c owns indices c*spc .. c*spc + spc - 1."""
+    seg = 64 * lane_syms
+    spc = -(-chunk_syms // seg)
+    return (n // chunk_syms) * spc + -(-(n % chunk_syms) // seg)
 
 
 def exp_encode(syms: np.ndarray, chunk_syms: int = 65536, lane_syms: int = 512, threads: int = 1,
@@ -171,7 +178,7 @@ def exp_encode(syms: np.ndarray, chunk_syms: int = 65536, lane_syms: int = 512, 
     sp = None
     if seeds is not None:
         seeds = np.ascontiguousarray(seeds, dtype=np.uint16).reshape(-1)
-        assert seeds.size >= 64 * (syms.size // (64 * lane_syms))
+        assert seeds.size >= 64 * segment_count(syms.size, chunk_syms, lane_syms)
         sp = _p(seeds, ctypes.c_uint16)
     r = lib().nzo_exp_encode(_p(syms, ctypes.c_uint8), syms.size, chunk_syms, lane_syms, sp,
                              _p(out, ctypes.c_uint8), cap, threads)
@@ -180,17 +187,20 @@ def exp_encode(syms: np.ndarray, chunk_syms: int = 65536, lane_syms: int = 512, 
     return out[:r].copy()
 
 
-def exp_decode(comp: np.ndarray, n: int, threads: int = 1, lane_syms: int | None = None):
-    """Returns (rc, symbols) or, with lane_syms given, (rc, symbols, seeds)."""
+def exp_decode(comp: np.ndarray, n: int, threads: int = 1, lane_syms: int | None = None,
+               chunk_syms: int = 65536):
+    """Returns (rc, symbols) or, with lane_syms given, (rc, symbols, seeds) where
+    seeds holds 64 values per segment (meaningful for full segments only)."""
     comp = _u8(comp)
     out = np.zeros(n, np.uint8)
     if lane_syms is None:
         rc = lib().nzo_exp_decode(_p(comp, ctypes.c_uint8), comp.size, n, _p(out, ctypes.c_uint8), None, threads)
         return int(rc), out
-    seeds = np.zeros(64 * (n // (64 * lane_syms)) + 64, np.uint16)
+    nseg = segment_count(n, chunk_syms, lane_syms)
+    seeds = np.zeros(64 * nseg + 64, np.uint16)
     rc = lib().nzo_exp_decode(_p(comp, ctypes.c_uint8), comp.size, n, _p(out, ctypes.c_uint8),
                               _p(seeds, ctypes.c_uint16), threads)
-    return int(rc), out, seeds[: 64 * (n // (64 * lane_syms))]
+    return int(rc), out, seeds[: 64 * nseg]
 
 
 def compress_bf16(bits: np.ndarray, s: int, chunk_syms: int = 65536, lane_syms: int = 512, threads: int = 1):
@@ -200,7 +210,7 @@ def compress_bf16(bits: np.ndarray, s: int, chunk_syms: int = 65536, lane_syms: 
     if cap == 0:
         raise ValueError("unsupported geometry")
     comp = np.zeros(cap, np.uint8)
-    frac = np.zeros(packed_stored_bytes(n, s, lane_syms), np.uint8)
+    frac = np.zeros(packed_stored_bytes(n, s, lane_syms, chunk_syms), np.uint8)
     r = lib().nzo_compress_bf16(_p(bits, ctypes.c_uint16), n, s, chunk_syms, lane_syms,
                                 _p(frac, ctypes.c_uint8), _p(comp, ctypes.c_uint8), cap, threads)
     if r < 0:

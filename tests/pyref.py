@@ -50,27 +50,30 @@ def decode_container(comp: bytes, n: int):
     """-> (symbols uint8[n], carried uint16[64 * full_segments])."""
     comp = bytes(comp)
     magic, version = _u32(comp, 0), _u32(comp, 4)
-    assert magic == 0x315A4E41 and version == 3
+    assert magic == 0x315A4E41 and version == 4
     assert _u32(comp, 8) | (_u32(comp, 12) << 32) == n
     chunk, lane = _u32(comp, 16), _u32(comp, 20)
     seg = 64 * lane
-    spc = chunk // seg
-    n_segs = (n + seg - 1) // seg
+    spc = -(-chunk // seg)  # the last segment of a chunk holds what remains
+    n_segs = (n // chunk) * spc + -(-(n % chunk) // seg)
     assert _u32(comp, 28) == n_segs
     dir_off, rec_off = _u32(comp, 32), _u32(comp, 36)
     out = np.zeros(n, np.uint8)
-    carried = np.zeros(64 * (n // seg), np.uint16)
+    carried = np.zeros(64 * n_segs, np.uint16)
     table = None
     for k in range(n_segs):
         o0, o1 = _u32(comp, dir_off + 4 * k), _u32(comp, dir_off + 4 * (k + 1))
         rec = comp[rec_off + 4 * o0: rec_off + 4 * o1]
-        sn = min(seg, n - k * seg)
+        cpos, kk = divmod(k, spc)
+        start = cpos * chunk + kk * seg
+        nominal = seg if kk + 1 < spc else chunk - (spc - 1) * seg
+        sn = min(nominal, n - start)
         if k % spc == 0:
             table, used = parse_table(rec)
             rec = rec[used:]
         if table == "raw":
-            out[k * seg: k * seg + sn] = np.frombuffer(rec[:sn], np.uint8)
-            if sn == seg:
+            out[start: start + sn] = np.frombuffer(rec[:sn], np.uint8)
+            if sn == nominal:
                 pad = (sn + 3) & ~3
                 carried[64 * k: 64 * k + 64] = np.frombuffer(rec[pad:pad + 128], "<u2")
             continue
@@ -99,14 +102,14 @@ def decode_container(comp: bytes, n: int):
                     x[lane_i] = freq[s] * (x[lane_i] >> 12) + slot - int(cum[s])
                     idx = (g * 64 + lane_i) * 8 + j
                     if idx < sn:
-                        out[k * seg + idx] = s
+                        out[start + idx] = s
                     if x[lane_i] < L:
                         x[lane_i] = (x[lane_i] << 16) | int(words[pos])
                         pos += 1
         assert pos <= len(words) and len(words) - pos <= 1
         for lane_i in range(64):
             assert x[lane_i] >> 16 == 1
-            if sn == seg:
+            if sn == nominal:
                 carried[64 * k + lane_i] = x[lane_i] & 0xFFFF
             else:
                 assert x[lane_i] == L

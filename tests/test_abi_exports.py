@@ -24,7 +24,7 @@ def test_header_symbols_are_exported():
     for name in names:
         assert hasattr(L, name), f"{name} declared in include/neuzip_hip.h but not exported"
     assert sorted(_lib.EXPORTS) == names  # the ctypes binding covers the whole header
-    assert L.nz_abi_version() == 3
+    assert L.nz_abi_version() == 4
 
 
 def test_size_helpers_match_oracle(oracle):
@@ -34,9 +34,9 @@ def test_size_helpers_match_oracle(oracle):
     for n in (0, 1, 7, 8, 9, 32767, 32768, 65536, 1_000_003):
         for s in (7, 3, 1, 0):
             assert L.nz_packed_bytes(n, s) == oracle.packed_bytes(n, s) == (n * (s + 1) + 7) // 8
-            for lane in (16, 128, 512, 1024):
-                assert L.nz_packed_stored_bytes(n, s, lane) == oracle.packed_stored_bytes(n, s, lane)
-        for lane, chunk in ((512, 65536), (128, 65536), (1024, 65536), (16, 1024), (2048, 1 << 20)):
+            for lane in (16, 128, 344, 512, 1024):
+                assert L.nz_packed_stored_bytes(n, s, 65536, lane) == oracle.packed_stored_bytes(n, s, lane, 65536)
+        for lane, chunk in ((512, 65536), (344, 65536), (128, 65536), (1024, 65536), (16, 1024), (2048, 1 << 20)):
             assert L.nz_exp_bound_bytes(n, chunk, lane) == oracle.exp_bound(n, chunk, lane)
             assert L.nz_encode_workspace_bytes(n, chunk, lane) > n
     assert L.nz_exp_bound_bytes(1000, 65536, 100) == 0  # unsupported geometry

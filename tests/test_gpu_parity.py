@@ -29,7 +29,7 @@ def gpu_encode(bits, s, chunk=65536, lane=512):
     assert cap > 0
     ws_bytes = L.nz_encode_workspace_bytes(n, chunk, lane)
     comp = torch.zeros(cap, dtype=torch.uint8, device="cuda")
-    packed = torch.zeros(max(8, L.nz_packed_stored_bytes(n, s, lane)), dtype=torch.uint8, device="cuda")
+    packed = torch.zeros(max(8, L.nz_packed_stored_bytes(n, s, chunk, lane)), dtype=torch.uint8, device="cuda")
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
     aux = torch.zeros(4, dtype=torch.int64, device="cuda")
     total = ctypes.c_uint64(0)
@@ -38,7 +38,7 @@ def gpu_encode(bits, s, chunk=65536, lane=512):
                      ws.data_ptr(), ws_bytes, aux.data_ptr(), aux.data_ptr() + 8, ctypes.byref(total), st)
     assert rc == 0, m.last_error()
     torch.cuda.synchronize()
-    return comp[: total.value].clone(), packed[: L.nz_packed_stored_bytes(n, s, lane)].clone()
+    return comp[: total.value].clone(), packed[: L.nz_packed_stored_bytes(n, s, chunk, lane)].clone()
 
 
 def gpu_decode(comp, packed, n, s, chunk=65536, lane=512, check=True):
@@ -73,8 +73,9 @@ def test_roundtrip_matches_oracle(oracle, n, s):
     assert np.array_equal(out, closed_form_recon(bits, s))
 
 
-@pytest.mark.parametrize("lane,chunk", [(128, 65536), (256, 65536), (512, 65536), (1024, 65536),
-                                        (16, 1024), (64, 4096), (2048, 1 << 20)])
+@pytest.mark.parametrize("lane,chunk", [(128, 65536), (256, 65536), (344, 65536), (352, 65536), (512, 65536),
+                                        (1024, 65536), (1000, 65536), (16, 1024), (24, 2560), (64, 4096),
+                                        (2048, 1 << 20)])
 def test_geometries(oracle, lane, chunk):
     n = 3 * chunk + 1234 if chunk <= 65536 else chunk + 777
     bits = bf16_bits_normal(n, seed=lane)

@@ -8,12 +8,13 @@ from hypothesis import given, settings, strategies as st
 import pyref
 from conftest import bf16_bits_normal, chunk_entropy_bytes, closed_form_recon, stress_bits
 
-GEOMS = ((16, 1024), (16, 8192), (64, 4096), (128, 65536), (512, 65536), (1024, 65536), (2048, 1 << 20))
+GEOMS = ((16, 1024), (16, 8192), (24, 2560), (64, 4096), (128, 65536), (344, 65536), (512, 65536),
+         (1024, 65536), (2048, 1 << 20))
 
 
 def roundtrip(oracle, syms, lane, chunk, seeds=None):
     comp = oracle.exp_encode(syms, chunk, lane, seeds=seeds)
-    rc, out, sd = oracle.exp_decode(comp, syms.size, lane_syms=lane)
+    rc, out, sd = oracle.exp_decode(comp, syms.size, lane_syms=lane, chunk_syms=chunk)
     assert rc == 0
     assert np.array_equal(out, syms)
     return comp, sd
@@ -32,9 +33,16 @@ def test_chunk_and_segment_boundaries(oracle, lane, chunk):
     seg = 64 * lane
     for n in (seg - 1, seg, seg + 1, chunk - 1, chunk, chunk + 1, 2 * chunk + seg + 5):
         syms = np.clip(rng.normal(118, 2.5, n), 0, 255).astype(np.uint8)
-        seeds = rng.integers(0, 65536, 64 * (n // seg)).astype(np.uint16)
+        nseg = oracle.segment_count(n, chunk, lane)
+        seeds = rng.integers(0, 65536, 64 * nseg).astype(np.uint16)
         comp, sd = roundtrip(oracle, syms, lane, chunk, seeds)
-        assert np.array_equal(sd, seeds)  # the carried bits come back from the final states
+        # the carried bits of every full segment come back from the final states
+        spc = -(-chunk // seg)
+        for k in range(nseg):
+            cpos, kk = divmod(k, spc)
+            nom = seg if kk + 1 < spc else chunk - (spc - 1) * seg
+            if cpos * chunk + kk * seg + nom <= n:
+                assert np.array_equal(sd[64 * k: 64 * k + 64], seeds[64 * k: 64 * k + 64])
         assert comp.size <= oracle.exp_bound(n, chunk, lane)
 
 
@@ -67,11 +75,12 @@ def test_python_decoder_agrees(alphabet, n, seed):
 
     rng = np.random.default_rng(seed)
     syms = rng.choice(np.array(alphabet, np.uint8), size=n)
-    seeds = rng.integers(0, 65536, 64 * (n // 1024)).astype(np.uint16)
+    seeds = rng.integers(0, 65536, 64 * O.segment_count(n, 2048, 16)).astype(np.uint16)
     comp = O.exp_encode(syms, 2048, 16, seeds=seeds)
     out, carried = pyref.decode_container(comp.tobytes(), n)
     assert np.array_equal(out, syms)
-    assert np.array_equal(carried, seeds)
+    full = 64 * (n // 1024)  # every 1024-symbol segment the stream does not end inside
+    assert np.array_equal(carried[:full], seeds[:full])
 
 
 def test_size_against_shannon_bound(oracle):
@@ -145,10 +154,12 @@ def test_corruption_is_detected(oracle):
 def test_geometry_validation(oracle):
     assert oracle.check_geometry(65536, 512) == 0
     assert oracle.check_geometry(65536, 1024) == 0
+    assert oracle.check_geometry(65536, 344) == 0  # 2 x 22016 + 21504: a ragged last segment
     assert oracle.check_geometry(65536, 64) != 0  # more than 8 segments per chunk
     assert oracle.check_geometry(65536, 8) != 0  # below the 16-symbol minimum
     assert oracle.check_geometry(65536, 100) != 0  # not a multiple of 8
-    assert oracle.check_geometry(60000, 512) != 0  # chunk not a multiple of the segment
+    assert oracle.check_geometry(60000, 512) != 0  # chunk not a multiple of 512
+    assert oracle.check_geometry(65536, 1016) != 0  # would leave a 512-symbol last segment
     assert oracle.exp_bound(1000, 65536, 100) == 0
 
 
@@ -158,6 +169,6 @@ def test_whole_tensor_with_carry(oracle, s):
     for n in (32768, 32768 * 3 + 17, 65536 * 2):
         bits = stress_bits(1, n, seed=n + s)
         comp, packed = oracle.compress_bf16(bits, s, 65536, 512)
-        assert packed.size == oracle.packed_bytes(n, s) - 128 * (n // 32768)
+        assert packed.size == oracle.packed_bytes(n, s) - 128 * (n // 32768) == oracle.packed_stored_bytes(n, s, 512)
         rc, out = oracle.decompress_bf16(comp, packed, n, s)
         assert rc == 0 and np.array_equal(out, closed_form_recon(bits, s))
