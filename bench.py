@@ -279,7 +279,7 @@ def run_gpt2m(args, torch):
             "decodes_per_step": n_dec / args.steps,
             "encodes_per_step": n_enc / args.steps,
             "compressed_tensors": len(comp_params),
-            "lane_symbols": "auto" if args.lane_symbols < 0 else (args.lane_symbols or 512),
+            "lane_symbols": "auto" if args.lane_symbols < 0 else (args.lane_symbols or 344),
             "stored_over_dense": round(sum(mgr.size(p._handle) for p in comp_params) /
                                        sum(2 * int(np.prod(p._shape)) for p in comp_params), 5),
             "first_loss": round(float(losses[0]), 4),

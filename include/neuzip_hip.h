@@ -45,7 +45,7 @@ extern "C" {
 #define NZ_ALGO_ANS 0
 
 #define NZ_DEFAULT_CHUNK 65536u   /* cuda/neuzip.cu:31 */
-#define NZ_DEFAULT_LANE_SYMS 512u /* two wavefronts per 64 KiB chunk */
+#define NZ_DEFAULT_LANE_SYMS 344u /* three wavefronts per 64 KiB chunk: 22016 + 22016 + 21504 */
 #define NZ_LANE_SYMS_AUTO 0xFFFFFFFFu /* nz_manager_create: choose per tensor */
 
 typedef struct nz_manager nz_manager;

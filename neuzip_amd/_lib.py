@@ -19,7 +19,7 @@ ERR_ARG, ERR_DTYPE, ERR_NOT_FOUND, ERR_HIP, ERR_CAPACITY, ERR_CORRUPT, ERR_ALIGN
 DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 ALGO_ANS = 0
 DEFAULT_CHUNK = 65536
-DEFAULT_LANE_SYMS = 512
+DEFAULT_LANE_SYMS = 344
 LANE_SYMS_AUTO = 0xFFFFFFFF
 
 EXPORTS = [

@@ -743,10 +743,15 @@ struct NzWaveDec {
       uint32_t w = *(lds_cu16*)(uintptr_t)at;
       // keep the word read unconditional: straight-line code, no exec-mask branch
       asm volatile("" : "+v"(w));
-      // renormalise: x = x << 16 | w, as one byte permute whose selector was
-      // chosen while the word was in flight
-      const uint32_t sel = need ? 0x05040100u : 0x07060504u;
-      x = __builtin_amdgcn_perm(x, w, sel);
+      // renormalise: x = x << 16 | w in the lanes that need it.  One byte permute
+      // under the ballot as exec mask (every lane of the wave is active here, so
+      // exec is all ones before and after); cheaper than select + permute.
+      asm volatile(
+          "s_mov_b64 exec, %[m]\n\t"
+          "v_perm_b32 %[x], %[x], %[w], %[sel]\n\t"
+          "s_mov_b64 exec, -1"
+          : [x] "+v"(x)
+          : [w] "v"(w), [m] "s"(m), [sel] "s"(0x05040100u));
       base += (uint32_t)__popcll(m);
     }
   }
