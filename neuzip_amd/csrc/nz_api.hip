@@ -325,7 +325,7 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   // Throughput of both codec directions is set by the number of wavefronts in
   // flight (one per 64 * lane_syms elements).  In auto mode a tensor too small
   // to give every SIMD two wavefronts at the default gets shorter segments,
-  // down to the 8 segments a chunk may hold, at ~8.5 bits per extra lane.
+  // down to the 8 segments a chunk may hold, at ~4.5 bits per extra lane.
   uint32_t lane_syms = m->lane_syms;
   if (m->auto_lanes) {
     while (lane_syms > 16 && nz_geom_check(m->chunk_syms, (lane_syms / 2 + 7) & ~7u) == 0 &&
