@@ -1,0 +1,112 @@
+"""The benchmark configurations at their full sizes on the GPU, through the C ABI.
+
+The oracle needs seconds for these sizes, so each case is checked three ways:
+bit-exact reconstruction against the closed form evaluated with torch integer
+ops on the device, container and packed stream byte-identical to the oracle's
+for the same input, and the stored size against the order-0 entropy bound."""
+import numpy as np
+import pytest
+
+from test_gpu_parity import gpu_decode, gpu_encode
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def _closed_form_dev(bits_i16, s):
+    a = bits_i16.to(torch.int32) & 0xFFFF
+    if s == 7:
+        return a
+    mag = a & 0x7FFF
+    rec = ((mag + (1 << (6 - s))) & 0x7FFF) & (0x7FFF ^ ((1 << (7 - s)) - 1))
+    return (a & 0x8000) | rec
+
+
+def _entropy_bound_bytes_dev(exps_i32, chunk=65536):
+    n = exps_i32.numel()
+    nch = (n + chunk - 1) // chunk
+    idx = torch.arange(n, device=exps_i32.device, dtype=torch.int64) // chunk
+    cnt = torch.bincount(idx * 256 + exps_i32.to(torch.int64), minlength=256 * nch).view(nch, 256).double()
+    tot = cnt.sum(1, keepdim=True)
+    p = cnt / tot
+    h = -(torch.where(cnt > 0, cnt * torch.log2(p.clamp_min(1e-300)), torch.zeros_like(cnt))).sum()
+    return float(h) / 8.0
+
+
+def _normal_weight(rows, cols, seed):
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    return (torch.randn(rows, cols, device="cuda", generator=g) * 0.02).to(torch.bfloat16).view(-1)
+
+
+def _stress_weight(rows, cols, seed):
+    """Student-t(3) * 0.02, 16 outlier columns at 50x, 1 % exact zeros, 0.1 %
+    subnormals with random sign and mantissa."""
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    z = torch.randn(rows, cols, device="cuda", generator=g)
+    chi = torch.zeros(rows, cols, device="cuda")
+    for _ in range(3):
+        chi += torch.randn(rows, cols, device="cuda", generator=g) ** 2
+    x = z / torch.sqrt(chi / 3.0) * 0.02
+    del z, chi
+    cols_out = torch.randperm(cols, device="cuda", generator=g)[:16]
+    x[:, cols_out] *= 50.0
+    bits = x.to(torch.bfloat16).view(torch.int16).view(-1).clone()
+    del x
+    n = bits.numel()
+    u = torch.rand(n, device="cuda", generator=g)
+    bits[u < 0.01] = 0
+    sub = (u >= 0.01) & (u < 0.011)
+    k = int(sub.sum())
+    mant = torch.randint(1, 128, (k,), device="cuda", generator=g, dtype=torch.int32)
+    sign = torch.randint(0, 2, (k,), device="cuda", generator=g, dtype=torch.int32) << 15
+    bits[sub] = (sign | mant).to(torch.int16)  # values >= 0x8000 wrap into the int16 view
+    return bits.view(torch.bfloat16)
+
+
+def _check(dense, s, oracle, max_over_bound, compare_oracle=True):
+    n = dense.numel()
+    bits_dev = dense.view(torch.int16)
+    host_bits = bits_dev.cpu().numpy().view(np.uint16)
+    print(f"case n={n} s={s}", flush=True)
+    comp, packed = gpu_encode(host_bits, s)
+    rc, out = gpu_decode(comp, packed, n, s)
+    assert rc == 0
+    want = _closed_form_dev(bits_dev, s)
+    got = torch.from_numpy(out.view(np.int16)).cuda().to(torch.int32) & 0xFFFF
+    assert torch.equal(got, want)
+    if compare_oracle:
+        o_comp, o_packed = oracle.compress_bf16(host_bits, s, 65536, 344, threads=8)
+        assert np.array_equal(comp.cpu().numpy(), o_comp)
+        assert np.array_equal(packed.cpu().numpy(), o_packed)
+    bound = _entropy_bound_bytes_dev((want >> 7) & 0xFF)
+    packed_ref = (n * (s + 1) + 7) // 8
+    effective = comp.numel() + packed.numel() - packed_ref
+    assert effective <= max_over_bound * bound, (effective, bound)
+    return (comp.numel() + packed.numel()) / (2.0 * n)
+
+
+@pytest.mark.parametrize("s,ratio", [(7, 0.659), (3, 0.409), (1, 0.284), (0, 0.221)])
+def test_truncation_sweep_16384x4096(oracle, s, ratio):
+    dense = _normal_weight(16384, 4096, 0)
+    stored = _check(dense, s, oracle, 1.01)
+    assert abs(stored - ratio) < 0.004, stored
+
+
+@pytest.mark.parametrize("s", [7, 3])
+def test_stress_layer_8192x28672(oracle, s):
+    dense = _stress_weight(8192, 28672, 11)
+    bits = dense.view(torch.int16).to(torch.int32) & 0xFFFF
+    # the generator produced what the case is about
+    assert int((bits == 0).sum()) > 0.009 * bits.numel()
+    assert int((((bits >> 7) & 0xFF) == 0).sum() - ((bits & 0x7FFF) == 0).sum()) > 0.0005 * bits.numel()
+    del bits
+    _check(dense, s, oracle, 1.01)
+
+
+def test_plumbing_case_4096x4096_gpu_equals_cpu(oracle):
+    """The CPU-runnable case (one 4096 x 4096 weight, lossless) gives the same
+    bytes on both sides and the expected stored size."""
+    dense = _normal_weight(4096, 4096, 0)
+    stored = _check(dense, 7, oracle, 1.01)
+    assert abs(stored - 0.659) < 0.004

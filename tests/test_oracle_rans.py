@@ -172,3 +172,17 @@ def test_whole_tensor_with_carry(oracle, s):
         assert packed.size == oracle.packed_bytes(n, s) - 128 * (n // 32768) == oracle.packed_stored_bytes(n, s, 512)
         rc, out = oracle.decompress_bf16(comp, packed, n, s)
         assert rc == 0 and np.array_equal(out, closed_form_recon(bits, s))
+
+
+def test_plumbing_case_4096x4096(oracle):
+    """One 4096 x 4096 weight from N(0, 0.02), lossless: split, entropy-code,
+    exact round trip, stored size about (8 + 2.546) / 16 of dense."""
+    n = 4096 * 4096
+    bits = bf16_bits_normal(n, 0)
+    comp, packed = oracle.compress_bf16(bits, 7, 65536, 344, threads=4)
+    rc, out = oracle.decompress_bf16(comp, packed, n, 7, threads=4)
+    assert rc == 0 and np.array_equal(out, bits)
+    assert abs((comp.size + packed.size) / (2.0 * n) - 0.659) < 0.004
+    exps = ((bits >> 7) & 0xFF).astype(np.uint8)
+    effective = comp.size + packed.size - n
+    assert effective <= 1.01 * chunk_entropy_bytes(exps)
