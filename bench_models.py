@@ -78,6 +78,27 @@ class LlamaBlock(torch.nn.Module):
         return x + self.down_proj(F.silu(self.gate_proj(h)) * self.up_proj(h))
 
 
+def _block_static(blk, x, posv, kc, vc, mask):
+    """One decode step of a LlamaBlock against a preallocated cache: the new key
+    and value go to row `posv` of kc / vc ([1, n_kv, Tmax, hd]); `mask` hides the
+    rows not written yet.  Shapes never change, so the step can be captured."""
+    B, T, _ = x.shape
+    h = blk.input_norm(x)
+    q = blk.q_proj(h).view(B, T, blk.n_q, blk.hd).transpose(1, 2)
+    k = blk.k_proj(h).view(B, T, blk.n_kv, blk.hd).transpose(1, 2)
+    v = blk.v_proj(h).view(B, T, blk.n_kv, blk.hd).transpose(1, 2)
+    q, k = _rope(q, posv), _rope(k, posv)
+    kc.index_copy_(2, posv, k)
+    vc.index_copy_(2, posv, v)
+    rep = blk.n_q // blk.n_kv
+    kk = kc.repeat_interleave(rep, dim=1)
+    vv = vc.repeat_interleave(rep, dim=1)
+    a = F.scaled_dot_product_attention(q, kk, vv, attn_mask=mask)
+    x = x + blk.o_proj(a.transpose(1, 2).reshape(B, T, -1))
+    h = blk.post_norm(x)
+    return x + blk.down_proj(F.silu(blk.gate_proj(h)) * blk.up_proj(h))
+
+
 class LlamaShaped(torch.nn.Module):
     """32 layers, d=4096, 32 q / 8 kv heads, FFN 14336, vocab 128256 by default."""
 
@@ -96,6 +117,34 @@ class LlamaShaped(torch.nn.Module):
         for blk, c in zip(self.layers, caches):
             x = blk(x, pos, c)
         return self.lm_head(self.norm(x[:, -1:]))
+
+    @torch.no_grad()
+    def static_caches(self, t_max):
+        dev = self.embed.weight.device
+        blk = self.layers[0]
+        mk = lambda: torch.zeros(1, blk.n_kv, t_max, blk.hd, dtype=self.embed.weight.dtype, device=dev)
+        return [mk() for _ in self.layers], [mk() for _ in self.layers]
+
+    @torch.no_grad()
+    def prefill_static(self, prompt, kcs, vcs):
+        """Eager prefill; leaves keys and values in the static caches; returns the logits of the last position."""
+        caches = [[None, None] for _ in self.layers]
+        logits = self.forward(prompt, 0, caches)
+        T = prompt.shape[1]
+        for (k, v), kc, vc in zip(caches, kcs, vcs):
+            kc[:, :, :T].copy_(k)
+            vc[:, :, :T].copy_(v)
+        return logits
+
+    @torch.no_grad()
+    def step_static(self, tok, pos, kcs, vcs):
+        """One token: `tok` [1, 1] int64, `pos` a 1-element int64 device tensor."""
+        t_max = kcs[0].shape[2]
+        mask = (torch.arange(t_max, device=tok.device) <= pos).view(1, 1, 1, t_max)
+        x = self.embed(tok)
+        for blk, kc, vc in zip(self.layers, kcs, vcs):
+            x = _block_static(blk, x, pos, kc, vc, mask)
+        return self.lm_head(self.norm(x))
 
     @torch.no_grad()
     def generate(self, prompt, steps):

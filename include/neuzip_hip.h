@@ -126,6 +126,15 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
 int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap_elems,
                     void* stream);
 
+/* Several Manager::read calls (cuda/high_level.cu:223-250) served by ONE kernel
+   launch: entry names[i] is decompressed into dev_outs[i] (capacity
+   cap_elems[i] elements).  The reference decompresses tensor by tensor; a
+   transformer block's weights are each too small to fill the GPU, together they
+   do.  Nothing is decoded when an argument is rejected.  Asynchronous on
+   `stream`; allocates nothing. */
+int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* dev_outs,
+                          const uint64_t* cap_elems, uint32_t count, void* stream);
+
 /* meta_cache lookup, cuda/high_level.cu:42-43,228-230. */
 int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype);
 

@@ -47,6 +47,7 @@ class _HipBackend:
                                        lane_symbols, ctypes.byref(self._h))
         _lib.raise_for(rc)
         self._device = torch.device("cuda", torch.cuda.current_device())
+        self._known = {}  # handle -> (encoded name, element count), dropped on write
 
     def close(self):
         if getattr(self, "_h", None) is not None and self._h:
@@ -73,17 +74,22 @@ class _HipBackend:
         flat = tensor.detach().contiguous().view(-1)
         if flat.data_ptr() % 16:
             flat = flat.clone()
+        self._known.pop(handle, None)
         rc = self._L.nz_manager_write(self._h, handle.encode(), flat.data_ptr(), flat.numel(), code,
                                       _stream_ptr(flat.device))
         _lib.raise_for(rc)
 
     def read(self, handle: str) -> torch.Tensor:
-        n = ctypes.c_uint64()
-        dt = ctypes.c_int()
-        _lib.raise_for(self._L.nz_manager_meta(self._h, handle.encode(), ctypes.byref(n), ctypes.byref(dt)))
-        out = torch.empty(n.value, dtype=torch.bfloat16, device=self._device)
-        rc = self._L.nz_manager_read(self._h, handle.encode(), out.data_ptr(), n.value,
-                                     _stream_ptr(self._device))
+        known = self._known.get(handle)
+        if known is None:
+            n = ctypes.c_uint64()
+            dt = ctypes.c_int()
+            name = handle.encode()
+            _lib.raise_for(self._L.nz_manager_meta(self._h, name, ctypes.byref(n), ctypes.byref(dt)))
+            known = self._known[handle] = (name, int(n.value))
+        name, numel = known
+        out = torch.empty(numel, dtype=torch.bfloat16, device=self._device)
+        rc = self._L.nz_manager_read(self._h, name, out.data_ptr(), numel, _stream_ptr(self._device))
         _lib.raise_for(rc)
         return out
 
@@ -100,6 +106,27 @@ class _HipBackend:
                                      _stream_ptr(out.device))
         _lib.raise_for(rc)
         return out
+
+    def batch_plan(self, handles):
+        """Argument block for :meth:`read_batch` over a fixed list of handles
+        (built once, reused for every call)."""
+        k = len(handles)
+        names = (ctypes.c_char_p * k)(*[h.encode() for h in handles])
+        caps = (ctypes.c_uint64 * k)(*[self.numel(h) for h in handles])
+        return names, caps, k
+
+    def read_batch(self, plan, outs) -> None:
+        """Decompress the planned handles into the bf16 tensors ``outs`` with one
+        kernel launch on the current stream (no allocation, no host sync)."""
+        names, caps, k = plan
+        if len(outs) != k:
+            raise ValueError("one output tensor per planned handle")
+        for i, o in enumerate(outs):
+            if o.dtype != torch.bfloat16 or not o.is_contiguous() or o.numel() < caps[i]:
+                raise ValueError("read_batch needs contiguous bfloat16 outputs of the stored sizes")
+        ptrs = (ctypes.c_void_p * k)(*[o.data_ptr() for o in outs])
+        rc = self._L.nz_manager_read_batch(self._h, names, ptrs, caps, k, _stream_ptr(outs[0].device) if k else None)
+        _lib.raise_for(rc)
 
     def size(self, handle: str) -> int:
         return int(self._L.nz_manager_size(self._h, handle.encode()))

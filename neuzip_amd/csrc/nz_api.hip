@@ -5,6 +5,7 @@
 // No torch types, no private streams: every kernel goes to the caller's stream.
 #include <hip/hip_runtime.h>
 
+#include <cstring>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -132,6 +133,26 @@ int decode_launch(const NzGeom& g, int precision, const void* comp, uint64_t com
     case 3: launch_decode<3>(g, comp, comp_bytes, packed, out, d_status, st); break;
     case 1: launch_decode<1>(g, comp, comp_bytes, packed, out, d_status, st); break;
     default: launch_decode<0>(g, comp, comp_bytes, packed, out, d_status, st); break;
+  }
+  NZ_HIP(hipGetLastError());
+  return NZ_OK;
+}
+
+template <int S>
+void launch_decode_batch(const NzBatch& b, uint32_t grid, uint32_t max_spc, uint32_t* d_status,
+                         hipStream_t st) {
+  const size_t lds = (2 * NZ_M + max_spc * NZ_RING_ALLOC_DWORDS) * 4;
+  hipLaunchKernelGGL(nz_decode_batch_kernel<S>, dim3(grid), dim3(64 * max_spc), lds, st, b, d_status);
+}
+
+int decode_batch_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int precision,
+                        uint32_t* d_status, hipStream_t st) {
+  if (grid == 0) return NZ_OK;
+  switch (precision) {
+    case 7: launch_decode_batch<7>(b, grid, max_spc, d_status, st); break;
+    case 3: launch_decode_batch<3>(b, grid, max_spc, d_status, st); break;
+    case 1: launch_decode_batch<1>(b, grid, max_spc, d_status, st); break;
+    default: launch_decode_batch<0>(b, grid, max_spc, d_status, st); break;
   }
   NZ_HIP(hipGetLastError());
   return NZ_OK;
@@ -438,6 +459,51 @@ int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap
   if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
   return decode_launch(g, m->precision, ent.comp, ent.comp_bytes, ent.packed, dev_out, m->d_status,
                        (hipStream_t)stream);
+}
+
+int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* dev_outs,
+                          const uint64_t* cap_elems, uint32_t count, void* stream) {
+  if (!m || (count && (!names || !dev_outs || !cap_elems)))
+    return fail(NZ_ERR_ARG, "null manager, names, outputs or capacities");
+  std::lock_guard<std::mutex> lock(m->mu);
+  // validate everything before the first launch: a failed call decodes nothing
+  for (uint32_t i = 0; i < count; ++i) {
+    if (!names[i]) return fail(NZ_ERR_ARG, "null name");
+    auto it = m->entries.find(names[i]);
+    if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+    const Entry& ent = it->second;
+    if (cap_elems[i] < ent.n) return fail(NZ_ERR_CAPACITY, "output smaller than the stored tensor");
+    if (ent.n && !dev_outs[i]) return fail(NZ_ERR_ARG, "null output pointer");
+    if ((uintptr_t)dev_outs[i] & 15) return fail(NZ_ERR_ALIGN, "dense output must be 16-byte aligned");
+  }
+  NzBatch b;
+  std::memset(&b, 0, sizeof(b));
+  uint32_t grid = 0, max_spc = 1;
+  auto flush = [&]() -> int {
+    int rc = decode_batch_launch(b, grid, max_spc, m->precision, m->d_status, (hipStream_t)stream);
+    b.count = 0;
+    grid = 0;
+    max_spc = 1;
+    return rc;
+  };
+  for (uint32_t i = 0; i < count; ++i) {
+    const Entry& ent = m->entries.find(names[i])->second;
+    if (ent.n == 0) continue;
+    NzGeom g;
+    if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
+    if (b.count == NZ_BATCH_MAX || (uint64_t)grid + g.n_chunks > 0x7FFFFFFFull)
+      if (int rc = flush()) return rc;
+    NzBatchItem& it = b.item[b.count++];
+    it.comp = (const uint8_t*)ent.comp;
+    it.comp_bytes = ent.comp_bytes;
+    it.packed = (const uint8_t*)ent.packed;
+    it.out = (uint16_t*)dev_outs[i];
+    it.g = g;
+    grid += (uint32_t)g.n_chunks;
+    it.chunk_end = grid;
+    if (g.spc > max_spc) max_spc = g.spc;
+  }
+  return b.count ? flush() : NZ_OK;
 }
 
 int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype) {

@@ -757,10 +757,13 @@ struct NzWaveDec {
   }
 };
 
+// One workgroup decodes chunk `c` of one tensor; wavefront k of the workgroup
+// takes segment k of the chunk (wavefronts beyond the chunk's segments only
+// help to build the slot table).
 template <int S>
-__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
-    const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
-    uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status) {
+__device__ __forceinline__ void nz_decode_chunk(
+    const uint8_t* __restrict__ comp, const uint64_t comp_bytes, const uint8_t* __restrict__ packed,
+    uint16_t* __restrict__ out, const NzGeom& g, uint32_t* __restrict__ d_status, const uint64_t c) {
   extern __shared__ uint32_t lds[];
   uint2* lut = reinterpret_cast<uint2*>(lds);                   // 4096 x 8 bytes
   uint32_t* rings = lds + 2 * NZ_M;                             // spc rings
@@ -771,7 +774,6 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
   const uint32_t tid = threadIdx.x;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keep it scalar
   const uint32_t lane = tid & 63;
-  const uint64_t c = blockIdx.x;
   const uint64_t seg0 = c * g.spc;
   const uint64_t chunk_base = c * g.chunk_syms;
   const uint32_t cn =
@@ -1034,4 +1036,42 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
       }
     }
   }
+}
+
+template <int S>
+__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
+    const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
+    uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status) {
+  nz_decode_chunk<S>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x);
+}
+
+// Several tensors in one launch: the grid is the concatenation of their
+// chunks, `chunk_end` the running total.  The items ride in the kernel
+// argument block, so a launch needs no device-side table.
+#define NZ_BATCH_MAX 16
+struct NzBatchItem {
+  const uint8_t* comp;
+  uint64_t comp_bytes;
+  const uint8_t* packed;
+  uint16_t* out;
+  NzGeom g;
+  uint32_t chunk_end;
+  uint32_t reserved;
+};
+struct NzBatch {
+  uint32_t count;
+  uint32_t reserved;
+  NzBatchItem item[NZ_BATCH_MAX];
+};
+
+template <int S>
+__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_batch_kernel(
+    const NzBatch b, uint32_t* __restrict__ d_status) {
+  uint32_t t = 0, first = 0;
+  while (t + 1 < b.count && blockIdx.x >= b.item[t].chunk_end) {
+    first = b.item[t].chunk_end;
+    ++t;
+  }
+  const NzBatchItem& it = b.item[t];
+  nz_decode_chunk<S>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status, blockIdx.x - first);
 }

@@ -29,6 +29,11 @@ class Linear(torch.nn.Module):
         return self._p
 
     def forward(self, x):
+        if not torch.is_grad_enabled():
+            # nothing to record for backward: same arithmetic without the autograd node
+            if torch.is_autocast_enabled():
+                x = x.to(torch.get_autocast_gpu_dtype())
+            return self._p.linear(x, self.bias)
         return CompressedLinear.apply(x, self._p, self.bias)
 
     def extra_repr(self) -> str:

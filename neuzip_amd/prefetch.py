@@ -1,16 +1,20 @@
-"""Decompress-ahead for a converted model.
+"""Per-block decompress(-ahead) for a converted model.
 
-The reference decompresses a weight inside the very call that needs it and
-blocks the host until it is there (cuda/high_level.cu:203,252-263).  Here the
-weight of the NEXT compressed Linear is decoded on a side stream while the
-current one runs its GEMM, so that by the time a layer is reached its dense
-weight is (partly) ready.  Only HIP streams and events are used; all streams
-have the default priority.
+The reference decompresses a weight inside the very call that needs it, one
+tensor per kernel sequence, and blocks the host until it is there
+(cuda/high_level.cu:203,252-263).  A single projection matrix is too small to
+fill an MI355X with decoder wavefronts, the seven of a transformer block
+together are not.  ``DecompressAhead`` therefore decodes all compressed Linear
+weights of one block with ONE kernel launch into a static dense buffer, at the
+moment the block's first Linear runs, and (``ahead=True``) already enqueues
+the next block's decode on a side stream so that it overlaps the current
+block's GEMMs.  Only HIP streams and events are used; all streams have the
+default priority; nothing is allocated after construction.
 
 Usage::
 
     manager.convert(model); model.cuda()
-    ahead = DecompressAhead(manager, model)      # forward order = module order
+    ahead = DecompressAhead(manager, model)      # blocks = elements of the model's ModuleLists
     with ahead:                                   # or ahead.enable() / ahead.disable()
         y = model(x)
 """
@@ -21,35 +25,68 @@ import torch
 from neuzip_amd.nn.linear import Linear
 
 
-class _Slot:
-    """One dense scratch buffer of the ring kept per weight size."""
+def _default_blocks(model: torch.nn.Module):
+    """Elements of every ModuleList that hold compressed Linears, in module order."""
+    blocks = []
+    for mod in model.modules():
+        if isinstance(mod, torch.nn.ModuleList):
+            for child in mod:
+                if any(isinstance(m, Linear) for m in child.modules()):
+                    blocks.append(child)
+    # a nested ModuleList would list a Linear twice: keep the outermost grouping
+    seen, out = set(), []
+    for b in blocks:
+        lins = [m for m in b.modules() if isinstance(m, Linear) and id(m) not in seen]
+        if lins:
+            seen.update(id(m) for m in lins)
+            out.append(lins)
+    return out
 
-    __slots__ = ("buf", "ready", "free", "handle")
+
+class _Slot:
+    """One static dense buffer able to hold the weights of any block."""
+
+    __slots__ = ("buf", "ready", "block", "used")
 
     def __init__(self, numel: int, device):
         self.buf = torch.empty(numel, dtype=torch.bfloat16, device=device)
-        self.ready = None   # recorded on the side stream when the decode is enqueued
-        self.free = None    # recorded on the consumer's stream after the GEMM that used the buffer
-        self.handle = None
+        self.ready = None  # event of a side-stream decode the consumer has not waited for yet
+        self.block = -1    # index of the block whose weights the buffer holds (or will hold)
+        self.used = False  # a forward pass already consumed this decode
 
 
 class DecompressAhead:
-    def __init__(self, manager, model: torch.nn.Module, depth: int = 1):
+    def __init__(self, manager, model: torch.nn.Module, blocks=None, ahead: bool = True, wrap: bool = True):
+        """``blocks``: modules whose compressed Linears are decoded together
+        (default: the elements of the model's ModuleLists); ``ahead``: decode
+        block k+1 on a side stream while block k computes; ``wrap``: after the
+        last block, already decode the first one for the next forward pass."""
         self.manager = manager
-        self.layers = [m for m in model.modules() if isinstance(m, Linear)]
-        self.handles = [m._p._handle for m in self.layers]
-        self.depth = max(1, int(depth))
-        self.stream = torch.cuda.Stream()  # default priority
-        self._pos = {h: i for i, h in enumerate(self.handles)}
+        self.wrap = bool(wrap)
         be = manager._be
-        self._numel = {h: be.numel(h) for h in self.handles}
-        # a ring of depth + 1 dense buffers per distinct weight size: one being
-        # consumed, `depth` being filled
+        groups = _default_blocks(model) if blocks is None else [
+            [m for m in b.modules() if isinstance(m, Linear)] for b in blocks]
+        self._handles = [[m._p._handle for m in g] for g in groups if g]
+        self._where = {}
+        for bi, hs in enumerate(self._handles):
+            for k, h in enumerate(hs):
+                self._where[h] = (bi, k)
+        self._plans = [be.batch_plan(hs) for hs in self._handles]
+        # element offsets of the block's tensors in a slot buffer, 16-byte aligned
+        self._offsets, need = [], 0
+        for hs in self._handles:
+            offs, at = [], 0
+            for h in hs:
+                offs.append(at)
+                at += (be.numel(h) + 7) & ~7
+            self._offsets.append(offs)
+            need = max(need, at)
         dev = torch.device("cuda", torch.cuda.current_device())
-        self._rings = {}
-        for n in set(self._numel.values()):
-            self._rings[n] = [[_Slot(n, dev) for _ in range(self.depth + 1)], 0]
-        self._ready = {}  # handle -> slot holding (or about to hold) its dense weight
+        self.ahead = bool(ahead) and len(self._handles) > 1
+        self._slots = [_Slot(need, dev) for _ in range(2 if self.ahead else 1)]
+        self._views = [[[s.buf[o:o + be.numel(h)] for o, h in zip(offs, hs)]
+                        for offs, hs in zip(self._offsets, self._handles)] for s in self._slots]
+        self.stream = torch.cuda.Stream() if self.ahead else None  # default priority
         self._enabled = False
 
     # -- context management ---------------------------------------------------
@@ -61,8 +98,7 @@ class DecompressAhead:
     def disable(self):
         if self._enabled:
             del self.manager.linear
-            torch.cuda.synchronize()
-            self._ready.clear()
+            self.join()
             self._enabled = False
 
     def __enter__(self):
@@ -73,48 +109,80 @@ class DecompressAhead:
         self.disable()
         return False
 
+    def join(self):
+        """Make the current stream wait for any decode still running on the side
+        stream and forget what the buffers hold (call before ending a stream
+        capture, and after the weights were rewritten)."""
+        cur = torch.cuda.current_stream()
+        for s in self._slots:
+            if s.ready is not None:
+                cur.wait_event(s.ready)
+            s.ready = None
+            s.block = -1
+            s.used = False
+
     # -- the hook ---------------------------------------------------------------
-    def _issue(self, handle: str, after: torch.cuda.Event) -> None:
-        if handle in self._ready:
-            return
-        ring = self._rings[self._numel[handle]]
-        slot = ring[0][ring[1]]
-        ring[1] = (ring[1] + 1) % len(ring[0])
-        if slot.handle is not None:
-            self._ready.pop(slot.handle, None)  # evicted before use
+    # Stream order does most of the work: the consumer stream decodes, computes
+    # and releases buffers in program order; the side stream is forked from the
+    # consumer stream at the entry of a block (one event) and joined at the
+    # entry of the next one (one event).
+    def _decode_here(self, bi: int, slot_i: int, cur) -> None:
+        slot = self._slots[slot_i]
+        if slot.ready is not None:  # an unused decode-ahead still owns the buffer
+            cur.wait_event(slot.ready)
+            slot.ready = None
+        self.manager._be.read_batch(self._plans[bi], self._views[slot_i][bi])
+        slot.block = bi
+        slot.used = False
+
+    def _decode_ahead(self, bi: int, slot_i: int, cur) -> None:
+        slot = self._slots[slot_i]
+        fork = torch.cuda.Event()
+        fork.record(cur)  # every earlier reader and writer of the buffer is before this point
         with torch.cuda.stream(self.stream):
-            self.stream.wait_event(after)          # not further ahead than `depth` layers
-            if slot.free is not None:
-                self.stream.wait_event(slot.free)  # the last consumer of this buffer is done
-            self.manager._be.read_into(handle, slot.buf)
+            self.stream.wait_event(fork)
+            self.manager._be.read_batch(self._plans[bi], self._views[slot_i][bi])
             slot.ready = torch.cuda.Event()
             slot.ready.record(self.stream)
-        slot.handle = handle
-        self._ready[handle] = slot
+        slot.block = bi
+        slot.used = False
+
+    def _weight(self, handle: str):
+        bi, k = self._where[handle]
+        slot_i = next((i for i, s in enumerate(self._slots) if s.block == bi), None)
+        if k == 0 and slot_i is not None and self._slots[slot_i].used:
+            self._slots[slot_i].block = -1  # left over from an earlier pass: decode again
+            slot_i = None
+        if k == 0 or slot_i is None:
+            cur = torch.cuda.current_stream()
+            if slot_i is None:
+                slot_i = next((i for i, s in enumerate(self._slots) if s.block < 0), 0)
+                self._decode_here(bi, slot_i, cur)
+            slot = self._slots[slot_i]
+            if slot.ready is not None:  # join the side stream once per block
+                cur.wait_event(slot.ready)
+                slot.ready = None
+            slot.used = True
+            if self.ahead and k == 0 and (self.wrap or bi + 1 < len(self._handles)):
+                nxt = (bi + 1) % len(self._handles)
+                other = 1 - slot_i
+                if self._slots[other].block != nxt or self._slots[other].used:
+                    if self._slots[other].ready is not None:  # never consumed: keep the streams joined
+                        cur.wait_event(self._slots[other].ready)
+                        self._slots[other].ready = None
+                    self._decode_ahead(nxt, other, cur)
+        elif self._slots[slot_i].ready is not None:  # the block was entered at another Linear than its first
+            torch.cuda.current_stream().wait_event(self._slots[slot_i].ready)
+            self._slots[slot_i].ready = None
+        return self._views[slot_i][bi][k]
 
     def _linear(self, handle: str, inputs: torch.Tensor, bias=None) -> torch.Tensor:
         shape = self.manager.meta_dict[handle]
-        cur = torch.cuda.current_stream()
-        i = self._pos.get(handle)
-        slot = self._ready.pop(handle, None)
-        if slot is None:
-            weight = self.manager._be.read(handle)
+        if handle in self._where:
+            weight = self._weight(handle)
         else:
-            cur.wait_event(slot.ready)
-            weight = slot.buf
-            slot.handle = None
-        if i is not None:
-            here = torch.cuda.Event()
-            here.record(cur)
-            n = len(self.handles)
-            for k in range(1, self.depth + 1):
-                self._issue(self.handles[(i + k) % n], here)
+            weight = self.manager._be.read(handle)
         weight = weight.view(shape)
         if bias is not None and inputs.dim() == 2:
-            out = torch.addmm(bias, inputs, weight.t())
-        else:
-            out = torch.nn.functional.linear(inputs, weight, bias)
-        if slot is not None:
-            slot.free = torch.cuda.Event()
-            slot.free.record(cur)
-        return out
+            return torch.addmm(bias, inputs, weight.t())
+        return torch.nn.functional.linear(inputs, weight, bias)

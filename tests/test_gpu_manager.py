@@ -6,7 +6,7 @@ from functools import partial
 import numpy as np
 import pytest
 
-from conftest import bf16_bits_normal, closed_form_recon
+from conftest import bf16_bits_normal, closed_form_recon, stress_bits
 
 pytestmark = pytest.mark.gpu
 
@@ -216,12 +216,36 @@ def test_dummy_backend():
     assert torch.equal(mgr.linear(h, x), torch.nn.functional.linear(x, w.cuda()))
 
 
-def test_decompress_ahead_matches_plain_forward():
+class _Block(torch.nn.Module):
+    def __init__(self, d, i):
+        super().__init__()
+        self.a = torch.nn.Linear(d, 2 * d, bias=(i % 2 == 0))
+        self.b = torch.nn.Linear(2 * d, d, bias=False)
+        self.c = torch.nn.Linear(d, d, bias=True)
+
+    def forward(self, x):
+        return x + self.c(self.b(torch.nn.functional.gelu(self.a(x))))
+
+
+class _Stack(torch.nn.Module):
+    def __init__(self, d, depth):
+        super().__init__()
+        self.inp = torch.nn.Linear(d, d)
+        self.blocks = torch.nn.ModuleList([_Block(d, i) for i in range(depth)])
+
+    def forward(self, x):
+        x = self.inp(x)
+        for b in self.blocks:
+            x = b(x)
+        return x
+
+
+@pytest.mark.parametrize("depth", [1, 2, 5])
+def test_decompress_ahead_matches_plain_forward(depth):
     import neuzip_amd
 
     torch.manual_seed(5)
-    layers = [torch.nn.Linear(256, 256, bias=(i % 2 == 0)) for i in range(6)]
-    model = torch.nn.Sequential(*layers).to(torch.bfloat16)
+    model = _Stack(256, depth).to(torch.bfloat16)
     for p in model.parameters():
         p.data.normal_(0, 0.02)
     mgr = neuzip_amd.Manager()
@@ -230,14 +254,116 @@ def test_decompress_ahead_matches_plain_forward():
     x = torch.randn(3, 256, device="cuda", dtype=torch.bfloat16)
     with torch.no_grad():
         want = model(x)
-        for depth in (1, 2):
-            ahead = neuzip_amd.DecompressAhead(mgr, model, depth=depth)
-            with ahead:
-                for _ in range(3):  # wraps around: the last layer prefetches the first
+        for ahead, wrap in ((False, True), (True, True), (True, False)):
+            print(f"case depth={depth} ahead={ahead} wrap={wrap}", flush=True)
+            da = neuzip_amd.DecompressAhead(mgr, model, ahead=ahead, wrap=wrap)
+            with da:
+                for _ in range(3):  # with wrap the last block prefetches the first
                     got = model(x)
                     assert torch.equal(got, want)
             assert torch.equal(model(x), want)  # hook removed again
     mgr._be.check()
+
+
+def test_decompress_ahead_sees_rewritten_weights():
+    import neuzip_amd
+
+    torch.manual_seed(6)
+    model = _Stack(128, 2).to(torch.bfloat16)
+    mgr = neuzip_amd.Manager()
+    mgr.convert(model)
+    model = model.cuda()
+    x = torch.randn(2, 128, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad(), neuzip_amd.DecompressAhead(mgr, model) as da:
+        y0 = model(x)
+        lin = model.blocks[0].a
+        mgr.write(lin.weight() * 2, lin.weight._handle)
+        da.join()
+        y1 = model(x)
+    with torch.no_grad():
+        assert torch.equal(y1, model(x))
+    assert not torch.equal(y0, y1)
+
+
+def test_decode_under_graph_capture_replays_exactly():
+    """The decode launches (per Linear, per block, per block with the side
+    stream) captured into a HIP graph: every replay, with eager work and host
+    synchronisation in between, gives the eager result for its input."""
+    import neuzip_amd
+
+    torch.manual_seed(7)
+    model = _Stack(256, 4).to(torch.bfloat16)
+    for p in model.parameters():
+        p.data.normal_(0, 0.02)
+    mgr = neuzip_amd.Manager()
+    mgr.convert(model)
+    model = model.cuda()
+    xs = [torch.randn(1, 256, device="cuda", dtype=torch.bfloat16) for _ in range(5)]
+    x_static = torch.zeros_like(xs[0])
+    with torch.no_grad():
+        wants = [model(x) for x in xs]
+        for mode in ("per_linear", "per_block", "per_block_ahead"):
+            print(f"case graph {mode}", flush=True)
+            da = None if mode == "per_linear" else neuzip_amd.DecompressAhead(
+                mgr, model, ahead=(mode == "per_block_ahead"), wrap=False)
+            if da:
+                da.enable()
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                model(x_static)
+                if da:
+                    da.join()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                y_static = model(x_static)
+                if da:
+                    da.join()
+            for x, want in zip(xs, wants):
+                x_static.copy_(x)
+                g.replay()
+                got = y_static.clone()
+                torch.cuda.synchronize()
+                assert torch.equal(got, want)
+                (x * 2).sum().item()  # eager work between replays
+            if da:
+                da.disable()
+            del g
+    mgr._be.check()
+
+
+def test_read_batch_equals_single_reads(oracle):
+    """One launch for several stored tensors, of different sizes and (auto mode)
+    different segment geometries, gives what the single reads give."""
+    import neuzip_amd
+
+    for lane in (0, "auto"):
+        mgr = neuzip_amd.Manager(lane_symbols=lane)
+        sizes = [1, 4096, 65536 * 3 + 17, 1 << 20, 300_001, 65536, 8, 2_000_000] + [70_001 + i for i in range(12)]
+        ws = [from_bits(stress_bits(1, n, seed=n % 89) if i % 2 else bf16_bits_normal(n, seed=i), (n,))
+              for i, n in enumerate(sizes)]
+        hs = [mgr.write(w) for w in ws]
+        be = mgr._be
+        print(f"case batch lane={lane}", flush=True)
+        plan = be.batch_plan(hs)  # 20 tensors: more than one launch's worth of arguments
+        outs = [torch.zeros((n + 7) & ~7, dtype=torch.bfloat16, device="cuda") for n in sizes]
+        be.read_batch(plan, outs)
+        for w, o, n in zip(ws, outs, sizes):
+            assert torch.equal(o[:n].view(torch.int16), w.view(torch.int16))
+        be.check()
+        # a rejected argument decodes nothing
+        import ctypes
+
+        outs2 = [torch.zeros_like(o) for o in outs[:4]]
+        names = (ctypes.c_char_p * 4)(*[h.encode() for h in hs[:3]], b"no such handle")
+        ptrs = (ctypes.c_void_p * 4)(*[o.data_ptr() for o in outs2])
+        caps = (ctypes.c_uint64 * 4)(*[o.numel() for o in outs2])
+        rc = be._L.nz_manager_read_batch(be._h, names, ptrs, caps, 4, torch.cuda.current_stream().cuda_stream)
+        assert rc != 0
+        torch.cuda.synchronize()
+        assert all(int(o.view(torch.int16).abs().max()) == 0 for o in outs2)
 
 
 def test_auto_lane_symbols(oracle):
