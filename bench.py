@@ -245,10 +245,22 @@ def run_llama8b(args, torch):
             measure(tag + "_graph", capture(finish=da.join))
         del da
         torch.cuda.empty_cache()
+    # decode fused into the matrix-vector product (single-token steps only; the
+    # prefill keeps the decompress-then-GEMM path)
+    fused = neuzip_amd.FusedGemv(mgr, model)
+    with torch.no_grad():
+        model.prefill_static(prompt, kcs, vcs)
+        pos_buf.fill_(T)
+        fused.trace(lambda: model.step_static(tok_buf, pos_buf, kcs, vcs))
+    with fused:
+        measure("fused_eager")
+        measure("fused_graph", capture())
     mgr._be.check()
 
     modes = [k[:-9] for k in res if k.endswith("_decode_s")]
-    same = all(bool(torch.equal(toks["dense_eager"], toks[m])) for m in modes)
+    same = all(bool(torch.equal(toks["dense_eager"], toks[m])) for m in modes if not m.startswith("fused"))
+    fused_same = bool(torch.equal(toks["fused_eager"], toks["fused_graph"]))
+    fused_prefix = int((toks["fused_eager"] != toks["dense_eager"]).int().cumsum(1).eq(0).sum())
     comp_modes = [m for m in modes if not m.startswith("dense")]
     tok_s = {m: round((steps - 1) / res[m + "_decode_s"], 2) for m in modes}
     total = {m: res[m + "_prefill_s"] + res[m + "_decode_s"] for m in modes}
@@ -266,7 +278,10 @@ def run_llama8b(args, torch):
             "workload": f"Llama-3-8B-shaped random-init decoder, {layers} layers, batch 1, {T}-token "
                         f"prompt + {steps} greedy steps, Linear weights compressed (precision {args.precision})",
             "best_mode": best,
-            "tokens_identical_in_all_modes": same,
+            "tokens_identical_in_all_decompress_modes": same,
+            "fused_graph_tokens_equal_fused_eager": fused_same,
+            "fused_leading_tokens_equal_to_dense": fused_prefix,
+            "fused_groups": sorted(len(g.handles) for g in fused._groups)[-4:],
             "decode_tok_s": tok_s,
             "prefill_s": {m: round(res[m + "_prefill_s"], 4) for m in modes},
             "total_s": {m: round(total[m], 4) for m in modes},

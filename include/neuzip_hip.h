@@ -135,6 +135,23 @@ int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap
 int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* dev_outs,
                           const uint64_t* cap_elems, uint32_t count, void* stream);
 
+/* Manager::linear / linear_without_bias (cuda/high_level.cu:252-263) for ONE
+   activation row: y_i = W_i x (+ bias_i) for up to 16 stored matrices W_i =
+   names[i] that share the input x, with the weights decoded on the fly and never
+   written to memory (the reference decompresses W, then calls matmul).  Each
+   stored tensor is read as a row-major matrix with rows of `in_features`
+   elements (a multiple of 512).  dev_x: in_features bf16, 16-byte aligned;
+   dev_y[i]: rows_i bf16; dev_bias: null, or per matrix null / rows_i bf16.
+   Sums are formed in fp32 per wavefront and row, then in 34.30 fixed point
+   across wavefronts, so the result does not depend on scheduling; a row whose
+   partial sums are NaN, infinite or beyond 2^26 in magnitude comes out as NaN.
+   Calls of one manager must be ordered on one stream (they share the
+   accumulators, which are allocated on first use and grown when needed; no
+   other call allocates).  Asynchronous on `stream`. */
+int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t count, const void* dev_x,
+                          uint32_t in_features, const void* const* dev_bias, void* const* dev_y,
+                          void* stream);
+
 /* meta_cache lookup, cuda/high_level.cu:42-43,228-230. */
 int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype);
 

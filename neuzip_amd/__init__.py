@@ -8,9 +8,10 @@ import torch
 
 from neuzip_amd import nn, ops
 from neuzip_amd.binding import Algorithm, Manager
+from neuzip_amd.fused import FusedGemv
 from neuzip_amd.prefetch import DecompressAhead
 
-__all__ = ["ops", "nn", "Algorithm", "Manager", "DecompressAhead", "lomo_hook", "compressed_lomo_hook"]
+__all__ = ["ops", "nn", "Algorithm", "Manager", "DecompressAhead", "FusedGemv", "lomo_hook", "compressed_lomo_hook"]
 
 
 def _current_lr(scheduler) -> float:

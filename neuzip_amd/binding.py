@@ -128,6 +128,21 @@ class _HipBackend:
         rc = self._L.nz_manager_read_batch(self._h, names, ptrs, caps, k, _stream_ptr(outs[0].device) if k else None)
         _lib.raise_for(rc)
 
+    def gemv_batch(self, names, x: torch.Tensor, biases, outs) -> None:
+        """``outs[i] = W_i @ x (+ biases[i])`` for the stored matrices ``names``
+        (a ctypes array of encoded handles) and ONE activation row ``x``; the
+        weights are decoded inside the kernel and never written out."""
+        k = len(names)
+        if x.dtype != torch.bfloat16 or not x.is_contiguous():
+            raise ValueError("gemv_batch needs a contiguous bfloat16 activation row")
+        ys = (ctypes.c_void_p * k)(*[o.data_ptr() for o in outs])
+        bs = None
+        if biases is not None and any(b is not None for b in biases):
+            bs = (ctypes.c_void_p * k)(*[None if b is None else b.data_ptr() for b in biases])
+        rc = self._L.nz_manager_gemv_batch(self._h, names, k, x.data_ptr(), x.numel(), bs, ys,
+                                           _stream_ptr(x.device))
+        _lib.raise_for(rc)
+
     def size(self, handle: str) -> int:
         return int(self._L.nz_manager_size(self._h, handle.encode()))
 

@@ -158,6 +158,22 @@ int decode_batch_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int p
   return NZ_OK;
 }
 
+int gemv_launch(const NzBatch& b, const NzGemvOut& o, uint32_t grid, uint32_t max_spc, uint32_t rows,
+                int precision, uint32_t* d_status, hipStream_t st) {
+  const size_t lds = (2 * NZ_M + max_spc * NZ_RING_ALLOC_DWORDS) * 4;
+  const dim3 gd(grid), bd(64 * max_spc);
+  switch (precision) {
+    case 7: hipLaunchKernelGGL(nz_decode_gemv_kernel<7>, gd, bd, lds, st, b, d_status); break;
+    case 3: hipLaunchKernelGGL(nz_decode_gemv_kernel<3>, gd, bd, lds, st, b, d_status); break;
+    case 1: hipLaunchKernelGGL(nz_decode_gemv_kernel<1>, gd, bd, lds, st, b, d_status); break;
+    default: hipLaunchKernelGGL(nz_decode_gemv_kernel<0>, gd, bd, lds, st, b, d_status); break;
+  }
+  NZ_HIP(hipGetLastError());
+  hipLaunchKernelGGL(nz_gemv_finish_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, o);
+  NZ_HIP(hipGetLastError());
+  return NZ_OK;
+}
+
 int make_geom(NzGeom* g, uint64_t n, uint32_t chunk, uint32_t lane_syms) {
   if (nz_geom_make(g, n, chunk, lane_syms))
     return fail(NZ_ERR_ARG,
@@ -189,6 +205,8 @@ struct nz_manager {
   uint64_t ws_bytes = 0;
   uint32_t* d_status = nullptr;
   uint64_t* h_pin = nullptr;  // pinned: [0] total, [1] status
+  long long* gemv_acc = nullptr;  // row accumulators of the matrix-vector product (all zero between calls)
+  uint64_t gemv_rows = 0;         // rows the accumulator buffer can hold
 };
 
 extern "C" {
@@ -332,6 +350,7 @@ void nz_manager_destroy(nz_manager* m) {
     if (kv.second.packed) (void)hipFree(kv.second.packed);
   }
   if (m->ws) (void)hipFree(m->ws);
+  if (m->gemv_acc) (void)hipFree(m->gemv_acc);
   if (m->d_status) (void)hipFree(m->d_status);
   if (m->h_pin) (void)hipHostFree(m->h_pin);
   delete m;
@@ -504,6 +523,72 @@ int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* 
     if (g.spc > max_spc) max_spc = g.spc;
   }
   return b.count ? flush() : NZ_OK;
+}
+
+int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t count, const void* dev_x,
+                          uint32_t in_features, const void* const* dev_bias, void* const* dev_y,
+                          void* stream) {
+  if (!m || !names || !dev_y || !dev_x) return fail(NZ_ERR_ARG, "null manager, names, input or outputs");
+  if (count == 0 || count > NZ_BATCH_MAX) return fail(NZ_ERR_ARG, "between 1 and 16 matrices per call");
+  if (in_features == 0 || in_features % NZ_GROUP_SYMS)
+    return fail(NZ_ERR_ARG, "in_features must be a multiple of 512");
+  if ((uintptr_t)dev_x & 15) return fail(NZ_ERR_ALIGN, "activation must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  std::lock_guard<std::mutex> lock(m->mu);
+  NzBatch b;
+  NzGemvOut o;
+  std::memset(&b, 0, sizeof(b));
+  std::memset(&o, 0, sizeof(o));
+  b.x = (const uint16_t*)dev_x;
+  b.in_features = in_features;
+  uint64_t grid = 0, rows = 0;
+  uint32_t max_spc = 1;
+  for (uint32_t i = 0; i < count; ++i) {
+    if (!names[i]) return fail(NZ_ERR_ARG, "null name");
+    auto it = m->entries.find(names[i]);
+    if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+    const Entry& ent = it->second;
+    if (ent.n == 0 || ent.n % in_features)
+      return fail(NZ_ERR_ARG, "stored tensor is not a matrix with rows of in_features elements");
+    if (!dev_y[i] || ((uintptr_t)dev_y[i] & 1)) return fail(NZ_ERR_ARG, "null or misaligned output pointer");
+    if (dev_bias && dev_bias[i] && ((uintptr_t)dev_bias[i] & 1)) return fail(NZ_ERR_ALIGN, "misaligned bias");
+    NzGeom g;
+    if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
+    NzBatchItem& bi = b.item[i];
+    bi.comp = (const uint8_t*)ent.comp;
+    bi.comp_bytes = ent.comp_bytes;
+    bi.packed = (const uint8_t*)ent.packed;
+    bi.g = g;
+    grid += g.n_chunks;
+    bi.chunk_end = (uint32_t)grid;
+    if (g.spc > max_spc) max_spc = g.spc;
+    NzGemvOutItem& oi = o.item[i];
+    oi.bias = dev_bias ? (const uint16_t*)dev_bias[i] : nullptr;
+    oi.y = (uint16_t*)dev_y[i];
+    bi.reserved = (uint32_t)rows;  // first row, turned into a pointer below
+    rows += ent.n / in_features;
+    oi.row_end = (uint32_t)rows;
+    if (grid > 0x7FFFFFFFull || rows > 0x7FFFFFFFull) return fail(NZ_ERR_ARG, "batch too large");
+  }
+  if (m->gemv_rows < rows) {
+    // the buffer in use may still be read by kernels on the stream
+    NZ_HIP(hipStreamSynchronize(st));
+    if (m->gemv_acc) NZ_HIP(hipFree(m->gemv_acc));
+    m->gemv_acc = nullptr;
+    m->gemv_rows = 0;
+    const uint64_t want = rows < 65536 ? 65536 : rows;
+    NZ_HIP(hipMalloc((void**)&m->gemv_acc, want * 16));
+    NZ_HIP(hipMemset(m->gemv_acc, 0, want * 16));
+    m->gemv_rows = want;
+  }
+  for (uint32_t i = 0; i < count; ++i) {
+    b.item[i].acc = m->gemv_acc + 2 * (uint64_t)b.item[i].reserved;
+    b.item[i].reserved = 0;
+    o.item[i].acc = b.item[i].acc;
+  }
+  b.count = count;
+  o.count = count;
+  return gemv_launch(b, o, (uint32_t)grid, max_spc, (uint32_t)rows, m->precision, m->d_status, st);
 }
 
 int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype) {

@@ -630,11 +630,10 @@ __device__ __forceinline__ uint64_t nz_load_sm(const uint8_t* p) {
   else return *p;
 }
 
-// Merge 8 exponents (byte 3 of ew[j]) with the group's packed bytes and store
-// 8 bf16 values with one 16-byte store.
+// Merge 8 exponents (byte 3 of ew[j]) with the group's packed bytes into 8
+// bf16 values.
 template <int S>
-__device__ __forceinline__ void nz_store_group(uint16_t* __restrict__ out, uint64_t sm,
-                                               const uint32_t (&ew)[8]) {
+__device__ __forceinline__ uint4 nz_merge_group(uint64_t sm, const uint32_t (&ew)[8]) {
   uint32_t o[4];
   if constexpr (S == 7) {
     // out16 = sign << 15 | exp << 7 | mant, byte b = sign << 7 | mant.  Per pair:
@@ -658,8 +657,96 @@ __device__ __forceinline__ void nz_store_group(uint16_t* __restrict__ out, uint6
       o[j >> 1] = nz_merge_one<S>(ew[j] >> 24, r0) | (nz_merge_one<S>(ew[j + 1] >> 24, r1) << 16);
     }
   }
-  *reinterpret_cast<uint4*>(out) = make_uint4(o[0], o[1], o[2], o[3]);
+  return make_uint4(o[0], o[1], o[2], o[3]);
 }
+
+// ... and store them with one 16-byte store.
+template <int S>
+__device__ __forceinline__ void nz_store_group(uint16_t* __restrict__ out, uint64_t sm,
+                                               const uint32_t (&ew)[8]) {
+  *reinterpret_cast<uint4*>(out) = nz_merge_group<S>(sm, ew);
+}
+
+// ----------------------------------------------------------------------------
+// y = W x for one activation row, W decoded on the fly and never written out
+// ----------------------------------------------------------------------------
+// A group of 512 consecutive weights lies inside one row of W (the row length
+// is a multiple of 512), so the row of a group is the same for all lanes.  A
+// lane keeps an fp32 partial sum of its 8-element dot products; when the wave
+// leaves a row the 64 partial sums are added in a fixed butterfly order and
+// lane 0 adds the result, converted to 34.30 fixed point, to the row's 64-bit
+// accumulator.  Integer addition is associative, so the value of y does not
+// depend on the order in which the wavefronts that share a row arrive.  A
+// partial sum that is NaN, infinite or beyond 2^26 sets the row's flag word
+// instead (the row then comes out as NaN).  Row r owns acc[2r] (sum) and
+// acc[2r + 1] (flag).
+#define NZ_GEMV_FRAC_BITS 30
+#define NZ_GEMV_PART_MAX 67108864.0f /* 2^26 */
+
+struct NzGemv {
+  const uint16_t* x;      // in_features bf16 values, 16-byte aligned
+  long long* acc;         // two words per row of this tensor (sum, flag), all zero on entry
+  uint32_t in_features;   // multiple of 512
+};
+
+typedef __attribute__((ext_vector_type(2))) __bf16 nz_bf16x2;
+
+__device__ __forceinline__ float nz_dot8(const uint4 w, const uint4 x, float acc) {
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(nz_bf16x2, w.x), __builtin_bit_cast(nz_bf16x2, x.x), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(nz_bf16x2, w.y), __builtin_bit_cast(nz_bf16x2, x.y), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(nz_bf16x2, w.z), __builtin_bit_cast(nz_bf16x2, x.z), acc, false);
+  acc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(nz_bf16x2, w.w), __builtin_bit_cast(nz_bf16x2, x.w), acc, false);
+  return acc;
+}
+
+// Position of a wavefront inside W while it walks its segment group by group.
+struct NzGemvWalk {
+  const uint4* xq;     // x as 8-element blocks, already offset by the lane
+  long long* acc;
+  uint64_t row;
+  uint32_t col;        // column of the current group's first element (uniform)
+  uint32_t in_features;
+  uint32_t pending;    // groups added since the last flush (uniform)
+  float sum;
+
+  __device__ __forceinline__ void start(const NzGemv& gv, uint64_t first_elem, uint32_t lane) {
+    xq = reinterpret_cast<const uint4*>(gv.x) + lane;
+    acc = gv.acc;
+    in_features = gv.in_features;
+    row = first_elem / in_features;
+    col = (uint32_t)(first_elem - row * in_features);
+    pending = 0;
+    sum = 0.f;
+  }
+  __device__ __forceinline__ uint32_t next_col() const {
+    return col + NZ_GROUP_SYMS == in_features ? 0u : col + NZ_GROUP_SYMS;
+  }
+  __device__ __forceinline__ uint4 load(uint32_t c) const { return xq[c / NZ_GROUP]; }
+  __device__ __forceinline__ void flush(uint32_t lane) {
+    float t = sum;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
+    if (lane == 0) {
+      unsigned long long* slot = reinterpret_cast<unsigned long long*>(acc + 2 * row);
+      if (fabsf(t) < NZ_GEMV_PART_MAX)  // false for NaN as well
+        atomicAdd(slot, (unsigned long long)__float2ll_rn(t * (float)(1u << NZ_GEMV_FRAC_BITS)));
+      else
+        atomicOr(slot + 1, 1ull);
+    }
+    sum = 0.f;
+    pending = 0;
+  }
+  // add the dot product of the current group, then step to the next group
+  __device__ __forceinline__ void add(const uint4 w, const uint4 x, uint32_t lane) {
+    sum = nz_dot8(w, x, sum);
+    ++pending;
+    col = next_col();
+    if (col == 0) {
+      flush(lane);
+      ++row;
+    }
+  }
+};
 
 // Decoder state of one wavefront.
 struct NzWaveDec {
@@ -760,10 +847,15 @@ struct NzWaveDec {
 // One workgroup decodes chunk `c` of one tensor; wavefront k of the workgroup
 // takes segment k of the chunk (wavefronts beyond the chunk's segments only
 // help to build the slot table).
-template <int S>
+// With GEMV the decoded values are not stored: they are multiplied with the
+// activation `gv.x` and summed into `gv.acc` (the tensor is a row-major matrix
+// with rows of gv.in_features elements, a multiple of 512, so that no group is
+// ragged and no group straddles two rows).
+template <int S, bool GEMV>
 __device__ __forceinline__ void nz_decode_chunk(
     const uint8_t* __restrict__ comp, const uint64_t comp_bytes, const uint8_t* __restrict__ packed,
-    uint16_t* __restrict__ out, const NzGeom& g, uint32_t* __restrict__ d_status, const uint64_t c) {
+    uint16_t* __restrict__ out, const NzGeom& g, uint32_t* __restrict__ d_status, const uint64_t c,
+    const NzGemv& gv) {
   extern __shared__ uint32_t lds[];
   uint2* lut = reinterpret_cast<uint2*>(lds);                   // 4096 x 8 bytes
   uint32_t* rings = lds + 2 * NZ_M;                             // spc rings
@@ -907,6 +999,8 @@ __device__ __forceinline__ void nz_decode_chunk(
   const uint64_t chunk_keep = (uint64_t)g.chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * g.spc;
   const uint8_t* pk = packed + c * chunk_keep + (uint64_t)wave * (g.seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES);
   uint16_t* dst = out + seg_base;
+  NzGemvWalk walk;
+  if constexpr (GEMV) walk.start(gv, seg_base, lane);
 
   if (mode == NZ_MODE_RAW) {
     const uint32_t padded = (seg_n + 3) & ~3u;
@@ -928,8 +1022,9 @@ __device__ __forceinline__ void nz_decode_chunk(
         uint32_t ew[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) ew[j] = (uint32_t)((sy >> (8 * j)) & 0xFFu) << 24;
-        nz_store_group<S>(dst + idx0, sm, ew);
-      } else {
+        if constexpr (GEMV) walk.add(nz_merge_group<S>(sm, ew), walk.load(walk.col), lane);
+        else nz_store_group<S>(dst + idx0, sm, ew);
+      } else if constexpr (!GEMV) {
         for (uint32_t j = 0; j < rem; ++j) {
           const uint32_t bit = (idx0 + j) * (S + 1);
           const uint32_t rp = ((uint32_t)pk[bit >> 3] >> (7u - S - (bit & 7u))) & ((2u << S) - 1u);
@@ -937,6 +1032,8 @@ __device__ __forceinline__ void nz_decode_chunk(
         }
       }
     }
+    if constexpr (GEMV)
+      if (walk.pending) walk.flush(lane);
     return;
   }
 
@@ -981,10 +1078,14 @@ __device__ __forceinline__ void nz_decode_chunk(
   const uint32_t lane_off = lane * (S + 1);
   const uint32_t last_off = whole ? (whole - 1) * NZ_LANES * (S + 1) + lane_off : 0u;
   uint64_t sm_next = whole ? nz_load_sm<S>(pk + lane_off) : 0;
+  uint4 xq_next = make_uint4(0, 0, 0, 0);
+  if constexpr (GEMV) xq_next = walk.load(walk.col);
   for (uint32_t gq = 0; gq < whole; ++gq) {
     const uint64_t sm = sm_next;
     const uint32_t noff = (gq + 1) * NZ_LANES * (S + 1) + lane_off;
     sm_next = nz_load_sm<S>(pk + (noff < last_off ? noff : last_off));
+    const uint4 xq = xq_next;
+    if constexpr (GEMV) xq_next = walk.load(walk.next_col());  // always inside x
     uint32_t ew[8];
     w.group(ew);
     // the merge starts only here: its wait for the packed bytes (fetched a group
@@ -992,9 +1093,12 @@ __device__ __forceinline__ void nz_decode_chunk(
     // wait for the previous group's store
     uint32_t sml = (uint32_t)sm, smh = (uint32_t)(sm >> 32);
     asm volatile("" : "+v"(sml), "+v"(smh), "+v"(ew[7]));
-    nz_store_group<S>(dst + (gq * NZ_LANES + lane) * NZ_GROUP, ((uint64_t)smh << 32) | sml, ew);
+    if constexpr (GEMV)
+      walk.add(nz_merge_group<S>(((uint64_t)smh << 32) | sml, ew), xq, lane);
+    else
+      nz_store_group<S>(dst + (gq * NZ_LANES + lane) * NZ_GROUP, ((uint64_t)smh << 32) | sml, ew);
   }
-  if (whole < body) {  // the ragged last group of the tensor
+  if (!GEMV && whole < body) {  // the ragged last group of the tensor
     const uint32_t idx0 = (whole * NZ_LANES + lane) * NZ_GROUP;
     uint32_t ew[8];
     w.group(ew);
@@ -1032,17 +1136,20 @@ __device__ __forceinline__ void nz_decode_chunk(
         const uint32_t idx0 = ((body + t) * NZ_LANES + lane) * NZ_GROUP;
         const uint32_t b = idx0 / 8 * (S + 1);
         const uint64_t sm = b >= keep ? nz_load_sm<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
-        nz_store_group<S>(dst + idx0, sm, ext[t]);
+        if constexpr (GEMV) walk.add(nz_merge_group<S>(sm, ext[t]), walk.load(walk.col), lane);
+        else nz_store_group<S>(dst + idx0, sm, ext[t]);
       }
     }
   }
+  if constexpr (GEMV)
+    if (walk.pending) walk.flush(lane);
 }
 
 template <int S>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
     uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status) {
-  nz_decode_chunk<S>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x);
+  nz_decode_chunk<S, false>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x, NzGemv{});
 }
 
 // Several tensors in one launch: the grid is the concatenation of their
@@ -1053,14 +1160,16 @@ struct NzBatchItem {
   const uint8_t* comp;
   uint64_t comp_bytes;
   const uint8_t* packed;
-  uint16_t* out;
+  uint16_t* out;       // dense output (decode) ...
+  long long* acc;      // ... or the row accumulators (matrix-vector product)
   NzGeom g;
   uint32_t chunk_end;
   uint32_t reserved;
 };
 struct NzBatch {
   uint32_t count;
-  uint32_t reserved;
+  uint32_t in_features;  // matrix-vector product only
+  const uint16_t* x;     // matrix-vector product only
   NzBatchItem item[NZ_BATCH_MAX];
 };
 
@@ -1073,5 +1182,61 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_batch_ke
     ++t;
   }
   const NzBatchItem& it = b.item[t];
-  nz_decode_chunk<S>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status, blockIdx.x - first);
+  nz_decode_chunk<S, false>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status, blockIdx.x - first,
+                            NzGemv{});
+}
+
+// The same walk over several matrices that multiply one activation row.
+template <int S>
+__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_gemv_kernel(
+    const NzBatch b, uint32_t* __restrict__ d_status) {
+  uint32_t t = 0, first = 0;
+  while (t + 1 < b.count && blockIdx.x >= b.item[t].chunk_end) {
+    first = b.item[t].chunk_end;
+    ++t;
+  }
+  const NzBatchItem& it = b.item[t];
+  const NzGemv gv{b.x, it.acc, b.in_features};
+  nz_decode_chunk<S, true>(it.comp, it.comp_bytes, it.packed, nullptr, it.g, d_status, blockIdx.x - first, gv);
+}
+
+// y = bf16(acc * 2^-30 + bias), and the accumulators return to zero for the next
+// product.  Flagged rows come out as NaN.
+struct NzGemvOutItem {
+  long long* acc;
+  const uint16_t* bias;  // or null
+  uint16_t* y;
+  uint32_t row_end;      // running total of rows
+  uint32_t reserved;
+};
+struct NzGemvOut {
+  uint32_t count;
+  uint32_t reserved;
+  NzGemvOutItem item[NZ_BATCH_MAX];
+};
+
+__device__ __forceinline__ float nz_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+__device__ __forceinline__ uint16_t nz_f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);  // NaN stays NaN
+  return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);                      // round to nearest even
+}
+
+__global__ __launch_bounds__(256) void nz_gemv_finish_kernel(const NzGemvOut o) {
+  const uint32_t r = blockIdx.x * 256 + threadIdx.x;
+  uint32_t t = 0, first = 0;
+  while (t + 1 < o.count && r >= o.item[t].row_end) {
+    first = o.item[t].row_end;
+    ++t;
+  }
+  const NzGemvOutItem& it = o.item[t];
+  if (r >= it.row_end) return;
+  const uint32_t i = r - first;
+  const longlong2 a = reinterpret_cast<longlong2*>(it.acc)[i];
+  reinterpret_cast<longlong2*>(it.acc)[i] = make_longlong2(0, 0);
+  float y;
+  if (a.y) y = __uint_as_float(0x7FC00000u);
+  else y = (float)((double)a.x * (1.0 / (double)(1u << NZ_GEMV_FRAC_BITS)));
+  if (it.bias) y += nz_bf16_to_f32(it.bias[i]);
+  it.y[i] = nz_f32_to_bf16(y);
 }

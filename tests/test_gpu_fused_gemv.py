@@ -1,0 +1,179 @@
+"""Fused decode + matrix-vector product against an fp64 product of the
+reconstructed weights (floating point: tolerance stated per assertion)."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import bf16_bits_normal, closed_form_recon, stress_bits
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def _bf16_to_f64(bits: np.ndarray) -> np.ndarray:
+    return (bits.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+
+
+def _weight(rows, cols, kind, seed):
+    bits = bf16_bits_normal(rows * cols, seed) if kind == "normal" else stress_bits(rows, cols, seed)
+    if kind == "stress":  # keep the product finite: no Inf/NaN patterns
+        bits = np.where(((bits >> 7) & 0xFF) == 0xFF, np.uint16(0x3C00), bits)
+    return bits
+
+
+def _gemv(mgr, handles, x, biases):
+    be = mgr._be
+    names = (ctypes.c_char_p * len(handles))(*[h.encode() for h in handles])
+    outs = [torch.full((int(np.prod(mgr.meta_dict[h])) // x.numel(),), 7.0, dtype=torch.bfloat16, device="cuda")
+            for h in handles]
+    be.gemv_batch(names, x, biases, outs)
+    torch.cuda.synchronize()
+    return outs
+
+
+def _check(y, w_bits, x, bias, s):
+    rows = y.numel()
+    w = _bf16_to_f64(closed_form_recon(w_bits, s)).reshape(rows, -1)
+    xv = x.double().cpu().numpy()
+    ref = w @ xv
+    if bias is not None:
+        ref = ref + bias.double().cpu().numpy()
+    got = y.double().cpu().numpy()
+    # bf16 output: half an ulp is 2^-9 relative; fp32 partial sums add a little
+    # relative to the sum of magnitudes
+    tol = 2.0 ** -8 * np.abs(ref) + 1e-5 * (np.abs(w) @ np.abs(xv)) + 1e-30
+    assert np.all(np.abs(got - ref) <= tol), float(np.max(np.abs(got - ref) / tol))
+
+
+@pytest.mark.parametrize("s", [7, 3, 0])
+@pytest.mark.parametrize("rows,cols,kind,lane", [
+    (64, 512, "normal", 0), (1000, 1024, "stress", 0), (4096, 4096, "normal", 0),
+    (333, 14336, "normal", 0), (512, 2048, "normal", 128), (96, 3584, "stress", "auto"),
+])
+def test_gemv_matches_fp64_product(rows, cols, kind, lane, s):
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=s, lane_symbols=lane)
+    bits = _weight(rows, cols, kind, seed=rows + s)
+    w = torch.from_numpy(bits.view(np.int16).copy()).cuda().view(torch.bfloat16).view(rows, cols)
+    h = mgr.write(w)
+    g = torch.Generator(device="cuda").manual_seed(rows)
+    x = torch.randn(cols, device="cuda", generator=g).to(torch.bfloat16)
+    bias = torch.randn(rows, device="cuda", generator=g).to(torch.bfloat16)
+    print(f"case gemv {rows}x{cols} {kind} lane={lane} s={s}", flush=True)
+    (y,) = _gemv(mgr, [h], x, None)
+    _check(y, bits, x, None, s)
+    (yb,) = _gemv(mgr, [h], x, [bias])
+    _check(yb, bits, x, bias, s)
+    # deterministic, and the accumulators are clean again after every call
+    (y2,) = _gemv(mgr, [h], x, None)
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+    mgr._be.check()
+
+
+def test_gemv_batch_equals_single_calls_and_rejects_bad_shapes():
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager()
+    cols = 1024
+    shapes = [(256, cols), (64, cols), (1024, cols), (8, cols)]
+    ws, hs = [], []
+    for i, (r, c) in enumerate(shapes):
+        bits = bf16_bits_normal(r * c, seed=40 + i)
+        w = torch.from_numpy(bits.view(np.int16).copy()).cuda().view(torch.bfloat16).view(r, c)
+        ws.append(w)
+        hs.append(mgr.write(w))
+    x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+    biases = [None, torch.randn(64, device="cuda").to(torch.bfloat16), None, None]
+    together = _gemv(mgr, hs, x, biases)
+    for h, b, y in zip(hs, biases, together):
+        (alone,) = _gemv(mgr, [h], x, [b])
+        assert torch.equal(alone.view(torch.int16), y.view(torch.int16))
+    # in_features must divide the tensor and be a multiple of 512; nothing is written otherwise
+    be = mgr._be
+    odd = mgr.write(torch.zeros(3, 700, dtype=torch.bfloat16, device="cuda"))
+    for handle, xin in ((odd, torch.zeros(700, dtype=torch.bfloat16, device="cuda")),
+                        (hs[0], torch.zeros(1536, dtype=torch.bfloat16, device="cuda"))):
+        out = torch.full((4096,), 7.0, dtype=torch.bfloat16, device="cuda")
+        names = (ctypes.c_char_p * 1)(handle.encode())
+        with pytest.raises(ValueError):
+            be.gemv_batch(names, xin, None, [out])
+        torch.cuda.synchronize()
+        assert bool((out == 7.0).all())
+    be.check()
+
+
+def test_gemv_non_finite_input_gives_nan_rows_then_recovers():
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager()
+    bits = bf16_bits_normal(128 * 512, seed=3)
+    w = torch.from_numpy(bits.view(np.int16).copy()).cuda().view(torch.bfloat16).view(128, 512)
+    h = mgr.write(w)
+    x = torch.randn(512, device="cuda").to(torch.bfloat16)
+    bad = x.clone()
+    bad[17] = float("inf")
+    (y,) = _gemv(mgr, [h], bad, None)
+    assert bool(torch.isnan(y).all())
+    (y,) = _gemv(mgr, [h], x, None)  # flags and sums were cleared
+    _check(y, bits, x, None, 7)
+
+
+class _Attn(torch.nn.Module):
+    def __init__(self, d):
+        super().__init__()
+        self.q = torch.nn.Linear(d, d, bias=False)
+        self.k = torch.nn.Linear(d, d // 2, bias=True)
+        self.v = torch.nn.Linear(d, d // 2, bias=False)
+        self.o = torch.nn.Linear(d, d, bias=True)
+
+    def forward(self, x):
+        q, k, v = self.q(x), self.k(x), self.v(x)
+        return x + self.o(q * torch.cat((k, v), dim=-1))
+
+
+def test_fused_gemv_module_groups_and_graph_replay():
+    import neuzip_amd
+
+    torch.manual_seed(11)
+    model = torch.nn.Sequential(_Attn(512), _Attn(512)).to(torch.bfloat16)
+    for p in model.parameters():
+        p.data.normal_(0, 0.05)
+    mgr = neuzip_amd.Manager()
+    mgr.convert(model)
+    model = model.cuda()
+    xs = [torch.randn(1, 1, 512, device="cuda").to(torch.bfloat16) for _ in range(4)]
+    x_static = torch.zeros_like(xs[0])
+    with torch.no_grad():
+        wants = [model(x) for x in xs]
+        many = torch.randn(3, 512, device="cuda").to(torch.bfloat16)
+        want_many = model(many)
+        fused = neuzip_amd.FusedGemv(mgr, model)
+        fused.trace(lambda: model(xs[0]))
+        assert sorted(len(g.handles) for g in fused._groups) == [1, 1, 3, 3]
+        with fused:
+            eager = [model(x) for x in xs]
+            for got, want in zip(eager, wants):
+                # every Linear output is rounded to bf16 on both paths: a few ulps through two blocks
+                assert torch.allclose(got.float(), want.float(), rtol=3e-2, atol=3e-2)
+            assert torch.equal(model(many), want_many)  # several rows: the ordinary path
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                model(x_static)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                y_static = model(x_static)
+            for x, want in zip(xs, eager):
+                x_static.copy_(x)
+                g.replay()
+                got = y_static.clone()
+                torch.cuda.synchronize()
+                assert torch.equal(got, want)  # the fused path itself is deterministic
+                (x * 2).sum().item()
+        assert torch.equal(model(xs[0]), wants[0])  # hook removed again
+    mgr._be.check()
