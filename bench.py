@@ -64,6 +64,8 @@ def parse_args():
     ap.add_argument("--decode-steps", type=int, default=128)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--seq-len", type=int, default=1024)
+    ap.add_argument("--no-llama", action="store_true",
+                    help="skip the 8B-shaped decoder that the default run appends to the codec line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run five plain 256 MiB device copies (to scale FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
@@ -137,13 +139,16 @@ def _timed(torch, fn):
     return time.perf_counter() - t0, out
 
 
-def run_llama8b(args, torch):
+def llama8b_measure(args, torch, full):
     """Llama-3-8B-shaped decoder, all Linear weights stored lossless-compressed,
     batch 1, 512-token prompt + 128 greedy steps, against the same model with
     dense weights.  Every mode runs the same static-cache decode step, eagerly
     or as a replayed HIP graph; compressed weights are decoded per Linear (the
     reference's granularity), or per transformer block with one launch, with or
-    without decoding the next block ahead on a side stream."""
+    without decoding the next block ahead on a side stream, or not at all as a
+    dense tensor (decode fused into the matrix-vector product).  `full` adds
+    the per-block modes; the lane setting -1 (auto) shortens the segments of
+    the smaller matrices."""
     import neuzip_amd
     from bench_models import LlamaShaped
 
@@ -234,7 +239,7 @@ def run_llama8b(args, torch):
 
     measure("per_linear_eager")
     measure("per_linear_graph", capture())
-    for ahead in (False, True):
+    for ahead in ((False, True) if full else ()):
         tag = "per_block_ahead" if ahead else "per_block"
         da = neuzip_amd.DecompressAhead(mgr, model, ahead=ahead)
         with da:
@@ -298,7 +303,13 @@ def run_llama8b(args, torch):
             "dense_model_bytes": dense_param_bytes,
         },
     }
-    print(json.dumps(out))
+    del fused, mgr, model, kcs, vcs
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_llama8b(args, torch):
+    print(json.dumps(llama8b_measure(args, torch, full=True)))
     return 0
 
 
@@ -556,6 +567,29 @@ def main():
                       f"({threads} threads over chunks), median",
             "matches_gpu_output": cpu_ok,
         }
+
+    # ---- the second half of the metric: tokens/s of an 8B-shaped compressed decoder ----
+    if not args.no_llama:
+        del codec, dense, out
+        torch.cuda.empty_cache()
+        import copy
+
+        largs = copy.copy(args)
+        largs.precision, largs.lane_symbols = 7, -1
+        try:
+            lm = llama8b_measure(largs, torch, full=False)
+            cfg = lm["config"]
+            result["llama8b_shape"] = {
+                "workload": cfg["workload"] + ", lane symbols chosen per tensor",
+                "decode_tok_s": cfg["decode_tok_s"],
+                "latency_ratio_eager": cfg["latency_ratio_eager"],
+                "latency_ratio_graph": cfg["latency_ratio_graph"],
+                "tokens_identical_in_all_decompress_modes": cfg["tokens_identical_in_all_decompress_modes"],
+                "fused_graph_tokens_equal_fused_eager": cfg["fused_graph_tokens_equal_fused_eager"],
+                "stored_over_dense": cfg["stored_over_dense"],
+            }
+        except Exception as e:  # the codec line above stands on its own
+            result["llama8b_shape"] = {"error": f"{type(e).__name__}: {e}"}
 
     print(json.dumps(result))
     return 0
