@@ -167,6 +167,19 @@ uint64_t nz_manager_packed_bytes(nz_manager* m, const char* name);
 int nz_manager_buffers(nz_manager* m, const char* name, const void** dev_comp,
                        uint64_t* comp_bytes, const void** dev_packed, uint64_t* packed_bytes);
 
+/* Copy an entry's two streams to host memory (sizes from nz_manager_exp_bytes /
+   nz_manager_packed_bytes) and back.  The reference keeps compressed tensors
+   only inside the process (cuda/high_level.cu:35-43; neuzip/nn/module.py:13
+   leaves 0-size parameters in a state_dict), so a converted model cannot be
+   checkpointed there; these two calls are what a save/load needs.  The
+   container names its own element count and geometry; import checks header,
+   directory and sizes against the manager (chunk_size, precision) and stores
+   nothing when they disagree.  Both calls block until the copies are done. */
+int nz_manager_export(nz_manager* m, const char* name, void* host_comp, uint64_t comp_cap,
+                      void* host_packed, uint64_t packed_cap, void* stream);
+int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, uint64_t comp_bytes,
+                      const void* host_packed, uint64_t packed_bytes, void* stream);
+
 /* compress_cache.erase(name), cuda/high_level.cu:137-140. */
 int nz_manager_erase(nz_manager* m, const char* name);
 

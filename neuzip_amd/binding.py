@@ -143,6 +143,28 @@ class _HipBackend:
                                            _stream_ptr(x.device))
         _lib.raise_for(rc)
 
+    def export(self, handle: str):
+        """The two stored streams of an entry as CPU uint8 tensors (container, packed)."""
+        name = handle.encode()
+        if self._L.nz_manager_meta(self._h, name, None, None):
+            _lib.raise_for(_lib.ERR_NOT_FOUND)
+        comp = torch.empty(self.exp_bytes(handle), dtype=torch.uint8)
+        packed = torch.empty(self.packed_bytes(handle), dtype=torch.uint8)
+        rc = self._L.nz_manager_export(self._h, name, comp.data_ptr(), comp.numel(), packed.data_ptr(),
+                                       packed.numel(), _stream_ptr(self._device))
+        _lib.raise_for(rc)
+        return comp, packed
+
+    def import_(self, handle: str, comp: torch.Tensor, packed: torch.Tensor) -> None:
+        """Store streams produced by :meth:`export` (checked against this manager's settings)."""
+        comp = comp.detach().to("cpu", torch.uint8).contiguous()
+        packed = packed.detach().to("cpu", torch.uint8).contiguous()
+        self._known.pop(handle, None)
+        rc = self._L.nz_manager_import(self._h, handle.encode(), comp.data_ptr(), comp.numel(),
+                                       packed.data_ptr() if packed.numel() else None, packed.numel(),
+                                       _stream_ptr(self._device))
+        _lib.raise_for(rc)
+
     def size(self, handle: str) -> int:
         return int(self._L.nz_manager_size(self._h, handle.encode()))
 
@@ -250,6 +272,8 @@ class Manager:
         if normalizer_size != 0:
             raise NotImplementedError("block normalizers (normalizer_size > 0) are not implemented")
         self._be = _HipBackend(precision, normalizer_size, chunk_size, lane_symbols)
+        self._settings = {"precision": int(precision), "normalizer_size": int(normalizer_size),
+                          "chunk_size": int(chunk_size)}
 
     # -- store ---------------------------------------------------------------
     def write(self, tensor: torch.Tensor, handle: Optional[str] = None) -> str:
@@ -271,6 +295,43 @@ class Manager:
         if bias is None:
             return self._be.linear_without_bias(handle, inputs, shape)
         return self._be.linear(handle, inputs, shape, bias)
+
+    # -- checkpointing (no counterpart in the reference, whose compressed tensors
+    #    live only inside the process: neuzip/nn/module.py:13) ------------------
+    def state_dict(self) -> dict:
+        """Everything needed to rebuild the store: settings, shapes and, per
+        handle, the entropy-coded exponent container and the packed
+        sign|mantissa stream as CPU uint8 tensors.  Plain containers and tensors
+        only, so ``torch.save`` / ``torch.load(weights_only=True)`` round-trip it."""
+        if isinstance(self._be, _DenseBackend):
+            raise RuntimeError("the dummy backend holds dense tensors: save the model's own state_dict")
+        entries = {}
+        for handle, shape in self.meta_dict.items():
+            comp, packed = self._be.export(handle)
+            entries[handle] = {"shape": [int(d) for d in shape], "container": comp, "packed": packed}
+        return {"neuzip_amd_format": _lib.load().nz_abi_version(), **self._settings, "entries": entries}
+
+    def load_state_dict(self, state: dict) -> None:
+        """Replace (or add) the entries named in ``state``; handles keep their
+        names, so the ``Parameter`` objects of a converted model see the loaded
+        weights.  Settings must match the manager's."""
+        if state.get("neuzip_amd_format") != _lib.load().nz_abi_version():
+            raise RuntimeError("checkpoint was written with another container format version")
+        for key, mine in self._settings.items():
+            if state.get(key) != mine:
+                raise RuntimeError(f"checkpoint has {key}={state.get(key)}, this manager {key}={mine}")
+        for handle, ent in state["entries"].items():
+            shape = torch.Size(ent["shape"])
+            self._be.import_(handle, ent["container"], ent["packed"])
+            if self._be.numel(handle) != shape.numel():
+                raise RuntimeError(f"entry {handle!r}: shape {tuple(shape)} does not match the stored element count")
+            self.meta_dict[handle] = shape
+
+    def save(self, path) -> None:
+        torch.save(self.state_dict(), path)
+
+    def load(self, path) -> None:
+        self.load_state_dict(torch.load(path, map_location="cpu", weights_only=True))
 
     # -- helpers -------------------------------------------------------------
     def convert(self, module: torch.nn.Module) -> torch.nn.Module:

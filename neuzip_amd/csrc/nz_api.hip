@@ -636,6 +636,91 @@ int nz_manager_buffers(nz_manager* m, const char* name, const void** dev_comp, u
   return NZ_OK;
 }
 
+int nz_manager_export(nz_manager* m, const char* name, void* host_comp, uint64_t comp_cap,
+                      void* host_packed, uint64_t packed_cap, void* stream) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  hipStream_t st = (hipStream_t)stream;
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  const Entry& ent = it->second;
+  if (comp_cap < ent.comp_bytes || packed_cap < ent.packed_bytes)
+    return fail(NZ_ERR_CAPACITY, "host buffers smaller than the stored streams");
+  if ((ent.comp_bytes && !host_comp) || (ent.packed_bytes && !host_packed))
+    return fail(NZ_ERR_ARG, "null host buffer");
+  if (ent.comp_bytes) NZ_HIP(hipMemcpyAsync(host_comp, ent.comp, ent.comp_bytes, hipMemcpyDeviceToHost, st));
+  if (ent.packed_bytes)
+    NZ_HIP(hipMemcpyAsync(host_packed, ent.packed, ent.packed_bytes, hipMemcpyDeviceToHost, st));
+  NZ_HIP(hipStreamSynchronize(st));
+  return NZ_OK;
+}
+
+int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, uint64_t comp_bytes,
+                      const void* host_packed, uint64_t packed_bytes, void* stream) {
+  if (!m || !name || !host_comp) return fail(NZ_ERR_ARG, "null manager, name or container");
+  hipStream_t st = (hipStream_t)stream;
+  // the container describes itself: check it against this manager before anything is stored
+  if (comp_bytes < NZ_HEADER_BYTES) return fail(NZ_ERR_CORRUPT, "container shorter than its header");
+  uint32_t h[16];
+  std::memcpy(h, host_comp, sizeof(h));
+  if (h[0] != NZ_MAGIC) return fail(NZ_ERR_CORRUPT, "not an exponent container");
+  if (h[1] != NZ_FORMAT_VERSION) return fail(NZ_ERR_CORRUPT, "container of another format version");
+  const uint64_t n = (uint64_t)h[2] | ((uint64_t)h[3] << 32);
+  const uint64_t total = (uint64_t)h[10] | ((uint64_t)h[11] << 32);
+  std::lock_guard<std::mutex> lock(m->mu);
+  if (h[4] != m->chunk_syms) return fail(NZ_ERR_ARG, "container was written with another chunk_size");
+  NzGeom g;
+  if (nz_geom_make(&g, n, h[4], h[5])) return fail(NZ_ERR_CORRUPT, "container header holds an unsupported geometry");
+  if (h[6] != (uint32_t)g.n_chunks || h[7] != (uint32_t)g.n_segs || h[8] != g.dir_off || h[9] != g.rec_off ||
+      total != comp_bytes || total > nz_geom_bound(&g) || total < g.rec_off + NZ_TAIL_PAD)
+    return fail(NZ_ERR_CORRUPT, "container header is inconsistent");
+  if (packed_bytes != nz_packed_stored_bytes_of(&g, m->precision))
+    return fail(NZ_ERR_ARG, "packed stream does not have the size this manager's precision gives");
+  if (packed_bytes && !host_packed) return fail(NZ_ERR_ARG, "null packed stream");
+  // the directory must be non-decreasing and end where the container ends
+  {
+    const uint8_t* c = (const uint8_t*)host_comp;
+    uint32_t prev = 0;
+    for (uint64_t i = 0; i <= g.n_segs; ++i) {
+      uint32_t v;
+      std::memcpy(&v, c + g.dir_off + 4 * i, 4);
+      if (v < prev) return fail(NZ_ERR_CORRUPT, "container directory is not monotone");
+      prev = v;
+    }
+    if (g.rec_off + 4 * (uint64_t)prev + NZ_TAIL_PAD != total)
+      return fail(NZ_ERR_CORRUPT, "container directory does not match its size");
+  }
+  Entry ent;
+  ent.n = n;
+  ent.dtype = NZ_DTYPE_BF16;
+  ent.lane_syms = h[5];
+  ent.comp_bytes = ent.comp_cap = comp_bytes;
+  ent.packed_bytes = packed_bytes;
+  ent.packed_cap = packed_bytes + 16;  // never a zero-byte allocation; the slack is zeroed
+  hipError_t e = hipMalloc(&ent.comp, ent.comp_cap);
+  if (e == hipSuccess) e = hipMalloc(&ent.packed, ent.packed_cap);
+  if (e == hipSuccess) e = hipMemcpyAsync(ent.comp, host_comp, comp_bytes, hipMemcpyHostToDevice, st);
+  if (e == hipSuccess && packed_bytes)
+    e = hipMemcpyAsync(ent.packed, host_packed, packed_bytes, hipMemcpyHostToDevice, st);
+  if (e == hipSuccess) e = hipMemsetAsync((uint8_t*)ent.packed + packed_bytes, 0, 16, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);  // the host buffers are the caller's again
+  if (e != hipSuccess) {
+    if (ent.comp) (void)hipFree(ent.comp);
+    if (ent.packed) (void)hipFree(ent.packed);
+    return fail(NZ_ERR_HIP, std::string("import: ") + hipGetErrorString(e));
+  }
+  auto it = m->entries.find(name);
+  if (it != m->entries.end()) {
+    // kernels reading the old buffers may still be in flight
+    (void)hipDeviceSynchronize();
+    if (it->second.comp) (void)hipFree(it->second.comp);
+    if (it->second.packed) (void)hipFree(it->second.packed);
+    m->entries.erase(it);
+  }
+  m->entries.emplace(name, ent);
+  return NZ_OK;
+}
+
 int nz_manager_erase(nz_manager* m, const char* name) {
   if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
   std::lock_guard<std::mutex> lock(m->mu);

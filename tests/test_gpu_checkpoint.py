@@ -1,0 +1,118 @@
+"""Saving and restoring the compressed store (export / import through the C ABI)."""
+import numpy as np
+import pytest
+
+from conftest import bf16_bits_normal, closed_form_recon, stress_bits
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def _tensor(bits, shape):
+    return torch.from_numpy(bits.view(np.int16).copy()).cuda().view(torch.bfloat16).view(shape)
+
+
+@pytest.mark.parametrize("precision,lane", [(7, 0), (3, "auto"), (0, 128)])
+def test_state_dict_round_trip(tmp_path, oracle, precision, lane):
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=precision, lane_symbols=lane)
+    shapes = [(300, 1000), (1,), (0,), (65536,), (17, 4099)]
+    bits = [stress_bits(1, int(np.prod(s)), seed=i) if i % 2 else bf16_bits_normal(int(np.prod(s)), seed=i)
+            for i, s in enumerate(shapes)]
+    hs = [mgr.write(_tensor(b, s)) for b, s in zip(bits, shapes)]
+    hs.append(mgr.write(_tensor(bits[0], shapes[0]), "named.weight"))
+    path = tmp_path / "store.pt"
+    mgr.save(path)
+    # what was exported is what the oracle writes for the same input
+    sd = mgr.state_dict()
+    lane0 = 344 if lane == 0 else (128 if lane == 128 else None)
+    if lane0:
+        o_comp, o_packed = oracle.compress_bf16(bits[0], precision, 65536, lane0)
+        assert np.array_equal(sd["entries"][hs[0]]["container"].numpy(), o_comp)
+        assert np.array_equal(sd["entries"][hs[0]]["packed"].numpy(), o_packed)
+
+    other = neuzip_amd.Manager(precision=precision, lane_symbols=lane)
+    other.write(torch.zeros(5, dtype=torch.bfloat16, device="cuda"), hs[0])  # replaced by the load
+    other.load(path)
+    for h, b, s in zip(hs, bits + [bits[0]], shapes + [shapes[0]]):
+        got = other.read(h)
+        assert got.shape == torch.Size(s)
+        assert np.array_equal(got.view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1),
+                              closed_form_recon(b, precision))
+        assert other.size(h) == mgr.size(h)
+    other._be.check()
+
+
+def test_load_rejects_what_does_not_fit():
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=7)
+    w = _tensor(bf16_bits_normal(200_000, 1), (200_000,))
+    h = mgr.write(w)
+    sd = mgr.state_dict()
+
+    with pytest.raises(RuntimeError, match="precision"):
+        neuzip_amd.Manager(precision=3).load_state_dict(sd)
+    with pytest.raises(RuntimeError, match="chunk_size"):
+        neuzip_amd.Manager(chunk_size=32768).load_state_dict(sd)
+
+    target = neuzip_amd.Manager(precision=7)  # keep the manager alive: its backend closes with it
+    be = target._be
+    comp, packed = sd["entries"][h]["container"], sd["entries"][h]["packed"]
+    for name, c, p in (
+        ("magic", torch.cat([torch.zeros(4, dtype=torch.uint8), comp[4:]]), packed),
+        ("short", comp[:-4], packed),
+        ("packed size", comp, packed[:-1]),
+        ("header only", comp[:64], packed),
+    ):
+        print("case", name, flush=True)
+        with pytest.raises((RuntimeError, ValueError)) as err:
+            be.import_("x", c, p)
+        assert "null manager" not in str(err.value)
+        assert be.size("x") == 0  # nothing was stored
+    # element count in the header changed: geometry no longer matches directory and sizes
+    bad = comp.clone()
+    bad[8] = (int(bad[8]) + 1) & 0xFF
+    with pytest.raises((RuntimeError, ValueError)):
+        be.import_("x", bad, packed)
+    # a damaged record passes the header checks and is reported by the decoder
+    bad = comp.clone()
+    bad[comp.numel() // 2] ^= 0x5A
+    be.import_("y", bad, packed)
+    out = be.read("y")
+    torch.cuda.synchronize()
+    ok = torch.equal(out, w)
+    try:
+        be.check()
+        flagged = False
+    except RuntimeError:
+        flagged = True
+    assert flagged or not ok
+
+
+def test_converted_model_resumes_from_checkpoint(tmp_path):
+    import neuzip_amd
+
+    def build(seed):
+        torch.manual_seed(seed)
+        m = torch.nn.Sequential(torch.nn.Linear(256, 512), torch.nn.GELU(), torch.nn.Linear(512, 256)).to(torch.bfloat16)
+        mgr = neuzip_amd.Manager()
+        mgr.convert(m)
+        return mgr, m.cuda()
+
+    mgr, model = build(1)
+    x = torch.randn(4, 256, device="cuda", dtype=torch.bfloat16)
+    with torch.no_grad():
+        want = model(x)
+    mgr.save(tmp_path / "w.pt")
+    torch.save(model.state_dict(), tmp_path / "m.pt")  # biases; the compressed weights are 0-size here
+
+    mgr2, model2 = build(2)  # other random weights under the same handles
+    with torch.no_grad():
+        assert not torch.equal(model2(x), want)
+    mgr2.load(tmp_path / "w.pt")
+    model2.load_state_dict(torch.load(tmp_path / "m.pt", weights_only=True))
+    with torch.no_grad():
+        assert torch.equal(model2(x), want)
