@@ -116,6 +116,62 @@ void nzo_merge_bf16_float(const uint8_t* exponents, const uint8_t* fractions, ui
   }
 }
 
+/* ---- block normalizers: kernels.cuh:94-118 (split side), :208-216 (merge side) ----
+ *
+ * Group j holds the elements [j*norm_size, (j+1)*norm_size) of the flat tensor.
+ *   split: absmax = max |float(x)| over the group (:97-100; elements past the end
+ *          count as 0, :92); fraction = the 23 mantissa bits of absmax (:104,
+ *          _float_to_fraction :36-38); every element is divided by the float
+ *          1.fraction (:108-112, _fraction_to_base_float :31-34) and cast back
+ *          to bf16, round to nearest even; the group stores fraction >> 15
+ *          (:116).  A bf16 absmax has 7 mantissa bits, so the stored byte loses
+ *          nothing: byte = mantissa << 1.
+ *   merge: out = bf16( 1.(byte << 15) * float(value) * +-1 )  (:208-216).
+ * The reference reduces with cub::BlockReduce<float, norm_size> inside a block of
+ * 1024 threads, which is only well defined for norm_size == 1024; for the other
+ * sizes this restates the intended group-wise maximum.  NaN inputs: the order of
+ * a float max with NaN operands is unspecified there -> PARITY UNPINNED; here the
+ * maximum is taken over the 15-bit magnitude patterns.
+ */
+static inline uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u = float_to_bits(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+size_t nzo_norm_count(uint64_t n, uint32_t norm_size) {
+  return norm_size ? (size_t)((n + norm_size - 1) / norm_size) : 0;
+}
+
+void nzo_block_normalize(const uint16_t* data, uint64_t n, uint32_t norm_size, uint8_t* norm_bytes,
+                         uint16_t* scaled) {
+  for (uint64_t g0 = 0; g0 < n; g0 += norm_size) {
+    uint64_t g1 = g0 + norm_size < n ? g0 + norm_size : n;
+    uint32_t amax = 0; /* bit pattern of |x|: ordered like the value for non-NaN */
+    for (uint64_t i = g0; i < g1; ++i) {
+      uint32_t a = data[i] & 0x7FFFu;
+      if (a > amax) amax = a;
+    }
+    uint32_t fraction = float_to_bits(bits_to_float(amax << 16)) & 0x7FFFFFu; /* :36-38 */
+    float base = bits_to_float((0x7Fu << 23) | fraction);                      /* :31-34 */
+    norm_bytes[g0 / norm_size] = (uint8_t)(fraction >> (23 - 8));              /* :116 */
+    for (uint64_t i = g0; i < g1; ++i) {
+      float x = bits_to_float((uint32_t)data[i] << 16);
+      scaled[i] = f32_to_bf16_rne(x / base); /* :111-112 */
+    }
+  }
+}
+
+void nzo_block_denormalize(const uint16_t* scaled, uint64_t n, uint32_t norm_size,
+                           const uint8_t* norm_bytes, uint16_t* data) {
+  for (uint64_t i = 0; i < n; ++i) {
+    float base = bits_to_float((0x7Fu << 23) | ((uint32_t)norm_bytes[i / norm_size] << (23 - 8)));
+    uint16_t v = scaled[i];
+    float mag = bits_to_float((uint32_t)(v & 0x7FFFu) << 16);
+    data[i] = f32_to_bf16_rne(base * mag * ((v >> 15) ? -1.0f : 1.0f)); /* :213-216 */
+  }
+}
+
 uint16_t nzo_recon_closed_form(uint16_t v, int s) {
   /* Independent statement of merge(split(v)): round-half-up of the 15-bit
      magnitude to a multiple of 2^(7-s), wrapping modulo 2^15. */

@@ -18,6 +18,12 @@
  *     which canonicalises NaN payloads in a way that depends on the device
  *     conversion routine -> the exact NaN bit pattern is PARITY UNPINNED.
  *
+ *     nzo_block_normalize / nzo_block_denormalize restate the block-normalizer
+ *     path (kernels.cuh:94-118, 208-216).  Pinned by an exact rational-arithmetic
+ *     model of "divide, round to nearest even" over all mantissa pairs and by
+ *     the invariants in the tests; NaN inputs and the reference's behaviour for
+ *     group sizes other than 1024 are PARITY UNPINNED (see the source).
+ *
  *  2. nzo_exp_* is the chunked, 64-way lane-interleaved rANS container that
  *     replaces the closed-source nvcomp ANS call sites
  *        cuda/high_level.cu:103-124 (compress) and :184-192 (decompress).
@@ -61,6 +67,12 @@ void nzo_merge_bf16(const uint8_t* exponents, const uint8_t* fractions, uint64_t
 void nzo_merge_bf16_float(const uint8_t* exponents, const uint8_t* fractions, uint64_t n, int s,
                           uint16_t* data);
 uint16_t nzo_recon_closed_form(uint16_t v, int s);
+/* block normalizers (kernels.cuh:94-118, 208-216): one byte per group of norm_size elements */
+size_t nzo_norm_count(uint64_t n, uint32_t norm_size);
+void nzo_block_normalize(const uint16_t* data, uint64_t n, uint32_t norm_size, uint8_t* norm_bytes,
+                         uint16_t* scaled);
+void nzo_block_denormalize(const uint16_t* scaled, uint64_t n, uint32_t norm_size,
+                           const uint8_t* norm_bytes, uint16_t* data);
 
 /* ---- frequency tables ---- */
 int nzo_normalize_freqs(const uint32_t cnt[256], uint64_t n, uint16_t freq[256]);

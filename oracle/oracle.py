@@ -48,6 +48,12 @@ def lib() -> ctypes.CDLL:
         L.nzo_merge_bf16_float.argtypes = [u8p, u8p, ctypes.c_uint64, ctypes.c_int, u16p]
         L.nzo_recon_closed_form.restype = ctypes.c_uint16
         L.nzo_recon_closed_form.argtypes = [ctypes.c_uint16, ctypes.c_int]
+        L.nzo_norm_count.restype = ctypes.c_size_t
+        L.nzo_norm_count.argtypes = [ctypes.c_uint64, ctypes.c_uint32]
+        L.nzo_block_normalize.restype = None
+        L.nzo_block_normalize.argtypes = [u16p, ctypes.c_uint64, ctypes.c_uint32, u8p, u16p]
+        L.nzo_block_denormalize.restype = None
+        L.nzo_block_denormalize.argtypes = [u16p, ctypes.c_uint64, ctypes.c_uint32, u8p, u16p]
         L.nzo_normalize_freqs.restype = ctypes.c_int
         L.nzo_normalize_freqs.argtypes = [u32p, ctypes.c_uint64, u16p]
         L.nzo_table_serialize.restype = ctypes.c_size_t
@@ -119,6 +125,35 @@ def reconstruct(bits: np.ndarray, s: int) -> np.ndarray:
     """merge(split(x)) — the tensor the reference would hand back for x."""
     e, f = split(bits, s)
     return merge(e, f, s)
+
+
+def block_normalize(bits: np.ndarray, norm_size: int):
+    """-> (one byte per group of norm_size elements, the normalized tensor as bf16 bits)"""
+    bits = _u16(bits)
+    n = bits.size
+    norm = np.zeros(lib().nzo_norm_count(n, norm_size), np.uint8)
+    scaled = np.empty(n, np.uint16)
+    if n:
+        lib().nzo_block_normalize(_p(bits, ctypes.c_uint16), n, norm_size, _p(norm, ctypes.c_uint8),
+                                  _p(scaled, ctypes.c_uint16))
+    return norm, scaled
+
+
+def block_denormalize(scaled: np.ndarray, norm_size: int, norm: np.ndarray) -> np.ndarray:
+    scaled, norm = _u16(scaled), _u8(norm)
+    out = np.empty(scaled.size, np.uint16)
+    if scaled.size:
+        lib().nzo_block_denormalize(_p(scaled, ctypes.c_uint16), scaled.size, norm_size,
+                                    _p(norm, ctypes.c_uint8), _p(out, ctypes.c_uint16))
+    return out
+
+
+def reconstruct_normalized(bits: np.ndarray, s: int, norm_size: int) -> np.ndarray:
+    """What the reference hands back for x with block normalizers of norm_size."""
+    if not norm_size:
+        return reconstruct(bits, s)
+    norm, scaled = block_normalize(bits, norm_size)
+    return block_denormalize(reconstruct(scaled, s), norm_size, norm)
 
 
 def recon_closed_form(v: int, s: int) -> int:
