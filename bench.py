@@ -97,7 +97,7 @@ class Codec:
         rc = self.L.nz_encode(dense.data_ptr(), self.n, self.s, self.chunk, self.lane,
                               self.packed.data_ptr(), self.comp.data_ptr(), self.cap,
                               self.ws.data_ptr(), self.ws_bytes, self.aux.data_ptr(),
-                              self.aux.data_ptr() + 8, ctypes.byref(total) if sync else None, st)
+                              self.aux.data_ptr() + 8, ctypes.byref(total) if sync else None, 0, None, st)
         if rc != 0:
             raise RuntimeError(self.m.last_error())
         if sync:
@@ -107,7 +107,7 @@ class Codec:
         st = self.torch.cuda.current_stream().cuda_stream
         rc = self.L.nz_decode(self.comp.data_ptr(), self.total, self.packed.data_ptr(), self.n,
                               self.s, self.chunk, self.lane, out.data_ptr(), self.status.data_ptr(),
-                              1 if check else 0, st)
+                              1 if check else 0, 0, None, st)
         if rc != 0:
             raise RuntimeError(self.m.last_error())
 

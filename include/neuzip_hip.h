@@ -74,12 +74,26 @@ uint64_t nz_exp_bound_bytes(uint64_t n, uint32_t chunk_size, uint32_t lane_syms)
 /* Device scratch needed by nz_encode for n elements. */
 uint64_t nz_encode_workspace_bytes(uint64_t n, uint32_t chunk_size, uint32_t lane_syms);
 
+/* Bytes of the block-normalizer array of n elements: one byte per group of
+   `normalizer_size` consecutive elements (cuda/high_level.cu:89-93), 0 without
+   normalizers.  normalizer_size is 0 or a power of two up to 1024, the sizes
+   cuda/neuzip.cu:47-105 instantiates. */
+uint64_t nz_norm_bytes(uint64_t n, uint32_t normalizer_size);
+
 /* ---- stateless kernels ------------------------------------------------ */
 
+/* Block normalizers (cuda/kernels.cuh:94-118 and :208-216) are part of the
+   three calls below: with normalizer_size > 0 every group of that many elements
+   is divided by 1.m before the split (m = the mantissa of the group's largest
+   magnitude; the byte m << 1 goes to dev_norm, nz_norm_bytes() bytes, 8-byte
+   aligned) and multiplied by it after the merge, both rounded to bf16.  With
+   normalizer_size == 0 dev_norm is ignored. */
+
 /* Manager::split, cuda/high_level.cu:265-321: unpacked exponent byte and
-   sign|mantissa byte per element, precision forced to 7 (:289). */
+   sign|mantissa byte per element, precision forced to 7 (:289).  dev_norm is
+   scratch here (the reference drops the bytes, :282-296). */
 int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fractions,
-             void* stream);
+             uint32_t normalizer_size, void* dev_norm, void* stream);
 
 /* Manager::_write_to_cache, cuda/high_level.cu:76-130: split, then entropy
    code the exponents.  `dev_packed` receives nz_packed_stored_bytes() bytes,
@@ -91,7 +105,8 @@ int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fr
 int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
               uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
               void* dev_workspace, uint64_t workspace_bytes, uint64_t* dev_total,
-              uint32_t* dev_status, uint64_t* host_total, void* stream);
+              uint32_t* dev_status, uint64_t* host_total, uint32_t normalizer_size, void* dev_norm,
+              void* stream);
 
 /* Manager::_decompress_and_merge, cuda/high_level.cu:169-206: entropy decode
    and merge in one kernel.  `dev_status` (device uint32, may be NULL) is
@@ -100,13 +115,14 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
    case.  chunk_size / lane_syms must be the ones used to encode. */
 int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed, uint64_t n,
               int precision, uint32_t chunk_size, uint32_t lane_syms, void* dev_bf16_out,
-              uint32_t* dev_status, int check, void* stream);
+              uint32_t* dev_status, int check, uint32_t normalizer_size, const void* dev_norm,
+              void* stream);
 
 /* ---- handle store: template struct Manager, cuda/high_level.cu:26-322 -- */
 
 /* Manager(algorithm, chunk_size) for the class Manager_f{precision}_n{normalizer_size}
    (cuda/neuzip.cu:19-38, neuzip/binding.py:69-70).  precision in {0,1,3,7};
-   normalizer_size must be 0 (block normalizers are not implemented);
+   normalizer_size 0 or a power of two up to 1024 (block normalizers, see above);
    lane_syms 0 selects NZ_DEFAULT_LANE_SYMS clipped to the chunk;
    NZ_LANE_SYMS_AUTO shortens the segments of tensors too small to fill the GPU
    at the default (more wavefronts, ~4.5 bits of container per extra lane). */
@@ -156,19 +172,21 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
 int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype);
 
 /* Manager::size(name), cuda/high_level.cu:208-221: bytes held for the entry
-   (entropy-coded exponents + packed sign/mantissa); 0 if unknown. */
+   (entropy-coded exponents + packed sign/mantissa + normalizer bytes of a
+   manager with normalizer_size > 0); 0 if unknown. */
 uint64_t nz_manager_size(nz_manager* m, const char* name);
 
 /* Bytes of the exponent container alone / of the packed stream alone. */
 uint64_t nz_manager_exp_bytes(nz_manager* m, const char* name);
 uint64_t nz_manager_packed_bytes(nz_manager* m, const char* name);
+uint64_t nz_manager_norm_bytes(nz_manager* m, const char* name); /* normalizer bytes, counted in size */
 
 /* Raw device pointers of an entry (valid until it is rewritten or erased). */
 int nz_manager_buffers(nz_manager* m, const char* name, const void** dev_comp,
                        uint64_t* comp_bytes, const void** dev_packed, uint64_t* packed_bytes);
 
-/* Copy an entry's two streams to host memory (sizes from nz_manager_exp_bytes /
-   nz_manager_packed_bytes) and back.  The reference keeps compressed tensors
+/* Copy an entry's streams (container, packed, normalizer bytes) to host memory
+   (sizes from nz_manager_exp_bytes / _packed_bytes / _norm_bytes) and back.  The reference keeps compressed tensors
    only inside the process (cuda/high_level.cu:35-43; neuzip/nn/module.py:13
    leaves 0-size parameters in a state_dict), so a converted model cannot be
    checkpointed there; these two calls are what a save/load needs.  The
@@ -176,9 +194,11 @@ int nz_manager_buffers(nz_manager* m, const char* name, const void** dev_comp,
    directory and sizes against the manager (chunk_size, precision) and stores
    nothing when they disagree.  Both calls block until the copies are done. */
 int nz_manager_export(nz_manager* m, const char* name, void* host_comp, uint64_t comp_cap,
-                      void* host_packed, uint64_t packed_cap, void* stream);
+                      void* host_packed, uint64_t packed_cap, void* host_norm, uint64_t norm_cap,
+                      void* stream);
 int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, uint64_t comp_bytes,
-                      const void* host_packed, uint64_t packed_bytes, void* stream);
+                      const void* host_packed, uint64_t packed_bytes, const void* host_norm,
+                      uint64_t norm_bytes, void* stream);
 
 /* compress_cache.erase(name), cuda/high_level.cu:137-140. */
 int nz_manager_erase(nz_manager* m, const char* name);

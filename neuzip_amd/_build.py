@@ -16,6 +16,11 @@ HIPCC_FLAGS = [
     "-shared",
     # packed-FP32 VALU forms are kept out of every code object built here
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the block-normalizer arithmetic must round like IEEE fp32 (exact division,
+    # gradual underflow), whatever the compiler's defaults are
+    "-fhip-fp32-correctly-rounded-divide-sqrt",
+    "-fno-gpu-flush-denormals-to-zero",
+    "-ffp-contract=off",
 ]
 
 

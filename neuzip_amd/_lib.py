@@ -24,10 +24,10 @@ LANE_SYMS_AUTO = 0xFFFFFFFF
 
 EXPORTS = [
     "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",
-    "nz_encode_workspace_bytes", "nz_split", "nz_encode", "nz_decode",
+    "nz_encode_workspace_bytes", "nz_norm_bytes", "nz_split", "nz_encode", "nz_decode",
     "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch",
     "nz_manager_meta", "nz_manager_size", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
-    "nz_manager_buffers", "nz_manager_erase", "nz_manager_check", "nz_manager_export", "nz_manager_import",
+    "nz_manager_norm_bytes", "nz_manager_buffers", "nz_manager_erase", "nz_manager_check", "nz_manager_export", "nz_manager_import",
 ]
 
 _lib = None
@@ -58,12 +58,14 @@ def load() -> ctypes.CDLL:
     L.nz_encode_workspace_bytes.restype = u64
     L.nz_encode_workspace_bytes.argtypes = [u64, u32, u32]
     L.nz_split.restype = i32
-    L.nz_split.argtypes = [vp, u64, vp, vp, vp]
+    L.nz_norm_bytes.restype = u64
+    L.nz_norm_bytes.argtypes = [u64, u32]
+    L.nz_split.argtypes = [vp, u64, vp, vp, u32, vp, vp]
     L.nz_encode.restype = i32
     L.nz_encode.argtypes = [vp, u64, i32, u32, u32, vp, vp, u64, vp, u64, vp, vp,
-                            ctypes.POINTER(u64), vp]
+                            ctypes.POINTER(u64), u32, vp, vp]
     L.nz_decode.restype = i32
-    L.nz_decode.argtypes = [vp, u64, vp, u64, i32, u32, u32, vp, vp, i32, vp]
+    L.nz_decode.argtypes = [vp, u64, vp, u64, i32, u32, u32, vp, vp, i32, u32, vp, vp]
     L.nz_manager_create.restype = i32
     L.nz_manager_create.argtypes = [i32, i32, i32, u32, u32, ctypes.POINTER(vp)]
     L.nz_manager_destroy.restype = None
@@ -73,9 +75,9 @@ def load() -> ctypes.CDLL:
     L.nz_manager_read.restype = i32
     L.nz_manager_read.argtypes = [vp, ctypes.c_char_p, vp, u64, vp]
     L.nz_manager_export.restype = i32
-    L.nz_manager_export.argtypes = [vp, ctypes.c_char_p, vp, u64, vp, u64, vp]
+    L.nz_manager_export.argtypes = [vp, ctypes.c_char_p, vp, u64, vp, u64, vp, u64, vp]
     L.nz_manager_import.restype = i32
-    L.nz_manager_import.argtypes = [vp, ctypes.c_char_p, vp, u64, vp, u64, vp]
+    L.nz_manager_import.argtypes = [vp, ctypes.c_char_p, vp, u64, vp, u64, vp, u64, vp]
     L.nz_manager_gemv_batch.restype = i32
     L.nz_manager_gemv_batch.argtypes = [vp, ctypes.POINTER(ctypes.c_char_p), u32, vp, u32, ctypes.POINTER(vp),
                                         ctypes.POINTER(vp), vp]
@@ -84,7 +86,7 @@ def load() -> ctypes.CDLL:
                                         ctypes.POINTER(u64), u32, vp]
     L.nz_manager_meta.restype = i32
     L.nz_manager_meta.argtypes = [vp, ctypes.c_char_p, ctypes.POINTER(u64), ctypes.POINTER(i32)]
-    for name in ("nz_manager_size", "nz_manager_exp_bytes", "nz_manager_packed_bytes"):
+    for name in ("nz_manager_size", "nz_manager_exp_bytes", "nz_manager_packed_bytes", "nz_manager_norm_bytes"):
         fn = getattr(L, name)
         fn.restype = u64
         fn.argtypes = [vp, ctypes.c_char_p]

@@ -47,6 +47,7 @@ class _HipBackend:
                                        lane_symbols, ctypes.byref(self._h))
         _lib.raise_for(rc)
         self._device = torch.device("cuda", torch.cuda.current_device())
+        self._normalizer = int(normalizer_size)
         self._known = {}  # handle -> (encoded name, element count), dropped on write
 
     def close(self):
@@ -144,24 +145,28 @@ class _HipBackend:
         _lib.raise_for(rc)
 
     def export(self, handle: str):
-        """The two stored streams of an entry as CPU uint8 tensors (container, packed)."""
+        """The stored streams of an entry as CPU uint8 tensors (container, packed, normalizer bytes)."""
         name = handle.encode()
         if self._L.nz_manager_meta(self._h, name, None, None):
             _lib.raise_for(_lib.ERR_NOT_FOUND)
         comp = torch.empty(self.exp_bytes(handle), dtype=torch.uint8)
         packed = torch.empty(self.packed_bytes(handle), dtype=torch.uint8)
+        norm = torch.empty(int(self._L.nz_manager_norm_bytes(self._h, name)), dtype=torch.uint8)
         rc = self._L.nz_manager_export(self._h, name, comp.data_ptr(), comp.numel(), packed.data_ptr(),
-                                       packed.numel(), _stream_ptr(self._device))
+                                       packed.numel(), norm.data_ptr() if norm.numel() else None, norm.numel(),
+                                       _stream_ptr(self._device))
         _lib.raise_for(rc)
-        return comp, packed
+        return comp, packed, norm
 
-    def import_(self, handle: str, comp: torch.Tensor, packed: torch.Tensor) -> None:
+    def import_(self, handle: str, comp: torch.Tensor, packed: torch.Tensor, norm: torch.Tensor = None) -> None:
         """Store streams produced by :meth:`export` (checked against this manager's settings)."""
         comp = comp.detach().to("cpu", torch.uint8).contiguous()
         packed = packed.detach().to("cpu", torch.uint8).contiguous()
+        norm = torch.empty(0, dtype=torch.uint8) if norm is None else norm.detach().to("cpu", torch.uint8).contiguous()
         self._known.pop(handle, None)
         rc = self._L.nz_manager_import(self._h, handle.encode(), comp.data_ptr(), comp.numel(),
                                        packed.data_ptr() if packed.numel() else None, packed.numel(),
+                                       norm.data_ptr() if norm.numel() else None, norm.numel(),
                                        _stream_ptr(self._device))
         _lib.raise_for(rc)
 
@@ -201,7 +206,11 @@ class _HipBackend:
         n = flat.numel()
         exps = torch.empty(n, dtype=torch.uint8, device=flat.device)
         fracs = torch.empty(n, dtype=torch.uint8, device=flat.device)
-        rc = self._L.nz_split(flat.data_ptr(), n, exps.data_ptr(), fracs.data_ptr(), _stream_ptr(flat.device))
+        norm = None
+        if self._normalizer:  # scratch: the reference computes the group bytes and drops them (high_level.cu:282-296)
+            norm = torch.empty(self._L.nz_norm_bytes(n, self._normalizer) + 8, dtype=torch.uint8, device=flat.device)
+        rc = self._L.nz_split(flat.data_ptr(), n, exps.data_ptr(), fracs.data_ptr(), self._normalizer,
+                              norm.data_ptr() if norm is not None else None, _stream_ptr(flat.device))
         _lib.raise_for(rc)
         return [exps, fracs]
 
@@ -269,8 +278,6 @@ class Manager:
             raise AttributeError(
                 f"module 'neuzip._cuda' has no attribute 'Manager_f{precision}_n{normalizer_size}'"
             )
-        if normalizer_size != 0:
-            raise NotImplementedError("block normalizers (normalizer_size > 0) are not implemented")
         self._be = _HipBackend(precision, normalizer_size, chunk_size, lane_symbols)
         self._settings = {"precision": int(precision), "normalizer_size": int(normalizer_size),
                           "chunk_size": int(chunk_size)}
@@ -307,8 +314,9 @@ class Manager:
             raise RuntimeError("the dummy backend holds dense tensors: save the model's own state_dict")
         entries = {}
         for handle, shape in self.meta_dict.items():
-            comp, packed = self._be.export(handle)
-            entries[handle] = {"shape": [int(d) for d in shape], "container": comp, "packed": packed}
+            comp, packed, norm = self._be.export(handle)
+            entries[handle] = {"shape": [int(d) for d in shape], "container": comp, "packed": packed,
+                               "normalizers": norm}
         return {"neuzip_amd_format": _lib.load().nz_abi_version(), **self._settings, "entries": entries}
 
     def load_state_dict(self, state: dict) -> None:
@@ -322,7 +330,7 @@ class Manager:
                 raise RuntimeError(f"checkpoint has {key}={state.get(key)}, this manager {key}={mine}")
         for handle, ent in state["entries"].items():
             shape = torch.Size(ent["shape"])
-            self._be.import_(handle, ent["container"], ent["packed"])
+            self._be.import_(handle, ent["container"], ent["packed"], ent.get("normalizers"))
             if self._be.numel(handle) != shape.numel():
                 raise RuntimeError(f"entry {handle!r}: shape {tuple(shape)} does not match the stored element count")
             self.meta_dict[handle] = shape

@@ -33,6 +33,15 @@ inline uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
 bool precision_ok(int p) { return p == 7 || p == 3 || p == 1 || p == 0; }
 
+// group sizes the reference instantiates (cuda/neuzip.cu:47-105): 0 = off, else a power of two up to 1024
+bool normalizer_ok(uint32_t ns) { return ns == 0 || (ns <= 1024 && (ns & (ns - 1)) == 0); }
+uint32_t log2_of(uint32_t v) {
+  uint32_t l = 0;
+  while ((1u << l) < v) ++l;
+  return l;
+}
+uint64_t norm_bytes_of(uint64_t n, uint32_t ns) { return ns ? (n + ns - 1) / ns : 0; }
+
 // Device scratch of one encode call.
 struct EncLayout {
   uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, hdr, total, status, bytes;
@@ -65,24 +74,35 @@ EncLayout enc_layout(const NzGeom& g) {
 
 template <int S>
 void launch_split_hist(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws,
-                       const EncLayout& L, hipStream_t st) {
+                       const EncLayout& L, const NzNorm& nm, hipStream_t st) {
   hipLaunchKernelGGL(nz_split_hist_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(NZ_SPLIT_THREADS), 0, st,
                      (const uint16_t*)in, g.n, g.chunk_syms, g.seg_syms, g.spc, packed, ws + L.carry,
                      ws + L.exps, (uint32_t*)(ws + L.enc_tab), ws + L.tab_ser,
-                     (NzChunkInfo*)(ws + L.info));
+                     (NzChunkInfo*)(ws + L.info), nm);
+}
+
+// group bytes of a tensor that is about to be split (nothing to do without normalizers)
+int launch_absmax(const void* in, uint64_t n, uint32_t ns, uint8_t* norm, hipStream_t st) {
+  if (!ns || !n) return NZ_OK;
+  hipLaunchKernelGGL(nz_absmax_kernel, dim3((uint32_t)((n + 2047) / 2048)), dim3(256), 0, st,
+                     (const uint16_t*)in, n, log2_of(ns), norm);
+  NZ_HIP(hipGetLastError());
+  return NZ_OK;
 }
 
 // Phase 1: everything up to the directory.  Header + directory land in `hdr`
 // (g.rec_off bytes), the container size in *d_total.
 int encode_phase1(const NzGeom& g, int precision, const void* in, uint8_t* packed, uint8_t* ws,
                   const EncLayout& L, uint8_t* hdr, uint64_t cap, uint64_t* d_total,
-                  uint32_t* d_status, hipStream_t st) {
+                  uint32_t* d_status, uint32_t ns, uint8_t* norm, hipStream_t st) {
   if (g.n_chunks > 0) {
+    if (int rc = launch_absmax(in, g.n, ns, norm, st)) return rc;
+    const NzNorm nm{ns ? norm : nullptr, log2_of(ns ? ns : 1)};
     switch (precision) {
-      case 7: launch_split_hist<7>(g, in, packed, ws, L, st); break;
-      case 3: launch_split_hist<3>(g, in, packed, ws, L, st); break;
-      case 1: launch_split_hist<1>(g, in, packed, ws, L, st); break;
-      default: launch_split_hist<0>(g, in, packed, ws, L, st); break;
+      case 7: launch_split_hist<7>(g, in, packed, ws, L, nm, st); break;
+      case 3: launch_split_hist<3>(g, in, packed, ws, L, nm, st); break;
+      case 1: launch_split_hist<1>(g, in, packed, ws, L, nm, st); break;
+      default: launch_split_hist<0>(g, in, packed, ws, L, nm, st); break;
     }
     hipLaunchKernelGGL(nz_rans_encode_kernel, dim3((uint32_t)g.n_chunks), dim3(64 * g.spc), 0, st,
                        ws + L.exps, g.n, g.chunk_syms, g.lane_syms, g.spc,
@@ -118,21 +138,27 @@ int encode_phase2(const NzGeom& g, uint8_t* ws, const EncLayout& L, const uint32
 
 template <int S>
 void launch_decode(const NzGeom& g, const void* comp, uint64_t comp_bytes, const void* packed,
-                   void* out, uint32_t* d_status, hipStream_t st) {
+                   void* out, uint32_t* d_status, const NzNorm& nm, hipStream_t st) {
   const size_t lds = (2 * NZ_M + g.spc * NZ_RING_ALLOC_DWORDS) * 4;
-  hipLaunchKernelGGL(nz_decode_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(64 * g.spc), lds, st,
-                     (const uint8_t*)comp, comp_bytes, (const uint8_t*)packed, (uint16_t*)out, g,
-                     d_status);
+  const dim3 gd((uint32_t)g.n_chunks), bd(64 * g.spc);
+  if (nm.bytes)
+    hipLaunchKernelGGL((nz_decode_kernel<S, true>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,
+                       (const uint8_t*)packed, (uint16_t*)out, g, d_status, nm);
+  else
+    hipLaunchKernelGGL((nz_decode_kernel<S, false>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,
+                       (const uint8_t*)packed, (uint16_t*)out, g, d_status, nm);
 }
 
 int decode_launch(const NzGeom& g, int precision, const void* comp, uint64_t comp_bytes,
-                  const void* packed, void* out, uint32_t* d_status, hipStream_t st) {
+                  const void* packed, void* out, uint32_t* d_status, uint32_t ns, const void* norm,
+                  hipStream_t st) {
   if (g.n_chunks == 0) return NZ_OK;
+  const NzNorm nm{ns ? (const uint8_t*)norm : nullptr, log2_of(ns ? ns : 1)};
   switch (precision) {
-    case 7: launch_decode<7>(g, comp, comp_bytes, packed, out, d_status, st); break;
-    case 3: launch_decode<3>(g, comp, comp_bytes, packed, out, d_status, st); break;
-    case 1: launch_decode<1>(g, comp, comp_bytes, packed, out, d_status, st); break;
-    default: launch_decode<0>(g, comp, comp_bytes, packed, out, d_status, st); break;
+    case 7: launch_decode<7>(g, comp, comp_bytes, packed, out, d_status, nm, st); break;
+    case 3: launch_decode<3>(g, comp, comp_bytes, packed, out, d_status, nm, st); break;
+    case 1: launch_decode<1>(g, comp, comp_bytes, packed, out, d_status, nm, st); break;
+    default: launch_decode<0>(g, comp, comp_bytes, packed, out, d_status, nm, st); break;
   }
   NZ_HIP(hipGetLastError());
   return NZ_OK;
@@ -142,7 +168,10 @@ template <int S>
 void launch_decode_batch(const NzBatch& b, uint32_t grid, uint32_t max_spc, uint32_t* d_status,
                          hipStream_t st) {
   const size_t lds = (2 * NZ_M + max_spc * NZ_RING_ALLOC_DWORDS) * 4;
-  hipLaunchKernelGGL(nz_decode_batch_kernel<S>, dim3(grid), dim3(64 * max_spc), lds, st, b, d_status);
+  if (b.item[0].norm)
+    hipLaunchKernelGGL((nz_decode_batch_kernel<S, true>), dim3(grid), dim3(64 * max_spc), lds, st, b, d_status);
+  else
+    hipLaunchKernelGGL((nz_decode_batch_kernel<S, false>), dim3(grid), dim3(64 * max_spc), lds, st, b, d_status);
 }
 
 int decode_batch_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int precision,
@@ -162,12 +191,17 @@ int gemv_launch(const NzBatch& b, const NzGemvOut& o, uint32_t grid, uint32_t ma
                 int precision, uint32_t* d_status, hipStream_t st) {
   const size_t lds = (2 * NZ_M + max_spc * NZ_RING_ALLOC_DWORDS) * 4;
   const dim3 gd(grid), bd(64 * max_spc);
+  const bool nrm = b.item[0].norm != nullptr;
+#define NZ_GEMV_CASE(S)                                                                              \
+  if (nrm) hipLaunchKernelGGL((nz_decode_gemv_kernel<S, true>), gd, bd, lds, st, b, d_status);       \
+  else hipLaunchKernelGGL((nz_decode_gemv_kernel<S, false>), gd, bd, lds, st, b, d_status)
   switch (precision) {
-    case 7: hipLaunchKernelGGL(nz_decode_gemv_kernel<7>, gd, bd, lds, st, b, d_status); break;
-    case 3: hipLaunchKernelGGL(nz_decode_gemv_kernel<3>, gd, bd, lds, st, b, d_status); break;
-    case 1: hipLaunchKernelGGL(nz_decode_gemv_kernel<1>, gd, bd, lds, st, b, d_status); break;
-    default: hipLaunchKernelGGL(nz_decode_gemv_kernel<0>, gd, bd, lds, st, b, d_status); break;
+    case 7: NZ_GEMV_CASE(7); break;
+    case 3: NZ_GEMV_CASE(3); break;
+    case 1: NZ_GEMV_CASE(1); break;
+    default: NZ_GEMV_CASE(0); break;
   }
+#undef NZ_GEMV_CASE
   NZ_HIP(hipGetLastError());
   hipLaunchKernelGGL(nz_gemv_finish_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, o);
   NZ_HIP(hipGetLastError());
@@ -191,12 +225,15 @@ struct Entry {
   uint64_t n = 0;
   int dtype = NZ_DTYPE_BF16;
   uint32_t lane_syms = 0;  // geometry this entry was written with
+  void* norm = nullptr;    // one byte per normalizer group (managers with normalizer_size > 0)
+  uint64_t norm_bytes = 0, norm_cap = 0;
 };
 
 }  // namespace
 
 struct nz_manager {
   int precision;
+  uint32_t normalizer = 0;  // elements per normalizer group, 0 = none
   uint32_t chunk_syms, lane_syms;
   bool auto_lanes = false;  // pick lane_syms per tensor so that small tensors still fill the GPU
   std::unordered_map<std::string, Entry> entries;  // compress_cache + meta_cache
@@ -235,17 +272,26 @@ uint64_t nz_encode_workspace_bytes(uint64_t n, uint32_t chunk_size, uint32_t lan
   return enc_layout(g).bytes;
 }
 
+uint64_t nz_norm_bytes(uint64_t n, uint32_t normalizer_size) {
+  return normalizer_ok(normalizer_size) ? norm_bytes_of(n, normalizer_size) : 0;
+}
+
 int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fractions,
-             void* stream) {
+             uint32_t normalizer_size, void* dev_norm, void* stream) {
+  if (!normalizer_ok(normalizer_size)) return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
   if (n == 0) return NZ_OK;
-  if (!dev_bf16 || !dev_exponents || !dev_fractions) return fail(NZ_ERR_ARG, "null pointer");
+  if (!dev_bf16 || !dev_exponents || !dev_fractions || (normalizer_size && !dev_norm))
+    return fail(NZ_ERR_ARG, "null pointer");
+  if (normalizer_size && ((uintptr_t)dev_norm & 7)) return fail(NZ_ERR_ALIGN, "normalizer bytes must be 8-byte aligned");
   if (((uintptr_t)dev_bf16 & 15) || ((uintptr_t)dev_exponents & 7) || ((uintptr_t)dev_fractions & 7))
     return fail(NZ_ERR_ALIGN, "nz_split: pointers must be 16-byte (input) / 8-byte (outputs) aligned");
   const uint64_t blocks = (n + 2047) / 2048;
   if (blocks > 0x7FFFFFFFull) return fail(NZ_ERR_ARG, "tensor too large");
+  if (int rc = launch_absmax(dev_bf16, n, normalizer_size, (uint8_t*)dev_norm, (hipStream_t)stream)) return rc;
+  const NzNorm nm{normalizer_size ? (const uint8_t*)dev_norm : nullptr, log2_of(normalizer_size ? normalizer_size : 1)};
   hipLaunchKernelGGL(nz_split_unpacked_kernel, dim3((uint32_t)blocks), dim3(256), 0,
                      (hipStream_t)stream, (const uint16_t*)dev_bf16, n, (uint8_t*)dev_exponents,
-                     (uint8_t*)dev_fractions);
+                     (uint8_t*)dev_fractions, nm);
   NZ_HIP(hipGetLastError());
   return NZ_OK;
 }
@@ -253,8 +299,12 @@ int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fr
 int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
               uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
               void* dev_workspace, uint64_t workspace_bytes, uint64_t* dev_total,
-              uint32_t* dev_status, uint64_t* host_total, void* stream) {
+              uint32_t* dev_status, uint64_t* host_total, uint32_t normalizer_size, void* dev_norm,
+              void* stream) {
   if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
+  if (!normalizer_ok(normalizer_size)) return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
+  if (normalizer_size && n && (!dev_norm || ((uintptr_t)dev_norm & 7)))
+    return fail(NZ_ERR_ARG, "normalizer bytes: null or not 8-byte aligned");
   NzGeom g;
   if (int rc = make_geom(&g, n, chunk_size, lane_syms)) return rc;
   if (!dev_comp || !dev_workspace || !dev_total || !dev_status || (n && (!dev_bf16 || !dev_packed)))
@@ -268,7 +318,7 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
   hipStream_t st = (hipStream_t)stream;
   uint8_t* ws = (uint8_t*)dev_workspace;
   if (int rc = encode_phase1(g, precision, dev_bf16, (uint8_t*)dev_packed, ws, L, (uint8_t*)dev_comp,
-                             comp_cap, dev_total, dev_status, st))
+                             comp_cap, dev_total, dev_status, normalizer_size, (uint8_t*)dev_norm, st))
     return rc;
   if (int rc = encode_phase2(g, ws, L, (const uint32_t*)((uint8_t*)dev_comp + g.dir_off),
                              (uint8_t*)dev_comp, comp_cap, st))
@@ -285,8 +335,12 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
 
 int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed, uint64_t n,
               int precision, uint32_t chunk_size, uint32_t lane_syms, void* dev_bf16_out,
-              uint32_t* dev_status, int check, void* stream) {
+              uint32_t* dev_status, int check, uint32_t normalizer_size, const void* dev_norm,
+              void* stream) {
   if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
+  if (!normalizer_ok(normalizer_size)) return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
+  if (normalizer_size && n && (!dev_norm || ((uintptr_t)dev_norm & 7)))
+    return fail(NZ_ERR_ARG, "normalizer bytes: null or not 8-byte aligned");
   NzGeom g;
   if (int rc = make_geom(&g, n, chunk_size, lane_syms)) return rc;
   if (n == 0) return NZ_OK;
@@ -297,7 +351,8 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
   if (check && !dev_status) return fail(NZ_ERR_ARG, "check requires dev_status");
   if (comp_bytes < g.rec_off + NZ_TAIL_PAD) return fail(NZ_ERR_CORRUPT, "container shorter than its directory");
   hipStream_t st = (hipStream_t)stream;
-  if (int rc = decode_launch(g, precision, dev_comp, comp_bytes, dev_packed, dev_bf16_out, dev_status, st))
+  if (int rc = decode_launch(g, precision, dev_comp, comp_bytes, dev_packed, dev_bf16_out, dev_status,
+                             normalizer_size, dev_norm, st))
     return rc;
   if (check) {
     uint32_t hs = 0;
@@ -317,7 +372,8 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   if (!out) return fail(NZ_ERR_ARG, "null out pointer");
   if (algorithm != NZ_ALGO_ANS) return fail(NZ_ERR_ALGO, "Unsupported algorithm");
   if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
-  if (normalizer_size != 0) return fail(NZ_ERR_ARG, "block normalizers are not implemented (normalizer_size must be 0)");
+  if (normalizer_size < 0 || !normalizer_ok((uint32_t)normalizer_size))
+    return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
   const bool auto_lanes = lane_syms == NZ_LANE_SYMS_AUTO;
   if (lane_syms == 0 || auto_lanes) {
     lane_syms = NZ_DEFAULT_LANE_SYMS;
@@ -328,6 +384,7 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   if (int rc = make_geom(&g, 0, chunk_size, lane_syms)) return rc;
   nz_manager* m = new nz_manager();
   m->precision = precision;
+  m->normalizer = (uint32_t)normalizer_size;
   m->chunk_syms = chunk_size;
   m->lane_syms = lane_syms;
   m->auto_lanes = auto_lanes;
@@ -348,6 +405,7 @@ void nz_manager_destroy(nz_manager* m) {
   for (auto& kv : m->entries) {
     if (kv.second.comp) (void)hipFree(kv.second.comp);
     if (kv.second.packed) (void)hipFree(kv.second.packed);
+    if (kv.second.norm) (void)hipFree(kv.second.norm);
   }
   if (m->ws) (void)hipFree(m->ws);
   if (m->gemv_acc) (void)hipFree(m->gemv_acc);
@@ -402,11 +460,27 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   ent.dtype = dtype;
   ent.lane_syms = lane_syms;
   ent.packed_bytes = nz_packed_stored_bytes_of(&g, m->precision);
+  ent.norm_bytes = norm_bytes_of(n, m->normalizer);
   auto release = [&](Entry& e) {
     if (e.comp) (void)hipFree(e.comp);
     if (e.packed) (void)hipFree(e.packed);
-    e.comp = e.packed = nullptr;
+    if (e.norm) (void)hipFree(e.norm);
+    e.comp = e.packed = e.norm = nullptr;
   };
+  if (ent.norm_bytes) {
+    if (old.norm && old.norm_cap >= ent.norm_bytes && old.norm_cap <= ent.norm_bytes + 4096) {
+      ent.norm = old.norm;
+      ent.norm_cap = old.norm_cap;
+      old.norm = nullptr;
+    } else {
+      ent.norm_cap = ent.norm_bytes + 8;
+      hipError_t e = hipMalloc(&ent.norm, ent.norm_cap);
+      if (e != hipSuccess) {
+        release(old);
+        return fail(NZ_ERR_HIP, std::string("hipMalloc(normalizers): ") + hipGetErrorString(e));
+      }
+    }
+  }
   if (old.packed && old.packed_cap >= ent.packed_bytes && old.packed_cap <= ent.packed_bytes + 4096) {
     ent.packed = old.packed;
     ent.packed_cap = old.packed_cap;
@@ -416,6 +490,7 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
     hipError_t e = hipMalloc(&ent.packed, ent.packed_cap);
     if (e != hipSuccess) {
       release(old);
+      release(ent);
       return fail(NZ_ERR_HIP, std::string("hipMalloc(packed): ") + hipGetErrorString(e));
     }
   }
@@ -426,7 +501,7 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   int rc = e == hipSuccess ? NZ_OK : fail(NZ_ERR_HIP, hipGetErrorString(e));
   if (rc == NZ_OK)
     rc = encode_phase1(g, m->precision, dev_data, (uint8_t*)ent.packed, ws, L, ws + L.hdr,
-                       ~0ull, d_total, d_estat, st);
+                       ~0ull, d_total, d_estat, m->normalizer, (uint8_t*)ent.norm, st);
   if (rc == NZ_OK) {
     e = hipMemcpyAsync(m->h_pin, d_total, 8, hipMemcpyDeviceToHost, st);
     if (e == hipSuccess) e = hipStreamSynchronize(st);  // the one host sync of a write
@@ -477,7 +552,7 @@ int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap
   NzGeom g;
   if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
   return decode_launch(g, m->precision, ent.comp, ent.comp_bytes, ent.packed, dev_out, m->d_status,
-                       (hipStream_t)stream);
+                       m->normalizer, ent.norm, (hipStream_t)stream);
 }
 
 int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* dev_outs,
@@ -517,6 +592,8 @@ int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* 
     it.comp_bytes = ent.comp_bytes;
     it.packed = (const uint8_t*)ent.packed;
     it.out = (uint16_t*)dev_outs[i];
+    it.norm = (const uint8_t*)ent.norm;
+    b.log2n = log2_of(m->normalizer ? m->normalizer : 1);
     it.g = g;
     grid += (uint32_t)g.n_chunks;
     it.chunk_end = grid;
@@ -541,6 +618,7 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
   std::memset(&o, 0, sizeof(o));
   b.x = (const uint16_t*)dev_x;
   b.in_features = in_features;
+  b.log2n = log2_of(m->normalizer ? m->normalizer : 1);
   uint64_t grid = 0, rows = 0;
   uint32_t max_spc = 1;
   for (uint32_t i = 0; i < count; ++i) {
@@ -558,6 +636,7 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
     bi.comp = (const uint8_t*)ent.comp;
     bi.comp_bytes = ent.comp_bytes;
     bi.packed = (const uint8_t*)ent.packed;
+    bi.norm = (const uint8_t*)ent.norm;
     bi.g = g;
     grid += g.n_chunks;
     bi.chunk_end = (uint32_t)grid;
@@ -606,7 +685,7 @@ uint64_t nz_manager_size(nz_manager* m, const char* name) {
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return 0;  // cuda/high_level.cu:209-211
-  return it->second.comp_bytes + it->second.packed_bytes;
+  return it->second.comp_bytes + it->second.packed_bytes + it->second.norm_bytes;
 }
 
 uint64_t nz_manager_exp_bytes(nz_manager* m, const char* name) {
@@ -636,18 +715,27 @@ int nz_manager_buffers(nz_manager* m, const char* name, const void** dev_comp, u
   return NZ_OK;
 }
 
+uint64_t nz_manager_norm_bytes(nz_manager* m, const char* name) {
+  if (!m || !name) return 0;
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  return it == m->entries.end() ? 0 : it->second.norm_bytes;
+}
+
 int nz_manager_export(nz_manager* m, const char* name, void* host_comp, uint64_t comp_cap,
-                      void* host_packed, uint64_t packed_cap, void* stream) {
+                      void* host_packed, uint64_t packed_cap, void* host_norm, uint64_t norm_cap,
+                      void* stream) {
   if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
   hipStream_t st = (hipStream_t)stream;
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
   const Entry& ent = it->second;
-  if (comp_cap < ent.comp_bytes || packed_cap < ent.packed_bytes)
+  if (comp_cap < ent.comp_bytes || packed_cap < ent.packed_bytes || norm_cap < ent.norm_bytes)
     return fail(NZ_ERR_CAPACITY, "host buffers smaller than the stored streams");
-  if ((ent.comp_bytes && !host_comp) || (ent.packed_bytes && !host_packed))
+  if ((ent.comp_bytes && !host_comp) || (ent.packed_bytes && !host_packed) || (ent.norm_bytes && !host_norm))
     return fail(NZ_ERR_ARG, "null host buffer");
+  if (ent.norm_bytes) NZ_HIP(hipMemcpyAsync(host_norm, ent.norm, ent.norm_bytes, hipMemcpyDeviceToHost, st));
   if (ent.comp_bytes) NZ_HIP(hipMemcpyAsync(host_comp, ent.comp, ent.comp_bytes, hipMemcpyDeviceToHost, st));
   if (ent.packed_bytes)
     NZ_HIP(hipMemcpyAsync(host_packed, ent.packed, ent.packed_bytes, hipMemcpyDeviceToHost, st));
@@ -656,7 +744,8 @@ int nz_manager_export(nz_manager* m, const char* name, void* host_comp, uint64_t
 }
 
 int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, uint64_t comp_bytes,
-                      const void* host_packed, uint64_t packed_bytes, void* stream) {
+                      const void* host_packed, uint64_t packed_bytes, const void* host_norm,
+                      uint64_t norm_bytes, void* stream) {
   if (!m || !name || !host_comp) return fail(NZ_ERR_ARG, "null manager, name or container");
   hipStream_t st = (hipStream_t)stream;
   // the container describes itself: check it against this manager before anything is stored
@@ -677,6 +766,9 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
   if (packed_bytes != nz_packed_stored_bytes_of(&g, m->precision))
     return fail(NZ_ERR_ARG, "packed stream does not have the size this manager's precision gives");
   if (packed_bytes && !host_packed) return fail(NZ_ERR_ARG, "null packed stream");
+  if (norm_bytes != norm_bytes_of(n, m->normalizer))
+    return fail(NZ_ERR_ARG, "normalizer bytes do not have the size this manager's normalizer_size gives");
+  if (norm_bytes && !host_norm) return fail(NZ_ERR_ARG, "null normalizer bytes");
   // the directory must be non-decreasing and end where the container ends
   {
     const uint8_t* c = (const uint8_t*)host_comp;
@@ -697,8 +789,13 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
   ent.comp_bytes = ent.comp_cap = comp_bytes;
   ent.packed_bytes = packed_bytes;
   ent.packed_cap = packed_bytes + 16;  // never a zero-byte allocation; the slack is zeroed
+  ent.norm_bytes = norm_bytes;
+  ent.norm_cap = norm_bytes ? norm_bytes + 8 : 0;
   hipError_t e = hipMalloc(&ent.comp, ent.comp_cap);
   if (e == hipSuccess) e = hipMalloc(&ent.packed, ent.packed_cap);
+  if (e == hipSuccess && norm_bytes) e = hipMalloc(&ent.norm, ent.norm_cap);
+  if (e == hipSuccess && norm_bytes)
+    e = hipMemcpyAsync(ent.norm, host_norm, norm_bytes, hipMemcpyHostToDevice, st);
   if (e == hipSuccess) e = hipMemcpyAsync(ent.comp, host_comp, comp_bytes, hipMemcpyHostToDevice, st);
   if (e == hipSuccess && packed_bytes)
     e = hipMemcpyAsync(ent.packed, host_packed, packed_bytes, hipMemcpyHostToDevice, st);
@@ -707,6 +804,7 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
   if (e != hipSuccess) {
     if (ent.comp) (void)hipFree(ent.comp);
     if (ent.packed) (void)hipFree(ent.packed);
+    if (ent.norm) (void)hipFree(ent.norm);
     return fail(NZ_ERR_HIP, std::string("import: ") + hipGetErrorString(e));
   }
   auto it = m->entries.find(name);
@@ -715,6 +813,8 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
     (void)hipDeviceSynchronize();
     if (it->second.comp) (void)hipFree(it->second.comp);
     if (it->second.packed) (void)hipFree(it->second.packed);
+  if (it->second.norm) (void)hipFree(it->second.norm);
+    if (it->second.norm) (void)hipFree(it->second.norm);
     m->entries.erase(it);
   }
   m->entries.emplace(name, ent);
@@ -730,6 +830,7 @@ int nz_manager_erase(nz_manager* m, const char* name) {
   NZ_HIP(hipDeviceSynchronize());
   if (it->second.comp) (void)hipFree(it->second.comp);
   if (it->second.packed) (void)hipFree(it->second.packed);
+  if (it->second.norm) (void)hipFree(it->second.norm);
   m->entries.erase(it);
   return NZ_OK;
 }

@@ -61,6 +61,121 @@ __device__ __forceinline__ uint32_t nz_merge_one(uint32_t exp, uint32_t repr) {
   return (sign << 15) | (exp << 7) | frac;
 }
 
+__device__ __forceinline__ float nz_bf16_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ uint32_t nz_f32_to_bf16(float f) {
+  const uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x0040u;  // NaN stays NaN
+  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;                      // round to nearest even
+}
+
+// ----------------------------------------------------------------------------
+// block normalizers (cuda/kernels.cuh:94-118 on the split side, :208-216 on the
+// merge side): every group of 2^log2n consecutive elements is divided by
+// 1.m, m = the 7 mantissa bits of the group's largest magnitude, before the
+// split, and multiplied by it again after the merge.  The group stores m << 1
+// (the top 8 of the 23 fraction bits of the float 1.m).  Division and product
+// run in fp32 and round to bf16, nearest even, exactly as the reference's
+// float expressions do (the quotient of two 8-bit significands never lies
+// close enough to a rounding boundary for the intermediate fp32 rounding to
+// matter).
+// ----------------------------------------------------------------------------
+struct NzNorm {
+  const uint8_t* bytes;  // one per group, null when the tensor is not normalized
+  uint32_t log2n;
+};
+
+__device__ __forceinline__ float nz_norm_base(uint32_t byte) {
+  return __uint_as_float(0x3F800000u | (byte << 15));
+}
+__device__ __forceinline__ uint32_t nz_norm_div(uint32_t h, uint32_t byte) {
+  return nz_f32_to_bf16(nz_bf16_to_f32(h) / nz_norm_base(byte));
+}
+__device__ __forceinline__ uint32_t nz_norm_mul(uint32_t h, uint32_t byte) {
+  return nz_f32_to_bf16(nz_bf16_to_f32(h) * nz_norm_base(byte));
+}
+
+// The group bytes of the 8 consecutive elements that start at e0 (a multiple of
+// 8), one per element: byte j of the result belongs to element e0 + j.
+__device__ __forceinline__ uint64_t nz_norm_load8(const NzNorm& nm, uint64_t e0) {
+  if (nm.log2n >= 3) return 0x0101010101010101ull * (uint64_t)nm.bytes[e0 >> nm.log2n];
+  if (nm.log2n == 0) return *reinterpret_cast<const uint64_t*>(nm.bytes + e0);
+  if (nm.log2n == 1) {
+    const uint32_t w = *reinterpret_cast<const uint32_t*>(nm.bytes + (e0 >> 1));
+    return (uint64_t)__builtin_amdgcn_perm(w, w, 0x01010000u) |
+           ((uint64_t)__builtin_amdgcn_perm(w, w, 0x03030202u) << 32);
+  }
+  const uint32_t w = *reinterpret_cast<const uint16_t*>(nm.bytes + (e0 >> 2));
+  return (uint64_t)((w & 0xFFu) * 0x01010101u) | ((uint64_t)((w >> 8) * 0x01010101u) << 32);
+}
+
+// 8 bf16 values times their group factors
+__device__ __forceinline__ uint4 nz_denorm8(const uint4 v, const uint64_t nb) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t b0 = (uint32_t)(nb >> (16 * k)) & 0xFFu, b1 = (uint32_t)(nb >> (16 * k + 8)) & 0xFFu;
+    o[k] = nz_norm_mul(w[k] & 0xFFFFu, b0) | (nz_norm_mul(w[k] >> 16, b1) << 16);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+__device__ __forceinline__ uint4 nz_norm8(const uint4 v, const uint64_t nb) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t b0 = (uint32_t)(nb >> (16 * k)) & 0xFFu, b1 = (uint32_t)(nb >> (16 * k + 8)) & 0xFFu;
+    o[k] = nz_norm_div(w[k] & 0xFFFFu, b0) | (nz_norm_div(w[k] >> 16, b1) << 16);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// One byte per group: the mantissa of the largest magnitude (patterns of |x|
+// order like the values).  A workgroup covers 2048 elements, a multiple of
+// every group size.
+__global__ __launch_bounds__(256) void nz_absmax_kernel(const uint16_t* __restrict__ in, uint64_t n,
+                                                        uint32_t log2n, uint8_t* __restrict__ norm) {
+  __shared__ uint32_t smax[256];
+  const uint32_t tid = threadIdx.x;
+  const uint64_t blk0 = (uint64_t)blockIdx.x * 2048;
+  const uint64_t e0 = blk0 + (uint64_t)tid * 8;
+  uint32_t mag[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) mag[j] = 0;
+  if (e0 + 8 <= n) {
+    const uint4 v = *reinterpret_cast<const uint4*>(in + e0);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) mag[j] = (w[j >> 1] >> (16 * (j & 1))) & 0x7FFFu;
+  } else {
+    for (uint32_t j = 0; j < 8 && e0 + j < n; ++j) mag[j] = in[e0 + j] & 0x7FFFu;
+  }
+  if (log2n < 3) {
+    const uint32_t gs = 1u << log2n;
+    for (uint32_t q = 0; q < 8; q += gs) {
+      if (e0 + q >= n) break;
+      uint32_t m = 0;
+      for (uint32_t j = 0; j < gs; ++j) m = mag[q + j] > m ? mag[q + j] : m;
+      norm[(e0 + q) >> log2n] = (uint8_t)((m & 0x7Fu) << 1);
+    }
+    return;
+  }
+  uint32_t m8 = 0;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) m8 = mag[j] > m8 ? mag[j] : m8;
+  smax[tid] = m8;
+  __syncthreads();
+  const uint32_t per = 1u << (log2n - 3);  // threads per group
+  if (tid < (256u >> (log2n - 3))) {
+    const uint64_t g0 = blk0 + ((uint64_t)tid << log2n);
+    if (g0 < n) {
+      uint32_t m = 0;
+      for (uint32_t q = 0; q < per; ++q) m = smax[tid * per + q] > m ? smax[tid * per + q] : m;
+      norm[g0 >> log2n] = (uint8_t)((m & 0x7Fu) << 1);
+    }
+  }
+}
+
 __device__ __forceinline__ uint32_t nz_lane_id() {
   return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 }
@@ -94,11 +209,13 @@ __device__ __forceinline__ uint32_t nz_get12(const uint8_t* p, uint32_t i) {
 __global__ __launch_bounds__(256) void nz_split_unpacked_kernel(const uint16_t* __restrict__ in,
                                                                 uint64_t n,
                                                                 uint8_t* __restrict__ exps,
-                                                                uint8_t* __restrict__ fracs) {
+                                                                uint8_t* __restrict__ fracs,
+                                                                const NzNorm nm) {
   uint64_t i0 = ((uint64_t)blockIdx.x * 256 + threadIdx.x) * 8;
   if (i0 >= n) return;
   if (i0 + 8 <= n) {
     uint4 v = *reinterpret_cast<const uint4*>(in + i0);
+    if (nm.bytes) v = nz_norm8(v, nz_norm_load8(nm, i0));
     uint32_t w[4] = {v.x, v.y, v.z, v.w};
     uint64_t e = 0, f = 0;
 #pragma unroll
@@ -112,8 +229,9 @@ __global__ __launch_bounds__(256) void nz_split_unpacked_kernel(const uint16_t* 
     *reinterpret_cast<uint64_t*>(fracs + i0) = f;
   } else {
     for (uint64_t i = i0; i < n; ++i) {
-      uint32_t ex, rp;
-      nz_split_one<7>(in[i], ex, rp);
+      uint32_t ex, rp, h = in[i];
+      if (nm.bytes) h = nz_norm_div(h, nm.bytes[i >> nm.log2n]);
+      nz_split_one<7>(h, ex, rp);
       exps[i] = (uint8_t)ex;
       fracs[i] = (uint8_t)rp;
     }
@@ -158,7 +276,8 @@ template <int S>
 __global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
     const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms, uint32_t spc,
     uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
-    uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info) {
+    uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info,
+    const NzNorm nm) {
   // 8 histogram copies (one per lane & 7) at a stride of 257 words: exponents of
   // weights cluster on a few values, so a single copy would serialise most of
   // a wavefront's atomics on one address; the odd stride keeps the copies of a
@@ -199,6 +318,7 @@ __global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
     const uint32_t rem = cn - i;
     if (rem >= 8) {
       uint4 v = *reinterpret_cast<const uint4*>(in + gi);
+      if (nm.bytes) v = nz_norm8(v, nz_norm_load8(nm, gi));
       uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
       for (int j = 0; j < 8; ++j) nz_split_one<S>((w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu, ex[j], rp[j]);
@@ -220,7 +340,9 @@ __global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
       // (cuda/kernels.cuh:92), and only ceil(rem*(S+1)/8) packed bytes exist.
       uint64_t f = 0;
       for (uint32_t j = 0; j < rem; ++j) {
-        nz_split_one<S>(in[gi + j], ex[0], rp[0]);
+        uint32_t h = in[gi + j];
+        if (nm.bytes) h = nz_norm_div(h, nm.bytes[(gi + j) >> nm.log2n]);
+        nz_split_one<S>(h, ex[0], rp[0]);
         exps[gi + j] = (uint8_t)ex[0];
         uint32_t bit = j * (S + 1);
         f |= (uint64_t)rp[0] << (8u * (bit >> 3) + (7u - S - (bit & 7u)));
@@ -660,13 +782,6 @@ __device__ __forceinline__ uint4 nz_merge_group(uint64_t sm, const uint32_t (&ew
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
 
-// ... and store them with one 16-byte store.
-template <int S>
-__device__ __forceinline__ void nz_store_group(uint16_t* __restrict__ out, uint64_t sm,
-                                               const uint32_t (&ew)[8]) {
-  *reinterpret_cast<uint4*>(out) = nz_merge_group<S>(sm, ew);
-}
-
 // ----------------------------------------------------------------------------
 // y = W x for one activation row, W decoded on the fly and never written out
 // ----------------------------------------------------------------------------
@@ -851,11 +966,13 @@ struct NzWaveDec {
 // activation `gv.x` and summed into `gv.acc` (the tensor is a row-major matrix
 // with rows of gv.in_features elements, a multiple of 512, so that no group is
 // ragged and no group straddles two rows).
-template <int S, bool GEMV>
+// With NORM every merged value is multiplied by its group's factor (`nm`)
+// before it is stored or used.
+template <int S, bool GEMV, bool NORM>
 __device__ __forceinline__ void nz_decode_chunk(
     const uint8_t* __restrict__ comp, const uint64_t comp_bytes, const uint8_t* __restrict__ packed,
     uint16_t* __restrict__ out, const NzGeom& g, uint32_t* __restrict__ d_status, const uint64_t c,
-    const NzGemv& gv) {
+    const NzGemv& gv, const NzNorm& nm) {
   extern __shared__ uint32_t lds[];
   uint2* lut = reinterpret_cast<uint2*>(lds);                   // 4096 x 8 bytes
   uint32_t* rings = lds + 2 * NZ_M;                             // spc rings
@@ -1022,13 +1139,17 @@ __device__ __forceinline__ void nz_decode_chunk(
         uint32_t ew[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) ew[j] = (uint32_t)((sy >> (8 * j)) & 0xFFu) << 24;
-        if constexpr (GEMV) walk.add(nz_merge_group<S>(sm, ew), walk.load(walk.col), lane);
-        else nz_store_group<S>(dst + idx0, sm, ew);
+        uint4 mv = nz_merge_group<S>(sm, ew);
+        if constexpr (NORM) mv = nz_denorm8(mv, nz_norm_load8(nm, seg_base + idx0));
+        if constexpr (GEMV) walk.add(mv, walk.load(walk.col), lane);
+        else *reinterpret_cast<uint4*>(dst + idx0) = mv;
       } else if constexpr (!GEMV) {
         for (uint32_t j = 0; j < rem; ++j) {
           const uint32_t bit = (idx0 + j) * (S + 1);
           const uint32_t rp = ((uint32_t)pk[bit >> 3] >> (7u - S - (bit & 7u))) & ((2u << S) - 1u);
-          dst[idx0 + j] = (uint16_t)nz_merge_one<S>(raw[idx0 + j], rp);
+          uint32_t h = nz_merge_one<S>(raw[idx0 + j], rp);
+          if constexpr (NORM) h = nz_norm_mul(h, nm.bytes[(seg_base + idx0 + j) >> nm.log2n]);
+          dst[idx0 + j] = (uint16_t)h;
         }
       }
     }
@@ -1080,12 +1201,18 @@ __device__ __forceinline__ void nz_decode_chunk(
   uint64_t sm_next = whole ? nz_load_sm<S>(pk + lane_off) : 0;
   uint4 xq_next = make_uint4(0, 0, 0, 0);
   if constexpr (GEMV) xq_next = walk.load(walk.col);
+  uint64_t nb_next = 0;
+  if constexpr (NORM)
+    if (whole) nb_next = nz_norm_load8(nm, seg_base + lane * NZ_GROUP);
   for (uint32_t gq = 0; gq < whole; ++gq) {
     const uint64_t sm = sm_next;
     const uint32_t noff = (gq + 1) * NZ_LANES * (S + 1) + lane_off;
     sm_next = nz_load_sm<S>(pk + (noff < last_off ? noff : last_off));
     const uint4 xq = xq_next;
     if constexpr (GEMV) xq_next = walk.load(walk.next_col());  // always inside x
+    const uint64_t nb = nb_next;
+    if constexpr (NORM)
+      nb_next = nz_norm_load8(nm, seg_base + ((gq + 1 < whole ? gq + 1 : gq) * NZ_LANES + lane) * NZ_GROUP);
     uint32_t ew[8];
     w.group(ew);
     // the merge starts only here: its wait for the packed bytes (fetched a group
@@ -1093,10 +1220,10 @@ __device__ __forceinline__ void nz_decode_chunk(
     // wait for the previous group's store
     uint32_t sml = (uint32_t)sm, smh = (uint32_t)(sm >> 32);
     asm volatile("" : "+v"(sml), "+v"(smh), "+v"(ew[7]));
-    if constexpr (GEMV)
-      walk.add(nz_merge_group<S>(((uint64_t)smh << 32) | sml, ew), xq, lane);
-    else
-      nz_store_group<S>(dst + (gq * NZ_LANES + lane) * NZ_GROUP, ((uint64_t)smh << 32) | sml, ew);
+    uint4 mv = nz_merge_group<S>(((uint64_t)smh << 32) | sml, ew);
+    if constexpr (NORM) mv = nz_denorm8(mv, nb);
+    if constexpr (GEMV) walk.add(mv, xq, lane);
+    else *reinterpret_cast<uint4*>(dst + (gq * NZ_LANES + lane) * NZ_GROUP) = mv;
   }
   if (!GEMV && whole < body) {  // the ragged last group of the tensor
     const uint32_t idx0 = (whole * NZ_LANES + lane) * NZ_GROUP;
@@ -1110,7 +1237,9 @@ __device__ __forceinline__ void nz_decode_chunk(
         uint32_t sym = 0;
 #pragma unroll
         for (int q = 0; q < 8; ++q) sym = (uint32_t)q == j ? (ew[q] >> 24) : sym;
-        dst[idx0 + j] = (uint16_t)nz_merge_one<S>(sym, rp);
+        uint32_t h = nz_merge_one<S>(sym, rp);
+        if constexpr (NORM) h = nz_norm_mul(h, nm.bytes[(seg_base + idx0 + j) >> nm.log2n]);
+        dst[idx0 + j] = (uint16_t)h;
       }
     }
   }
@@ -1136,8 +1265,10 @@ __device__ __forceinline__ void nz_decode_chunk(
         const uint32_t idx0 = ((body + t) * NZ_LANES + lane) * NZ_GROUP;
         const uint32_t b = idx0 / 8 * (S + 1);
         const uint64_t sm = b >= keep ? nz_load_sm<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
-        if constexpr (GEMV) walk.add(nz_merge_group<S>(sm, ext[t]), walk.load(walk.col), lane);
-        else nz_store_group<S>(dst + idx0, sm, ext[t]);
+        uint4 mv = nz_merge_group<S>(sm, ext[t]);
+        if constexpr (NORM) mv = nz_denorm8(mv, nz_norm_load8(nm, seg_base + idx0));
+        if constexpr (GEMV) walk.add(mv, walk.load(walk.col), lane);
+        else *reinterpret_cast<uint4*>(dst + idx0) = mv;
       }
     }
   }
@@ -1145,11 +1276,11 @@ __device__ __forceinline__ void nz_decode_chunk(
     if (walk.pending) walk.flush(lane);
 }
 
-template <int S>
+template <int S, bool NORM>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
-    uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status) {
-  nz_decode_chunk<S, false>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x, NzGemv{});
+    uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status, const NzNorm nm) {
+  nz_decode_chunk<S, false, NORM>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x, NzGemv{}, nm);
 }
 
 // Several tensors in one launch: the grid is the concatenation of their
@@ -1162,6 +1293,7 @@ struct NzBatchItem {
   const uint8_t* packed;
   uint16_t* out;       // dense output (decode) ...
   long long* acc;      // ... or the row accumulators (matrix-vector product)
+  const uint8_t* norm; // group bytes of a normalized tensor
   NzGeom g;
   uint32_t chunk_end;
   uint32_t reserved;
@@ -1170,10 +1302,12 @@ struct NzBatch {
   uint32_t count;
   uint32_t in_features;  // matrix-vector product only
   const uint16_t* x;     // matrix-vector product only
+  uint32_t log2n;        // normalized tensors only
+  uint32_t reserved;
   NzBatchItem item[NZ_BATCH_MAX];
 };
 
-template <int S>
+template <int S, bool NORM>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_batch_kernel(
     const NzBatch b, uint32_t* __restrict__ d_status) {
   uint32_t t = 0, first = 0;
@@ -1182,12 +1316,12 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_batch_ke
     ++t;
   }
   const NzBatchItem& it = b.item[t];
-  nz_decode_chunk<S, false>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status, blockIdx.x - first,
-                            NzGemv{});
+  nz_decode_chunk<S, false, NORM>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status,
+                                  blockIdx.x - first, NzGemv{}, NzNorm{it.norm, b.log2n});
 }
 
 // The same walk over several matrices that multiply one activation row.
-template <int S>
+template <int S, bool NORM>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_gemv_kernel(
     const NzBatch b, uint32_t* __restrict__ d_status) {
   uint32_t t = 0, first = 0;
@@ -1197,7 +1331,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_gemv_ker
   }
   const NzBatchItem& it = b.item[t];
   const NzGemv gv{b.x, it.acc, b.in_features};
-  nz_decode_chunk<S, true>(it.comp, it.comp_bytes, it.packed, nullptr, it.g, d_status, blockIdx.x - first, gv);
+  nz_decode_chunk<S, true, NORM>(it.comp, it.comp_bytes, it.packed, nullptr, it.g, d_status,
+                                 blockIdx.x - first, gv, NzNorm{it.norm, b.log2n});
 }
 
 // y = bf16(acc * 2^-30 + bias), and the accumulators return to zero for the next
@@ -1215,13 +1350,6 @@ struct NzGemvOut {
   NzGemvOutItem item[NZ_BATCH_MAX];
 };
 
-__device__ __forceinline__ float nz_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
-__device__ __forceinline__ uint16_t nz_f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u);  // NaN stays NaN
-  return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);                      // round to nearest even
-}
-
 __global__ __launch_bounds__(256) void nz_gemv_finish_kernel(const NzGemvOut o) {
   const uint32_t r = blockIdx.x * 256 + threadIdx.x;
   uint32_t t = 0, first = 0;
@@ -1238,5 +1366,5 @@ __global__ __launch_bounds__(256) void nz_gemv_finish_kernel(const NzGemvOut o) 
   if (a.y) y = __uint_as_float(0x7FC00000u);
   else y = (float)((double)a.x * (1.0 / (double)(1u << NZ_GEMV_FRAC_BITS)));
   if (it.bias) y += nz_bf16_to_f32(it.bias[i]);
-  it.y[i] = nz_f32_to_bf16(y);
+  it.y[i] = (uint16_t)nz_f32_to_bf16(y);
 }

@@ -7,6 +7,8 @@ the fixtures pin THIS build's semantics against accidental change:
                     precision, cross-checked here against the independent
                     closed form before being written
   containers.npz    container + stored packed bytes of three seeded inputs
+  normalizers.npz   group bytes and reconstruction of two seeded inputs stored
+                    with block normalizers
 
 Run from the repository root:  python tests/golden/make_golden.py
 """
@@ -28,6 +30,17 @@ CASES = {
     "normal_70000_s7": ("normal", 70000, 12, 7, 65536, 512),
     "stress_70000_s3": ("stress", 70000, 13, 3, 65536, 512),
 }
+
+
+NORM_CASES = {
+    # name: (generator, n, seed, precision, normalizer_size)
+    "stress_5000_s3_n512": ("stress", 5000, 21, 3, 512),
+    "normal_3000_s0_n8": ("normal", 3000, 22, 0, 8),
+}
+
+
+def finite(bits):
+    return np.where((bits & 0x7F80) == 0x7F80, np.uint16(0x3F80) | (bits & 0x8000), bits).astype(np.uint16)
 
 
 def make_bits(kind, n, seed):
@@ -57,7 +70,16 @@ def main():
         cont[name + "_comp"] = comp
         cont[name + "_packed"] = packed
     np.savez_compressed(os.path.join(HERE, "containers.npz"), **cont)
-    for f in ("recon_tables.npz", "containers.npz"):
+    nrm = {}
+    for name, (kind, n, seed, s, ns) in NORM_CASES.items():
+        bits = finite(make_bits(kind, n, seed))
+        norm, scaled = O.block_normalize(bits, ns)
+        nrm[name + "_bits"] = bits
+        nrm[name + "_norm"] = norm
+        nrm[name + "_scaled"] = scaled
+        nrm[name + "_recon"] = O.reconstruct_normalized(bits, s, ns)
+    np.savez_compressed(os.path.join(HERE, "normalizers.npz"), **nrm)
+    for f in ("recon_tables.npz", "containers.npz", "normalizers.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")
 
 

@@ -48,15 +48,15 @@ def test_argument_errors_without_a_gpu():
 
     L = _lib.load()
     # precision / geometry / null checks happen before any HIP call
-    assert L.nz_decode(None, 0, None, 16, 5, 65536, 512, None, None, 0, None) == _lib.ERR_ARG
+    assert L.nz_decode(None, 0, None, 16, 5, 65536, 512, None, None, 0, 0, None, None) == _lib.ERR_ARG
     assert "precision" in _lib.last_error()
-    assert L.nz_decode(None, 0, None, 16, 7, 65536, 100, None, None, 0, None) == _lib.ERR_ARG
-    assert L.nz_decode(None, 0, None, 16, 7, 65536, 512, None, None, 0, None) == _lib.ERR_ARG
-    assert L.nz_decode(None, 0, None, 0, 7, 65536, 512, None, None, 0, None) == _lib.OK  # empty tensor
+    assert L.nz_decode(None, 0, None, 16, 7, 65536, 100, None, None, 0, 0, None, None) == _lib.ERR_ARG
+    assert L.nz_decode(None, 0, None, 16, 7, 65536, 512, None, None, 0, 0, None, None) == _lib.ERR_ARG
+    assert L.nz_decode(None, 0, None, 0, 7, 65536, 512, None, None, 0, 0, None, None) == _lib.OK  # empty tensor
     h = ctypes.c_void_p()
     assert L.nz_manager_create(3, 7, 0, 65536, 0, ctypes.byref(h)) == _lib.ERR_ALGO
     assert _lib.last_error() == "Unsupported algorithm"  # cuda/high_level.cu:67
     assert L.nz_manager_create(0, 5, 0, 65536, 0, ctypes.byref(h)) == _lib.ERR_ARG
-    assert L.nz_manager_create(0, 7, 32, 65536, 0, ctypes.byref(h)) == _lib.ERR_ARG
+    assert L.nz_manager_create(0, 7, 33, 65536, 0, ctypes.byref(h)) == _lib.ERR_ARG  # not a power of two
     with pytest.raises(RuntimeError):
         _lib.raise_for(_lib.ERR_ALGO)

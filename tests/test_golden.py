@@ -15,13 +15,13 @@ def _load(name):
     return np.load(os.path.join(sys_path_golden, name))
 
 
-def _cases():
+def _cases(which="CASES"):
     import importlib.util
 
     spec = importlib.util.spec_from_file_location("make_golden", os.path.join(sys_path_golden, "make_golden.py"))
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
-    return mod.CASES
+    return getattr(mod, which)
 
 
 def test_oracle_matches_recon_tables(oracle):
@@ -75,3 +75,26 @@ def test_gpu_matches_containers():
         rc, out = gpu_decode(torch.from_numpy(c[name + "_comp"]).cuda(), torch.from_numpy(c[name + "_packed"]).cuda(),
                              n, s, chunk, lane)
         assert rc == 0 and np.array_equal(out, closed_form_recon(bits, s))
+
+
+def test_oracle_matches_normalizer_fixtures(oracle):
+    c = _load("normalizers.npz")
+    for name, (kind, n, seed, s, ns) in _cases("NORM_CASES").items():
+        bits = c[name + "_bits"]
+        norm, scaled = oracle.block_normalize(bits, ns)
+        assert np.array_equal(norm, c[name + "_norm"]) and np.array_equal(scaled, c[name + "_scaled"]), name
+        assert np.array_equal(oracle.reconstruct_normalized(bits, s, ns), c[name + "_recon"]), name
+
+
+@pytest.mark.gpu
+def test_gpu_matches_normalizer_fixtures():
+    from test_gpu_parity import gpu_decode, gpu_encode
+
+    c = _load("normalizers.npz")
+    for name, (kind, n, seed, s, ns) in _cases("NORM_CASES").items():
+        print(f"case golden normalizer {name}", flush=True)
+        bits = c[name + "_bits"]
+        comp, packed, nb = gpu_encode(bits, s, norm_size=ns)
+        assert np.array_equal(nb.cpu().numpy(), c[name + "_norm"]), name
+        rc, out = gpu_decode(comp, packed, n, s, norm_size=ns, norm=nb)
+        assert rc == 0 and np.array_equal(out, c[name + "_recon"]), name

@@ -21,7 +21,8 @@ def _to_dev(bits: np.ndarray):
     return torch.from_numpy(bits.view(np.int16).copy()).cuda()
 
 
-def gpu_encode(bits, s, chunk=65536, lane=344):
+def gpu_encode(bits, s, chunk=65536, lane=344, norm_size=0):
+    """-> (container, stored packed stream[, normalizer bytes when norm_size > 0]) as device tensors"""
     L, m = _lib()
     n = bits.size
     d_in = _to_dev(bits) if n else torch.empty(0, dtype=torch.int16, device="cuda")
@@ -34,22 +35,28 @@ def gpu_encode(bits, s, chunk=65536, lane=344):
     aux = torch.zeros(4, dtype=torch.int64, device="cuda")
     total = ctypes.c_uint64(0)
     st = torch.cuda.current_stream().cuda_stream
+    norm = torch.zeros(L.nz_norm_bytes(n, norm_size) + 8, dtype=torch.uint8, device="cuda")
     rc = L.nz_encode(d_in.data_ptr(), n, s, chunk, lane, packed.data_ptr(), comp.data_ptr(), cap,
-                     ws.data_ptr(), ws_bytes, aux.data_ptr(), aux.data_ptr() + 8, ctypes.byref(total), st)
+                     ws.data_ptr(), ws_bytes, aux.data_ptr(), aux.data_ptr() + 8, ctypes.byref(total),
+                     norm_size, norm.data_ptr(), st)
     assert rc == 0, m.last_error()
     torch.cuda.synchronize()
-    return comp[: total.value].clone(), packed[: L.nz_packed_stored_bytes(n, s, chunk, lane)].clone()
+    res = comp[: total.value].clone(), packed[: L.nz_packed_stored_bytes(n, s, chunk, lane)].clone()
+    return res + (norm[: L.nz_norm_bytes(n, norm_size)].clone(),) if norm_size else res
 
 
-def gpu_decode(comp, packed, n, s, chunk=65536, lane=344, check=True):
+def gpu_decode(comp, packed, n, s, chunk=65536, lane=344, check=True, norm_size=0, norm=None):
     L, m = _lib()
+    if norm_size:
+        norm = torch.cat([norm, torch.zeros(8, dtype=torch.uint8, device="cuda")])
     out = torch.zeros(max(n, 8), dtype=torch.int16, device="cuda")
     status = torch.zeros(2, dtype=torch.int32, device="cuda")
     if packed.numel() < 8:
         packed = torch.cat([packed, torch.zeros(8, dtype=torch.uint8, device="cuda")])
     st = torch.cuda.current_stream().cuda_stream
     rc = L.nz_decode(comp.data_ptr(), comp.numel(), packed.data_ptr(), n, s, chunk, lane,
-                     out.data_ptr(), status.data_ptr(), 1 if check else 0, st)
+                     out.data_ptr(), status.data_ptr(), 1 if check else 0, norm_size,
+                     norm.data_ptr() if norm_size else None, st)
     torch.cuda.synchronize()
     return rc, out[:n].cpu().numpy().view(np.uint16)
 
@@ -176,7 +183,7 @@ def test_split_api(oracle):
         d = _to_dev(bits) if n else torch.empty(0, dtype=torch.int16, device="cuda")
         e = torch.zeros(max(n, 8), dtype=torch.uint8, device="cuda")
         f = torch.zeros(max(n, 8), dtype=torch.uint8, device="cuda")
-        rc = L.nz_split(d.data_ptr(), n, e.data_ptr(), f.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        rc = L.nz_split(d.data_ptr(), n, e.data_ptr(), f.data_ptr(), 0, None, torch.cuda.current_stream().cuda_stream)
         assert rc == 0, m.last_error()
         torch.cuda.synchronize()
         oe, of = oracle.split(bits, 7)

@@ -183,5 +183,3 @@ def test_manager_argument_errors():
         neuzip_amd.Manager(normalizer_size=3)
     with pytest.raises(RuntimeError, match="Unsupported algorithm"):
         neuzip_amd.Manager(algorithm=A.zstd)
-    with pytest.raises(NotImplementedError):
-        neuzip_amd.Manager(normalizer_size=32)
