@@ -168,6 +168,16 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
                           uint32_t in_features, const void* const* dev_bias, void* const* dev_y,
                           void* stream);
 
+/* Embedding lookup on a stored table (neuzip/nn/embedding.py:30-39 decompresses
+   the WHOLE table for every forward): row dev_indices[i] (int64) of the table
+   `name`, read as rows of row_len elements, goes to dev_out[i * row_len ...];
+   only the chunks that hold the requested rows are decoded.  An index outside
+   the table gives a row of zeros and makes the next nz_manager_check fail.
+   Uses the manager's write scratch (grown when needed: calls must be ordered on
+   one stream with the writes).  Asynchronous on `stream`. */
+int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indices, uint64_t count,
+                           uint32_t row_len, void* dev_out, void* stream);
+
 /* meta_cache lookup, cuda/high_level.cu:42-43,228-230. */
 int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype);
 

@@ -25,7 +25,7 @@ LANE_SYMS_AUTO = 0xFFFFFFFF
 EXPORTS = [
     "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",
     "nz_encode_workspace_bytes", "nz_norm_bytes", "nz_split", "nz_encode", "nz_decode",
-    "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch",
+    "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
     "nz_manager_meta", "nz_manager_size", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
     "nz_manager_norm_bytes", "nz_manager_buffers", "nz_manager_erase", "nz_manager_check", "nz_manager_export", "nz_manager_import",
 ]
@@ -78,6 +78,8 @@ def load() -> ctypes.CDLL:
     L.nz_manager_export.argtypes = [vp, ctypes.c_char_p, vp, u64, vp, u64, vp, u64, vp]
     L.nz_manager_import.restype = i32
     L.nz_manager_import.argtypes = [vp, ctypes.c_char_p, vp, u64, vp, u64, vp, u64, vp]
+    L.nz_manager_gather_rows.restype = i32
+    L.nz_manager_gather_rows.argtypes = [vp, ctypes.c_char_p, vp, u64, u32, vp, vp]
     L.nz_manager_gemv_batch.restype = i32
     L.nz_manager_gemv_batch.argtypes = [vp, ctypes.POINTER(ctypes.c_char_p), u32, vp, u32, ctypes.POINTER(vp),
                                         ctypes.POINTER(vp), vp]

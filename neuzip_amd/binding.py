@@ -129,6 +129,17 @@ class _HipBackend:
         rc = self._L.nz_manager_read_batch(self._h, names, ptrs, caps, k, _stream_ptr(outs[0].device) if k else None)
         _lib.raise_for(rc)
 
+    def gather_rows(self, handle: str, indices: torch.Tensor, row_len: int) -> torch.Tensor:
+        """Rows ``indices`` (any integer shape) of the stored table with rows of
+        ``row_len`` elements -> ``[indices.numel(), row_len]``; only the chunks
+        that hold those rows are decoded."""
+        idx = indices.reshape(-1).to(device=self._device, dtype=torch.int64).contiguous()
+        out = torch.empty(idx.numel(), row_len, dtype=torch.bfloat16, device=self._device)
+        rc = self._L.nz_manager_gather_rows(self._h, handle.encode(), idx.data_ptr(), idx.numel(), row_len,
+                                            out.data_ptr(), _stream_ptr(self._device))
+        _lib.raise_for(rc)
+        return out
+
     def gemv_batch(self, names, x: torch.Tensor, biases, outs) -> None:
         """``outs[i] = W_i @ x (+ biases[i])`` for the stored matrices ``names``
         (a ctypes array of encoded handles) and ONE activation row ``x``; the
@@ -302,6 +313,17 @@ class Manager:
         if bias is None:
             return self._be.linear_without_bias(handle, inputs, shape)
         return self._be.linear(handle, inputs, shape, bias)
+
+    def gather_rows(self, handle: str, indices: torch.Tensor) -> torch.Tensor:
+        """Rows ``indices`` of the stored 2-D table ``handle`` as ``[indices.numel(), row_len]``
+        (no counterpart in the reference, which decompresses the whole table:
+        neuzip/nn/embedding.py:30-39)."""
+        shape = self.meta_dict[handle]
+        if len(shape) != 2:
+            raise ValueError("gather_rows needs a stored 2-D table")
+        if isinstance(self._be, _DenseBackend):
+            return self._be.read(handle).reshape(shape)[indices.reshape(-1)]
+        return self._be.gather_rows(handle, indices, int(shape[1]))
 
     # -- checkpointing (no counterpart in the reference, whose compressed tensors
     #    live only inside the process: neuzip/nn/module.py:13) ------------------

@@ -208,6 +208,20 @@ int gemv_launch(const NzBatch& b, const NzGemvOut& o, uint32_t grid, uint32_t ma
   return NZ_OK;
 }
 
+template <int S>
+void launch_decode_rows(const NzGeom& g, const void* comp, uint64_t comp_bytes, const void* packed,
+                        uint16_t* scratch, uint32_t* d_status, const NzNorm& nm, const long long* idx,
+                        uint32_t count, uint32_t row_len, uint32_t cpr, hipStream_t st) {
+  const size_t lds = (2 * NZ_M + g.spc * NZ_RING_ALLOC_DWORDS) * 4;
+  const dim3 gd(count * cpr), bd(64 * g.spc);
+  if (nm.bytes)
+    hipLaunchKernelGGL((nz_decode_rows_kernel<S, true>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,
+                       (const uint8_t*)packed, scratch, g, d_status, nm, idx, row_len, cpr);
+  else
+    hipLaunchKernelGGL((nz_decode_rows_kernel<S, false>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,
+                       (const uint8_t*)packed, scratch, g, d_status, nm, idx, row_len, cpr);
+}
+
 int make_geom(NzGeom* g, uint64_t n, uint32_t chunk, uint32_t lane_syms) {
   if (nz_geom_make(g, n, chunk, lane_syms))
     return fail(NZ_ERR_ARG,
@@ -670,6 +684,52 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
   return gemv_launch(b, o, (uint32_t)grid, max_spc, (uint32_t)rows, m->precision, m->d_status, st);
 }
 
+int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indices, uint64_t count,
+                           uint32_t row_len, void* dev_out, void* stream) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  if (count == 0) return NZ_OK;
+  if (!dev_indices || !dev_out) return fail(NZ_ERR_ARG, "null indices or output");
+  if (((uintptr_t)dev_indices & 7) || ((uintptr_t)dev_out & 1)) return fail(NZ_ERR_ALIGN, "misaligned indices or output");
+  hipStream_t st = (hipStream_t)stream;
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  const Entry& ent = it->second;
+  if (row_len == 0 || ent.n == 0 || ent.n % row_len)
+    return fail(NZ_ERR_ARG, "stored tensor is not a table with rows of row_len elements");
+  NzGeom g;
+  if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
+  // chunks a row can touch, wherever it starts
+  const uint32_t cpr = (uint32_t)(((uint64_t)row_len + g.chunk_syms - 2) / g.chunk_syms + 1);
+  if (count * (uint64_t)cpr > 0x7FFFFFFFull || count > 0xFFFFull * 0xFFFFull)
+    return fail(NZ_ERR_ARG, "too many rows for one call");
+  // one chunk-sized slot per (row, touched chunk): taken from the encode scratch of this manager
+  const uint64_t need = count * (uint64_t)cpr * g.chunk_syms * 2;
+  if (m->ws_bytes < need) {
+    NZ_HIP(hipStreamSynchronize(st));
+    if (m->ws) NZ_HIP(hipFree(m->ws));
+    m->ws = nullptr;
+    m->ws_bytes = 0;
+    NZ_HIP(hipMalloc(&m->ws, need));
+    m->ws_bytes = need;
+  }
+  const NzNorm nm{m->normalizer ? (const uint8_t*)ent.norm : nullptr, log2_of(m->normalizer ? m->normalizer : 1)};
+  const long long* idx = (const long long*)dev_indices;
+  uint16_t* scratch = (uint16_t*)m->ws;
+  switch (m->precision) {
+    case 7: launch_decode_rows<7>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx, (uint32_t)count, row_len, cpr, st); break;
+    case 3: launch_decode_rows<3>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx, (uint32_t)count, row_len, cpr, st); break;
+    case 1: launch_decode_rows<1>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx, (uint32_t)count, row_len, cpr, st); break;
+    default: launch_decode_rows<0>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx, (uint32_t)count, row_len, cpr, st); break;
+  }
+  NZ_HIP(hipGetLastError());
+  const uint32_t bx = (row_len + 255) / 256 < 64 ? (row_len + 255) / 256 : 64;
+  hipLaunchKernelGGL(nz_copy_rows_kernel, dim3(bx, (uint32_t)count), dim3(256), 0, st, (const uint16_t*)scratch,
+                     idx, ent.n / row_len, row_len, g.chunk_syms, cpr, (uint16_t*)dev_out);
+  NZ_HIP(hipGetLastError());
+  return NZ_OK;
+}
+
 int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype) {
   if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
   std::lock_guard<std::mutex> lock(m->mu);
@@ -843,6 +903,7 @@ int nz_manager_check(nz_manager* m, void* stream) {
   NZ_HIP(hipMemsetAsync(m->d_status, 0, 4, st));
   NZ_HIP(hipStreamSynchronize(st));
   const uint32_t hs = (uint32_t)m->h_pin[1];
+  if (hs == 8u) return fail(NZ_ERR_CORRUPT, "a row gather was given an index outside the table");
   if (hs) return fail(NZ_ERR_CORRUPT, "a read saw a container that failed validation (status " + std::to_string(hs) + ")");
   return NZ_OK;
 }

@@ -1368,3 +1368,48 @@ __global__ __launch_bounds__(256) void nz_gemv_finish_kernel(const NzGemvOut o) 
   if (it.bias) y += nz_bf16_to_f32(it.bias[i]);
   it.y[i] = (uint16_t)nz_f32_to_bf16(y);
 }
+
+// ----------------------------------------------------------------------------
+// row gather (embedding lookup): decode only the chunks that hold the rows asked
+// for.  Workgroup (i, k) decodes the k-th chunk touched by row indices[i] into
+// slot i * cpr + k of `scratch` (a slot is one chunk of bf16 values); the copy
+// kernel then lifts the row out of its slots.  An index outside the table sets
+// status bit 8 and yields a row of zeros.
+// ----------------------------------------------------------------------------
+template <int S, bool NORM>
+__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_rows_kernel(
+    const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
+    uint16_t* __restrict__ scratch, NzGeom g, uint32_t* __restrict__ d_status, const NzNorm nm,
+    const long long* __restrict__ indices, uint32_t row_len, uint32_t cpr) {
+  const uint32_t i = blockIdx.x / cpr, k = blockIdx.x - i * cpr;
+  const long long idx = indices[i];
+  if (idx < 0 || (uint64_t)idx >= g.n / row_len) {
+    if (threadIdx.x == 0 && k == 0) atomicOr(d_status, 8u);
+    return;
+  }
+  const uint64_t first = (uint64_t)idx * row_len, last = first + row_len - 1;
+  const uint64_t c = first / g.chunk_syms + k;
+  if (c > last / g.chunk_syms) return;
+  // the chunk function writes element e of the tensor to out[e]: shift `out` so
+  // that the chunk's first element lands at the start of this workgroup's slot
+  uint16_t* out = scratch + ((int64_t)blockIdx.x - (int64_t)c) * (int64_t)g.chunk_syms;
+  nz_decode_chunk<S, false, NORM>(comp, comp_bytes, packed, out, g, d_status, c, NzGemv{}, nm);
+}
+
+__global__ __launch_bounds__(256) void nz_copy_rows_kernel(const uint16_t* __restrict__ scratch,
+                                                           const long long* __restrict__ indices,
+                                                           uint64_t rows, uint32_t row_len,
+                                                           uint32_t chunk_syms, uint32_t cpr,
+                                                           uint16_t* __restrict__ out) {
+  const uint32_t i = blockIdx.y;
+  const long long idx = indices[i];
+  const bool ok = idx >= 0 && (uint64_t)idx < rows;
+  const uint64_t first = ok ? (uint64_t)idx * row_len : 0;
+  const uint64_t c0 = first / chunk_syms;
+  for (uint32_t e = blockIdx.x * 256 + threadIdx.x; e < row_len; e += gridDim.x * 256) {
+    const uint64_t ge = first + e;
+    const uint64_t c = ge / chunk_syms;
+    const uint16_t v = ok ? scratch[((uint64_t)i * cpr + (c - c0)) * chunk_syms + (ge - c * chunk_syms)] : 0;
+    out[(uint64_t)i * row_len + e] = v;
+  }
+}

@@ -1,4 +1,5 @@
+from neuzip_amd.nn.embedding import Embedding
 from neuzip_amd.nn.linear import Linear
 from neuzip_amd.nn.module import Parameter
 
-__all__ = ["Parameter", "Linear"]
+__all__ = ["Parameter", "Linear", "Embedding"]

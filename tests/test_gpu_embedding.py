@@ -1,0 +1,92 @@
+"""Row gather on a stored table and the compressed Embedding module."""
+import numpy as np
+import pytest
+
+from conftest import bf16_bits_normal, stress_bits
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+def _table(rows, dim, seed, kind="normal"):
+    bits = bf16_bits_normal(rows * dim, seed) if kind == "normal" else stress_bits(rows, dim, seed)
+    bits = np.where((bits & 0x7F80) == 0x7F80, np.uint16(0x3F80), bits).astype(np.uint16)
+    return torch.from_numpy(bits.view(np.int16).copy()).cuda().view(torch.bfloat16).view(rows, dim)
+
+
+@pytest.mark.parametrize("rows,dim,precision,norm,lane", [
+    (1000, 64, 7, 0, 0),        # many rows per chunk
+    (300, 4096, 7, 0, 0),       # 16 rows per chunk
+    (37, 100_000, 7, 0, 0),     # a row spans several chunks and starts anywhere inside one
+    (513, 768, 3, 512, "auto"),
+    (129, 40, 0, 8, 128),       # odd row length: rows straddle groups of 8
+])
+def test_gather_rows_equals_full_read(rows, dim, precision, norm, lane):
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=precision, normalizer_size=norm, lane_symbols=lane)
+    h = mgr.write(_table(rows, dim, seed=rows, kind="stress" if norm else "normal"))
+    full = mgr.read(h)
+    g = torch.Generator().manual_seed(rows)
+    for count in (1, 7, 200):
+        idx = torch.randint(0, rows, (count,), generator=g)
+        idx[0], idx[-1] = rows - 1, 0
+        print(f"case gather rows={rows} dim={dim} count={count}", flush=True)
+        got = mgr.gather_rows(h, idx.cuda())
+        assert got.shape == (count, dim)
+        assert torch.equal(got, full[idx.cuda()])
+    mgr._be.check()
+    # an index outside the table: zeros, and the manager reports it
+    got = mgr.gather_rows(h, torch.tensor([0, rows, -1, 1]).cuda())
+    assert torch.equal(got[0], full[0]) and torch.equal(got[3], full[1])
+    assert int(got[1].view(torch.int16).abs().max()) == 0 and int(got[2].view(torch.int16).abs().max()) == 0
+    with pytest.raises(RuntimeError, match="outside the table"):
+        mgr._be.check()
+
+
+def test_embedding_module_and_unroll_convert():
+    import neuzip_amd
+    from neuzip_amd.utils import _unroll_convert
+
+    torch.manual_seed(3)
+
+    class Tiny(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.emb = torch.nn.Embedding(500, 128, padding_idx=0)
+            self.blocks = torch.nn.ModuleList([torch.nn.Linear(128, 128) for _ in range(2)])
+            self.lm_head = torch.nn.Linear(128, 500, bias=False)
+
+        def forward(self, ids):
+            x = self.emb(ids)
+            for b in self.blocks:
+                x = torch.relu(b(x))
+            return self.lm_head(x)
+
+    dense = Tiny().to(torch.bfloat16).cuda()
+    ids = torch.randint(0, 500, (3, 17), device="cuda")
+    with torch.no_grad():
+        want = dense(ids)
+    mgr = neuzip_amd.Manager()
+    model = _unroll_convert(mgr, dense)
+    assert isinstance(model.emb, neuzip_amd.nn.Embedding) and repr(model.emb).startswith("Embedding(!")
+    assert isinstance(model.lm_head, neuzip_amd.nn.Linear)  # unlike convert(), nothing is skipped
+    assert all(isinstance(b, neuzip_amd.nn.Linear) for b in model.blocks)
+    assert model.emb.weight.numel() == 0 and mgr.size(model.emb.weight._handle) > 0
+    with torch.no_grad():
+        assert torch.equal(model(ids), want)
+
+    # max_norm goes through torch's own renormalisation
+    e = torch.nn.Embedding(50, 64, max_norm=0.5).to(torch.bfloat16).cuda()
+    w0 = e.weight.data.clone()
+    ce = neuzip_amd.nn.Embedding(mgr, e)
+    ids = torch.randint(0, 50, (9,), device="cuda")
+    with torch.no_grad():
+        ref = torch.nn.functional.embedding(ids, w0.clone(), None, 0.5, 2.0)
+        assert torch.equal(ce(ids), ref)
+    # the dummy backend keeps the module usable
+    dm = neuzip_amd.Manager(algorithm=neuzip_amd.Algorithm.dummy)
+    de = neuzip_amd.nn.Embedding(dm, torch.nn.Embedding(20, 8).to(torch.bfloat16).cuda())
+    assert de(torch.tensor([[1, 2]]).cuda()).shape == (1, 2, 8)
+    mgr._be.check()
