@@ -37,6 +37,7 @@ HBM_PEAK_GBPS = 8000.0
 # (rows, cols, precision, chunk_size, lane_symbols). A live run cannot read these counters, so any
 # other workload reports null.
 MEASURED_TRAFFIC = {
+    (16384, 4096, 7, 131072, 256): 233_203_000,
     (16384, 4096, 7, 65536, 344): 230_958_000,
 }
 
@@ -49,7 +50,8 @@ def parse_args():
     ap.add_argument("--rows", type=int, default=16384)
     ap.add_argument("--cols", type=int, default=4096)
     ap.add_argument("--precision", type=int, default=7, choices=[7, 3, 1, 0])
-    ap.add_argument("--chunk-size", type=int, default=65536)
+    ap.add_argument("--chunk-size", type=int, default=0,
+                    help="elements per frequency table; 0 = library default (131072), 65536 = the reference's nvcomp chunk")
     ap.add_argument("--lane-symbols", type=int, default=0, help="0 = library default; -1 = per-tensor (model workloads)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -230,7 +232,7 @@ def llama8b_measure(args, torch, full):
     measure("dense_graph", capture())
     dense_param_bytes = sum(p.numel() * p.element_size() for p in model.parameters())
 
-    mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size,
+    mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size or None,
                              lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
     t_conv, _ = sync_time(lambda: mgr.convert(model))
     torch.cuda.empty_cache()
@@ -325,7 +327,7 @@ def run_gpt2m(args, torch):
         torch.set_default_dtype(torch.bfloat16)
         model = GPT2Shaped(layers=layers, ctx=args.seq_len)
         torch.set_default_dtype(torch.float32)
-    mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size,
+    mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size or None,
                              lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
     mgr.convert(model)
     comp_params = [p for p in model.parameters() if isinstance(p, neuzip_amd.nn.Parameter)]
@@ -390,7 +392,7 @@ def run_gpt2m(args, torch):
             "decodes_per_step": n_dec / args.steps,
             "encodes_per_step": n_enc / args.steps,
             "compressed_tensors": len(comp_params),
-            "lane_symbols": "auto" if args.lane_symbols < 0 else (args.lane_symbols or 344),
+            "lane_symbols": "auto" if args.lane_symbols < 0 else (args.lane_symbols or "default"),
             "stored_over_dense": round(sum(mgr.size(p._handle) for p in comp_params) /
                                        sum(2 * int(np.prod(p._shape)) for p in comp_params), 5),
             "first_loss": round(float(losses[0]), 4),
@@ -433,12 +435,14 @@ def main():
         return run_gpt2m(args, torch)
 
     n = args.rows * args.cols
-    lane = args.lane_symbols or lib_mod.DEFAULT_LANE_SYMS
+    chunk = args.chunk_size or lib_mod.DEFAULT_CHUNK
+    lane = args.lane_symbols or (lib_mod.DEFAULT_LANE_SYMS if chunk == lib_mod.DEFAULT_CHUNK else
+                                 lib_mod.LANE_SYMS_64K if chunk == 65536 else max(16, chunk // 512))
     torch.manual_seed(args.seed)
     dense = (torch.randn(args.rows, args.cols, device="cuda") * 0.02).to(torch.bfloat16).view(-1)
     out = torch.empty_like(dense)
 
-    codec = Codec(torch, L, lib_mod, n, args.precision, args.chunk_size, lane)
+    codec = Codec(torch, L, lib_mod, n, args.precision, chunk, lane)
     codec.encode(dense)
     codec.decode(out, check=True)
     torch.cuda.synchronize()
@@ -497,7 +501,7 @@ def main():
                         f"fused rANS decode + merge, precision {args.precision}",
             "elements": n,
             "precision": args.precision,
-            "chunk_size": args.chunk_size,
+            "chunk_size": chunk,
             "lane_symbols": lane,
             "bit_exact": bit_exact,
             "compressed_exponent_bytes": codec.total,
@@ -511,7 +515,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": MEASURED_TRAFFIC.get((args.rows, args.cols, args.precision, args.chunk_size, lane)),
+            "traffic": MEASURED_TRAFFIC.get((args.rows, args.cols, args.precision, chunk, lane)),
             "kernel": f"nz_decode_kernel<{args.precision}>",
             "algorithmic_bytes_per_launch": algo_bytes,
             "mean_launch_us": round(mean_launch * 1e6, 2),
@@ -523,7 +527,7 @@ def main():
     if not args.no_sweep:
         sweep = {}
         for s in (7, 3, 1, 0):
-            c2 = codec if s == args.precision else Codec(torch, L, lib_mod, n, s, args.chunk_size, lane)
+            c2 = codec if s == args.precision else Codec(torch, L, lib_mod, n, s, chunk, lane)
             c2.encode(dense)
             k = max(5, args.steps // 10)
             w_d, m_d, _ = time_launches(torch, lambda: c2.decode(out), k, 3)

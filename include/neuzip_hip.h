@@ -44,8 +44,13 @@ extern "C" {
 /* algorithm codes: cuda/algorithms.cuh:8. Only ANS exists here. */
 #define NZ_ALGO_ANS 0
 
-#define NZ_DEFAULT_CHUNK 65536u   /* cuda/neuzip.cu:31 */
-#define NZ_DEFAULT_LANE_SYMS 344u /* three wavefronts per 64 KiB chunk: 22016 + 22016 + 21504 */
+/* The library's own geometry (chunk_size 0): tables shared by 128 Ki elements,
+   eight wavefronts of 256 symbols per lane each.  The reference hands nvcomp
+   chunks of 64 Ki (cuda/neuzip.cu:31); that size is honoured when asked for,
+   its best segment length being 344 (22016 + 22016 + 21504 elements). */
+#define NZ_DEFAULT_CHUNK 131072u
+#define NZ_DEFAULT_LANE_SYMS 256u
+#define NZ_LANE_SYMS_64K 344u
 #define NZ_LANE_SYMS_AUTO 0xFFFFFFFFu /* nz_manager_create: choose per tensor */
 
 typedef struct nz_manager nz_manager;
@@ -123,9 +128,12 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
 /* Manager(algorithm, chunk_size) for the class Manager_f{precision}_n{normalizer_size}
    (cuda/neuzip.cu:19-38, neuzip/binding.py:69-70).  precision in {0,1,3,7};
    normalizer_size 0 or a power of two up to 1024 (block normalizers, see above);
-   lane_syms 0 selects NZ_DEFAULT_LANE_SYMS clipped to the chunk;
+   chunk_size 0 selects NZ_DEFAULT_CHUNK; lane_syms 0 the best segment length
+   for the chunk (NZ_DEFAULT_LANE_SYMS, NZ_LANE_SYMS_64K, or the chunk cut in 1..8);
    NZ_LANE_SYMS_AUTO shortens the segments of tensors too small to fill the GPU
-   at the default (more wavefronts, ~4.5 bits of container per extra lane). */
+   at the default (more wavefronts, ~4.5 bits of container per extra lane; with
+   chunk_size 0 such tensors are stored with 64 Ki chunks).  Every entry records
+   the geometry it was written with. */
 int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_t chunk_size,
                       uint32_t lane_syms, nz_manager** out);
 void nz_manager_destroy(nz_manager* m);
@@ -201,7 +209,7 @@ int nz_manager_buffers(nz_manager* m, const char* name, const void** dev_comp,
    leaves 0-size parameters in a state_dict), so a converted model cannot be
    checkpointed there; these two calls are what a save/load needs.  The
    container names its own element count and geometry; import checks header,
-   directory and sizes against the manager (chunk_size, precision) and stores
+   directory and sizes against the manager (precision, normalizer_size) and stores
    nothing when they disagree.  Both calls block until the copies are done. */
 int nz_manager_export(nz_manager* m, const char* name, void* host_comp, uint64_t comp_cap,
                       void* host_packed, uint64_t packed_cap, void* host_norm, uint64_t norm_cap,

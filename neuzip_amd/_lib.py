@@ -18,8 +18,9 @@ OK = 0
 ERR_ARG, ERR_DTYPE, ERR_NOT_FOUND, ERR_HIP, ERR_CAPACITY, ERR_CORRUPT, ERR_ALIGN, ERR_ALGO = range(-1, -9, -1)
 DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 ALGO_ANS = 0
-DEFAULT_CHUNK = 65536
-DEFAULT_LANE_SYMS = 344
+DEFAULT_CHUNK = 131072
+DEFAULT_LANE_SYMS = 256
+LANE_SYMS_64K = 344
 LANE_SYMS_AUTO = 0xFFFFFFFF
 
 EXPORTS = [

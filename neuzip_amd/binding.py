@@ -264,14 +264,18 @@ class Manager:
         algorithm: Algorithm = Algorithm.ans,
         precision: int = 7,
         normalizer_size=None,
-        chunk_size=2**16,
+        chunk_size=None,
         lane_symbols: int = 0,
     ) -> None:
-        """``lane_symbols`` (extension; 0 = library default of 344, three
-        wavefronts per 64 KiB chunk) is the number of exponents each of the 64
-        rANS lanes of a wavefront codes per segment: smaller values expose more
-        wavefronts per chunk at the price of about 4.5 bits of container per
-        lane and segment.  ``"auto"`` keeps the default
+        """``chunk_size`` is the number of exponents that share one frequency
+        table.  The reference passes its value (default ``2**16``) to nvcomp as
+        the chunk size; here ``None`` selects the library's own table scope of
+        ``2**17`` elements decoded by eight wavefronts, which is both smaller and
+        faster on this hardware, and ``2**16`` (or any supported value) is
+        honoured when given.  ``lane_symbols`` (extension; 0 = the best value
+        for the chunk) is the number of exponents each of the 64 rANS lanes of a
+        wavefront codes per segment: smaller values expose more wavefronts per
+        chunk at the price of about 4.5 bits of container per lane and segment.  ``"auto"`` keeps the default
         for large tensors and shortens the segments of small ones so that they
         still fill the GPU (meant for training, where every weight is decoded
         three times and encoded once per step)."""
@@ -289,9 +293,9 @@ class Manager:
             raise AttributeError(
                 f"module 'neuzip._cuda' has no attribute 'Manager_f{precision}_n{normalizer_size}'"
             )
-        self._be = _HipBackend(precision, normalizer_size, chunk_size, lane_symbols)
-        self._settings = {"precision": int(precision), "normalizer_size": int(normalizer_size),
-                          "chunk_size": int(chunk_size)}
+        self._be = _HipBackend(precision, normalizer_size, int(chunk_size or 0), lane_symbols)
+        # what a checkpoint must agree on (the chunk geometry travels inside every container)
+        self._settings = {"precision": int(precision), "normalizer_size": int(normalizer_size)}
 
     # -- store ---------------------------------------------------------------
     def write(self, tensor: torch.Tensor, handle: Optional[str] = None) -> str:

@@ -239,6 +239,7 @@ struct Entry {
   uint64_t n = 0;
   int dtype = NZ_DTYPE_BF16;
   uint32_t lane_syms = 0;  // geometry this entry was written with
+  uint32_t chunk_syms = 0;
   void* norm = nullptr;    // one byte per normalizer group (managers with normalizer_size > 0)
   uint64_t norm_bytes = 0, norm_cap = 0;
 };
@@ -249,7 +250,8 @@ struct nz_manager {
   int precision;
   uint32_t normalizer = 0;  // elements per normalizer group, 0 = none
   uint32_t chunk_syms, lane_syms;
-  bool auto_lanes = false;  // pick lane_syms per tensor so that small tensors still fill the GPU
+  bool own_chunk = false;   // chunk_size 0 was given: the library's own table scope
+  bool auto_lanes = false;  // pick the geometry per tensor so that small tensors still fill the GPU
   std::unordered_map<std::string, Entry> entries;  // compress_cache + meta_cache
   std::mutex mu;
   void* ws = nullptr;
@@ -389,8 +391,18 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   if (normalizer_size < 0 || !normalizer_ok((uint32_t)normalizer_size))
     return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
   const bool auto_lanes = lane_syms == NZ_LANE_SYMS_AUTO;
+  const bool own_chunk = chunk_size == 0;
+  if (own_chunk) {
+    chunk_size = NZ_DEFAULT_CHUNK;
+    // an explicit segment length too short for eight segments to cover the
+    // default chunk goes with the smaller table scope
+    if (lane_syms != 0 && !auto_lanes && (uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size)
+      chunk_size = 65536;
+  }
   if (lane_syms == 0 || auto_lanes) {
-    lane_syms = NZ_DEFAULT_LANE_SYMS;
+    // the best measured segment length for the chunk: 8 segments of 256 per lane
+    // in a 128 Ki chunk, three ragged segments (344 per lane) in a 64 Ki chunk
+    lane_syms = chunk_size == NZ_DEFAULT_CHUNK ? NZ_DEFAULT_LANE_SYMS : NZ_LANE_SYMS_64K;
     while (lane_syms > 8 && (uint64_t)lane_syms * NZ_LANES > chunk_size) lane_syms /= 2;
     while ((uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size) lane_syms *= 2;
   }
@@ -400,6 +412,7 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   m->precision = precision;
   m->normalizer = (uint32_t)normalizer_size;
   m->chunk_syms = chunk_size;
+  m->own_chunk = own_chunk;
   m->lane_syms = lane_syms;
   m->auto_lanes = auto_lanes;
   hipError_t e = hipMalloc((void**)&m->d_status, 256);
@@ -436,16 +449,21 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   if ((uintptr_t)dev_data & 15) return fail(NZ_ERR_ALIGN, "dense input must be 16-byte aligned");
   // Throughput of both codec directions is set by the number of wavefronts in
   // flight (one per 64 * lane_syms elements).  In auto mode a tensor too small
-  // to give every SIMD two wavefronts at the default gets shorter segments,
-  // down to the 8 segments a chunk may hold, at ~4.5 bits per extra lane.
-  uint32_t lane_syms = m->lane_syms;
+  // to give every SIMD two wavefronts at the default gets shorter segments
+  // (and, with the library's own chunk, the smaller 64 Ki table scope that
+  // allows them), at ~4.5 bits per extra lane.
+  uint32_t lane_syms = m->lane_syms, chunk_syms = m->chunk_syms;
   if (m->auto_lanes) {
-    while (lane_syms > 16 && nz_geom_check(m->chunk_syms, (lane_syms / 2 + 7) & ~7u) == 0 &&
+    if (m->own_chunk && n / ((uint64_t)lane_syms * NZ_LANES) < 2048) {
+      chunk_syms = 65536;
+      lane_syms = 176;
+    }
+    while (lane_syms > 16 && nz_geom_check(chunk_syms, (lane_syms / 2 + 7) & ~7u) == 0 &&
            n / ((uint64_t)lane_syms * NZ_LANES) < 2048)
       lane_syms = (lane_syms / 2 + 7) & ~7u;
   }
   NzGeom g;
-  if (int rc = make_geom(&g, n, m->chunk_syms, lane_syms)) return rc;
+  if (int rc = make_geom(&g, n, chunk_syms, lane_syms)) return rc;
   hipStream_t st = (hipStream_t)stream;
   std::lock_guard<std::mutex> lock(m->mu);
 
@@ -473,6 +491,7 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
   ent.n = n;
   ent.dtype = dtype;
   ent.lane_syms = lane_syms;
+  ent.chunk_syms = chunk_syms;
   ent.packed_bytes = nz_packed_stored_bytes_of(&g, m->precision);
   ent.norm_bytes = norm_bytes_of(n, m->normalizer);
   auto release = [&](Entry& e) {
@@ -564,7 +583,7 @@ int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap
   if (!dev_out) return fail(NZ_ERR_ARG, "null output pointer");
   if ((uintptr_t)dev_out & 15) return fail(NZ_ERR_ALIGN, "dense output must be 16-byte aligned");
   NzGeom g;
-  if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
+  if (int rc = make_geom(&g, ent.n, ent.chunk_syms, ent.lane_syms)) return rc;
   return decode_launch(g, m->precision, ent.comp, ent.comp_bytes, ent.packed, dev_out, m->d_status,
                        m->normalizer, ent.norm, (hipStream_t)stream);
 }
@@ -598,7 +617,7 @@ int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* 
     const Entry& ent = m->entries.find(names[i])->second;
     if (ent.n == 0) continue;
     NzGeom g;
-    if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
+    if (int rc = make_geom(&g, ent.n, ent.chunk_syms, ent.lane_syms)) return rc;
     if (b.count == NZ_BATCH_MAX || (uint64_t)grid + g.n_chunks > 0x7FFFFFFFull)
       if (int rc = flush()) return rc;
     NzBatchItem& it = b.item[b.count++];
@@ -645,7 +664,7 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
     if (!dev_y[i] || ((uintptr_t)dev_y[i] & 1)) return fail(NZ_ERR_ARG, "null or misaligned output pointer");
     if (dev_bias && dev_bias[i] && ((uintptr_t)dev_bias[i] & 1)) return fail(NZ_ERR_ALIGN, "misaligned bias");
     NzGeom g;
-    if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
+    if (int rc = make_geom(&g, ent.n, ent.chunk_syms, ent.lane_syms)) return rc;
     NzBatchItem& bi = b.item[i];
     bi.comp = (const uint8_t*)ent.comp;
     bi.comp_bytes = ent.comp_bytes;
@@ -698,7 +717,7 @@ int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indi
   if (row_len == 0 || ent.n == 0 || ent.n % row_len)
     return fail(NZ_ERR_ARG, "stored tensor is not a table with rows of row_len elements");
   NzGeom g;
-  if (int rc = make_geom(&g, ent.n, m->chunk_syms, ent.lane_syms)) return rc;
+  if (int rc = make_geom(&g, ent.n, ent.chunk_syms, ent.lane_syms)) return rc;
   // chunks a row can touch, wherever it starts
   const uint32_t cpr = (uint32_t)(((uint64_t)row_len + g.chunk_syms - 2) / g.chunk_syms + 1);
   if (count * (uint64_t)cpr > 0x7FFFFFFFull || count > 0xFFFFull * 0xFFFFull)
@@ -817,7 +836,6 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
   const uint64_t n = (uint64_t)h[2] | ((uint64_t)h[3] << 32);
   const uint64_t total = (uint64_t)h[10] | ((uint64_t)h[11] << 32);
   std::lock_guard<std::mutex> lock(m->mu);
-  if (h[4] != m->chunk_syms) return fail(NZ_ERR_ARG, "container was written with another chunk_size");
   NzGeom g;
   if (nz_geom_make(&g, n, h[4], h[5])) return fail(NZ_ERR_CORRUPT, "container header holds an unsupported geometry");
   if (h[6] != (uint32_t)g.n_chunks || h[7] != (uint32_t)g.n_segs || h[8] != g.dir_off || h[9] != g.rec_off ||
@@ -846,6 +864,7 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
   ent.n = n;
   ent.dtype = NZ_DTYPE_BF16;
   ent.lane_syms = h[5];
+  ent.chunk_syms = h[4];
   ent.comp_bytes = ent.comp_cap = comp_bytes;
   ent.packed_bytes = packed_bytes;
   ent.packed_cap = packed_bytes + 16;  // never a zero-byte allocation; the slack is zeroed

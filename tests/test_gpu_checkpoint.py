@@ -13,7 +13,7 @@ def _tensor(bits, shape):
     return torch.from_numpy(bits.view(np.int16).copy()).cuda().view(torch.bfloat16).view(shape)
 
 
-@pytest.mark.parametrize("precision,lane", [(7, 0), (3, "auto"), (0, 128)])
+@pytest.mark.parametrize("precision,lane", [(7, 0), (3, "auto"), (0, 512), (1, 128)])
 def test_state_dict_round_trip(tmp_path, oracle, precision, lane):
     import neuzip_amd
 
@@ -27,9 +27,9 @@ def test_state_dict_round_trip(tmp_path, oracle, precision, lane):
     mgr.save(path)
     # what was exported is what the oracle writes for the same input
     sd = mgr.state_dict()
-    lane0 = 344 if lane == 0 else (128 if lane == 128 else None)
-    if lane0:
-        o_comp, o_packed = oracle.compress_bf16(bits[0], precision, 65536, lane0)
+    geom = {0: (131072, 256), 512: (131072, 512), 128: (65536, 128)}.get(lane)  # "auto" picks per tensor
+    if geom:
+        o_comp, o_packed = oracle.compress_bf16(bits[0], precision, *geom)
         assert np.array_equal(sd["entries"][hs[0]]["container"].numpy(), o_comp)
         assert np.array_equal(sd["entries"][hs[0]]["packed"].numpy(), o_packed)
 
@@ -55,8 +55,10 @@ def test_load_rejects_what_does_not_fit():
 
     with pytest.raises(RuntimeError, match="precision"):
         neuzip_amd.Manager(precision=3).load_state_dict(sd)
-    with pytest.raises(RuntimeError, match="chunk_size"):
-        neuzip_amd.Manager(chunk_size=32768).load_state_dict(sd)
+    # the chunk geometry travels with the container: a manager created for another one reads it
+    other = neuzip_amd.Manager(chunk_size=32768)
+    other.load_state_dict(sd)
+    assert torch.equal(other.read(h), w)
 
     target = neuzip_amd.Manager(precision=7)  # keep the manager alive: its backend closes with it
     be = target._be

@@ -37,7 +37,7 @@ def test_write_read_size(oracle, precision):
         out = mgr.read(h)
         assert out.shape == torch.Size(shp) and out.dtype == torch.bfloat16 and not out.requires_grad
         assert np.array_equal(bits_of(out), oracle.reconstruct(bits_of(w), precision))
-        o_comp, o_packed = oracle.compress_bf16(bits_of(w), precision, 65536, 344)
+        o_comp, o_packed = oracle.compress_bf16(bits_of(w), precision, 131072, 256)
         assert mgr.size(h) == o_comp.size + o_packed.size  # exponents + packed bytes held
         assert mgr._be.packed_bytes(h) == o_packed.size
     assert mgr.size("nope") == 0  # cuda/high_level.cu:209-211
@@ -371,11 +371,17 @@ def test_auto_lane_symbols(oracle):
     are those of the oracle at that geometry, and reads are exact."""
     import neuzip_amd
 
-    mgr = neuzip_amd.Manager(lane_symbols="auto")
-    for n, lane in ((1 << 20, 176), (40_000_000, 176), (70_000_000, 344)):
-        w = from_bits(bf16_bits_normal(n, seed=n % 97), (n,))
-        h = mgr.write(w)
-        o_comp, o_packed = oracle.compress_bf16(bits_of(w), 7, 65536, lane, threads=8)
-        assert mgr.size(h) == o_comp.size + o_packed.size
-        assert torch.equal(mgr.read(h), w)
+    for chunk_arg, cases in (
+        (None, ((1 << 20, 65536, 176), (40_000_000, 131072, 256), (70_000_000, 131072, 256))),
+        (65536, ((1 << 20, 65536, 176), (40_000_000, 65536, 176), (70_000_000, 65536, 344))),
+    ):
+        mgr = neuzip_amd.Manager(chunk_size=chunk_arg, lane_symbols="auto")
+        for n, chunk, lane in cases:
+            print(f"case auto chunk_arg={chunk_arg} n={n}", flush=True)
+            w = from_bits(bf16_bits_normal(n, seed=n % 97), (n,))
+            h = mgr.write(w)
+            o_comp, o_packed = oracle.compress_bf16(bits_of(w), 7, chunk, lane, threads=8)
+            assert mgr.size(h) == o_comp.size + o_packed.size
+            assert torch.equal(mgr.read(h), w)
+            del w
     mgr._be.check()
