@@ -218,6 +218,12 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
                       const void* host_packed, uint64_t packed_bytes, const void* host_norm,
                       uint64_t norm_bytes, void* stream);
 
+/* Release the manager's scratch (the workspace of the largest write so far, the
+   accumulators of the matrix-vector product); it is allocated again on demand.
+   The reference allocates its scratch per call (cuda/high_level.cu:81-108).
+   Waits for the device. */
+int nz_manager_trim(nz_manager* m);
+
 /* compress_cache.erase(name), cuda/high_level.cu:137-140. */
 int nz_manager_erase(nz_manager* m, const char* name);
 

@@ -190,6 +190,9 @@ class _HipBackend:
     def packed_bytes(self, handle: str) -> int:
         return int(self._L.nz_manager_packed_bytes(self._h, handle.encode()))
 
+    def trim(self) -> None:
+        _lib.raise_for(self._L.nz_manager_trim(self._h))
+
     def check(self) -> None:
         _lib.raise_for(self._L.nz_manager_check(self._h, _stream_ptr(self._device)))
 
@@ -369,7 +372,14 @@ class Manager:
 
     # -- helpers -------------------------------------------------------------
     def convert(self, module: torch.nn.Module) -> torch.nn.Module:
-        return _convert(self, module)
+        module = _convert(self, module)
+        self.trim()  # the encode workspace of the largest layer is not needed to serve the model
+        return module
+
+    def trim(self) -> None:
+        """Free the scratch the backend keeps between calls (re-allocated on demand)."""
+        if hasattr(self._be, "trim"):
+            self._be.trim()
 
     def split(self, tensor: torch.Tensor):
         exp, frac = self._be.split(tensor)

@@ -914,6 +914,20 @@ int nz_manager_erase(nz_manager* m, const char* name) {
   return NZ_OK;
 }
 
+int nz_manager_trim(nz_manager* m) {
+  if (!m) return fail(NZ_ERR_ARG, "null manager");
+  std::lock_guard<std::mutex> lock(m->mu);
+  // kernels of earlier writes, gathers or products may still use the scratch
+  NZ_HIP(hipDeviceSynchronize());
+  if (m->ws) NZ_HIP(hipFree(m->ws));
+  m->ws = nullptr;
+  m->ws_bytes = 0;
+  if (m->gemv_acc) NZ_HIP(hipFree(m->gemv_acc));
+  m->gemv_acc = nullptr;
+  m->gemv_rows = 0;
+  return NZ_OK;
+}
+
 int nz_manager_check(nz_manager* m, void* stream) {
   if (!m) return fail(NZ_ERR_ARG, "null manager");
   hipStream_t st = (hipStream_t)stream;

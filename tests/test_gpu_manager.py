@@ -385,3 +385,26 @@ def test_auto_lane_symbols(oracle):
             assert torch.equal(mgr.read(h), w)
             del w
     mgr._be.check()
+
+
+def test_trim_releases_the_write_scratch():
+    """After trim the manager holds little more than the compressed bytes."""
+    import neuzip_amd
+
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    mgr = neuzip_amd.Manager()
+    n = 32 * 1024 * 1024
+    w = from_bits(bf16_bits_normal(n, seed=4), (n,))
+    free0 = torch.cuda.mem_get_info()[0]
+    h = mgr.write(w)
+    held_with_scratch = free0 - torch.cuda.mem_get_info()[0]
+    mgr.trim()
+    held = free0 - torch.cuda.mem_get_info()[0]
+    stored = mgr.size(h)
+    assert held_with_scratch > 2 * stored           # the encode workspace dominates
+    assert stored <= held <= stored + (64 << 20)    # allocator granularity aside
+    assert torch.equal(mgr.read(h), w)              # reads need no scratch
+    mgr.write(w * 2, h)                             # and a write brings it back
+    assert torch.equal(mgr.read(h), w * 2)
+    mgr._be.check()
