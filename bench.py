@@ -327,18 +327,38 @@ def run_gpt2m(args, torch):
         torch.set_default_dtype(torch.bfloat16)
         model = GPT2Shaped(layers=layers, ctx=args.seq_len)
         torch.set_default_dtype(torch.float32)
+    def train_step(opts):
+        ids = torch.randint(0, 50257, (args.batch, args.seq_len), device="cuda")
+        logits = model(ids[:, :-1])
+        loss = torch.nn.functional.cross_entropy(logits.float().reshape(-1, logits.shape[-1]), ids[:, 1:].reshape(-1))
+        loss.backward()
+        for o in opts:
+            o.step()
+        return loss.detach()
+
+    # the same model with dense bf16 weights and torch's AdamW, for scale
+    opt = torch.optim.AdamW(model.parameters(), lr=1e-4)
+    for _ in range(args.warmup):
+        train_step([opt])
+        opt.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        train_step([opt])
+        opt.zero_grad(set_to_none=True)
+    torch.cuda.synchronize()
+    dense_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    del opt
+    torch.cuda.empty_cache()
+
     mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size or None,
                              lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
     mgr.convert(model)
     comp_params = [p for p in model.parameters() if isinstance(p, neuzip_amd.nn.Parameter)]
     rest = [p for p in model.parameters() if not isinstance(p, neuzip_amd.nn.Parameter)]
-    opt_c = CompressedAdamW(comp_params, lr=1e-4)
-    opt_d = torch.optim.AdamW(rest, lr=1e-4)
-
     # time every codec call with events on the stream it runs on
     be = mgr._be
     spans = []
-    raw_read, raw_write = be.read, be.write
 
     def timed(fn, kind):
         def wrapper(*a, **k):
@@ -350,30 +370,44 @@ def run_gpt2m(args, torch):
             return r
         return wrapper
 
-    be.read, be.write = timed(raw_read, "decode"), timed(raw_write, "encode")
+    be.read, be.write = timed(be.read, "decode"), timed(be.write, "encode")
+    be.read_batch = timed(be.read_batch, "decode")
 
-    def step():
-        ids = torch.randint(0, 50257, (args.batch, args.seq_len), device="cuda")
-        logits = model(ids[:, :-1])
-        loss = torch.nn.functional.cross_entropy(logits.float().reshape(-1, logits.shape[-1]), ids[:, 1:].reshape(-1))
-        loss.backward()
-        opt_c.step()
-        opt_d.step()
-        opt_d.zero_grad(set_to_none=True)
-        return loss
+    def run(group):
+        """-> per-step figures with the Linears decoded one by one (group 1) or per block"""
+        opt_c = CompressedAdamW(comp_params, lr=1e-4, group=group)
+        opt_d = torch.optim.AdamW(rest, lr=1e-4)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    spans.clear()
-    t0 = time.perf_counter()
-    losses = [step() for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    dec = sum(a.elapsed_time(b) for k, a, b in spans if k == "decode") * 1e-3
-    enc = sum(a.elapsed_time(b) for k, a, b in spans if k == "encode") * 1e-3
-    n_dec = sum(1 for k, _, _ in spans if k == "decode")
-    n_enc = sum(1 for k, _, _ in spans if k == "encode")
+        def step():
+            loss = train_step([opt_c, opt_d])
+            opt_d.zero_grad(set_to_none=True)
+            return loss
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        spans.clear()
+        t0 = time.perf_counter()
+        losses = [step() for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        dec = sum(a.elapsed_time(b) for k, a, b in spans if k == "decode") * 1e-3
+        enc = sum(a.elapsed_time(b) for k, a, b in spans if k == "encode") * 1e-3
+        return {
+            "ms_per_step": round(wall / args.steps * 1e3, 3),
+            "codec_share_of_step": round((dec + enc) / wall, 4),
+            "decode_s_per_step": round(dec / args.steps, 5),
+            "encode_s_per_step": round(enc / args.steps, 5),
+            "decode_launches_per_step": sum(1 for k, _, _ in spans if k == "decode") / args.steps,
+            "encodes_per_step": sum(1 for k, _, _ in spans if k == "encode") / args.steps,
+            "first_loss": round(float(losses[0]), 4),
+            "last_loss": round(float(losses[-1]), 4),
+        }, wall
+
+    per_linear, _ = run(1)
+    per_block_linears = len(comp_params) // max(1, layers)
+    with neuzip_amd.DecompressAhead(mgr, model, ahead=False):
+        per_block, wall = run(per_block_linears)
     mgr._be.check()
     tokens = args.batch * (args.seq_len - 1) * args.steps
     out = {
@@ -381,22 +415,18 @@ def run_gpt2m(args, torch):
         "value": round(tokens / wall, 1),
         "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(wall / args.steps * 1e3, 3),
+        "ms_per_step": per_block["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {
             "workload": f"GPT-2-medium-shaped random-init model, {layers} layers, batch {args.batch} x seq {args.seq_len}, "
                         f"bf16 weights compressed (precision {args.precision}), re-compressed after each AdamW step",
-            "codec_share_of_step": round((dec + enc) / wall, 4),
-            "decode_s_per_step": round(dec / args.steps, 5),
-            "encode_s_per_step": round(enc / args.steps, 5),
-            "decodes_per_step": n_dec / args.steps,
-            "encodes_per_step": n_enc / args.steps,
+            "dense_bf16_torch_adamw_ms_per_step": round(dense_ms, 3),
+            "decode_per_block": per_block,
+            "decode_per_linear": per_linear,
             "compressed_tensors": len(comp_params),
             "lane_symbols": "auto" if args.lane_symbols < 0 else (args.lane_symbols or "default"),
             "stored_over_dense": round(sum(mgr.size(p._handle) for p in comp_params) /
                                        sum(2 * int(np.prod(p._shape)) for p in comp_params), 5),
-            "first_loss": round(float(losses[0]), 4),
-            "last_loss": round(float(losses[-1]), 4),
         },
     }
     print(json.dumps(out))

@@ -210,8 +210,12 @@ class CompressedAdamW:
     same handle (the read -> update -> write idiom of neuzip/__init__.py:25-35
     with Adam moments kept dense in fp32)."""
 
-    def __init__(self, params, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01):
+    def __init__(self, params, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, group=1):
+        """``group``: parameters are read, updated and written back ``group`` at a
+        time (the Linears of one block), so that a per-block decode serves all
+        of them before the first write makes it stale."""
         self.params = list(params)
+        self.group = max(1, int(group))
         self.lr, self.b1, self.b2, self.eps, self.wd = lr, betas[0], betas[1], eps, weight_decay
         self.state = {}
         self.t = 0
@@ -221,22 +225,25 @@ class CompressedAdamW:
         self.t += 1
         c1 = 1.0 - self.b1 ** self.t
         c2 = 1.0 - self.b2 ** self.t
-        for p in self.params:
-            g = p._gradient
-            if g is None:
-                continue
-            st = self.state.get(p._handle)
-            if st is None:
-                st = (torch.zeros_like(g, dtype=torch.float32), torch.zeros_like(g, dtype=torch.float32))
-                self.state[p._handle] = st
-            m, v = st
-            gf = g.float()
-            m.mul_(self.b1).add_(gf, alpha=1 - self.b1)
-            v.mul_(self.b2).addcmul_(gf, gf, value=1 - self.b2)
-            w = p()  # decompress
-            wf = w.float()
-            wf.mul_(1 - self.lr * self.wd)
-            wf.addcdiv_(m, (v / c2).sqrt_().add_(self.eps), value=-self.lr / c1)
-            p._manager.write(wf.to(w.dtype), p._handle)  # re-compress
-            p._gradient = None
-            p.grad = None
+        todo = [p for p in self.params if p._gradient is not None]
+        for at in range(0, len(todo), self.group):
+            batch = todo[at:at + self.group]
+            new = []
+            for p in batch:
+                g = p._gradient
+                st = self.state.get(p._handle)
+                if st is None:
+                    st = (torch.zeros_like(g, dtype=torch.float32), torch.zeros_like(g, dtype=torch.float32))
+                    self.state[p._handle] = st
+                m, v = st
+                gf = g.float()
+                m.mul_(self.b1).add_(gf, alpha=1 - self.b1)
+                v.mul_(self.b2).addcmul_(gf, gf, value=1 - self.b2)
+                wf = p.shared().float()  # decompress (read only: the float copy is what changes)
+                wf.mul_(1 - self.lr * self.wd)
+                wf.addcdiv_(m, (v / c2).sqrt_().add_(self.eps), value=-self.lr / c1)
+                new.append(wf.to(torch.bfloat16))
+            for p, w in zip(batch, new):
+                p._manager.write(w, p._handle)  # re-compress
+                p._gradient = None
+                p.grad = None

@@ -284,6 +284,7 @@ class Manager:
         three times and encoded once per step)."""
         normalizer_size = 0 if normalizer_size is None else normalizer_size
         self.meta_dict = {}  # handle -> original shape
+        self._writes = 0     # bumped by every write: lets caches of decoded weights notice
         if algorithm == Algorithm.dummy:
             self._be = _DenseBackend()
             return
@@ -304,6 +305,7 @@ class Manager:
     def write(self, tensor: torch.Tensor, handle: Optional[str] = None) -> str:
         key = str(len(self.meta_dict)) if handle is None else handle
         self.meta_dict[key] = tensor.shape
+        self._writes += 1
         self._be.write(key, tensor)  # note the argument order of the backend
         return key
 
@@ -311,6 +313,12 @@ class Manager:
         shape = self.meta_dict[handle]  # KeyError for an unknown handle, as in the reference
         flat = self._be.read(handle)
         return flat.requires_grad_(False).reshape(shape)
+
+    def read_shared(self, handle: str) -> torch.Tensor:
+        """Like ``read``, but the result may be a view of a buffer that the next
+        call on this manager reuses: for callers that only read the weight and
+        drop it at once (the backward pass of a compressed Linear)."""
+        return self.read(handle)
 
     def size(self, handle: str) -> int:
         return self._be.size(handle)
@@ -359,6 +367,7 @@ class Manager:
                 raise RuntimeError(f"checkpoint has {key}={state.get(key)}, this manager {key}={mine}")
         for handle, ent in state["entries"].items():
             shape = torch.Size(ent["shape"])
+            self._writes += 1
             self._be.import_(handle, ent["container"], ent["packed"], ent.get("normalizers"))
             if self._be.numel(handle) != shape.numel():
                 raise RuntimeError(f"entry {handle!r}: shape {tuple(shape)} does not match the stored element count")

@@ -25,6 +25,13 @@ class Parameter(torch.nn.Parameter):
         dense = self._manager.read(self._handle)
         return dense.reshape(self._shape).to(self.device).requires_grad_(False)
 
+    @torch.no_grad()
+    def shared(self) -> torch.Tensor:
+        """The dense weight for a caller that only reads it and drops it at once
+        (may be a view of a buffer the manager reuses)."""
+        dense = self._manager.read_shared(self._handle) if hasattr(self._manager, "read_shared") else self()
+        return dense.reshape(self._shape)
+
     def linear(self, inputs, bias=None):
         return self._manager.linear(self._handle, inputs, bias).to(self.device)
 

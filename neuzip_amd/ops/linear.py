@@ -37,7 +37,7 @@ class CompressedLinear(torch.autograd.Function):
 
         x2d = _as_rows(x)
         go2d = _as_rows(grad_output)
-        dense_w = _p()
+        dense_w = _p.shared()
 
         grad_x = torch.mm(go2d, dense_w).reshape(x.shape).to(ctx._inputs_dtype)
         del dense_w

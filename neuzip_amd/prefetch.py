@@ -46,13 +46,13 @@ def _default_blocks(model: torch.nn.Module):
 class _Slot:
     """One static dense buffer able to hold the weights of any block."""
 
-    __slots__ = ("buf", "ready", "block", "used")
+    __slots__ = ("buf", "ready", "block", "stamp")
 
     def __init__(self, numel: int, device):
         self.buf = torch.empty(numel, dtype=torch.bfloat16, device=device)
         self.ready = None  # event of a side-stream decode the consumer has not waited for yet
         self.block = -1    # index of the block whose weights the buffer holds (or will hold)
-        self.used = False  # a forward pass already consumed this decode
+        self.stamp = -1    # the manager's write counter when the block was decoded
 
 
 class DecompressAhead:
@@ -88,16 +88,19 @@ class DecompressAhead:
                         for offs, hs in zip(self._offsets, self._handles)] for s in self._slots]
         self.stream = torch.cuda.Stream() if self.ahead else None  # default priority
         self._enabled = False
+        self._last, self._step = -1, 1  # block visited last, direction of the walk
 
     # -- context management ---------------------------------------------------
     def enable(self):
         if not self._enabled:
-            self.manager.linear = self._linear  # instance attribute shadows the method
+            self.manager.linear = self._linear  # instance attributes shadow the methods
+            self.manager.read_shared = self._read_shared
             self._enabled = True
 
     def disable(self):
         if self._enabled:
             del self.manager.linear
+            del self.manager.read_shared
             self.join()
             self._enabled = False
 
@@ -112,14 +115,16 @@ class DecompressAhead:
     def join(self):
         """Make the current stream wait for any decode still running on the side
         stream and forget what the buffers hold (call before ending a stream
-        capture, and after the weights were rewritten)."""
+        capture).  Writes through the manager need no call: a decoded block is
+        used only while the manager's write counter is what it was at decode time."""
         cur = torch.cuda.current_stream()
         for s in self._slots:
             if s.ready is not None:
                 cur.wait_event(s.ready)
             s.ready = None
             s.block = -1
-            s.used = False
+            s.stamp = -1
+        self._last, self._step = -1, 1
 
     # -- the hook ---------------------------------------------------------------
     # Stream order does most of the work: the consumer stream decodes, computes
@@ -133,7 +138,7 @@ class DecompressAhead:
             slot.ready = None
         self.manager._be.read_batch(self._plans[bi], self._views[slot_i][bi])
         slot.block = bi
-        slot.used = False
+        slot.stamp = self.manager._writes
 
     def _decode_ahead(self, bi: int, slot_i: int, cur) -> None:
         slot = self._slots[slot_i]
@@ -145,15 +150,20 @@ class DecompressAhead:
             slot.ready = torch.cuda.Event()
             slot.ready.record(self.stream)
         slot.block = bi
-        slot.used = False
+        slot.stamp = self.manager._writes
 
     def _weight(self, handle: str):
         bi, k = self._where[handle]
+        now = self.manager._writes
         slot_i = next((i for i, s in enumerate(self._slots) if s.block == bi), None)
-        if k == 0 and slot_i is not None and self._slots[slot_i].used:
-            self._slots[slot_i].block = -1  # left over from an earlier pass: decode again
+        if slot_i is not None and self._slots[slot_i].stamp != now:
+            self._slots[slot_i].block = -1  # decoded before a later write: decode again
             slot_i = None
-        if k == 0 or slot_i is None:
+        entering = bi != self._last
+        if entering:
+            self._step = -1 if bi < self._last else 1  # backward passes walk the blocks in reverse
+            self._last = bi
+        if entering or slot_i is None:
             cur = torch.cuda.current_stream()
             if slot_i is None:
                 slot_i = next((i for i, s in enumerate(self._slots) if s.block < 0), 0)
@@ -162,19 +172,24 @@ class DecompressAhead:
             if slot.ready is not None:  # join the side stream once per block
                 cur.wait_event(slot.ready)
                 slot.ready = None
-            slot.used = True
-            if self.ahead and k == 0 and (self.wrap or bi + 1 < len(self._handles)):
-                nxt = (bi + 1) % len(self._handles)
+            nxt = bi + self._step
+            if self.ahead and entering and (self.wrap or 0 <= nxt < len(self._handles)):
+                nxt %= len(self._handles)
                 other = 1 - slot_i
-                if self._slots[other].block != nxt or self._slots[other].used:
+                if self._slots[other].block != nxt or self._slots[other].stamp != now:
                     if self._slots[other].ready is not None:  # never consumed: keep the streams joined
                         cur.wait_event(self._slots[other].ready)
                         self._slots[other].ready = None
                     self._decode_ahead(nxt, other, cur)
-        elif self._slots[slot_i].ready is not None:  # the block was entered at another Linear than its first
+        elif self._slots[slot_i].ready is not None:
             torch.cuda.current_stream().wait_event(self._slots[slot_i].ready)
             self._slots[slot_i].ready = None
         return self._views[slot_i][bi][k]
+
+    def _read_shared(self, handle: str) -> torch.Tensor:
+        if handle in self._where:
+            return self._weight(handle).view(self.manager.meta_dict[handle])
+        return type(self.manager).read_shared(self.manager, handle)
 
     def _linear(self, handle: str, inputs: torch.Tensor, bias=None) -> torch.Tensor:
         shape = self.manager.meta_dict[handle]
