@@ -372,6 +372,7 @@ def run_gpt2m(args, torch):
 
     be.read, be.write = timed(be.read, "decode"), timed(be.write, "encode")
     be.read_batch = timed(be.read_batch, "decode")
+    be.write_batch = timed(be.write_batch, "encode")
 
     def run(group):
         """-> per-step figures with the Linears decoded one by one (group 1) or per block"""

@@ -243,7 +243,10 @@ class CompressedAdamW:
                 wf.mul_(1 - self.lr * self.wd)
                 wf.addcdiv_(m, (v / c2).sqrt_().add_(self.eps), value=-self.lr / c1)
                 new.append(wf.to(torch.bfloat16))
-            for p, w in zip(batch, new):
-                p._manager.write(w, p._handle)  # re-compress
+            if len(batch) > 1:
+                batch[0]._manager.write_many(new, [p._handle for p in batch])  # re-compress, one sync
+            else:
+                batch[0]._manager.write(new[0], batch[0]._handle)
+            for p in batch:
                 p._gradient = None
                 p.grad = None

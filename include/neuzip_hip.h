@@ -144,6 +144,15 @@ void nz_manager_destroy(nz_manager* m);
 int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint64_t n,
                      int dtype, void* stream);
 
+/* Up to 16 writes with ONE host synchronisation: the device work of all tensors
+   is enqueued back to back, the container sizes come back together, then the
+   exact-size buffers are filled (an optimizer step that re-compresses the
+   weights of a block pays one sync instead of one per weight,
+   cuda/high_level.cu:114-115 per call).  Same semantics per entry as
+   nz_manager_write; a name may appear only once. */
+int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* const* dev_data,
+                           const uint64_t* ns, uint32_t count, int dtype, void* stream);
+
 /* Manager::read(name), cuda/high_level.cu:223-250, into caller-owned memory of
    at least `cap_elems` elements.  Asynchronous on `stream` (the reference
    blocks the host here, :203; callers that need that call hipStreamSynchronize). */

@@ -26,7 +26,7 @@ LANE_SYMS_AUTO = 0xFFFFFFFF
 EXPORTS = [
     "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",
     "nz_encode_workspace_bytes", "nz_norm_bytes", "nz_split", "nz_encode", "nz_decode",
-    "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
+    "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_write_batch", "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
     "nz_manager_meta", "nz_manager_size", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
     "nz_manager_norm_bytes", "nz_manager_buffers", "nz_manager_erase", "nz_manager_check", "nz_manager_export", "nz_manager_import", "nz_manager_trim",
 ]
@@ -73,6 +73,9 @@ def load() -> ctypes.CDLL:
     L.nz_manager_destroy.argtypes = [vp]
     L.nz_manager_write.restype = i32
     L.nz_manager_write.argtypes = [vp, ctypes.c_char_p, vp, u64, i32, vp]
+    L.nz_manager_write_batch.restype = i32
+    L.nz_manager_write_batch.argtypes = [vp, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(vp), ctypes.POINTER(u64),
+                                         u32, i32, vp]
     L.nz_manager_read.restype = i32
     L.nz_manager_read.argtypes = [vp, ctypes.c_char_p, vp, u64, vp]
     L.nz_manager_trim.restype = i32

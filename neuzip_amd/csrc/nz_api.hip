@@ -257,7 +257,7 @@ struct nz_manager {
   void* ws = nullptr;
   uint64_t ws_bytes = 0;
   uint32_t* d_status = nullptr;
-  uint64_t* h_pin = nullptr;  // pinned: [0] total, [1] status
+  uint64_t* h_pin = nullptr;  // pinned: [0..15] container sizes of a write batch, [16] status
   long long* gemv_acc = nullptr;  // row accumulators of the matrix-vector product (all zero between calls)
   uint64_t gemv_rows = 0;         // rows the accumulator buffer can hold
 };
@@ -417,7 +417,7 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   m->auto_lanes = auto_lanes;
   hipError_t e = hipMalloc((void**)&m->d_status, 256);
   if (e == hipSuccess) e = hipMemset(m->d_status, 0, 256);
-  if (e == hipSuccess) e = hipHostMalloc((void**)&m->h_pin, 64, hipHostMallocDefault);
+  if (e == hipSuccess) e = hipHostMalloc((void**)&m->h_pin, 256, hipHostMallocDefault);
   if (e != hipSuccess) {
     if (m->d_status) (void)hipFree(m->d_status);
     delete m;
@@ -441,17 +441,36 @@ void nz_manager_destroy(nz_manager* m) {
   delete m;
 }
 
-int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint64_t n, int dtype,
-                     void* stream) {
-  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
-  if (dtype != NZ_DTYPE_BF16) return fail(NZ_ERR_DTYPE, "Unsupported data type");
-  if (n && !dev_data) return fail(NZ_ERR_ARG, "null data pointer");
-  if ((uintptr_t)dev_data & 15) return fail(NZ_ERR_ALIGN, "dense input must be 16-byte aligned");
-  // Throughput of both codec directions is set by the number of wavefronts in
-  // flight (one per 64 * lane_syms elements).  In auto mode a tensor too small
-  // to give every SIMD two wavefronts at the default gets shorter segments
-  // (and, with the library's own chunk, the smaller 64 Ki table scope that
-  // allows them), at ~4.5 bits per extra lane.
+}  // extern "C"
+
+// ---- write: begin (everything up to the directory, on the device) | one host
+// ---- synchronisation for the sizes | finish (exact-size buffer, compaction) ----
+
+#define NZ_WRITE_BATCH_MAX 16
+
+namespace {
+
+struct PendingWrite {
+  std::string name;
+  Entry ent, old;
+  NzGeom g;
+  EncLayout L;
+  uint8_t* ws = nullptr;
+};
+
+void release_entry(Entry& e) {
+  if (e.comp) (void)hipFree(e.comp);
+  if (e.packed) (void)hipFree(e.packed);
+  if (e.norm) (void)hipFree(e.norm);
+  e.comp = e.packed = e.norm = nullptr;
+}
+
+// Geometry of a tensor of n elements.  Throughput of both codec directions is
+// set by the number of wavefronts in flight (one per 64 * lane_syms elements).
+// In auto mode a tensor too small to give every SIMD two wavefronts at the
+// default gets shorter segments (and, with the library's own chunk, the smaller
+// 64 Ki table scope that allows them), at ~4.5 bits per extra lane.
+int pick_geometry(const nz_manager* m, uint64_t n, NzGeom* g, uint32_t* chunk_out, uint32_t* lane_out) {
   uint32_t lane_syms = m->lane_syms, chunk_syms = m->chunk_syms;
   if (m->auto_lanes) {
     if (m->own_chunk && n / ((uint64_t)lane_syms * NZ_LANES) < 2048) {
@@ -462,44 +481,36 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
            n / ((uint64_t)lane_syms * NZ_LANES) < 2048)
       lane_syms = (lane_syms / 2 + 7) & ~7u;
   }
-  NzGeom g;
-  if (int rc = make_geom(&g, n, chunk_syms, lane_syms)) return rc;
-  hipStream_t st = (hipStream_t)stream;
-  std::lock_guard<std::mutex> lock(m->mu);
+  *chunk_out = chunk_syms;
+  *lane_out = lane_syms;
+  return make_geom(g, n, chunk_syms, lane_syms);
+}
 
-  const EncLayout L = enc_layout(g);
-  if (m->ws_bytes < L.bytes) {
-    // the previous scratch may still be in use by kernels on the stream
-    NZ_HIP(hipStreamSynchronize(st));
-    if (m->ws) NZ_HIP(hipFree(m->ws));
-    m->ws = nullptr;
-    m->ws_bytes = 0;
-    NZ_HIP(hipMalloc(&m->ws, L.bytes));
-    m->ws_bytes = L.bytes;
-  }
-  uint8_t* ws = (uint8_t*)m->ws;
-
-  // cuda/high_level.cu:137-140: an existing entry is replaced.  Its buffers are
-  // reused when large enough, which also avoids a device-wide hipFree stall.
-  Entry old;
+// Takes the entry `name` out of the store (cuda/high_level.cu:137-140: an existing
+// entry is replaced; its buffers are reused when large enough, which also avoids
+// a device-wide hipFree stall), allocates what has a known size and enqueues
+// everything up to the directory into the scratch slice `ws`.
+int write_begin(nz_manager* m, const char* name, const void* dev_data, uint64_t n, int dtype,
+                uint32_t chunk_syms, uint32_t lane_syms, const NzGeom& g, uint8_t* ws, PendingWrite* pw,
+                hipStream_t st) {
+  pw->name = name;
+  pw->g = g;
+  pw->L = enc_layout(g);
+  pw->ws = ws;
   auto it = m->entries.find(name);
   if (it != m->entries.end()) {
-    old = it->second;
+    pw->old = it->second;
     m->entries.erase(it);
   }
-  Entry ent;
+  Entry& ent = pw->ent;
+  Entry& old = pw->old;
   ent.n = n;
   ent.dtype = dtype;
   ent.lane_syms = lane_syms;
   ent.chunk_syms = chunk_syms;
   ent.packed_bytes = nz_packed_stored_bytes_of(&g, m->precision);
   ent.norm_bytes = norm_bytes_of(n, m->normalizer);
-  auto release = [&](Entry& e) {
-    if (e.comp) (void)hipFree(e.comp);
-    if (e.packed) (void)hipFree(e.packed);
-    if (e.norm) (void)hipFree(e.norm);
-    e.comp = e.packed = e.norm = nullptr;
-  };
+  hipError_t e = hipSuccess;
   if (ent.norm_bytes) {
     if (old.norm && old.norm_cap >= ent.norm_bytes && old.norm_cap <= ent.norm_bytes + 4096) {
       ent.norm = old.norm;
@@ -507,68 +518,119 @@ int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint
       old.norm = nullptr;
     } else {
       ent.norm_cap = ent.norm_bytes + 8;
-      hipError_t e = hipMalloc(&ent.norm, ent.norm_cap);
-      if (e != hipSuccess) {
-        release(old);
-        return fail(NZ_ERR_HIP, std::string("hipMalloc(normalizers): ") + hipGetErrorString(e));
-      }
+      e = hipMalloc(&ent.norm, ent.norm_cap);
     }
   }
-  if (old.packed && old.packed_cap >= ent.packed_bytes && old.packed_cap <= ent.packed_bytes + 4096) {
-    ent.packed = old.packed;
-    ent.packed_cap = old.packed_cap;
-    old.packed = nullptr;
-  } else {
-    ent.packed_cap = ent.packed_bytes ? ent.packed_bytes : 8;
-    hipError_t e = hipMalloc(&ent.packed, ent.packed_cap);
-    if (e != hipSuccess) {
-      release(old);
-      release(ent);
-      return fail(NZ_ERR_HIP, std::string("hipMalloc(packed): ") + hipGetErrorString(e));
+  if (e == hipSuccess) {
+    if (old.packed && old.packed_cap >= ent.packed_bytes && old.packed_cap <= ent.packed_bytes + 4096) {
+      ent.packed = old.packed;
+      ent.packed_cap = old.packed_cap;
+      old.packed = nullptr;
+    } else {
+      ent.packed_cap = ent.packed_bytes ? ent.packed_bytes : 8;
+      e = hipMalloc(&ent.packed, ent.packed_cap);
     }
   }
+  if (e == hipSuccess) e = hipMemsetAsync(ws + pw->L.status, 0, 4, st);
+  if (e != hipSuccess) return fail(NZ_ERR_HIP, std::string("write: ") + hipGetErrorString(e));
+  return encode_phase1(g, m->precision, dev_data, (uint8_t*)ent.packed, ws, pw->L, ws + pw->L.hdr, ~0ull,
+                       (uint64_t*)(ws + pw->L.total), (uint32_t*)(ws + pw->L.status), m->normalizer,
+                       (uint8_t*)ent.norm, st);
+}
 
-  uint64_t* d_total = (uint64_t*)(ws + L.total);
-  uint32_t* d_estat = (uint32_t*)(ws + L.status);
-  hipError_t e = hipMemsetAsync(d_estat, 0, 4, st);
-  int rc = e == hipSuccess ? NZ_OK : fail(NZ_ERR_HIP, hipGetErrorString(e));
-  if (rc == NZ_OK)
-    rc = encode_phase1(g, m->precision, dev_data, (uint8_t*)ent.packed, ws, L, ws + L.hdr,
-                       ~0ull, d_total, d_estat, m->normalizer, (uint8_t*)ent.norm, st);
+// With the container size known on the host: exact-size buffer, header copy, compaction.
+int write_finish(nz_manager* m, PendingWrite* pw, uint64_t total, hipStream_t st) {
+  Entry& ent = pw->ent;
+  Entry& old = pw->old;
+  const NzGeom& g = pw->g;
+  ent.comp_bytes = total;
+  hipError_t e = hipSuccess;
+  if (old.comp && old.comp_cap >= ent.comp_bytes && old.comp_cap <= ent.comp_bytes + ent.comp_bytes / 16 + 4096) {
+    ent.comp = old.comp;
+    ent.comp_cap = old.comp_cap;
+    old.comp = nullptr;
+  } else {
+    // a little headroom: the next write of this handle (an optimizer step
+    // later) is a few bytes longer or shorter and can reuse the buffer
+    ent.comp_cap = ent.comp_bytes + ent.comp_bytes / 64 + 1024;
+    e = hipMalloc(&ent.comp, ent.comp_cap);
+  }
+  if (e == hipSuccess)
+    e = hipMemcpyAsync(ent.comp, pw->ws + pw->L.hdr, g.rec_off + (g.n_segs ? 0 : NZ_TAIL_PAD),
+                       hipMemcpyDeviceToDevice, st);
+  if (e != hipSuccess) return fail(NZ_ERR_HIP, std::string("write: ") + hipGetErrorString(e));
+  if (int rc = encode_phase2(g, pw->ws, pw->L, (const uint32_t*)(pw->ws + pw->L.hdr + g.dir_off),
+                             (uint8_t*)ent.comp, ent.comp_cap, st))
+    return rc;
+  m->entries.emplace(pw->name, ent);
+  ent = Entry();  // now owned by the store
+  return NZ_OK;
+}
+
+int grow_workspace(nz_manager* m, uint64_t bytes, hipStream_t st) {
+  if (m->ws_bytes >= bytes) return NZ_OK;
+  // the previous scratch may still be in use by kernels on the stream
+  NZ_HIP(hipStreamSynchronize(st));
+  if (m->ws) NZ_HIP(hipFree(m->ws));
+  m->ws = nullptr;
+  m->ws_bytes = 0;
+  NZ_HIP(hipMalloc(&m->ws, bytes));
+  m->ws_bytes = bytes;
+  return NZ_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* const* dev_data,
+                           const uint64_t* ns, uint32_t count, int dtype, void* stream) {
+  if (!m || (count && (!names || !dev_data || !ns))) return fail(NZ_ERR_ARG, "null manager, names, data or sizes");
+  if (dtype != NZ_DTYPE_BF16) return fail(NZ_ERR_DTYPE, "Unsupported data type");
+  if (count > NZ_WRITE_BATCH_MAX) return fail(NZ_ERR_ARG, "at most 16 tensors per batch");
+  hipStream_t st = (hipStream_t)stream;
+  // check everything and size the scratch before anything is touched
+  NzGeom g[NZ_WRITE_BATCH_MAX];
+  uint32_t chunk[NZ_WRITE_BATCH_MAX], lane[NZ_WRITE_BATCH_MAX];
+  uint64_t at[NZ_WRITE_BATCH_MAX + 1];
+  at[0] = 0;
+  for (uint32_t i = 0; i < count; ++i) {
+    if (!names[i]) return fail(NZ_ERR_ARG, "null name");
+    for (uint32_t j = 0; j < i; ++j)
+      if (std::strcmp(names[i], names[j]) == 0) return fail(NZ_ERR_ARG, "a name appears twice in the batch");
+    if (ns[i] && !dev_data[i]) return fail(NZ_ERR_ARG, "null data pointer");
+    if ((uintptr_t)dev_data[i] & 15) return fail(NZ_ERR_ALIGN, "dense input must be 16-byte aligned");
+    if (int rc = pick_geometry(m, ns[i], &g[i], &chunk[i], &lane[i])) return rc;
+    at[i + 1] = at[i] + enc_layout(g[i]).bytes;
+  }
+  std::lock_guard<std::mutex> lock(m->mu);
+  if (int rc = grow_workspace(m, at[count], st)) return rc;
+  PendingWrite pw[NZ_WRITE_BATCH_MAX];
+  int rc = NZ_OK;
+  uint32_t begun = 0;
+  for (; begun < count && rc == NZ_OK; ++begun)
+    rc = write_begin(m, names[begun], dev_data[begun], ns[begun], dtype, chunk[begun], lane[begun], g[begun],
+                     (uint8_t*)m->ws + at[begun], &pw[begun], st);
   if (rc == NZ_OK) {
-    e = hipMemcpyAsync(m->h_pin, d_total, 8, hipMemcpyDeviceToHost, st);
-    if (e == hipSuccess) e = hipStreamSynchronize(st);  // the one host sync of a write
+    hipError_t e = hipSuccess;
+    for (uint32_t i = 0; i < count && e == hipSuccess; ++i)
+      e = hipMemcpyAsync(&m->h_pin[i], pw[i].ws + pw[i].L.total, 8, hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);  // the one host sync of the batch
     if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("size readback: ") + hipGetErrorString(e));
   }
-  if (rc == NZ_OK) {
-    ent.comp_bytes = m->h_pin[0];
-    if (old.comp && old.comp_cap >= ent.comp_bytes && old.comp_cap <= ent.comp_bytes + ent.comp_bytes / 16 + 4096) {
-      ent.comp = old.comp;
-      ent.comp_cap = old.comp_cap;
-      old.comp = nullptr;
-    } else {
-      // a little headroom: the next write of this handle (an optimizer step
-      // later) is a few bytes longer or shorter and can reuse the buffer
-      ent.comp_cap = ent.comp_bytes + ent.comp_bytes / 64 + 1024;
-      e = hipMalloc(&ent.comp, ent.comp_cap);
-      if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("hipMalloc(comp): ") + hipGetErrorString(e));
-    }
+  for (uint32_t i = 0; i < count && rc == NZ_OK; ++i) rc = write_finish(m, &pw[i], m->h_pin[i], st);
+  // whatever did not make it into the store is released, old buffers in any case
+  for (uint32_t i = 0; i < begun; ++i) {
+    release_entry(pw[i].old);
+    release_entry(pw[i].ent);
   }
-  if (rc == NZ_OK) {
-    e = hipMemcpyAsync(ent.comp, ws + L.hdr, g.rec_off + (g.n_segs ? 0 : NZ_TAIL_PAD),
-                       hipMemcpyDeviceToDevice, st);
-    if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("header copy: ") + hipGetErrorString(e));
-  }
-  if (rc == NZ_OK)
-    rc = encode_phase2(g, ws, L, (const uint32_t*)(ws + L.hdr + g.dir_off), (uint8_t*)ent.comp,
-                       ent.comp_cap, st);
-  release(old);
-  if (rc != NZ_OK) {
-    release(ent);
-    return rc;
-  }
-  m->entries.emplace(name, ent);
-  return NZ_OK;
+  return rc;
+}
+
+int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint64_t n, int dtype,
+                     void* stream) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  return nz_manager_write_batch(m, &name, &dev_data, &n, 1, dtype, stream);
 }
 
 int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap_elems,
@@ -932,10 +994,11 @@ int nz_manager_check(nz_manager* m, void* stream) {
   if (!m) return fail(NZ_ERR_ARG, "null manager");
   hipStream_t st = (hipStream_t)stream;
   std::lock_guard<std::mutex> lock(m->mu);
-  NZ_HIP(hipMemcpyAsync(&m->h_pin[1], m->d_status, 4, hipMemcpyDeviceToHost, st));
+  m->h_pin[16] = 0;
+  NZ_HIP(hipMemcpyAsync(&m->h_pin[16], m->d_status, 4, hipMemcpyDeviceToHost, st));
   NZ_HIP(hipMemsetAsync(m->d_status, 0, 4, st));
   NZ_HIP(hipStreamSynchronize(st));
-  const uint32_t hs = (uint32_t)m->h_pin[1];
+  const uint32_t hs = (uint32_t)m->h_pin[16];
   if (hs == 8u) return fail(NZ_ERR_CORRUPT, "a row gather was given an index outside the table");
   if (hs) return fail(NZ_ERR_CORRUPT, "a read saw a container that failed validation (status " + std::to_string(hs) + ")");
   return NZ_OK;

@@ -447,3 +447,25 @@ def test_trim_releases_the_write_scratch():
     mgr.write(w * 2, h)                             # and a write brings it back
     assert torch.equal(mgr.read(h), w * 2)
     mgr._be.check()
+
+
+def test_write_many_equals_single_writes(oracle):
+    import neuzip_amd
+
+    for lane in (0, "auto"):
+        one, many = neuzip_amd.Manager(lane_symbols=lane), neuzip_amd.Manager(lane_symbols=lane)
+        sizes = [(64, 1000), (3,), (0,), (300_000,), (1 << 20,)] + [(1000 + i,) for i in range(14)]  # 19 tensors
+        ws = [from_bits(bf16_bits_normal(int(np.prod(s)), seed=i), s) for i, s in enumerate(sizes)]
+        hs = [f"w{i}" for i in range(len(ws))]
+        many.write(ws[3], hs[0])  # replaced by the batch
+        for w, h in zip(ws, hs):
+            one.write(w, h)
+        many.write_many(ws, hs)
+        for w, h in zip(ws, hs):
+            assert many.size(h) == one.size(h)
+            assert torch.equal(many.read(h), w) and many.read(h).shape == w.shape
+        a, b = one._be.export(hs[4]), many._be.export(hs[4])
+        assert all(torch.equal(x, y) for x, y in zip(a, b))
+        with pytest.raises(ValueError):
+            many.write_many(ws[:2], ["same", "same"])
+        many._be.check()
