@@ -114,8 +114,9 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
               void* stream);
 
 /* Manager::_decompress_and_merge, cuda/high_level.cu:169-206: entropy decode
-   and merge in one kernel.  `dev_status` (device uint32, may be NULL) is
-   OR-ed with a non-zero value when the container fails validation; with
+   and merge in one kernel.  `dev_status` (device uint32, zeroed by the
+   caller) is OR-ed with a non-zero value when the container fails validation
+   (bit 4: the header does not name n / chunk_size / lane_syms as passed); with
    `check` != 0 the call synchronises and returns NZ_ERR_CORRUPT in that
    case.  chunk_size / lane_syms must be the ones used to encode. */
 int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed, uint64_t n,

@@ -364,7 +364,7 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
   if ((uintptr_t)dev_bf16_out & 15) return fail(NZ_ERR_ALIGN, "dense output must be 16-byte aligned");
   if (((uintptr_t)dev_comp & 15) || ((uintptr_t)dev_packed & 7))
     return fail(NZ_ERR_ALIGN, "comp/packed buffers must be 16/8-byte aligned");
-  if (check && !dev_status) return fail(NZ_ERR_ARG, "check requires dev_status");
+  if (!dev_status) return fail(NZ_ERR_ARG, "dev_status is required (the kernel reports there)");
   if (comp_bytes < g.rec_off + NZ_TAIL_PAD) return fail(NZ_ERR_CORRUPT, "container shorter than its directory");
   hipStream_t st = (hipStream_t)stream;
   if (int rc = decode_launch(g, precision, dev_comp, comp_bytes, dev_packed, dev_bf16_out, dev_status,

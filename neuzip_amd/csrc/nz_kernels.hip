@@ -990,6 +990,14 @@ __device__ __forceinline__ void nz_decode_chunk(
   const uint32_t nseg = (cn + g.seg_syms - 1) / g.seg_syms;
   const uint32_t* dir = reinterpret_cast<const uint32_t*>(comp + g.dir_off);
 
+  // the container must be the one the caller's geometry describes
+  if (c == 0 && tid == 0) {
+    const uint32_t* h = reinterpret_cast<const uint32_t*>(comp);
+    if (h[0] != NZ_MAGIC || h[1] != NZ_FORMAT_VERSION || h[2] != (uint32_t)g.n || h[3] != (uint32_t)(g.n >> 32) ||
+        h[4] != g.chunk_syms || h[5] != g.lane_syms)
+      atomicOr(d_status, 16u);
+  }
+
   // record of the chunk's first segment starts with the table
   const uint64_t f0 = dir[seg0], f1 = dir[seg0 + 1];
   if (f1 <= f0 || g.rec_off + 4 * f1 > comp_bytes) {

@@ -161,6 +161,23 @@ def test_corrupt_container_is_reported(oracle):
     assert rc == -6
 
 
+def test_geometry_mismatch_is_reported(oracle):
+    """A container decoded with another geometry than it was written with is
+    refused (the header names its own), not turned into garbage."""
+    from neuzip_amd import _lib
+
+    n = 200_000
+    bits = bf16_bits_normal(n, 8)
+    comp, packed = gpu_encode(bits, 7, 65536, 344)
+    for chunk, lane in ((65536, 512), (131072, 256)):
+        print(f"case mismatch chunk={chunk} lane={lane}", flush=True)
+        pk = torch.cat([packed, torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")])  # sizes differ per geometry
+        rc, _ = gpu_decode(comp, pk, n, 7, chunk, lane)
+        assert rc == _lib.ERR_CORRUPT
+    rc, out = gpu_decode(comp, packed, n, 7, 65536, 344)
+    assert rc == 0 and np.array_equal(out, bits)
+
+
 def test_ratio_close_to_entropy(oracle):
     n = 4096 * 4096
     bits = bf16_bits_normal(n, seed=0)
