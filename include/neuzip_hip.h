@@ -176,9 +176,10 @@ int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* 
    stored tensor is read as a row-major matrix with rows of `in_features`
    elements (a multiple of 512).  dev_x: in_features bf16, 16-byte aligned;
    dev_y[i]: rows_i bf16; dev_bias: null, or per matrix null / rows_i bf16.
-   Sums are formed in fp32 per wavefront and row, then in 34.30 fixed point
+   Sums are formed in fp32 per wavefront and row, then in 24.40 fixed point
    across wavefronts, so the result does not depend on scheduling; a row whose
-   partial sums are NaN, infinite or beyond 2^26 in magnitude comes out as NaN.
+   partial sums are NaN, infinite or beyond 2^18 in magnitude comes out as NaN; sums
+   are resolved to 2^-40.
    Calls of one manager must be ordered on one stream (they share the
    accumulators, which are allocated on first use and grown when needed; no
    other call allocates).  Asynchronous on `stream`. */

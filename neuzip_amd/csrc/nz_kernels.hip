@@ -789,14 +789,16 @@ __device__ __forceinline__ uint4 nz_merge_group(uint64_t sm, const uint32_t (&ew
 // is a multiple of 512), so the row of a group is the same for all lanes.  A
 // lane keeps an fp32 partial sum of its 8-element dot products; when the wave
 // leaves a row the 64 partial sums are added in a fixed butterfly order and
-// lane 0 adds the result, converted to 34.30 fixed point, to the row's 64-bit
+// lane 0 adds the result, converted to 24.40 fixed point, to the row's 64-bit
 // accumulator.  Integer addition is associative, so the value of y does not
 // depend on the order in which the wavefronts that share a row arrive.  A
-// partial sum that is NaN, infinite or beyond 2^26 sets the row's flag word
+// partial sum that is NaN, infinite or beyond 2^18 sets the row's flag word
 // instead (the row then comes out as NaN).  Row r owns acc[2r] (sum) and
 // acc[2r + 1] (flag).
-#define NZ_GEMV_FRAC_BITS 30
-#define NZ_GEMV_PART_MAX 67108864.0f /* 2^26 */
+// 40 fraction bits: an absolute resolution of 9e-13 per partial sum; up to 16
+// partial sums below 2^18 in magnitude cannot overflow 64 bits.
+#define NZ_GEMV_FRAC_BITS 40
+#define NZ_GEMV_PART_MAX 262144.0f /* 2^18 */
 
 struct NzGemv {
   const uint16_t* x;      // in_features bf16 values, 16-byte aligned
@@ -844,7 +846,7 @@ struct NzGemvWalk {
     if (lane == 0) {
       unsigned long long* slot = reinterpret_cast<unsigned long long*>(acc + 2 * row);
       if (fabsf(t) < NZ_GEMV_PART_MAX)  // false for NaN as well
-        atomicAdd(slot, (unsigned long long)__float2ll_rn(t * (float)(1u << NZ_GEMV_FRAC_BITS)));
+        atomicAdd(slot, (unsigned long long)__float2ll_rn(t * (float)(1ull << NZ_GEMV_FRAC_BITS)));
       else
         atomicOr(slot + 1, 1ull);
     }
@@ -1343,7 +1345,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_gemv_ker
                                  blockIdx.x - first, gv, NzNorm{it.norm, b.log2n});
 }
 
-// y = bf16(acc * 2^-30 + bias), and the accumulators return to zero for the next
+// y = bf16(acc * 2^-40 + bias), and the accumulators return to zero for the next
 // product.  Flagged rows come out as NaN.
 struct NzGemvOutItem {
   long long* acc;
@@ -1372,7 +1374,7 @@ __global__ __launch_bounds__(256) void nz_gemv_finish_kernel(const NzGemvOut o) 
   reinterpret_cast<longlong2*>(it.acc)[i] = make_longlong2(0, 0);
   float y;
   if (a.y) y = __uint_as_float(0x7FC00000u);
-  else y = (float)((double)a.x * (1.0 / (double)(1u << NZ_GEMV_FRAC_BITS)));
+  else y = (float)((double)a.x * (1.0 / (double)(1ull << NZ_GEMV_FRAC_BITS)));
   if (it.bias) y += nz_bf16_to_f32(it.bias[i]);
   it.y[i] = (uint16_t)nz_f32_to_bf16(y);
 }
