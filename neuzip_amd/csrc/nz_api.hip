@@ -106,14 +106,11 @@ int encode_phase1(const NzGeom& g, int precision, const void* in, uint8_t* packe
     }
     hipLaunchKernelGGL(nz_rans_encode_kernel, dim3((uint32_t)g.n_chunks), dim3(64 * g.spc), 0, st,
                        ws + L.exps, g.n, g.chunk_syms, g.lane_syms, g.spc,
-                       (const uint32_t*)(ws + L.enc_tab), (const NzChunkInfo*)(ws + L.info),
+                       (const uint32_t*)(ws + L.enc_tab), (NzChunkInfo*)(ws + L.info),
                        (const uint16_t*)(ws + L.carry), (uint16_t*)(ws + L.slots),
                        (uint32_t*)(ws + L.states),
-                       (uint32_t*)(ws + L.seg_words), (uint32_t*)(ws + L.seg_sbytes));
-    hipLaunchKernelGGL(nz_chunk_finalize_kernel, dim3((uint32_t)((g.n_chunks + 255) / 256)),
-                       dim3(256), 0, st, g.n, g.chunk_syms, g.seg_syms, g.spc, g.n_chunks,
-                       (NzChunkInfo*)(ws + L.info), (const uint32_t*)(ws + L.seg_words),
-                       (const uint32_t*)(ws + L.seg_sbytes), (uint32_t*)(ws + L.seg_units));
+                       (uint32_t*)(ws + L.seg_words), (uint32_t*)(ws + L.seg_sbytes),
+                       (uint32_t*)(ws + L.seg_units));
   }
   hipLaunchKernelGGL(nz_scan_kernel, dim3(1), dim3(1024), 0, st,
                      (const uint32_t*)(ws + L.seg_units), g, hdr, cap, d_total, d_status);

@@ -5,9 +5,8 @@
 //                              + per-chunk exponent histogram, 12-bit frequency
 //                              table and its serialized form
 //   nz_rans_encode_kernel      nvcomp ANS compress       cuda/high_level.cu:103-115
-//   nz_chunk_finalize_kernel   \ exact-size compaction    cuda/high_level.cu:117-124
-//   nz_scan_kernel              > (done on the device, no host round trip
-//   nz_compact_kernel          /  between the kernels)
+//   nz_scan_kernel             \ exact-size compaction    cuda/high_level.cu:117-124
+//   nz_compact_kernel          / (done on the device, no host round trip between the kernels)
 //   nz_decode_kernel           nvcomp ANS decompress + kernel_aligned_merge fused:
 //                              cuda/high_level.cu:184-201, cuda/kernels.cuh:167-217
 //
@@ -471,6 +470,39 @@ __global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
 }
 
 // ----------------------------------------------------------------------------
+// per chunk: coded or raw, and the record size of each of its segments (run by one
+// thread of the encode kernel once all segments of the chunk are coded)
+// ----------------------------------------------------------------------------
+__device__ __forceinline__ void nz_chunk_finalize(uint64_t c, uint64_t n, uint32_t chunk_syms,
+                                                  uint32_t seg_syms, uint32_t spc, NzChunkInfo* info,
+                                                  const uint32_t* seg_words, const uint32_t* seg_state_bytes,
+                                                  uint32_t* seg_units) {
+  const uint64_t base = c * chunk_syms;
+  const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
+  const uint32_t nseg = (cn + seg_syms - 1) / seg_syms;
+  const uint32_t tab_len = info[c].tab_len;
+  uint64_t rans_total = tab_len, raw_total = 4;
+  for (uint32_t k = 0; k < nseg; ++k) {
+    const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
+    const uint32_t w = seg_words[c * spc + k];
+    rans_total += seg_state_bytes[c * spc + k] + 2 * (uint64_t)((w + 1) & ~1u);
+    raw_total += ((sn + 3) & ~3u) + (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
+  }
+  const bool raw = rans_total >= raw_total;
+  info[c].raw = raw ? 1u : 0u;
+  for (uint32_t k = 0; k < nseg; ++k) {
+    const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
+    const uint32_t w = seg_words[c * spc + k];
+    uint32_t bytes;
+    if (raw)
+      bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u) +
+              (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
+    else bytes = (k == 0 ? tab_len : 0u) + seg_state_bytes[c * spc + k] + 2u * ((w + 1) & ~1u);
+    seg_units[c * spc + k] = bytes / 4;
+  }
+}
+
+// ----------------------------------------------------------------------------
 // rANS encode: one workgroup per chunk, one wavefront per segment
 // ----------------------------------------------------------------------------
 //
@@ -479,13 +511,14 @@ __global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
 // slot back to front, so that the decoder reads front to back), then
 // x = (x / f) << 12 | (x % f) + cum.  A segment's slot holds one word per
 // symbol, the most any input can emit, so there is no overflow path; a chunk
-// that codes to more than its raw size is stored raw by the finalize kernel.
+// that codes to more than its raw size is stored raw (decided at the end of this
+// kernel, once all segments of the chunk are coded).
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_kernel(
     const uint8_t* __restrict__ exps, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
-    uint32_t spc, const uint32_t* __restrict__ enc_tab, const NzChunkInfo* __restrict__ info,
+    uint32_t spc, const uint32_t* __restrict__ enc_tab, NzChunkInfo* __restrict__ info,
     const uint16_t* __restrict__ carry, uint16_t* __restrict__ slots,
     uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words,
-    uint32_t* __restrict__ seg_state_bytes) {
+    uint32_t* __restrict__ seg_state_bytes, uint32_t* __restrict__ seg_units) {
   __shared__ uint32_t sbuf[NZ_MAX_SEGS_PER_CHUNK][NZ_STATE_MAX_BYTES / 4];
   // per symbol: x = freq << 20 (renormalisation threshold), y = freq, z = cum,
   // w = bits of 1.0f / freq
@@ -503,7 +536,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
   const uint32_t seg_syms = lane_syms * NZ_LANES;
   const uint64_t seg = c * spc + wave;
   const uint64_t seg_base = c * chunk_syms + (uint64_t)wave * seg_syms;
-  if (seg_base >= n) return;
+  if (seg_base < n) {  // wavefronts beyond the tensor only take part in the barrier below
   const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, wave);
   const uint32_t seg_n = (uint32_t)((n - seg_base) < nom ? (n - seg_base) : nom);
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
@@ -576,42 +609,10 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
     seg_words[seg] = cap_words - pos;
     seg_state_bytes[seg] = sbytes;
   }
-}
-
-// ----------------------------------------------------------------------------
-// per chunk: coded or raw, and the record size of each of its segments
-// ----------------------------------------------------------------------------
-__global__ void nz_chunk_finalize_kernel(uint64_t n, uint32_t chunk_syms, uint32_t seg_syms,
-                                         uint32_t spc, uint64_t n_chunks,
-                                         NzChunkInfo* __restrict__ info,
-                                         const uint32_t* __restrict__ seg_words,
-                                         const uint32_t* __restrict__ seg_state_bytes,
-                                         uint32_t* __restrict__ seg_units) {
-  const uint64_t c = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (c >= n_chunks) return;
-  const uint64_t base = c * chunk_syms;
-  const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
-  const uint32_t nseg = (cn + seg_syms - 1) / seg_syms;
-  const uint32_t tab_len = info[c].tab_len;
-  uint64_t rans_total = tab_len, raw_total = 4;
-  for (uint32_t k = 0; k < nseg; ++k) {
-    const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
-    const uint32_t w = seg_words[c * spc + k];
-    rans_total += seg_state_bytes[c * spc + k] + 2 * (uint64_t)((w + 1) & ~1u);
-    raw_total += ((sn + 3) & ~3u) + (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
   }
-  const bool raw = rans_total >= raw_total;
-  info[c].raw = raw ? 1u : 0u;
-  for (uint32_t k = 0; k < nseg; ++k) {
-    const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
-    const uint32_t w = seg_words[c * spc + k];
-    uint32_t bytes;
-    if (raw)
-      bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u) +
-              (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
-    else bytes = (k == 0 ? tab_len : 0u) + seg_state_bytes[c * spc + k] + 2u * ((w + 1) & ~1u);
-    seg_units[c * spc + k] = bytes / 4;
-  }
+  // every segment of the chunk is coded: decide coded-or-raw and size the records
+  __syncthreads();
+  if (threadIdx.x == 0) nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units);
 }
 
 // ----------------------------------------------------------------------------
@@ -719,10 +720,19 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
   if (tid < sbytes / 4) sdst[tid] = states[seg * (NZ_STATE_MAX_BYTES / 4) + tid];
   const uint32_t w = seg_words[seg];
   const uint32_t cap_words = g.seg_syms;
+  // the words sit at the end of the segment's slot, 2-byte aligned; they are moved
+  // as dwords (two aligned loads and a funnel shift when the source is off by one
+  // word; the load past the last word stays inside the scratch buffer)
   const uint16_t* src = slots + seg * cap_words + (cap_words - w);
-  uint16_t* wdst = reinterpret_cast<uint16_t*>(dst + off + sbytes);
-  for (uint32_t i = tid; i < w; i += 256) wdst[i] = src[i];
-  if ((w & 1) && tid == 0) wdst[w] = 0;
+  const uint32_t mis = (uint32_t)((reinterpret_cast<uintptr_t>(src) >> 1) & 1u);
+  const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src - mis);
+  uint32_t* wdst = reinterpret_cast<uint32_t*>(dst + off + sbytes);
+  const uint32_t nd = (w + 1) / 2;
+  for (uint32_t i = tid; i < nd; i += 256) {
+    uint32_t v = mis ? __builtin_amdgcn_alignbit(s32[i + 1], s32[i], 16) : s32[i];
+    if ((w & 1) && i == nd - 1) v &= 0xFFFFu;  // the padding word of an odd count is zero
+    wdst[i] = v;
+  }
 }
 
 // ----------------------------------------------------------------------------
