@@ -73,12 +73,14 @@ EncLayout enc_layout(const NzGeom& g) {
 }
 
 template <int S>
-void launch_split_hist(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws,
-                       const EncLayout& L, const NzNorm& nm, hipStream_t st) {
-  hipLaunchKernelGGL(nz_split_hist_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(NZ_SPLIT_THREADS), 0, st,
-                     (const uint16_t*)in, g.n, g.chunk_syms, g.seg_syms, g.spc, packed, ws + L.carry,
+void launch_split_encode(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws,
+                         const EncLayout& L, const NzNorm& nm, hipStream_t st) {
+  hipLaunchKernelGGL(nz_split_encode_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(NZ_SPLIT_THREADS), 0, st,
+                     (const uint16_t*)in, g.n, g.chunk_syms, g.lane_syms, g.spc, packed, ws + L.carry,
                      ws + L.exps, (uint32_t*)(ws + L.enc_tab), ws + L.tab_ser,
-                     (NzChunkInfo*)(ws + L.info), nm);
+                     (NzChunkInfo*)(ws + L.info), nm, (uint16_t*)(ws + L.slots), (uint32_t*)(ws + L.states),
+                     (uint32_t*)(ws + L.seg_words), (uint32_t*)(ws + L.seg_sbytes),
+                     (uint32_t*)(ws + L.seg_units));
 }
 
 // group bytes of a tensor that is about to be split (nothing to do without normalizers)
@@ -99,18 +101,11 @@ int encode_phase1(const NzGeom& g, int precision, const void* in, uint8_t* packe
     if (int rc = launch_absmax(in, g.n, ns, norm, st)) return rc;
     const NzNorm nm{ns ? norm : nullptr, log2_of(ns ? ns : 1)};
     switch (precision) {
-      case 7: launch_split_hist<7>(g, in, packed, ws, L, nm, st); break;
-      case 3: launch_split_hist<3>(g, in, packed, ws, L, nm, st); break;
-      case 1: launch_split_hist<1>(g, in, packed, ws, L, nm, st); break;
-      default: launch_split_hist<0>(g, in, packed, ws, L, nm, st); break;
+      case 7: launch_split_encode<7>(g, in, packed, ws, L, nm, st); break;
+      case 3: launch_split_encode<3>(g, in, packed, ws, L, nm, st); break;
+      case 1: launch_split_encode<1>(g, in, packed, ws, L, nm, st); break;
+      default: launch_split_encode<0>(g, in, packed, ws, L, nm, st); break;
     }
-    hipLaunchKernelGGL(nz_rans_encode_kernel, dim3((uint32_t)g.n_chunks), dim3(64 * g.spc), 0, st,
-                       ws + L.exps, g.n, g.chunk_syms, g.lane_syms, g.spc,
-                       (const uint32_t*)(ws + L.enc_tab), (NzChunkInfo*)(ws + L.info),
-                       (const uint16_t*)(ws + L.carry), (uint16_t*)(ws + L.slots),
-                       (uint32_t*)(ws + L.states),
-                       (uint32_t*)(ws + L.seg_words), (uint32_t*)(ws + L.seg_sbytes),
-                       (uint32_t*)(ws + L.seg_units));
   }
   hipLaunchKernelGGL(nz_scan_kernel, dim3(1), dim3(1024), 0, st,
                      (const uint32_t*)(ws + L.seg_units), g, hdr, cap, d_total, d_status);

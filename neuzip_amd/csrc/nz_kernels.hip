@@ -1,10 +1,10 @@
 // gfx950 (CDNA4, wave64) kernels of the NeuZip bf16 codec.
 //
 //   nz_split_unpacked_kernel   Manager::split            cuda/high_level.cu:265-321
-//   nz_split_hist_kernel       kernel_aligned_split      cuda/kernels.cuh:62-156
+//   nz_split_encode_kernel     kernel_aligned_split      cuda/kernels.cuh:62-156
 //                              + per-chunk exponent histogram, 12-bit frequency
-//                              table and its serialized form
-//   nz_rans_encode_kernel      nvcomp ANS compress       cuda/high_level.cu:103-115
+//                              table and its serialized form, then
+//                              nvcomp ANS compress       cuda/high_level.cu:103-115
 //   nz_scan_kernel             \ exact-size compaction    cuda/high_level.cu:117-124
 //   nz_compact_kernel          / (done on the device, no host round trip between the kernels)
 //   nz_decode_kernel           nvcomp ANS decompress + kernel_aligned_merge fused:
@@ -272,7 +272,7 @@ __device__ __forceinline__ uint32_t nz_block_max(uint32_t v, uint32_t* red) {
 }
 
 template <int S>
-__global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_hist_kernel(
+__device__ __forceinline__ void nz_split_hist_body(
     const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms, uint32_t spc,
     uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
     uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info,
@@ -513,7 +513,7 @@ __device__ __forceinline__ void nz_chunk_finalize(uint64_t c, uint64_t n, uint32
 // symbol, the most any input can emit, so there is no overflow path; a chunk
 // that codes to more than its raw size is stored raw (decided at the end of this
 // kernel, once all segments of the chunk are coded).
-__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_kernel(
+__device__ __forceinline__ void nz_rans_encode_body(
     const uint8_t* __restrict__ exps, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
     uint32_t spc, const uint32_t* __restrict__ enc_tab, NzChunkInfo* __restrict__ info,
     const uint16_t* __restrict__ carry, uint16_t* __restrict__ slots,
@@ -536,7 +536,10 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
   const uint32_t seg_syms = lane_syms * NZ_LANES;
   const uint64_t seg = c * spc + wave;
   const uint64_t seg_base = c * chunk_syms + (uint64_t)wave * seg_syms;
-  if (seg_base < n) {  // wavefronts beyond the tensor only take part in the barrier below
+  // wavefronts without a segment leave: their slots go to the next chunk's
+  // split phase, which then overlaps this chunk's coding
+  if (wave >= spc) return;
+  if (seg_base < n) {  // a wavefront beyond the tensor's end only takes part in the barrier below
   const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, wave);
   const uint32_t seg_n = (uint32_t)((n - seg_base) < nom ? (n - seg_base) : nom);
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
@@ -613,6 +616,31 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_rans_encode_ker
   // every segment of the chunk is coded: decide coded-or-raw and size the records
   __syncthreads();
   if (threadIdx.x == 0) nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units);
+}
+
+// ----------------------------------------------------------------------------
+// One workgroup of 1024 threads per chunk: split + histogram + table with all
+// sixteen wavefronts (bandwidth-bound), then the chunk's segments are coded by
+// one wavefront each (latency-bound) from the exponents the workgroup has just
+// written.  Workgroups of different chunks are in different phases at any
+// time, so the two kinds of work overlap on the chip.
+// ----------------------------------------------------------------------------
+template <int S>
+__global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_encode_kernel(
+    const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms, uint32_t spc,
+    uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
+    uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info,
+    const NzNorm nm, uint16_t* __restrict__ slots, uint32_t* __restrict__ states,
+    uint32_t* __restrict__ seg_words, uint32_t* __restrict__ seg_state_bytes,
+    uint32_t* __restrict__ seg_units) {
+  nz_split_hist_body<S>(in, n, chunk_syms, lane_syms * NZ_LANES, spc, packed, carry, exps, enc_tab, tab_ser,
+                        info, nm);
+  // exponents, table, carried bytes and chunk info of this chunk are read back below
+  __threadfence_block();
+  __syncthreads();
+  nz_rans_encode_body(exps, n, chunk_syms, lane_syms, spc, enc_tab, info,
+                      reinterpret_cast<const uint16_t*>(carry), slots, states, seg_words, seg_state_bytes,
+                      seg_units);
 }
 
 // ----------------------------------------------------------------------------
