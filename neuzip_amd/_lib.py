@@ -26,9 +26,11 @@ LANE_SYMS_AUTO = 0xFFFFFFFF
 EXPORTS = [
     "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",
     "nz_encode_workspace_bytes", "nz_norm_bytes", "nz_split", "nz_encode", "nz_decode",
-    "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_write_batch", "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
+    "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_write_batch",
+    "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
     "nz_manager_meta", "nz_manager_size", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
-    "nz_manager_norm_bytes", "nz_manager_buffers", "nz_manager_erase", "nz_manager_check", "nz_manager_export", "nz_manager_import", "nz_manager_trim",
+    "nz_manager_norm_bytes", "nz_manager_buffers", "nz_manager_erase", "nz_manager_check",
+    "nz_manager_export", "nz_manager_import", "nz_manager_trim",
 ]
 
 _lib = None

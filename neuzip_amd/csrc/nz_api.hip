@@ -44,7 +44,8 @@ uint64_t norm_bytes_of(uint64_t n, uint32_t ns) { return ns ? (n + ns - 1) / ns 
 
 // Device scratch of one encode call.
 struct EncLayout {
-  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, hdr, total, status, bytes;
+  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, hdr, total,
+      status, bytes;
 };
 
 EncLayout enc_layout(const NzGeom& g) {
@@ -286,11 +287,13 @@ uint64_t nz_norm_bytes(uint64_t n, uint32_t normalizer_size) {
 
 int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fractions,
              uint32_t normalizer_size, void* dev_norm, void* stream) {
-  if (!normalizer_ok(normalizer_size)) return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
+  if (!normalizer_ok(normalizer_size))
+    return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
   if (n == 0) return NZ_OK;
   if (!dev_bf16 || !dev_exponents || !dev_fractions || (normalizer_size && !dev_norm))
     return fail(NZ_ERR_ARG, "null pointer");
-  if (normalizer_size && ((uintptr_t)dev_norm & 7)) return fail(NZ_ERR_ALIGN, "normalizer bytes must be 8-byte aligned");
+  if (normalizer_size && ((uintptr_t)dev_norm & 7))
+    return fail(NZ_ERR_ALIGN, "normalizer bytes must be 8-byte aligned");
   if (((uintptr_t)dev_bf16 & 15) || ((uintptr_t)dev_exponents & 7) || ((uintptr_t)dev_fractions & 7))
     return fail(NZ_ERR_ALIGN, "nz_split: pointers must be 16-byte (input) / 8-byte (outputs) aligned");
   const uint64_t blocks = (n + 2047) / 2048;
@@ -310,7 +313,8 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
               uint32_t* dev_status, uint64_t* host_total, uint32_t normalizer_size, void* dev_norm,
               void* stream) {
   if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
-  if (!normalizer_ok(normalizer_size)) return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
+  if (!normalizer_ok(normalizer_size))
+    return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
   if (normalizer_size && n && (!dev_norm || ((uintptr_t)dev_norm & 7)))
     return fail(NZ_ERR_ARG, "normalizer bytes: null or not 8-byte aligned");
   NzGeom g;
@@ -346,7 +350,8 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
               uint32_t* dev_status, int check, uint32_t normalizer_size, const void* dev_norm,
               void* stream) {
   if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
-  if (!normalizer_ok(normalizer_size)) return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
+  if (!normalizer_ok(normalizer_size))
+    return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
   if (normalizer_size && n && (!dev_norm || ((uintptr_t)dev_norm & 7)))
     return fail(NZ_ERR_ARG, "normalizer bytes: null or not 8-byte aligned");
   NzGeom g;
@@ -762,7 +767,8 @@ int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indi
   if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
   if (count == 0) return NZ_OK;
   if (!dev_indices || !dev_out) return fail(NZ_ERR_ARG, "null indices or output");
-  if (((uintptr_t)dev_indices & 7) || ((uintptr_t)dev_out & 1)) return fail(NZ_ERR_ALIGN, "misaligned indices or output");
+  if (((uintptr_t)dev_indices & 7) || ((uintptr_t)dev_out & 1))
+    return fail(NZ_ERR_ALIGN, "misaligned indices or output");
   hipStream_t st = (hipStream_t)stream;
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
@@ -789,12 +795,16 @@ int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indi
   const NzNorm nm{m->normalizer ? (const uint8_t*)ent.norm : nullptr, log2_of(m->normalizer ? m->normalizer : 1)};
   const long long* idx = (const long long*)dev_indices;
   uint16_t* scratch = (uint16_t*)m->ws;
+#define NZ_ROWS_CASE(S)                                                                              \
+  launch_decode_rows<S>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx,     \
+                        (uint32_t)count, row_len, cpr, st)
   switch (m->precision) {
-    case 7: launch_decode_rows<7>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx, (uint32_t)count, row_len, cpr, st); break;
-    case 3: launch_decode_rows<3>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx, (uint32_t)count, row_len, cpr, st); break;
-    case 1: launch_decode_rows<1>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx, (uint32_t)count, row_len, cpr, st); break;
-    default: launch_decode_rows<0>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx, (uint32_t)count, row_len, cpr, st); break;
+    case 7: NZ_ROWS_CASE(7); break;
+    case 3: NZ_ROWS_CASE(3); break;
+    case 1: NZ_ROWS_CASE(1); break;
+    default: NZ_ROWS_CASE(0); break;
   }
+#undef NZ_ROWS_CASE
   NZ_HIP(hipGetLastError());
   const uint32_t bx = (row_len + 255) / 256 < 64 ? (row_len + 255) / 256 : 64;
   hipLaunchKernelGGL(nz_copy_rows_kernel, dim3(bx, (uint32_t)count), dim3(256), 0, st, (const uint16_t*)scratch,
@@ -992,7 +1002,9 @@ int nz_manager_check(nz_manager* m, void* stream) {
   NZ_HIP(hipStreamSynchronize(st));
   const uint32_t hs = (uint32_t)m->h_pin[16];
   if (hs == 8u) return fail(NZ_ERR_CORRUPT, "a row gather was given an index outside the table");
-  if (hs) return fail(NZ_ERR_CORRUPT, "a read saw a container that failed validation (status " + std::to_string(hs) + ")");
+  if (hs)
+    return fail(NZ_ERR_CORRUPT,
+                "a read saw a container that failed validation (status " + std::to_string(hs) + ")");
   return NZ_OK;
 }
 
