@@ -76,7 +76,7 @@ def _check(dense, s, oracle, max_over_bound, compare_oracle=True):
     got = torch.from_numpy(out.view(np.int16)).cuda().to(torch.int32) & 0xFFFF
     assert torch.equal(got, want)
     if compare_oracle:
-        o_comp, o_packed = oracle.compress_bf16(host_bits, s, 65536, 344, threads=8)
+        o_comp, o_packed = oracle.compress_bf16(host_bits, s, 131072, 256, threads=8)
         assert np.array_equal(comp.cpu().numpy(), o_comp)
         assert np.array_equal(packed.cpu().numpy(), o_packed)
     bound = _entropy_bound_bytes_dev((want >> 7) & 0xFF)

@@ -36,7 +36,7 @@ def test_encode_decode_match_oracle(oracle, norm, s):
         comp, packed, nb = gpu_encode(bits, s, norm_size=norm)
         o_norm, o_scaled = oracle.block_normalize(bits, norm)
         assert np.array_equal(nb.cpu().numpy(), o_norm)
-        o_comp, o_packed = oracle.compress_bf16(o_scaled, s, 65536, 344)
+        o_comp, o_packed = oracle.compress_bf16(o_scaled, s, 131072, 256)
         assert np.array_equal(packed.cpu().numpy(), o_packed)
         assert np.array_equal(comp.cpu().numpy(), o_comp)
         rc, out = gpu_decode(comp, packed, n, s, norm_size=norm, norm=nb)

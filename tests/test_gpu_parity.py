@@ -21,7 +21,7 @@ def _to_dev(bits: np.ndarray):
     return torch.from_numpy(bits.view(np.int16).copy()).cuda()
 
 
-def gpu_encode(bits, s, chunk=65536, lane=344, norm_size=0):
+def gpu_encode(bits, s, chunk=131072, lane=256, norm_size=0):
     """-> (container, stored packed stream[, normalizer bytes when norm_size > 0]) as device tensors"""
     L, m = _lib()
     n = bits.size
@@ -45,7 +45,7 @@ def gpu_encode(bits, s, chunk=65536, lane=344, norm_size=0):
     return res + (norm[: L.nz_norm_bytes(n, norm_size)].clone(),) if norm_size else res
 
 
-def gpu_decode(comp, packed, n, s, chunk=65536, lane=344, check=True, norm_size=0, norm=None):
+def gpu_decode(comp, packed, n, s, chunk=131072, lane=256, check=True, norm_size=0, norm=None):
     L, m = _lib()
     if norm_size:
         norm = torch.cat([norm, torch.zeros(8, dtype=torch.uint8, device="cuda")])
@@ -71,7 +71,7 @@ def test_roundtrip_matches_oracle(oracle, n, s):
     print(f"case n={n} s={s}", flush=True)
     comp, packed = gpu_encode(bits, s)
     # container and packed stream are byte-identical to the oracle's
-    o_comp, o_packed = oracle.compress_bf16(bits, s, 65536, 344)
+    o_comp, o_packed = oracle.compress_bf16(bits, s, 131072, 256)
     assert np.array_equal(packed.cpu().numpy(), o_packed)
     assert np.array_equal(comp.cpu().numpy(), o_comp)
     rc, out = gpu_decode(comp, packed, n, s)
@@ -82,7 +82,8 @@ def test_roundtrip_matches_oracle(oracle, n, s):
 
 @pytest.mark.parametrize("lane,chunk", [(128, 65536), (256, 65536), (344, 65536), (352, 65536), (512, 65536),
                                         (1024, 65536), (1000, 65536), (16, 1024), (24, 2560), (64, 4096),
-                                        (2048, 1 << 20)])
+                                        (2048, 1 << 20), (256, 131072), (344, 131072), (2048, 131072),
+                                        (512, 262144)])
 def test_geometries(oracle, lane, chunk):
     n = 3 * chunk + 1234 if chunk <= 65536 else chunk + 777
     bits = bf16_bits_normal(n, seed=lane)
@@ -125,10 +126,10 @@ def test_incompressible_goes_raw(oracle):
     bits = rng.integers(0, 65536, n).astype(np.uint16)
     print("case raw", flush=True)
     comp, packed = gpu_encode(bits, 7)
-    o_comp, _ = oracle.compress_bf16(bits, 7, 65536, 344)
+    o_comp, _ = oracle.compress_bf16(bits, 7, 131072, 256)
     assert np.array_equal(comp.cpu().numpy(), o_comp)
     L, _m = _lib()
-    assert comp.numel() <= L.nz_exp_bound_bytes(n, 65536, 344)
+    assert comp.numel() <= L.nz_exp_bound_bytes(n, 131072, 256)
     rc, out = gpu_decode(comp, packed, n, 7)
     assert rc == 0 and np.array_equal(out, bits)
 
@@ -139,7 +140,7 @@ def test_constant_and_two_symbol(oracle):
                        ("two", np.where(np.arange(70_000) % 97 == 0, 0x3C00, 0x0080).astype(np.uint16))):
         print(f"case {name}", flush=True)
         comp, packed = gpu_encode(bits, 7)
-        o_comp, _ = oracle.compress_bf16(bits, 7, 65536, 344)
+        o_comp, _ = oracle.compress_bf16(bits, 7, 131072, 256)
         assert np.array_equal(comp.cpu().numpy(), o_comp)
         rc, out = gpu_decode(comp, packed, bits.size, 7)
         assert rc == 0 and np.array_equal(out, bits)

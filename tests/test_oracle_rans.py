@@ -9,7 +9,7 @@ import pyref
 from conftest import bf16_bits_normal, chunk_entropy_bytes, closed_form_recon, stress_bits
 
 GEOMS = ((16, 1024), (16, 8192), (24, 2560), (64, 4096), (128, 65536), (344, 65536), (512, 65536),
-         (1024, 65536), (2048, 1 << 20))
+         (1024, 65536), (2048, 1 << 20), (256, 131072), (344, 131072), (512, 262144))
 
 
 def roundtrip(oracle, syms, lane, chunk, seeds=None):
