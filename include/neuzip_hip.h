@@ -176,10 +176,12 @@ int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* 
    stored tensor is read as a row-major matrix with rows of `in_features`
    elements (a multiple of 512).  dev_x: in_features bf16, 16-byte aligned;
    dev_y[i]: rows_i bf16; dev_bias: null, or per matrix null / rows_i bf16.
-   Sums are formed in fp32 per wavefront and row, then in 24.40 fixed point
-   across wavefronts, so the result does not depend on scheduling; a row whose
-   partial sums are NaN, infinite or beyond 2^18 in magnitude comes out as NaN; sums
-   are resolved to 2^-40.
+   Sums are formed in fp32 per wavefront and row; a row that several
+   wavefronts share is summed across them in 24.40 fixed point, so the result
+   does not depend on scheduling (such a row comes out as NaN when one of its
+   partial sums is NaN, infinite or beyond 2^18 in magnitude, and is resolved
+   to 2^-40); the wavefront that completes a row rounds and stores it, so the
+   whole product is one kernel launch.
    Calls of one manager must be ordered on one stream (they share the
    accumulators, which are allocated on first use and grown when needed; no
    other call allocates).  Asynchronous on `stream`. */

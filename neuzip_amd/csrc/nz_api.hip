@@ -180,8 +180,8 @@ int decode_batch_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int p
   return NZ_OK;
 }
 
-int gemv_launch(const NzBatch& b, const NzGemvOut& o, uint32_t grid, uint32_t max_spc, uint32_t rows,
-                int precision, uint32_t* d_status, hipStream_t st) {
+int gemv_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int precision, uint32_t* d_status,
+                hipStream_t st) {
   const size_t lds = (2 * NZ_M + max_spc * NZ_RING_ALLOC_DWORDS) * 4;
   const dim3 gd(grid), bd(64 * max_spc);
   const bool nrm = b.item[0].norm != nullptr;
@@ -195,8 +195,6 @@ int gemv_launch(const NzBatch& b, const NzGemvOut& o, uint32_t grid, uint32_t ma
     default: NZ_GEMV_CASE(0); break;
   }
 #undef NZ_GEMV_CASE
-  NZ_HIP(hipGetLastError());
-  hipLaunchKernelGGL(nz_gemv_finish_kernel, dim3((rows + 255) / 256), dim3(256), 0, st, o);
   NZ_HIP(hipGetLastError());
   return NZ_OK;
 }
@@ -705,9 +703,7 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
   hipStream_t st = (hipStream_t)stream;
   std::lock_guard<std::mutex> lock(m->mu);
   NzBatch b;
-  NzGemvOut o;
   std::memset(&b, 0, sizeof(b));
-  std::memset(&o, 0, sizeof(o));
   b.x = (const uint16_t*)dev_x;
   b.in_features = in_features;
   b.log2n = log2_of(m->normalizer ? m->normalizer : 1);
@@ -733,12 +729,10 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
     grid += g.n_chunks;
     bi.chunk_end = (uint32_t)grid;
     if (g.spc > max_spc) max_spc = g.spc;
-    NzGemvOutItem& oi = o.item[i];
-    oi.bias = dev_bias ? (const uint16_t*)dev_bias[i] : nullptr;
-    oi.y = (uint16_t*)dev_y[i];
+    bi.bias = dev_bias ? (const uint16_t*)dev_bias[i] : nullptr;
+    bi.y = (uint16_t*)dev_y[i];
     bi.reserved = (uint32_t)rows;  // first row, turned into a pointer below
     rows += ent.n / in_features;
-    oi.row_end = (uint32_t)rows;
     if (grid > 0x7FFFFFFFull || rows > 0x7FFFFFFFull) return fail(NZ_ERR_ARG, "batch too large");
   }
   if (m->gemv_rows < rows) {
@@ -755,11 +749,9 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
   for (uint32_t i = 0; i < count; ++i) {
     b.item[i].acc = m->gemv_acc + 2 * (uint64_t)b.item[i].reserved;
     b.item[i].reserved = 0;
-    o.item[i].acc = b.item[i].acc;
   }
   b.count = count;
-  o.count = count;
-  return gemv_launch(b, o, (uint32_t)grid, max_spc, (uint32_t)rows, m->precision, m->d_status, st);
+  return gemv_launch(b, (uint32_t)grid, max_spc, m->precision, m->d_status, st);
 }
 
 int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indices, uint64_t count,
@@ -1001,6 +993,8 @@ int nz_manager_check(nz_manager* m, void* stream) {
   NZ_HIP(hipMemsetAsync(m->d_status, 0, 4, st));
   NZ_HIP(hipStreamSynchronize(st));
   const uint32_t hs = (uint32_t)m->h_pin[16];
+  // a product that met a broken container left rows half summed: start clean
+  if (hs && m->gemv_acc) NZ_HIP(hipMemset(m->gemv_acc, 0, m->gemv_rows * 16));
   if (hs == 8u) return fail(NZ_ERR_CORRUPT, "a row gather was given an index outside the table");
   if (hs)
     return fail(NZ_ERR_CORRUPT,

@@ -825,14 +825,10 @@ __device__ __forceinline__ uint4 nz_merge_group(uint64_t sm, const uint32_t (&ew
 // ----------------------------------------------------------------------------
 // A group of 512 consecutive weights lies inside one row of W (the row length
 // is a multiple of 512), so the row of a group is the same for all lanes.  A
-// lane keeps an fp32 partial sum of its 8-element dot products; when the wave
-// leaves a row the 64 partial sums are added in a fixed butterfly order and
-// lane 0 adds the result, converted to 24.40 fixed point, to the row's 64-bit
-// accumulator.  Integer addition is associative, so the value of y does not
-// depend on the order in which the wavefronts that share a row arrive.  A
-// partial sum that is NaN, infinite or beyond 2^18 sets the row's flag word
-// instead (the row then comes out as NaN).  Row r owns acc[2r] (sum) and
-// acc[2r + 1] (flag).
+// lane keeps an fp32 partial sum of its 8-element dot products; what happens
+// when the wave leaves a row is described at NzGemvWalk.  Row r owns acc[2r]
+// (fixed-point sum) and acc[2r + 1] (contribution count in the low half, flag
+// in bit 32).
 // 40 fraction bits: an absolute resolution of 9e-13 per partial sum; up to 16
 // partial sums below 2^18 in magnitude cannot overflow 64 bits.
 #define NZ_GEMV_FRAC_BITS 40
@@ -840,7 +836,9 @@ __device__ __forceinline__ uint4 nz_merge_group(uint64_t sm, const uint32_t (&ew
 
 struct NzGemv {
   const uint16_t* x;      // in_features bf16 values, 16-byte aligned
-  long long* acc;         // two words per row of this tensor (sum, flag), all zero on entry
+  long long* acc;         // two words per row of this tensor (sum | count and flag), all zero between calls
+  uint16_t* y;            // one bf16 per row
+  const uint16_t* bias;   // one bf16 per row, or null
   uint32_t in_features;   // multiple of 512
 };
 
@@ -855,38 +853,100 @@ __device__ __forceinline__ float nz_dot8(const uint4 w, const uint4 x, float acc
 }
 
 // Position of a wavefront inside W while it walks its segment group by group.
+//
+// When the wave leaves a row it adds its 64 partial sums in a fixed butterfly
+// order.  A row that lies inside the wave's segment is complete then: bias
+// added, rounded, stored.  A row shared with other segments goes through the
+// row's accumulator pair: the sum in 24.40 fixed point (integer addition is
+// associative, so the result does not depend on which wave arrives first; a
+// partial sum that is NaN, infinite or beyond 2^18 sets a flag instead and the
+// row comes out as NaN), and a counter of contributions; the wave that brings
+// the count to the number of segments the row touches converts, stores and
+// returns both words to zero.
 struct NzGemvWalk {
   const uint4* xq;     // x as 8-element blocks, already offset by the lane
-  long long* acc;
+  NzGemv gv;
   uint64_t row;
+  uint64_t seg_first, seg_end;  // elements of the tensor this wave covers
   uint32_t col;        // column of the current group's first element (uniform)
-  uint32_t in_features;
   uint32_t pending;    // groups added since the last flush (uniform)
+  uint32_t seg_syms, last_syms, spc, k;  // segment lengths of a chunk, this wave's segment inside it
   float sum;
 
-  __device__ __forceinline__ void start(const NzGemv& gv, uint64_t first_elem, uint32_t lane) {
-    xq = reinterpret_cast<const uint4*>(gv.x) + lane;
-    acc = gv.acc;
-    in_features = gv.in_features;
-    row = first_elem / in_features;
-    col = (uint32_t)(first_elem - row * in_features);
+  __device__ __forceinline__ void start(const NzGemv& g, const NzGeom& geom, uint64_t first_elem,
+                                        uint32_t seg_n, uint32_t wave_in_chunk, uint32_t lane) {
+    gv = g;
+    xq = reinterpret_cast<const uint4*>(g.x) + lane;
+    row = first_elem / g.in_features;
+    col = (uint32_t)(first_elem - row * g.in_features);
+    seg_first = first_elem;
+    seg_end = first_elem + seg_n;
+    seg_syms = geom.seg_syms;
+    spc = geom.spc;
+    last_syms = geom.chunk_syms - (geom.spc - 1) * geom.seg_syms;  // the chunk's (shorter) last segment
+    k = wave_in_chunk;
     pending = 0;
     sum = 0.f;
   }
   __device__ __forceinline__ uint32_t next_col() const {
-    return col + NZ_GROUP_SYMS == in_features ? 0u : col + NZ_GROUP_SYMS;
+    return col + NZ_GROUP_SYMS == gv.in_features ? 0u : col + NZ_GROUP_SYMS;
   }
   __device__ __forceinline__ uint4 load(uint32_t c) const { return xq[c / NZ_GROUP]; }
+  // Segments the row [first, last] touches, this wave's included: walk over the
+  // segment boundaries to the left and to the right (a row rarely spans more
+  // than two or three segments; no division).
+  __device__ __forceinline__ uint32_t segments_of_row(uint64_t first, uint64_t last) const {
+    uint32_t count = 1;
+    uint64_t at = seg_first;
+    uint32_t kk = k;
+    while (at > first) {  // the segment before `at` also holds part of the row
+      kk = kk ? kk - 1 : spc - 1;
+      at -= kk == spc - 1 ? last_syms : seg_syms;
+      ++count;
+    }
+    at = seg_end;
+    kk = k;
+    while (at <= last) {  // so does the segment that starts at `at`
+      kk = kk + 1 == spc ? 0 : kk + 1;
+      at += kk == spc - 1 ? last_syms : seg_syms;
+      ++count;
+    }
+    return count;
+  }
+  __device__ __forceinline__ void store_row(float v) const {
+    if (gv.bias) v += nz_bf16_to_f32(gv.bias[row]);
+    gv.y[row] = (uint16_t)nz_f32_to_bf16(v);
+  }
   __device__ __forceinline__ void flush(uint32_t lane) {
     float t = sum;
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
     if (lane == 0) {
-      unsigned long long* slot = reinterpret_cast<unsigned long long*>(acc + 2 * row);
-      if (fabsf(t) < NZ_GEMV_PART_MAX)  // false for NaN as well
-        atomicAdd(slot, (unsigned long long)__float2ll_rn(t * (float)(1ull << NZ_GEMV_FRAC_BITS)));
-      else
-        atomicOr(slot + 1, 1ull);
+      const uint64_t first = row * gv.in_features, last = first + gv.in_features - 1;
+      if (first >= seg_first && last < seg_end) {
+        store_row(t);
+      } else {
+        // Device-scope atomics execute at the L2 in the order they are issued by
+        // this lane when each one waits for the value the previous returned, so
+        // no cache flush is needed: the count is issued only after the sum's old
+        // value has come back, the exchanges only after the count's.
+        unsigned long long* slot = reinterpret_cast<unsigned long long*>(gv.acc + 2 * row);
+        unsigned long long r0;
+        if (fabsf(t) < NZ_GEMV_PART_MAX)  // false for NaN as well
+          r0 = atomicAdd(slot, (unsigned long long)__float2ll_rn(t * (float)(1ull << NZ_GEMV_FRAC_BITS)));
+        else
+          r0 = atomicOr(slot + 1, 1ull << 32);
+        uint32_t zero;  // 0, but only the hardware knows: ties the next atomic to the returned value
+        asm volatile("v_and_b32 %0, 0, %1" : "=v"(zero) : "v"((uint32_t)r0));
+        const uint32_t expected = segments_of_row(first, last);
+        const unsigned long long before = atomicAdd(slot + 1, 1ull + zero);
+        if ((uint32_t)before + 1u == expected) {
+          const long long a = (long long)atomicExch(slot, 0ull);
+          const unsigned long long f = atomicExch(slot + 1, 0ull);
+          store_row((f >> 32) ? __uint_as_float(0x7FC00000u)
+                              : (float)((double)a * (1.0 / (double)(1ull << NZ_GEMV_FRAC_BITS))));
+        }
+      }
     }
     sum = 0.f;
     pending = 0;
@@ -1165,7 +1225,7 @@ __device__ __forceinline__ void nz_decode_chunk(
   const uint8_t* pk = packed + c * chunk_keep + (uint64_t)wave * (g.seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES);
   uint16_t* dst = out + seg_base;
   NzGemvWalk walk;
-  if constexpr (GEMV) walk.start(gv, seg_base, lane);
+  if constexpr (GEMV) walk.start(gv, g, seg_base, seg_n, wave, lane);
 
   if (mode == NZ_MODE_RAW) {
     const uint32_t padded = (seg_n + 3) & ~3u;
@@ -1340,7 +1400,9 @@ struct NzBatchItem {
   uint64_t comp_bytes;
   const uint8_t* packed;
   uint16_t* out;       // dense output (decode) ...
-  long long* acc;      // ... or the row accumulators (matrix-vector product)
+  long long* acc;      // ... or the row accumulators, output and bias (matrix-vector product)
+  uint16_t* y;
+  const uint16_t* bias;
   const uint8_t* norm; // group bytes of a normalized tensor
   NzGeom g;
   uint32_t chunk_end;
@@ -1378,43 +1440,9 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_gemv_ker
     ++t;
   }
   const NzBatchItem& it = b.item[t];
-  const NzGemv gv{b.x, it.acc, b.in_features};
+  const NzGemv gv{b.x, it.acc, it.y, it.bias, b.in_features};
   nz_decode_chunk<S, true, NORM>(it.comp, it.comp_bytes, it.packed, nullptr, it.g, d_status,
                                  blockIdx.x - first, gv, NzNorm{it.norm, b.log2n});
-}
-
-// y = bf16(acc * 2^-40 + bias), and the accumulators return to zero for the next
-// product.  Flagged rows come out as NaN.
-struct NzGemvOutItem {
-  long long* acc;
-  const uint16_t* bias;  // or null
-  uint16_t* y;
-  uint32_t row_end;      // running total of rows
-  uint32_t reserved;
-};
-struct NzGemvOut {
-  uint32_t count;
-  uint32_t reserved;
-  NzGemvOutItem item[NZ_BATCH_MAX];
-};
-
-__global__ __launch_bounds__(256) void nz_gemv_finish_kernel(const NzGemvOut o) {
-  const uint32_t r = blockIdx.x * 256 + threadIdx.x;
-  uint32_t t = 0, first = 0;
-  while (t + 1 < o.count && r >= o.item[t].row_end) {
-    first = o.item[t].row_end;
-    ++t;
-  }
-  const NzGemvOutItem& it = o.item[t];
-  if (r >= it.row_end) return;
-  const uint32_t i = r - first;
-  const longlong2 a = reinterpret_cast<longlong2*>(it.acc)[i];
-  reinterpret_cast<longlong2*>(it.acc)[i] = make_longlong2(0, 0);
-  float y;
-  if (a.y) y = __uint_as_float(0x7FC00000u);
-  else y = (float)((double)a.x * (1.0 / (double)(1ull << NZ_GEMV_FRAC_BITS)));
-  if (it.bias) y += nz_bf16_to_f32(it.bias[i]);
-  it.y[i] = (uint16_t)nz_f32_to_bf16(y);
 }
 
 // ----------------------------------------------------------------------------
