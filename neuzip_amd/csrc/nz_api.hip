@@ -132,7 +132,7 @@ int encode_phase2(const NzGeom& g, uint8_t* ws, const EncLayout& L, const uint32
 template <int S>
 void launch_decode(const NzGeom& g, const void* comp, uint64_t comp_bytes, const void* packed,
                    void* out, uint32_t* d_status, const NzNorm& nm, hipStream_t st) {
-  const size_t lds = (2 * NZ_M + g.spc * NZ_RING_ALLOC_DWORDS) * 4;
+  const size_t lds = NZ_DEC_LDS_BYTES(g.spc);
   const dim3 gd((uint32_t)g.n_chunks), bd(64 * g.spc);
   if (nm.bytes)
     hipLaunchKernelGGL((nz_decode_kernel<S, true>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,
@@ -160,7 +160,7 @@ int decode_launch(const NzGeom& g, int precision, const void* comp, uint64_t com
 template <int S>
 void launch_decode_batch(const NzBatch& b, uint32_t grid, uint32_t max_spc, uint32_t* d_status,
                          hipStream_t st) {
-  const size_t lds = (2 * NZ_M + max_spc * NZ_RING_ALLOC_DWORDS) * 4;
+  const size_t lds = NZ_DEC_LDS_BYTES(max_spc);
   if (b.item[0].norm)
     hipLaunchKernelGGL((nz_decode_batch_kernel<S, true>), dim3(grid), dim3(64 * max_spc), lds, st, b, d_status);
   else
@@ -182,7 +182,7 @@ int decode_batch_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int p
 
 int gemv_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int precision, uint32_t* d_status,
                 hipStream_t st) {
-  const size_t lds = (2 * NZ_M + max_spc * NZ_RING_ALLOC_DWORDS) * 4;
+  const size_t lds = NZ_DEC_LDS_BYTES(max_spc);
   const dim3 gd(grid), bd(64 * max_spc);
   const bool nrm = b.item[0].norm != nullptr;
 #define NZ_GEMV_CASE(S)                                                                              \
@@ -203,7 +203,7 @@ template <int S>
 void launch_decode_rows(const NzGeom& g, const void* comp, uint64_t comp_bytes, const void* packed,
                         uint16_t* scratch, uint32_t* d_status, const NzNorm& nm, const long long* idx,
                         uint32_t count, uint32_t row_len, uint32_t cpr, hipStream_t st) {
-  const size_t lds = (2 * NZ_M + g.spc * NZ_RING_ALLOC_DWORDS) * 4;
+  const size_t lds = NZ_DEC_LDS_BYTES(g.spc);
   const dim3 gd(count * cpr), bd(64 * g.spc);
   if (nm.bytes)
     hipLaunchKernelGGL((nz_decode_rows_kernel<S, true>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,

@@ -185,15 +185,19 @@ __device__ __forceinline__ uint32_t nz_rank_below(uint64_t mask) {
 }
 
 // inclusive prefix sum over the 64 lanes of a wavefront
+// Inclusive prefix sum over the 64 lanes with data-parallel-primitive moves:
+// four shifted adds inside each row of 16 lanes, then the last lane of row 0
+// and 2 is added to rows 1 and 3, and lane 31 to rows 2 and 3.
 __device__ __forceinline__ uint32_t nz_wave_scan(uint32_t v, uint32_t lane) {
-#pragma unroll
-  for (int o = 1; o < 64; o <<= 1) {
-    const uint32_t t = __shfl_up(v, o, 64);
-    if (lane >= (uint32_t)o) v += t;
-  }
+  (void)lane;
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xF, 0xF, false);  // row_shr:1
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xF, 0xF, false);  // row_shr:2
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xF, 0xF, false);  // row_shr:4
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xF, 0xF, false);  // row_shr:8
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xA, 0xF, false);  // row_bcast:15
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xC, 0xF, false);  // row_bcast:31
   return v;
 }
-
 __device__ __forceinline__ uint32_t nz_get12(const uint8_t* p, uint32_t i) {
   uint32_t bit = 12u * i;
   const uint8_t* q = p + (bit >> 3);
@@ -770,16 +774,20 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
 // LDS: a 4096-entry slot table of 8-byte entries
 //          lo = freq | symbol << 24      hi = slot - cum[symbol]
 //      (so that one v_mad_u32_u24 of lo's low 24 bits gives the next state and
-//      the symbol is a whole byte for v_perm_b32) and a ring of 1024
-//      renormalisation words (2 KiB) per wavefront; the table-parse scratch
-//      aliases the rings (it is dead before the first ring is filled).  Up to
-//      four wavefronts per chunk need at most 40 KiB, so four workgroups share
-//      the 160 KiB of a CU.
+//      the symbol is a whole byte for v_perm_b32), per wavefront a ring of
+//      1024 16-bit units (2 KiB) that is a sliding window over the segment's
+//      record (it first holds the record's head: table, coder states, first
+//      words), and the 257 cumulative frequencies of the table parse.  Eight
+//      wavefronts per chunk need 49 KiB, so three workgroups share the 160 KiB
+//      of a CU.
 // A rANS step per lane: one table read, one multiply-add, and when the state
 // falls below 2^16 a 16-bit word taken at (words consumed so far by the wave +
 // rank of the lane among the lanes that need one).
 
 #define NZ_RING_ALLOC_DWORDS NZ_RING_DWORDS
+#define NZ_DEC_CUM_DWORDS (512 + 256 + 4)  /* table-parse results: runs, windows, flags */
+// dynamic LDS of a decode workgroup whose chunks have up to `spc` segments
+#define NZ_DEC_LDS_BYTES(spc) ((size_t)(2 * NZ_M + (spc) * NZ_RING_ALLOC_DWORDS + NZ_DEC_CUM_DWORDS) * 4)
 
 // S+1 packed bytes of one 8-element group, as a little-endian integer
 template <int S>
@@ -966,10 +974,10 @@ struct NzGemvWalk {
 // Decoder state of one wavefront.
 struct NzWaveDec {
   const uint2* lut;
-  uint32_t* ring32;       // 1024 dwords = 2048 words
-  const uint8_t* words;   // first renormalisation word of the record (uniform)
+  uint32_t* ring32;       // 512 dwords = 1024 words: a window of the record
+  const uint8_t* words;   // start of the record (uniform); word indices count from here
   const uint8_t* last16;  // last 16-byte block that may be loaded: container end - 16 (uniform)
-  uint32_t nwords;        // words the record holds
+  uint32_t nwords;        // 16-bit units the record holds, table and states included
   uint32_t lane;
   uint32_t x;             // this lane's rANS state
   uint32_t base;          // words consumed by the wave
@@ -991,19 +999,23 @@ struct NzWaveDec {
     *reinterpret_cast<uint4*>(ring32 + (d & (NZ_RING_DWORDS - 1))) = v;
   }
 
-  __device__ __forceinline__ void start(uint32_t x0) {
-    x = x0;
-    // fill the whole ring: 512 dwords = 1024 words ahead
+  // Stage the first 512 dwords of the record (table of a chunk's first record,
+  // coder states, first words) into the ring.
+  __device__ __forceinline__ void stage() {
     uint4 v[2];
 #pragma unroll
     for (uint32_t q = 0; q < 2; ++q) v[q] = fetch(256 * q + 4 * lane);
 #pragma unroll
     for (uint32_t q = 0; q < 2; ++q) commit(256 * q + 4 * lane, v[q]);
     filled = 512;
-    base = 0;
+  }
+
+  // Start decoding from state x0; the words begin `first_word` 16-bit units
+  // into the record (at most 348, so at least 676 words are staged ahead).
+  __device__ __forceinline__ void start(uint32_t x0, uint32_t first_word) {
+    x = x0;
+    base = first_word;
     r = make_uint4(0, 0, 0, 0);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
   }
 
   // Decode the next 8 symbols of every lane into byte 3 of ew[0..7].
@@ -1076,9 +1088,11 @@ __device__ __forceinline__ void nz_decode_chunk(
   extern __shared__ uint32_t lds[];
   uint2* lut = reinterpret_cast<uint2*>(lds);                   // 4096 x 8 bytes
   uint32_t* rings = lds + 2 * NZ_M;                             // spc rings
-  uint32_t* scratch = rings;                                    // 106 + 257 dwords, dead before the rings fill
-  uint8_t* tb = reinterpret_cast<uint8_t*>(scratch);            // table bytes (424)
-  uint32_t* cum = scratch + NZ_TABLE_MAX_BYTES / 4;             // 257 entries
+  uint32_t* tmeta = rings + g.spc * NZ_RING_ALLOC_DWORDS;       // what the table parse leaves for the fill:
+  uint2* runs = reinterpret_cast<uint2*>(tmeta);                //   per live symbol (freq | symbol << 24, first slot)
+  uint2* wins = runs + 256;                                     //   per 32 slots (bitmap of run starts, runs before)
+  uint32_t* tflag = reinterpret_cast<uint32_t*>(wins + 128);    //   [0] frequencies sum to 4096, [1] table bytes
+  const uint8_t* tb = reinterpret_cast<const uint8_t*>(rings);  // table bytes: start of the first record
 
   const uint32_t tid = threadIdx.x;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keep it scalar
@@ -1098,17 +1112,65 @@ __device__ __forceinline__ void nz_decode_chunk(
       atomicOr(d_status, 16u);
   }
 
-  // record of the chunk's first segment starts with the table
-  const uint64_t f0 = dir[seg0], f1 = dir[seg0 + 1];
+  // Two rounds of global loads, then only LDS: every wavefront reads the
+  // chunk's directory entries itself, then stages the first 2 KiB of its
+  // record into its ring (for the chunk's first record that window begins with
+  // the table, which all wavefronts parse from there) and fetches the packed
+  // bytes of its first group.
+  const uint32_t dv = lane <= nseg ? dir[seg0 + lane] : 0u;
+  const uint64_t f0 = __builtin_amdgcn_readlane(dv, 0), f1 = __builtin_amdgcn_readlane(dv, 1);
   if (f1 <= f0 || g.rec_off + 4 * f1 > comp_bytes) {
     if (tid == 0) atomicOr(d_status, 2u);
     return;
   }
-  const uint8_t* rec0 = comp + g.rec_off + 4 * f0;
-  const uint32_t rec0_bytes = (uint32_t)(4 * (f1 - f0));
-  // stage up to 424 table bytes
-  for (uint32_t i = tid; i < NZ_TABLE_MAX_BYTES / 4; i += blockDim.x)
-    scratch[i] = (4 * i < rec0_bytes) ? reinterpret_cast<const uint32_t*>(rec0)[i] : 0u;
+  const bool has_seg = wave < nseg;
+  const uint32_t wk = has_seg ? wave : 0u;  // wavefronts without a segment only help with the table
+  const uint64_t seg_base = chunk_base + (uint64_t)wk * g.seg_syms;
+  const uint32_t nom = nz_seg_nominal(g.chunk_syms, g.seg_syms, g.spc, wk);
+  const uint32_t seg_n = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
+  const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
+  const uint64_t o0 = __builtin_amdgcn_readlane(dv, wk), o1 = __builtin_amdgcn_readlane(dv, wk + 1);
+  const bool bad_rec = o1 < o0 || g.rec_off + 4 * o1 > comp_bytes;
+  const uint64_t rec_pos = g.rec_off + 4 * o0;  // uniform: the readlanes above are scalar
+  const uint32_t rec_all = (uint32_t)(4 * (o1 - o0));
+  // stored packed layout: every full segment keeps seg_p - 128 bytes, its last
+  // 128 bytes ride in the coder states (or behind the symbols of a raw record)
+  const bool carry = seg_n == nom;
+  const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
+  const uint64_t chunk_keep = (uint64_t)g.chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * g.spc;
+  const uint8_t* pk = packed + c * chunk_keep + (uint64_t)wk * (g.seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES);
+  uint16_t* dst = out + seg_base;
+  // groups whose packed bytes are (partly) carried are merged after the loop
+  const uint32_t tailg = carry ? (S == 0 ? 2u : 1u) : 0u;
+  const uint32_t body = ngroups - tailg;
+  // Groups in which every lane has 8 elements run without any predicate; the
+  // packed bytes are fetched one group ahead of their use (the address of the
+  // fetch past the last group is clamped, its value unused).
+  const uint32_t whole = seg_n / NZ_GROUP_SYMS < body ? seg_n / NZ_GROUP_SYMS : body;
+  const uint32_t lane_off = lane * (S + 1);
+  const uint32_t last_off = whole ? (whole - 1) * NZ_LANES * (S + 1) + lane_off : 0u;
+  NzWaveDec w;
+  w.lut = lut;
+  w.ring32 = rings + wk * NZ_RING_ALLOC_DWORDS;
+  w.words = comp + rec_pos;
+  w.last16 = comp + comp_bytes - NZ_TAIL_PAD;
+  w.nwords = rec_all / 2;
+  w.lane = lane;
+  w.filled = 0;
+  uint64_t sm_next = 0, nb_next = 0;
+  uint4 xq_next = make_uint4(0, 0, 0, 0);
+  NzGemvWalk walk;
+  if (has_seg && !bad_rec) {
+    w.stage();
+    if constexpr (GEMV) {
+      walk.start(gv, g, seg_base, seg_n, wk, lane);
+      xq_next = walk.load(walk.col);
+    }
+    if (whole) {
+      sm_next = nz_load_sm<S>(pk + lane_off);
+      if constexpr (NORM) nb_next = nz_norm_load8(nm, seg_base + lane * NZ_GROUP);
+    }
+  }
   __syncthreads();
   const uint32_t mode = tb[0];
   uint32_t tab_len = 4;
@@ -1118,114 +1180,117 @@ __device__ __forceinline__ void nz_decode_chunk(
       if (tid == 0) atomicOr(d_status, 2u);
       return;
     }
-    uint32_t head, kk = 0;
-    if (mode == NZ_MODE_BITMAP) {
-      head = 33;
-      for (int b = 0; b < 32; ++b) kk += __popc((uint32_t)tb[1 + b]);
-    } else {
-      head = 1 + 2 * mode;
-      for (uint32_t r = 0; r < mode; ++r) kk += (uint32_t)tb[2 + 2 * r] + 1u;
-    }
-    if (kk > 256) kk = 256;  // corrupt input: stay inside the staged bytes
-    tab_len = (head + (12 * kk + 7) / 8 + 3) & ~3u;
-    // frequency of every symbol -> cum[sym + 1] for now
-    for (uint32_t sym = tid; sym < 256; sym += blockDim.x) {
-      uint32_t live = 0, rank = 0;
+    // Wavefront 0 parses the table, four symbols per lane, and leaves for the
+    // fill below: the live symbols in order (`runs`: frequency, symbol, first
+    // slot) and, per window of 32 slots, which slots start a run and how many
+    // runs start before the window (`wins`).
+    if (wave == 0) {
+      uint32_t head, kk = 0, live4 = 0, rank0 = 0;  // rank0: table rank of this lane's first live symbol
+      uint32_t rk[4] = {0, 0, 0, 0};
       if (mode == NZ_MODE_BITMAP) {
-        live = (tb[1 + (sym >> 3)] >> (sym & 7)) & 1u;
-        for (uint32_t b = 0; b < (sym >> 3); ++b) rank += __popc((uint32_t)tb[1 + b]);
-        rank += __popc((uint32_t)tb[1 + (sym >> 3)] & ((1u << (sym & 7)) - 1u));
+        head = 33;
+        live4 = ((uint32_t)tb[1 + (lane >> 1)] >> (4 * (lane & 1))) & 15u;
+        const uint32_t c = (uint32_t)__popc(live4);
+        const uint32_t ci = nz_wave_scan(c, lane);
+        kk = __builtin_amdgcn_readlane(ci, 63);
+        rank0 = ci - c;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) rk[j] = rank0 + (uint32_t)__popc(live4 & ((1u << j) - 1u));
       } else {
+        head = 1 + 2 * mode;
         uint32_t acc = 0;
         for (uint32_t r = 0; r < mode; ++r) {
           const uint32_t st = tb[1 + 2 * r], ln = (uint32_t)tb[2 + 2 * r] + 1u;
-          if (sym >= st && sym < st + ln) {
-            live = 1;
-            rank = acc + sym - st;
+#pragma unroll
+          for (uint32_t j = 0; j < 4; ++j) {
+            const uint32_t sym = 4 * lane + j;
+            if (sym >= st && sym < st + ln) {
+              live4 |= 1u << j;
+              rk[j] = acc + sym - st;
+            }
           }
           acc += ln;
         }
+        kk = acc;
       }
-      if (rank > 255) rank = 255;
-      cum[sym + 1] = live ? nz_get12(tb + head, rank) : 0u;
-    }
-    __syncthreads();
-    // inclusive scan by wavefront 0, four symbols per lane
-    if (wave == 0) {
-      uint32_t a0 = cum[4 * lane + 1], a1 = cum[4 * lane + 2], a2 = cum[4 * lane + 3],
-               a3 = cum[4 * lane + 4];
-      uint32_t tot = a0 + a1 + a2 + a3, incl = tot;
+      if (kk > 256) kk = 256;  // corrupt input: stay inside the staged bytes
+      uint32_t fr[4], tot = 0;
 #pragma unroll
-      for (int o = 1; o < 64; o <<= 1) {
-        uint32_t t = __shfl_up(incl, o, 64);
-        if (lane >= (uint32_t)o) incl += t;
+      for (uint32_t j = 0; j < 4; ++j) {
+        fr[j] = ((live4 >> j) & 1u) ? nz_get12(tb + head, rk[j] > 255 ? 255u : rk[j]) : 0u;
+        tot += fr[j];
       }
-      uint32_t ex = incl - tot;
-      cum[4 * lane + 1] = ex + a0;
-      cum[4 * lane + 2] = ex + a0 + a1;
-      cum[4 * lane + 3] = ex + a0 + a1 + a2;
-      cum[4 * lane + 4] = incl;
-      if (lane == 0) cum[0] = 0;
+      // one scan for both the cumulative frequency (below 2^20) and the number of
+      // symbols with a nonzero frequency (from bit 20 up)
+      uint32_t nz4 = 0;
+#pragma unroll
+      for (uint32_t j = 0; j < 4; ++j) nz4 += fr[j] ? 1u : 0u;
+      const uint32_t mine = tot | (nz4 << 20);
+      const uint32_t incl = nz_wave_scan(mine, lane);
+      const uint32_t all = __builtin_amdgcn_readlane(incl, 63);
+      const bool sums = (all & 0xFFFFFu) == NZ_M;
+      wins[lane] = make_uint2(0u, 0u);
+      wins[lane + 64] = make_uint2(0u, 0u);
+      if (lane == 0) {
+        tflag[0] = sums ? 1u : 0u;
+        tflag[1] = (head + (12 * kk + 7) / 8 + 3) & ~3u;
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (sums) {  // only then do the first slots stay below 4096
+        uint32_t first = (incl - mine) & 0xFFFFFu, k = (incl - mine) >> 20;
+#pragma unroll
+        for (uint32_t j = 0; j < 4; ++j) {
+          if (fr[j]) {
+            runs[k] = make_uint2(fr[j] | ((4 * lane + j) << 24), first);
+            atomicOr(&wins[first >> 5].x, 1u << (first & 31));
+            ++k;
+            first += fr[j];
+          }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        // runs that start before each window: prefix of the bitmap's popcounts
+        const uint32_t b0 = wins[2 * lane].x, b1 = wins[2 * lane + 1].x;
+        const uint32_t c0 = (uint32_t)__popc(b0), c1 = (uint32_t)__popc(b1);
+        const uint32_t pi = nz_wave_scan(c0 + c1, lane);
+        wins[2 * lane].y = pi - c0 - c1;
+        wins[2 * lane + 1].y = pi - c1;
+      }
     }
     __syncthreads();
-    if (cum[256] != NZ_M) {
+    if (!tflag[0]) {
       if (tid == 0) atomicOr(d_status, 2u);
       return;
     }
-    // slot table: the lanes of a wave hold (cum, freq) of four symbols each; the
-    // live symbols are walked with ballot/readlane and every thread of the
-    // workgroup fills a stride of the symbol's slot range.
+    tab_len = tflag[1];
+    // slot table: consecutive threads fill consecutive slots.  The run of a
+    // slot is the number of runs that start at or before it, minus one.
     {
-      uint32_t cv[5];
-#pragma unroll
-      for (int j = 0; j < 5; ++j) cv[j] = cum[4 * lane + j];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint32_t fj = cv[j + 1] - cv[j];
-        uint64_t live = __ballot(fj != 0);
-        while (live) {
-          const int l = __builtin_ctzll(live);
-          live &= live - 1;
-          const uint32_t f = __builtin_amdgcn_readlane(fj, l);
-          const uint32_t cb = __builtin_amdgcn_readlane(cv[j], l);
-          const uint32_t elo = f | ((uint32_t)(4 * l + j) << 24);
-          for (uint32_t i = tid; i < f; i += blockDim.x) lut[cb + i] = make_uint2(elo, i);
-        }
+      const uint32_t below = (2u << (tid & 31)) - 1u;  // bits of a window up to this thread's slot
+      for (uint32_t slot = tid; slot < NZ_M; slot += blockDim.x) {
+        const uint2 wn = wins[slot >> 5];
+        const uint32_t k = wn.y + (uint32_t)__popc(wn.x & below) - 1u;
+        const uint2 rn = runs[k & 255u];
+        lut[slot] = make_uint2(rn.x, slot - rn.y);
       }
     }
   }
   __syncthreads();
 
-  if (wave >= nseg) return;
-  const uint64_t seg = seg0 + wave;
-  const uint64_t seg_base = chunk_base + (uint64_t)wave * g.seg_syms;
-  const uint32_t nom = nz_seg_nominal(g.chunk_syms, g.seg_syms, g.spc, wave);
-  const uint32_t seg_n = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
-  const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
-  uint64_t o0 = dir[seg], o1 = dir[seg + 1];
-  if (o1 < o0 || g.rec_off + 4 * o1 > comp_bytes) {
+  if (!has_seg) return;
+  if (bad_rec) {
     if (lane == 0) atomicOr(d_status, 2u);
     return;
   }
-  uint64_t rec_start = g.rec_off + 4 * o0;
-  uint64_t rec_bytes = 4 * (o1 - o0);
-  if (wave == 0) {
-    if (rec_bytes < tab_len) {
-      if (lane == 0) atomicOr(d_status, 2u);
-      return;
-    }
-    rec_start += tab_len;
-    rec_bytes -= tab_len;
+  // the chunk's first record begins with the table
+  const uint32_t rec_skip = wave == 0 ? tab_len : 0u;
+  if (rec_all < rec_skip) {
+    if (lane == 0) atomicOr(d_status, 2u);
+    return;
   }
-  // stored packed layout: every full segment keeps seg_p - 128 bytes, its last
-  // 128 bytes ride in the coder states (or behind the symbols of a raw record)
-  const bool carry = seg_n == nom;
-  const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
-  const uint64_t chunk_keep = (uint64_t)g.chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * g.spc;
-  const uint8_t* pk = packed + c * chunk_keep + (uint64_t)wave * (g.seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES);
-  uint16_t* dst = out + seg_base;
-  NzGemvWalk walk;
-  if constexpr (GEMV) walk.start(gv, g, seg_base, seg_n, wave, lane);
+  const uint64_t rec_start = rec_pos + rec_skip;
+  const uint32_t rec_bytes = rec_all - rec_skip;
 
   if (mode == NZ_MODE_RAW) {
     const uint32_t padded = (seg_n + 3) & ~3u;
@@ -1270,11 +1335,9 @@ __device__ __forceinline__ void nz_decode_chunk(
     if (lane == 0) atomicOr(d_status, 2u);
     return;
   }
-  // the record position is the same for all lanes: keep it in scalar registers
-  const uint64_t rs = ((uint64_t)__builtin_amdgcn_readfirstlane((uint32_t)(rec_start >> 32)) << 32) |
-                      __builtin_amdgcn_readfirstlane((uint32_t)rec_start);
-  // final encoder states: 64 two-bit length codes, then a nibble stream
-  const uint32_t* rec32 = reinterpret_cast<const uint32_t*>(comp + rs);
+  // final encoder states, read from the staged window: 64 two-bit length
+  // codes, then a nibble stream
+  const uint32_t* rec32 = w.ring32 + rec_skip / 4;
   const uint32_t nn = 5u + ((rec32[lane >> 4] >> (2 * (lane & 15))) & 3u);
   const uint32_t incl = nz_wave_scan(nn, lane);
   const uint32_t at = incl - nn;
@@ -1283,35 +1346,12 @@ __device__ __forceinline__ void nz_decode_chunk(
     if (lane == 0) atomicOr(d_status, 2u);
     return;
   }
-  // the 8 bytes read here may reach into the words or the next record; the
-  // container's closing padding keeps them in bounds
+  // the 8 bytes read here may reach into the words: still inside the window
   const uint32_t fb = 16u + (at >> 1);
   const uint64_t win = (uint64_t)rec32[fb >> 2] | ((uint64_t)rec32[(fb >> 2) + 1] << 32);
   const uint32_t x0 = (uint32_t)(win >> (8 * (fb & 3) + 4 * (at & 1))) & (0xFFFFFFFFu >> (32 - 4 * nn));
-  NzWaveDec w;
-  w.lut = lut;
-  w.ring32 = rings + wave * NZ_RING_ALLOC_DWORDS;
-  w.words = comp + rs + sbytes;
-  w.last16 = comp + comp_bytes - NZ_TAIL_PAD;
-  w.nwords = __builtin_amdgcn_readfirstlane((uint32_t)((rec_bytes - sbytes) / 2));
-  w.lane = lane;
-  w.start(x0);
+  w.start(x0, (rec_skip + sbytes) / 2);
 
-  // groups whose packed bytes are (partly) carried are merged after the loop
-  const uint32_t tailg = carry ? (S == 0 ? 2u : 1u) : 0u;
-  const uint32_t body = ngroups - tailg;
-  // Groups in which every lane has 8 elements run without any predicate; the
-  // packed bytes are fetched one group ahead of their use (the address of the
-  // fetch past the last group is clamped, its value unused).
-  const uint32_t whole = seg_n / NZ_GROUP_SYMS < body ? seg_n / NZ_GROUP_SYMS : body;
-  const uint32_t lane_off = lane * (S + 1);
-  const uint32_t last_off = whole ? (whole - 1) * NZ_LANES * (S + 1) + lane_off : 0u;
-  uint64_t sm_next = whole ? nz_load_sm<S>(pk + lane_off) : 0;
-  uint4 xq_next = make_uint4(0, 0, 0, 0);
-  if constexpr (GEMV) xq_next = walk.load(walk.col);
-  uint64_t nb_next = 0;
-  if constexpr (NORM)
-    if (whole) nb_next = nz_norm_load8(nm, seg_base + lane * NZ_GROUP);
   for (uint32_t gq = 0; gq < whole; ++gq) {
     const uint64_t sm = sm_next;
     const uint32_t noff = (gq + 1) * NZ_LANES * (S + 1) + lane_off;
