@@ -784,7 +784,9 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
 // falls below 2^16 a 16-bit word taken at (words consumed so far by the wave +
 // rank of the lane among the lanes that need one).
 
-#define NZ_RING_ALLOC_DWORDS NZ_RING_DWORDS
+// a ring is followed by a copy of its first 64 words, so that the 64 words a
+// step may touch never wrap
+#define NZ_RING_ALLOC_DWORDS (NZ_RING_DWORDS + 32)
 #define NZ_DEC_CUM_DWORDS (512 + 256 + 4)  /* table-parse results: runs, windows, flags */
 // dynamic LDS of a decode workgroup whose chunks have up to `spc` segments
 #define NZ_DEC_LDS_BYTES(spc) ((size_t)(2 * NZ_M + (spc) * NZ_RING_ALLOC_DWORDS + NZ_DEC_CUM_DWORDS) * 4)
@@ -976,7 +978,8 @@ struct NzWaveDec {
   const uint2* lut;
   uint32_t* ring32;       // 512 dwords = 1024 words: a window of the record
   const uint8_t* words;   // start of the record (uniform); word indices count from here
-  const uint8_t* last16;  // last 16-byte block that may be loaded: container end - 16 (uniform)
+  uint32_t lim;           // largest byte offset from `words` that may be loaded: container end - 16 (uniform)
+  uint32_t ring_addr;     // LDS byte address of the ring (uniform)
   uint32_t nwords;        // 16-bit units the record holds, table and states included
   uint32_t lane;
   uint32_t x;             // this lane's rANS state
@@ -989,14 +992,25 @@ struct NzWaveDec {
   // unconditional and in bounds; words past the record are never consumed by
   // a valid stream.
   __device__ __forceinline__ uint4 fetch(uint32_t d) const {
-    const uint8_t* p = words + 4ull * d;
-    p = p < last16 ? p : last16;
-    const uint32_t* q = reinterpret_cast<const uint32_t*>(p);
+    const uint32_t off = 4u * d < lim ? 4u * d : lim;
+    const uint32_t* q = reinterpret_cast<const uint32_t*>(words + off);
     return make_uint4(q[0], q[1], q[2], q[3]);
   }
 
   __device__ __forceinline__ void commit(uint32_t d, const uint4& v) {
-    *reinterpret_cast<uint4*>(ring32 + (d & (NZ_RING_DWORDS - 1))) = v;
+    const uint32_t i = d & (NZ_RING_DWORDS - 1);
+    *reinterpret_cast<uint4*>(ring32 + i) = v;
+    if (i < 32) *reinterpret_cast<uint4*>(ring32 + NZ_RING_DWORDS + i) = v;  // the copy behind the end
+  }
+
+  // record at comp + pos of a container of comp_bytes (pos + 16 <= comp_bytes)
+  __device__ __forceinline__ void attach(const uint8_t* comp, uint64_t comp_bytes, uint64_t pos, uint32_t* ring) {
+    typedef __attribute__((address_space(3))) uint32_t lds_u32;
+    ring32 = ring;
+    ring_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((lds_u32*)ring));
+    words = comp + pos;
+    const uint64_t room = comp_bytes - NZ_TAIL_PAD - pos;
+    lim = room < 0xFFFFFFF0ull ? (uint32_t)room : 0xFFFFFFF0u;
   }
 
   // Stage the first 512 dwords of the record (table of a chunk's first record,
@@ -1036,12 +1050,7 @@ struct NzWaveDec {
       __builtin_amdgcn_wave_barrier();
     }
     r = fetch(filled + 4 * lane);
-    // LDS byte address of the ring (4 KiB aligned inside the workgroup's LDS)
-    typedef __attribute__((address_space(3))) uint32_t lds_u32;
     typedef __attribute__((address_space(3))) const uint16_t lds_cu16;
-    const uint32_t ring_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((lds_u32*)ring32));
-    uint32_t wmask = 2 * NZ_RING_WORDS - 2;  // kept in a VGPR: v_and_or_b32 takes one scalar operand
-    asm volatile("" : "+v"(wmask));
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const uint2 e = lut[x & (NZ_M - 1)];
@@ -1051,9 +1060,9 @@ struct NzWaveDec {
       const uint64_t m = __ballot(need);
       const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
                                                       __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-      // word (base + rank) mod 2048 of the ring: add-shift, then bitfield insert
-      uint32_t at;
-      asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(at) : "v"((rank + base) << 1), "v"(wmask), "s"(ring_addr));
+      // word base + rank of the record: the ring position of `base` is scalar
+      // arithmetic, the lane adds its rank (never past the copy behind the end)
+      const uint32_t at = ring_addr + 2u * (base & (NZ_RING_WORDS - 1)) + 2u * rank;
       uint32_t w = *(lds_cu16*)(uintptr_t)at;
       // keep the word read unconditional: straight-line code, no exec-mask branch
       asm volatile("" : "+v"(w));
@@ -1119,7 +1128,7 @@ __device__ __forceinline__ void nz_decode_chunk(
   // bytes of its first group.
   const uint32_t dv = lane <= nseg ? dir[seg0 + lane] : 0u;
   const uint64_t f0 = __builtin_amdgcn_readlane(dv, 0), f1 = __builtin_amdgcn_readlane(dv, 1);
-  if (f1 <= f0 || g.rec_off + 4 * f1 > comp_bytes) {
+  if (f1 <= f0 || g.rec_off + 4 * f1 + NZ_TAIL_PAD > comp_bytes) {
     if (tid == 0) atomicOr(d_status, 2u);
     return;
   }
@@ -1130,7 +1139,7 @@ __device__ __forceinline__ void nz_decode_chunk(
   const uint32_t seg_n = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
   const uint64_t o0 = __builtin_amdgcn_readlane(dv, wk), o1 = __builtin_amdgcn_readlane(dv, wk + 1);
-  const bool bad_rec = o1 < o0 || g.rec_off + 4 * o1 > comp_bytes;
+  const bool bad_rec = o1 < o0 || g.rec_off + 4 * o1 + NZ_TAIL_PAD > comp_bytes;
   const uint64_t rec_pos = g.rec_off + 4 * o0;  // uniform: the readlanes above are scalar
   const uint32_t rec_all = (uint32_t)(4 * (o1 - o0));
   // stored packed layout: every full segment keeps seg_p - 128 bytes, its last
@@ -1151,9 +1160,7 @@ __device__ __forceinline__ void nz_decode_chunk(
   const uint32_t last_off = whole ? (whole - 1) * NZ_LANES * (S + 1) + lane_off : 0u;
   NzWaveDec w;
   w.lut = lut;
-  w.ring32 = rings + wk * NZ_RING_ALLOC_DWORDS;
-  w.words = comp + rec_pos;
-  w.last16 = comp + comp_bytes - NZ_TAIL_PAD;
+  w.attach(comp, comp_bytes, bad_rec ? 0 : rec_pos, rings + wk * NZ_RING_ALLOC_DWORDS);
   w.nwords = rec_all / 2;
   w.lane = lane;
   w.filled = 0;
