@@ -817,7 +817,8 @@ __device__ __forceinline__ uint4 nz_merge_group(uint64_t sm, const uint32_t (&ew
       const uint32_t t = q << 7;
       const uint32_t w = k < 2 ? lo : hi;
       const uint32_t u = __builtin_amdgcn_perm(0u, w, (k & 1) ? 0x03030202u : 0x01010000u);
-      o[k] = (t & 0x7F807F80u) | (u & ~0x7F807F80u);
+      // bitfield insert: (mask & t) | (~mask & u)
+      asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(o[k]) : "s"(0x7F807F80u), "v"(t), "v"(u));
     }
   } else {
 #pragma unroll
