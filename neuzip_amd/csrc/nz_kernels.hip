@@ -821,11 +821,34 @@ __device__ __forceinline__ uint4 nz_merge_group(uint64_t sm, const uint32_t (&ew
       asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(o[k]) : "s"(0x7F807F80u), "v"(t), "v"(u));
     }
   } else {
+    // Fewer mantissa bits: the same shape.  A byte that holds an element's sign
+    // in bit 7 and its mantissa bits right below goes into both bytes of the
+    // element's half (sign on bit 15, mantissa from bit 6 down); what else the
+    // byte holds is masked away, and the exponents, alone in their word, are
+    // or-ed in.
+    const uint32_t lo = (uint32_t)sm;
+    constexpr uint32_t keep = 0x80008000u | (((0x7Fu << (7 - S)) & 0x7Fu) * 0x00010001u);
+    constexpr int NV = S == 3 ? 2 : (S == 1 ? 4 : 8);
+    uint32_t v[NV];  // v[i]: the packed bytes shifted left by i fields
 #pragma unroll
-    for (int j = 0; j < 8; j += 2) {
-      uint32_t r0 = (uint32_t)(sm >> nz_field_shift<S>(j)) & ((2u << S) - 1u);
-      uint32_t r1 = (uint32_t)(sm >> nz_field_shift<S>(j + 1)) & ((2u << S) - 1u);
-      o[j >> 1] = nz_merge_one<S>(ew[j] >> 24, r0) | (nz_merge_one<S>(ew[j + 1] >> 24, r1) << 16);
+    for (int i = 0; i < NV; ++i) v[i] = lo << (i * (S + 1));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t q = __builtin_amdgcn_perm(ew[2 * k + 1], ew[2 * k], 0x0c070c03u);
+      const uint32_t t = q << 7;
+      uint32_t u;
+      if constexpr (S == 3) {
+        // byte k holds elements 2k (high nibble) and 2k + 1
+        u = __builtin_amdgcn_perm(v[1], v[0], (uint32_t)(4 + k) * 0x01010000u + (uint32_t)k * 0x0101u);
+      } else if constexpr (S == 1) {
+        // byte k / 2 holds elements 4 (k / 2) .. + 3, two bits each
+        const uint32_t b = (uint32_t)k >> 1;
+        u = __builtin_amdgcn_perm(v[2 * (k & 1) + 1], v[2 * (k & 1)], (4 + b) * 0x01010000u + b * 0x0101u);
+      } else {
+        // one byte holds the eight signs, element 0 in bit 7
+        u = __builtin_amdgcn_perm(v[2 * k + 1], v[2 * k], 0x04040000u);
+      }
+      o[k] = (u & keep) | t;
     }
   }
   return make_uint4(o[0], o[1], o[2], o[3]);
