@@ -198,6 +198,21 @@ __device__ __forceinline__ uint32_t nz_wave_scan(uint32_t v, uint32_t lane) {
   v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xC, 0xF, false);  // row_bcast:31
   return v;
 }
+// Sum of a float over the 64 lanes, by the same moves as nz_wave_scan (a fixed
+// order of additions); every lane gets the total.
+__device__ __forceinline__ float nz_wave_sum(float v) {
+#define NZ_DPP_ADD(ctrl, rows)                                                                      \
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rows, 0xF, false))
+  NZ_DPP_ADD(0x111, 0xF);
+  NZ_DPP_ADD(0x112, 0xF);
+  NZ_DPP_ADD(0x114, 0xF);
+  NZ_DPP_ADD(0x118, 0xF);
+  NZ_DPP_ADD(0x142, 0xA);
+  NZ_DPP_ADD(0x143, 0xC);
+#undef NZ_DPP_ADD
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
 __device__ __forceinline__ uint32_t nz_get12(const uint8_t* p, uint32_t i) {
   uint32_t bit = 12u * i;
   const uint8_t* q = p + (bit >> 3);
@@ -888,8 +903,7 @@ __device__ __forceinline__ float nz_dot8(const uint4 w, const uint4 x, float acc
 
 // Position of a wavefront inside W while it walks its segment group by group.
 //
-// When the wave leaves a row it adds its 64 partial sums in a fixed butterfly
-// order.  A row that lies inside the wave's segment is complete then: bias
+// When the wave leaves a row it adds its 64 partial sums in a fixed order.  A row that lies inside the wave's segment is complete then: bias
 // added, rounded, stored.  A row shared with other segments goes through the
 // row's accumulator pair: the sum in 24.40 fixed point (integer addition is
 // associative, so the result does not depend on which wave arrives first; a
@@ -952,9 +966,7 @@ struct NzGemvWalk {
     gv.y[row] = (uint16_t)nz_f32_to_bf16(v);
   }
   __device__ __forceinline__ void flush(uint32_t lane) {
-    float t = sum;
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) t += __shfl_xor(t, o, 64);
+    const float t = nz_wave_sum(sum);
     if (lane == 0) {
       const uint64_t first = row * gv.in_features, last = first + gv.in_features - 1;
       if (first >= seg_first && last < seg_end) {
