@@ -299,10 +299,14 @@ class Manager:
         honoured when given.  ``lane_symbols`` (extension; 0 = the best value
         for the chunk) is the number of exponents each of the 64 rANS lanes of a
         wavefront codes per segment: smaller values expose more wavefronts per
-        chunk at the price of about 4.5 bits of container per lane and segment.  ``"auto"`` keeps the default
-        for large tensors and shortens the segments of small ones so that they
-        still fill the GPU (meant for training, where every weight is decoded
-        three times and encoded once per step)."""
+        chunk at the price of about 4.5 bits of container per lane and segment.
+        ``"auto"`` picks the geometry per tensor from its size and from how many
+        decode workgroups the device holds at once: small tensors get shorter
+        segments (and smaller chunks) so that they still fill the GPU, mid-sized
+        ones slightly longer segments so that two of them decoded by one launch
+        run as a single round of workgroups (meant for single-token inference
+        and for training, where every weight is decoded three times and encoded
+        once per step)."""
         normalizer_size = 0 if normalizer_size is None else normalizer_size
         self.meta_dict = {}  # handle -> original shape
         self._writes = 0     # bumped by every write: lets caches of decoded weights notice

@@ -406,12 +406,16 @@ def test_read_batch_equals_single_reads(oracle):
 
 
 def test_auto_lane_symbols(oracle):
-    """Per-tensor geometry: small tensors get shorter segments, the stored bytes
-    are those of the oracle at that geometry, and reads are exact."""
+    """Per-tensor geometry: small tensors get shorter segments (32 Ki or 64 Ki
+    chunks of eight segments), tensors whose chunks would take between half and
+    all of the device's 768 workgroup slots get longer ones (at most 384
+    chunks), the stored bytes are those of the oracle at that geometry, and
+    reads are exact."""
     import neuzip_amd
 
     for chunk_arg, cases in (
-        (None, ((1 << 20, 65536, 176), (40_000_000, 131072, 256), (70_000_000, 131072, 256))),
+        (None, ((1 << 20, 32768, 64), (25_165_824, 32768, 64), (40_000_000, 65536, 128), (14336 * 4096, 155648, 304),
+                (70_000_000, 184320, 360), (110_000_000, 131072, 256))),
         (65536, ((1 << 20, 65536, 176), (40_000_000, 65536, 176), (70_000_000, 65536, 344))),
     ):
         mgr = neuzip_amd.Manager(chunk_size=chunk_arg, lane_symbols="auto")
