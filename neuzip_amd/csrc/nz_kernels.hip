@@ -1215,7 +1215,10 @@ __device__ __forceinline__ void nz_decode_chunk(
     }
   }
   __syncthreads();
-  const uint32_t mode = tb[0];
+  // the first 32 table bytes hold the mode and all run descriptors there can be
+  const uint4 h0 = reinterpret_cast<const uint4*>(tb)[0], h1 = reinterpret_cast<const uint4*>(tb)[1];
+  const uint32_t bm_byte = tb[1 + (lane >> 1)];  // bitmap mode: the byte with this lane's four symbols
+  const uint32_t mode = h0.x & 0xFFu;
   uint32_t tab_len = 4;
 
   if (mode != NZ_MODE_RAW) {
@@ -1228,58 +1231,59 @@ __device__ __forceinline__ void nz_decode_chunk(
     // slot) and, per window of 32 slots, which slots start a run and how many
     // runs start before the window (`wins`).
     if (wave == 0) {
-      uint32_t head, kk = 0, live4 = 0, rank0 = 0;  // rank0: table rank of this lane's first live symbol
-      uint32_t rk[4] = {0, 0, 0, 0};
+      wins[lane] = make_uint2(0u, 0u);
+      wins[lane + 64] = make_uint2(0u, 0u);
+      uint32_t head, kk = 0, live4 = 0;
+      uint32_t rk[4] = {0, 0, 0, 0};  // rank of the symbol among those the table lists
       if (mode == NZ_MODE_BITMAP) {
         head = 33;
-        live4 = ((uint32_t)tb[1 + (lane >> 1)] >> (4 * (lane & 1))) & 15u;
+        live4 = (bm_byte >> (4 * (lane & 1))) & 15u;
         const uint32_t c = (uint32_t)__popc(live4);
         const uint32_t ci = nz_wave_scan(c, lane);
         kk = __builtin_amdgcn_readlane(ci, 63);
-        rank0 = ci - c;
 #pragma unroll
-        for (uint32_t j = 0; j < 4; ++j) rk[j] = rank0 + (uint32_t)__popc(live4 & ((1u << j) - 1u));
+        for (uint32_t j = 0; j < 4; ++j) rk[j] = ci - c + (uint32_t)__popc(live4 & ((1u << j) - 1u));
       } else {
         head = 1 + 2 * mode;
+        const uint32_t hw[8] = {h0.x, h0.y, h0.z, h0.w, h1.x, h1.y, h1.z, h1.w};
         uint32_t acc = 0;
-        for (uint32_t r = 0; r < mode; ++r) {
-          const uint32_t st = tb[1 + 2 * r], ln = (uint32_t)tb[2 + 2 * r] + 1u;
 #pragma unroll
-          for (uint32_t j = 0; j < 4; ++j) {
-            const uint32_t sym = 4 * lane + j;
-            if (sym >= st && sym < st + ln) {
-              live4 |= 1u << j;
-              rk[j] = acc + sym - st;
+        for (uint32_t r = 0; r < NZ_MAX_RUNS; ++r) {
+          if (r < mode) {
+            const uint32_t st = (hw[(1 + 2 * r) >> 2] >> (8 * ((1 + 2 * r) & 3))) & 0xFFu;
+            const uint32_t ln = ((hw[(2 + 2 * r) >> 2] >> (8 * ((2 + 2 * r) & 3))) & 0xFFu) + 1u;
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) {
+              const uint32_t sym = 4 * lane + j;
+              if (sym >= st && sym < st + ln) {
+                live4 |= 1u << j;
+                rk[j] = acc + sym - st;
+              }
             }
+            acc += ln;
           }
-          acc += ln;
         }
         kk = acc;
       }
       if (kk > 256) kk = 256;  // corrupt input: stay inside the staged bytes
-      uint32_t fr[4], tot = 0;
+      uint32_t fr[4], tot = 0, nz4 = 0;
 #pragma unroll
       for (uint32_t j = 0; j < 4; ++j) {
-        fr[j] = ((live4 >> j) & 1u) ? nz_get12(tb + head, rk[j] > 255 ? 255u : rk[j]) : 0u;
+        const uint32_t f = nz_get12(tb + head, rk[j] > 255 ? 255u : rk[j]);  // read in any case: no branch
+        fr[j] = ((live4 >> j) & 1u) ? f : 0u;
         tot += fr[j];
+        nz4 += fr[j] ? 1u : 0u;
       }
       // one scan for both the cumulative frequency (below 2^20) and the number of
       // symbols with a nonzero frequency (from bit 20 up)
-      uint32_t nz4 = 0;
-#pragma unroll
-      for (uint32_t j = 0; j < 4; ++j) nz4 += fr[j] ? 1u : 0u;
       const uint32_t mine = tot | (nz4 << 20);
       const uint32_t incl = nz_wave_scan(mine, lane);
       const uint32_t all = __builtin_amdgcn_readlane(incl, 63);
       const bool sums = (all & 0xFFFFFu) == NZ_M;
-      wins[lane] = make_uint2(0u, 0u);
-      wins[lane + 64] = make_uint2(0u, 0u);
       if (lane == 0) {
         tflag[0] = sums ? 1u : 0u;
         tflag[1] = (head + (12 * kk + 7) / 8 + 3) & ~3u;
       }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
       if (sums) {  // only then do the first slots stay below 4096
         uint32_t first = (incl - mine) & 0xFFFFFu, k = (incl - mine) >> 20;
 #pragma unroll
@@ -1302,13 +1306,10 @@ __device__ __forceinline__ void nz_decode_chunk(
       }
     }
     __syncthreads();
-    if (!tflag[0]) {
-      if (tid == 0) atomicOr(d_status, 2u);
-      return;
-    }
-    tab_len = tflag[1];
     // slot table: consecutive threads fill consecutive slots.  The run of a
-    // slot is the number of runs that start at or before it, minus one.
+    // slot is the number of runs that start at or before it, minus one.  (Of a
+    // table whose frequencies do not sum to 4096 nothing was written: the fill
+    // then reads zeros and the chunk is given up right after.)
     {
       const uint32_t below = (2u << (tid & 31)) - 1u;  // bits of a window up to this thread's slot
       for (uint32_t slot = tid; slot < NZ_M; slot += blockDim.x) {
@@ -1318,6 +1319,11 @@ __device__ __forceinline__ void nz_decode_chunk(
         lut[slot] = make_uint2(rn.x, slot - rn.y);
       }
     }
+    if (!tflag[0]) {
+      if (tid == 0) atomicOr(d_status, 2u);
+      return;
+    }
+    tab_len = tflag[1];
   }
   __syncthreads();
 
