@@ -802,9 +802,14 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(
 // a ring is followed by a copy of its first 64 words, so that the 64 words a
 // step may touch never wrap
 #define NZ_RING_ALLOC_DWORDS (NZ_RING_DWORDS + 32)
-#define NZ_DEC_CUM_DWORDS (512 + 256 + 4)  /* table-parse results: runs, windows, flags */
+// What the table parse leaves for the slot-table fill (runs, windows, flags)
+// lies in the last slots of the table itself; those are filled last, from
+// registers.
+#define NZ_TMETA_DWORDS (512 + 256 + 4)
+#define NZ_TMETA_SLOT ((uint32_t)(NZ_M - 416))  /* first slot under it; a multiple of 32 */
+static_assert(2 * (NZ_M - NZ_TMETA_SLOT) >= NZ_TMETA_DWORDS && NZ_TMETA_SLOT % 32 == 0, "parse results fit under the tail");
 // dynamic LDS of a decode workgroup whose chunks have up to `spc` segments
-#define NZ_DEC_LDS_BYTES(spc) ((size_t)(2 * NZ_M + (spc) * NZ_RING_ALLOC_DWORDS + NZ_DEC_CUM_DWORDS) * 4)
+#define NZ_DEC_LDS_BYTES(spc) ((size_t)(2 * NZ_M + (spc) * NZ_RING_ALLOC_DWORDS) * 4)
 
 // S+1 packed bytes of one 8-element group, as a little-endian integer
 template <int S>
@@ -1064,7 +1069,8 @@ struct NzWaveDec {
   // into the record (at most 348, so at least 676 words are staged ahead).
   __device__ __forceinline__ void start(uint32_t x0, uint32_t first_word) {
     x = x0;
-    base = first_word;
+    base = __builtin_amdgcn_readfirstlane(first_word);  // the same in all lanes: keep it scalar
+    filled = __builtin_amdgcn_readfirstlane(filled);
     r = make_uint4(0, 0, 0, 0);
   }
 
@@ -1133,7 +1139,7 @@ __device__ __forceinline__ void nz_decode_chunk(
   extern __shared__ uint32_t lds[];
   uint2* lut = reinterpret_cast<uint2*>(lds);                   // 4096 x 8 bytes
   uint32_t* rings = lds + 2 * NZ_M;                             // spc rings
-  uint32_t* tmeta = rings + g.spc * NZ_RING_ALLOC_DWORDS;       // what the table parse leaves for the fill:
+  uint32_t* tmeta = lds + 2 * NZ_TMETA_SLOT;                    // what the table parse leaves for the fill:
   uint2* runs = reinterpret_cast<uint2*>(tmeta);                //   per live symbol (freq | symbol << 24, first slot)
   uint2* wins = runs + 256;                                     //   per 32 slots (bitmap of run starts, runs before)
   uint32_t* tflag = reinterpret_cast<uint32_t*>(wins + 128);    //   [0] frequencies sum to 4096, [1] table bytes
@@ -1309,21 +1315,39 @@ __device__ __forceinline__ void nz_decode_chunk(
     // slot table: consecutive threads fill consecutive slots.  The run of a
     // slot is the number of runs that start at or before it, minus one.  (Of a
     // table whose frequencies do not sum to 4096 nothing was written: the fill
-    // then reads zeros and the chunk is given up right after.)
+    // then reads zeros and the chunk is given up right after.)  The last slots
+    // lie under the parse results: their entries wait in registers until every
+    // thread has read what it needs.
     {
       const uint32_t below = (2u << (tid & 31)) - 1u;  // bits of a window up to this thread's slot
-      for (uint32_t slot = tid; slot < NZ_M; slot += blockDim.x) {
+      const auto entry_of = [&](uint32_t slot) {
         const uint2 wn = wins[slot >> 5];
         const uint32_t k = wn.y + (uint32_t)__popc(wn.x & below) - 1u;
         const uint2 rn = runs[k & 255u];
-        lut[slot] = make_uint2(rn.x, slot - rn.y);
+        return make_uint2(rn.x, slot - rn.y);
+      };
+      for (uint32_t slot = tid; slot < NZ_TMETA_SLOT; slot += blockDim.x) lut[slot] = entry_of(slot);
+      // (NZ_TMETA_SLOT is a multiple of 32, so `below` fits these slots as well)
+      constexpr uint32_t LAST = (NZ_M - NZ_TMETA_SLOT + 63) / 64;  // per thread, for the smallest workgroup
+      uint2 last[LAST];
+#pragma unroll
+      for (uint32_t i = 0; i < LAST; ++i) {
+        const uint32_t slot = NZ_TMETA_SLOT + tid + i * blockDim.x;
+        last[i] = slot < NZ_M ? entry_of(slot) : make_uint2(0u, 0u);
       }
+      const uint32_t table_ok = tflag[0], table_len = tflag[1];
+      __syncthreads();
+#pragma unroll
+      for (uint32_t i = 0; i < LAST; ++i) {
+        const uint32_t slot = NZ_TMETA_SLOT + tid + i * blockDim.x;
+        if (slot < NZ_M) lut[slot] = last[i];
+      }
+      if (!table_ok) {
+        if (tid == 0) atomicOr(d_status, 2u);
+        return;
+      }
+      tab_len = table_len;
     }
-    if (!tflag[0]) {
-      if (tid == 0) atomicOr(d_status, 2u);
-      return;
-    }
-    tab_len = tflag[1];
   }
   __syncthreads();
 
