@@ -51,7 +51,8 @@ def parse_args():
     ap.add_argument("--precision", type=int, default=7, choices=[7, 3, 1, 0])
     ap.add_argument("--chunk-size", type=int, default=0,
                     help="elements per frequency table; 0 = library default (131072), 65536 = the reference's nvcomp chunk")
-    ap.add_argument("--lane-symbols", type=int, default=0, help="0 = library default; -1 = per-tensor (model workloads)")
+    ap.add_argument("--lane-symbols", type=int, default=None,
+                    help="0 = library default; -1 = chosen per tensor (the default of the model workloads)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
@@ -448,6 +449,9 @@ def main():
     if not torch.cuda.is_available():
         print("no GPU visible", file=sys.stderr)
         return 2
+
+    if args.lane_symbols is None:  # model workloads: tensors of many sizes, geometry per tensor
+        args.lane_symbols = 0 if args.workload == "tensor" else -1
 
     if args.calibrate_copy:
         src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
