@@ -414,7 +414,7 @@ def test_auto_lane_symbols(oracle):
     import neuzip_amd
 
     for chunk_arg, cases in (
-        (None, ((1 << 20, 32768, 64), (25_165_824, 32768, 64), (40_000_000, 65536, 128), (14336 * 4096, 155648, 304),
+        (None, ((1000, 32768, 64), (40_001, 32768, 64), (1 << 20, 32768, 64), (25_165_824, 32768, 64), (40_000_000, 65536, 128), (14336 * 4096, 155648, 304),
                 (70_000_000, 184320, 360), (110_000_000, 131072, 256))),
         (65536, ((1 << 20, 65536, 176), (40_000_000, 65536, 176), (70_000_000, 65536, 344))),
     ):
