@@ -336,19 +336,25 @@ def run_gpt2m(args, torch):
             o.step()
         return loss.detach()
 
-    # the same model with dense bf16 weights and torch's AdamW, for scale
+    # the same model with dense bf16 weights and torch's AdamW: for scale, and (lossless
+    # setting) as the loss curve the compressed run has to reproduce
+    state0 = {k: v.clone() for k, v in model.state_dict().items()}
     opt = torch.optim.AdamW(model.parameters(), lr=1e-4)
+    torch.manual_seed(args.seed + 1)
+    dense_losses = []
     for _ in range(args.warmup):
-        train_step([opt])
+        dense_losses.append(train_step([opt]))
         opt.zero_grad(set_to_none=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        train_step([opt])
+        dense_losses.append(train_step([opt]))
         opt.zero_grad(set_to_none=True)
     torch.cuda.synchronize()
     dense_ms = (time.perf_counter() - t0) / args.steps * 1e3
     del opt
+    model.load_state_dict(state0)
+    del state0
     torch.cuda.empty_cache()
 
     mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size or None,
@@ -384,8 +390,7 @@ def run_gpt2m(args, torch):
             opt_d.zero_grad(set_to_none=True)
             return loss
 
-        for _ in range(args.warmup):
-            step()
+        warm = [step() for _ in range(args.warmup)]
         torch.cuda.synchronize()
         spans.clear()
         t0 = time.perf_counter()
@@ -403,12 +408,19 @@ def run_gpt2m(args, torch):
             "encodes_per_step": sum(1 for k, _, _ in spans if k == "encode") / args.steps,
             "first_loss": round(float(losses[0]), 4),
             "last_loss": round(float(losses[-1]), 4),
-        }, wall
+        }, wall, warm + losses
 
-    per_linear, _ = run(1)
+    # per block first: it starts from the very weights, data and optimizer state the dense run
+    # started from, so with a lossless manager its losses must be the dense run's, bit for bit
     per_block_linears = len(comp_params) // max(1, layers)
+    torch.manual_seed(args.seed + 1)
     with neuzip_amd.DecompressAhead(mgr, model, ahead=False):
-        per_block, wall = run(per_block_linears)
+        per_block, wall, comp_losses = run(per_block_linears)
+    same = sum(1 for a, b in zip(dense_losses, comp_losses) if torch.equal(a, b))
+    per_block["steps_with_the_dense_runs_loss"] = f"{same} of {len(dense_losses)}"
+    per_block["dense_first_loss"] = round(float(dense_losses[args.warmup]), 4)
+    per_block["dense_last_loss"] = round(float(dense_losses[-1]), 4)
+    per_linear, _, _ = run(1)
     mgr._be.check()
     tokens = args.batch * (args.seq_len - 1) * args.steps
     out = {

@@ -207,8 +207,10 @@ class GPT2Shaped(torch.nn.Module):
 
 class CompressedAdamW:
     """AdamW for compressed parameters: decompress, update, re-compress under the
-    same handle (the read -> update -> write idiom of neuzip/__init__.py:25-35
-    with Adam moments kept dense in fp32)."""
+    same handle (the read -> update -> write idiom of neuzip/__init__.py:25-35).
+    The update itself is torch's own multi-tensor AdamW on the decoded weights,
+    with moments in the weights' dtype as ``torch.optim.AdamW`` keeps them, so a
+    lossless manager trains exactly like the dense model."""
 
     def __init__(self, params, lr=1e-4, betas=(0.9, 0.999), eps=1e-8, weight_decay=0.01, group=1):
         """``group``: parameters are read, updated and written back ``group`` at a
@@ -218,35 +220,32 @@ class CompressedAdamW:
         self.group = max(1, int(group))
         self.lr, self.b1, self.b2, self.eps, self.wd = lr, betas[0], betas[1], eps, weight_decay
         self.state = {}
-        self.t = 0
 
     @torch.no_grad()
     def step(self):
-        self.t += 1
-        c1 = 1.0 - self.b1 ** self.t
-        c2 = 1.0 - self.b2 ** self.t
+        from torch.optim.adamw import adamw
+
         todo = [p for p in self.params if p._gradient is not None]
         for at in range(0, len(todo), self.group):
             batch = todo[at:at + self.group]
-            new = []
+            weights, grads, m1, m2, steps = [], [], [], [], []
             for p in batch:
-                g = p._gradient
+                w = p.shared()  # decompress; updated in place, then written back under the same handle
                 st = self.state.get(p._handle)
                 if st is None:
-                    st = (torch.zeros_like(g, dtype=torch.float32), torch.zeros_like(g, dtype=torch.float32))
+                    st = (torch.zeros_like(w), torch.zeros_like(w), torch.tensor(0.0, dtype=torch.float32))
                     self.state[p._handle] = st
-                m, v = st
-                gf = g.float()
-                m.mul_(self.b1).add_(gf, alpha=1 - self.b1)
-                v.mul_(self.b2).addcmul_(gf, gf, value=1 - self.b2)
-                wf = p.shared().float()  # decompress (read only: the float copy is what changes)
-                wf.mul_(1 - self.lr * self.wd)
-                wf.addcdiv_(m, (v / c2).sqrt_().add_(self.eps), value=-self.lr / c1)
-                new.append(wf.to(torch.bfloat16))
+                weights.append(w)
+                grads.append(p._gradient.to(w.dtype).view_as(w))
+                m1.append(st[0])
+                m2.append(st[1])
+                steps.append(st[2])
+            adamw(weights, grads, m1, m2, [], steps, foreach=True, amsgrad=False, beta1=self.b1, beta2=self.b2,
+                  lr=self.lr, weight_decay=self.wd, eps=self.eps, maximize=False)
             if len(batch) > 1:
-                batch[0]._manager.write_many(new, [p._handle for p in batch])  # re-compress, one sync
+                batch[0]._manager.write_many(weights, [p._handle for p in batch])  # re-compress, one sync
             else:
-                batch[0]._manager.write(new[0], batch[0]._handle)
+                batch[0]._manager.write(weights[0], batch[0]._handle)
             for p in batch:
                 p._gradient = None
                 p.grad = None
