@@ -73,17 +73,6 @@ EncLayout enc_layout(const NzGeom& g) {
   return L;
 }
 
-template <int S>
-void launch_split_encode(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws,
-                         const EncLayout& L, const NzNorm& nm, hipStream_t st) {
-  hipLaunchKernelGGL(nz_split_encode_kernel<S>, dim3((uint32_t)g.n_chunks), dim3(NZ_SPLIT_THREADS), 0, st,
-                     (const uint16_t*)in, g.n, g.chunk_syms, g.lane_syms, g.spc, packed, ws + L.carry,
-                     ws + L.exps, (uint32_t*)(ws + L.enc_tab), ws + L.tab_ser,
-                     (NzChunkInfo*)(ws + L.info), nm, (uint16_t*)(ws + L.slots), (uint32_t*)(ws + L.states),
-                     (uint32_t*)(ws + L.seg_words), (uint32_t*)(ws + L.seg_sbytes),
-                     (uint32_t*)(ws + L.seg_units));
-}
-
 // group bytes of a tensor that is about to be split (nothing to do without normalizers)
 int launch_absmax(const void* in, uint64_t n, uint32_t ns, uint8_t* norm, hipStream_t st) {
   if (!ns || !n) return NZ_OK;
@@ -93,37 +82,82 @@ int launch_absmax(const void* in, uint64_t n, uint32_t ns, uint8_t* norm, hipStr
   return NZ_OK;
 }
 
-// Phase 1: everything up to the directory.  Header + directory land in `hdr`
-// (g.rec_off bytes), the container size in *d_total.
-int encode_phase1(const NzGeom& g, int precision, const void* in, uint8_t* packed, uint8_t* ws,
-                  const EncLayout& L, uint8_t* hdr, uint64_t cap, uint64_t* d_total,
-                  uint32_t* d_status, uint32_t ns, uint8_t* norm, hipStream_t st) {
-  if (g.n_chunks > 0) {
-    if (int rc = launch_absmax(in, g.n, ns, norm, st)) return rc;
-    const NzNorm nm{ns ? norm : nullptr, log2_of(ns ? ns : 1)};
+// One tensor of an encode call, as the kernels see it.  `hdr` is where header
+// and directory are built, `comp`/`comp_cap` where the records go (known only
+// after phase 1 when the buffer is sized to fit).
+NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws, const EncLayout& L,
+                   uint8_t* hdr, uint8_t* comp, uint64_t comp_cap, uint64_t* d_total, uint32_t* d_status,
+                   uint32_t ns, uint8_t* norm) {
+  NzEncItem it{};
+  it.in = (const uint16_t*)in;
+  it.packed = packed;
+  it.ws = ws;
+  it.hdr = hdr;
+  it.comp = comp;
+  it.comp_cap = comp_cap;
+  it.d_total = d_total;
+  it.d_status = d_status;
+  it.nm = NzNorm{ns ? norm : nullptr, log2_of(ns ? ns : 1)};
+  it.g = g;
+  it.exps = L.exps;
+  it.enc_tab = L.enc_tab;
+  it.tab_ser = L.tab_ser;
+  it.info = L.info;
+  it.carry = L.carry;
+  it.slots = L.slots;
+  it.states = L.states;
+  it.seg_words = L.seg_words;
+  it.seg_sbytes = L.seg_sbytes;
+  it.seg_units = L.seg_units;
+  return it;
+}
+
+// running totals of chunks and segments; false when they do not fit a grid
+bool enc_batch_close(NzEncBatch* b) {
+  uint64_t chunks = 0, segs = 0;
+  for (uint32_t i = 0; i < b->count; ++i) {
+    chunks += b->item[i].g.n_chunks;
+    segs += b->item[i].g.n_segs;
+    if (chunks > 0x7FFFFFFFull || segs > 0x7FFFFFFFull) return false;
+    b->item[i].chunk_end = (uint32_t)chunks;
+    b->item[i].seg_end = (uint32_t)segs;
+  }
+  return true;
+}
+
+// Phase 1 for all tensors of the batch: everything up to the directory.  Header
+// + directory land in each item's `hdr`, the container size in its *d_total.
+int encode_phase1(NzEncBatch* b, int precision, uint32_t ns, hipStream_t st) {
+  if (!enc_batch_close(b)) return fail(NZ_ERR_ARG, "too many chunks for one launch");
+  for (uint32_t i = 0; i < b->count; ++i)
+    if (int rc = launch_absmax(b->item[i].in, b->item[i].g.n, ns, const_cast<uint8_t*>(b->item[i].nm.bytes), st))
+      return rc;
+  const uint32_t chunks = b->count ? b->item[b->count - 1].chunk_end : 0;
+  if (chunks) {
+    const dim3 grid(chunks), block(NZ_SPLIT_THREADS);
     switch (precision) {
-      case 7: launch_split_encode<7>(g, in, packed, ws, L, nm, st); break;
-      case 3: launch_split_encode<3>(g, in, packed, ws, L, nm, st); break;
-      case 1: launch_split_encode<1>(g, in, packed, ws, L, nm, st); break;
-      default: launch_split_encode<0>(g, in, packed, ws, L, nm, st); break;
+      case 7: hipLaunchKernelGGL(nz_split_encode_kernel<7>, grid, block, 0, st, *b); break;
+      case 3: hipLaunchKernelGGL(nz_split_encode_kernel<3>, grid, block, 0, st, *b); break;
+      case 1: hipLaunchKernelGGL(nz_split_encode_kernel<1>, grid, block, 0, st, *b); break;
+      default: hipLaunchKernelGGL(nz_split_encode_kernel<0>, grid, block, 0, st, *b); break;
     }
   }
-  hipLaunchKernelGGL(nz_scan_kernel, dim3(1), dim3(1024), 0, st,
-                     (const uint32_t*)(ws + L.seg_units), g, hdr, cap, d_total, d_status);
+  if (b->count) hipLaunchKernelGGL(nz_scan_kernel, dim3(b->count), dim3(1024), 0, st, *b);
   NZ_HIP(hipGetLastError());
   return NZ_OK;
 }
 
-// Phase 2: place the records behind a header/directory already at `comp`.
-int encode_phase2(const NzGeom& g, uint8_t* ws, const EncLayout& L, const uint32_t* dir,
-                  uint8_t* comp, uint64_t cap, hipStream_t st) {
-  if (g.n_segs > 0) {
-    hipLaunchKernelGGL(nz_compact_kernel, dim3((uint32_t)g.n_segs), dim3(256), 0, st,
-                       ws + L.exps, g, (const NzChunkInfo*)(ws + L.info), ws + L.tab_ser,
-                       ws + L.carry, (const uint16_t*)(ws + L.slots),
-                       (const uint32_t*)(ws + L.states),
-                       (const uint32_t*)(ws + L.seg_words), (const uint32_t*)(ws + L.seg_sbytes), dir,
-                       comp, cap);
+// Phase 2: the records (and, where it was built elsewhere, header and directory)
+// go to each item's `comp`.
+int encode_phase2(NzEncBatch* b, hipStream_t st) {
+  const uint32_t segs = b->count ? b->item[b->count - 1].seg_end : 0;
+  for (uint32_t i = 0; i < b->count; ++i) {  // a tensor without segments has no workgroup to move its header
+    const NzEncItem& it = b->item[i];
+    if (it.g.n_segs == 0 && it.hdr != it.comp)
+      NZ_HIP(hipMemcpyAsync(it.comp, it.hdr, it.g.rec_off + NZ_TAIL_PAD, hipMemcpyDeviceToDevice, st));
+  }
+  if (segs) {
+    hipLaunchKernelGGL(nz_compact_kernel, dim3(segs), dim3(256), 0, st, *b);
     NZ_HIP(hipGetLastError());
   }
   return NZ_OK;
@@ -328,12 +362,12 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
   if (comp_cap < nz_geom_bound(&g)) return fail(NZ_ERR_CAPACITY, "dev_comp smaller than nz_exp_bound_bytes");
   hipStream_t st = (hipStream_t)stream;
   uint8_t* ws = (uint8_t*)dev_workspace;
-  if (int rc = encode_phase1(g, precision, dev_bf16, (uint8_t*)dev_packed, ws, L, (uint8_t*)dev_comp,
-                             comp_cap, dev_total, dev_status, normalizer_size, (uint8_t*)dev_norm, st))
-    return rc;
-  if (int rc = encode_phase2(g, ws, L, (const uint32_t*)((uint8_t*)dev_comp + g.dir_off),
-                             (uint8_t*)dev_comp, comp_cap, st))
-    return rc;
+  NzEncBatch b{};
+  b.count = 1;
+  b.item[0] = enc_item(g, dev_bf16, (uint8_t*)dev_packed, ws, L, (uint8_t*)dev_comp, (uint8_t*)dev_comp, comp_cap,
+                       dev_total, dev_status, normalizer_size, (uint8_t*)dev_norm);
+  if (int rc = encode_phase1(&b, precision, normalizer_size, st)) return rc;
+  if (int rc = encode_phase2(&b, st)) return rc;
   if (host_total) {
     uint32_t hs = 0;
     NZ_HIP(hipMemcpyAsync(host_total, dev_total, 8, hipMemcpyDeviceToHost, st));
@@ -517,13 +551,19 @@ int pick_geometry(const nz_manager* m, uint64_t n, NzGeom* g, uint32_t* chunk_ou
   return make_geom(g, n, chunk_syms, lane_syms);
 }
 
+// The manager's 256-byte device block: [0, 4) status of decode launches, [64, 192)
+// container sizes of a write batch, [192, 256) its status words.
+uint64_t* write_totals(nz_manager* m) { return reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(m->d_status) + 64); }
+uint32_t* write_status(nz_manager* m) { return reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(m->d_status) + 192); }
+
 // Takes the entry `name` out of the store (cuda/high_level.cu:137-140: an existing
 // entry is replaced; its buffers are reused when large enough, which also avoids
-// a device-wide hipFree stall), allocates what has a known size and enqueues
-// everything up to the directory into the scratch slice `ws`.
+// a device-wide hipFree stall), allocates what has a known size and describes
+// the tensor to the encode kernels (`item`; scratch slice `ws`, container size
+// and status in slot `slot` of the manager's device block).
 int write_begin(nz_manager* m, const char* name, const void* dev_data, uint64_t n, int dtype,
                 uint32_t chunk_syms, uint32_t lane_syms, const NzGeom& g, uint8_t* ws, PendingWrite* pw,
-                hipStream_t st) {
+                uint32_t slot, NzEncItem* item) {
   pw->name = name;
   pw->g = g;
   pw->L = enc_layout(g);
@@ -562,18 +602,18 @@ int write_begin(nz_manager* m, const char* name, const void* dev_data, uint64_t 
       e = hipMalloc(&ent.packed, ent.packed_cap);
     }
   }
-  if (e == hipSuccess) e = hipMemsetAsync(ws + pw->L.status, 0, 4, st);
   if (e != hipSuccess) return fail(NZ_ERR_HIP, std::string("write: ") + hipGetErrorString(e));
-  return encode_phase1(g, m->precision, dev_data, (uint8_t*)ent.packed, ws, pw->L, ws + pw->L.hdr, ~0ull,
-                       (uint64_t*)(ws + pw->L.total), (uint32_t*)(ws + pw->L.status), m->normalizer,
-                       (uint8_t*)ent.norm, st);
+  // header and directory are built in the scratch; where the records go is decided
+  // once the size is known
+  *item = enc_item(g, dev_data, (uint8_t*)ent.packed, ws, pw->L, ws + pw->L.hdr, nullptr, ~0ull,
+                   write_totals(m) + slot, write_status(m) + slot, m->normalizer, (uint8_t*)ent.norm);
+  return NZ_OK;
 }
 
-// With the container size known on the host: exact-size buffer, header copy, compaction.
-int write_finish(nz_manager* m, PendingWrite* pw, uint64_t total, hipStream_t st) {
+// With the container size known on the host: a buffer of that size for the records.
+int write_place(PendingWrite* pw, uint64_t total, NzEncItem* item) {
   Entry& ent = pw->ent;
   Entry& old = pw->old;
-  const NzGeom& g = pw->g;
   ent.comp_bytes = total;
   hipError_t e = hipSuccess;
   if (old.comp && old.comp_cap >= ent.comp_bytes && old.comp_cap <= ent.comp_bytes + ent.comp_bytes / 16 + 4096) {
@@ -586,15 +626,9 @@ int write_finish(nz_manager* m, PendingWrite* pw, uint64_t total, hipStream_t st
     ent.comp_cap = ent.comp_bytes + ent.comp_bytes / 64 + 1024;
     e = hipMalloc(&ent.comp, ent.comp_cap);
   }
-  if (e == hipSuccess)
-    e = hipMemcpyAsync(ent.comp, pw->ws + pw->L.hdr, g.rec_off + (g.n_segs ? 0 : NZ_TAIL_PAD),
-                       hipMemcpyDeviceToDevice, st);
   if (e != hipSuccess) return fail(NZ_ERR_HIP, std::string("write: ") + hipGetErrorString(e));
-  if (int rc = encode_phase2(g, pw->ws, pw->L, (const uint32_t*)(pw->ws + pw->L.hdr + g.dir_off),
-                             (uint8_t*)ent.comp, ent.comp_cap, st))
-    return rc;
-  m->entries.emplace(pw->name, ent);
-  ent = Entry();  // now owned by the store
+  item->comp = (uint8_t*)ent.comp;
+  item->comp_cap = ent.comp_cap;
   return NZ_OK;
 }
 
@@ -639,17 +673,37 @@ int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* 
   PendingWrite pw[NZ_WRITE_BATCH_MAX];
   int rc = NZ_OK;
   uint32_t begun = 0;
+  NzEncBatch b{};
   for (; begun < count && rc == NZ_OK; ++begun)
     rc = write_begin(m, names[begun], dev_data[begun], ns[begun], dtype, chunk[begun], lane[begun], g[begun],
-                     (uint8_t*)m->ws + at[begun], &pw[begun], st);
-  if (rc == NZ_OK) {
-    hipError_t e = hipSuccess;
-    for (uint32_t i = 0; i < count && e == hipSuccess; ++i)
-      e = hipMemcpyAsync(&m->h_pin[i], pw[i].ws + pw[i].L.total, 8, hipMemcpyDeviceToHost, st);
-    if (e == hipSuccess) e = hipStreamSynchronize(st);  // the one host sync of the batch
-    if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("size readback: ") + hipGetErrorString(e));
+                     (uint8_t*)m->ws + at[begun], &pw[begun], begun, &b.item[begun]);
+  b.count = count;
+  // phase 1 of all tensors: one launch per kernel, then the one host
+  // synchronisation of the batch for the container sizes
+  uint64_t* h_totals = m->h_pin;
+  uint32_t* h_status = reinterpret_cast<uint32_t*>(m->h_pin + 17);
+  if (rc == NZ_OK && count) {
+    hipError_t e = hipMemsetAsync(write_status(m), 0, 64, st);
+    if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("write: ") + hipGetErrorString(e));
+    if (rc == NZ_OK) rc = encode_phase1(&b, m->precision, m->normalizer, st);
+    if (rc == NZ_OK) {
+      e = hipMemcpyAsync(h_totals, write_totals(m), 8 * count, hipMemcpyDeviceToHost, st);
+      if (e == hipSuccess) e = hipMemcpyAsync(h_status, write_status(m), 4 * count, hipMemcpyDeviceToHost, st);
+      if (e == hipSuccess) e = hipStreamSynchronize(st);
+      if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("size readback: ") + hipGetErrorString(e));
+    }
+    for (uint32_t i = 0; i < count && rc == NZ_OK; ++i)
+      if (h_status[i] & 1u) rc = fail(NZ_ERR_CAPACITY, "container too large for its directory");
   }
-  for (uint32_t i = 0; i < count && rc == NZ_OK; ++i) rc = write_finish(m, &pw[i], m->h_pin[i], st);
+  // phase 2: exact-size buffers, then one launch moves all records
+  for (uint32_t i = 0; i < count && rc == NZ_OK; ++i) rc = write_place(&pw[i], h_totals[i], &b.item[i]);
+  if (rc == NZ_OK && count) rc = encode_phase2(&b, st);
+  if (rc == NZ_OK) {
+    for (uint32_t i = 0; i < count; ++i) {
+      m->entries.emplace(pw[i].name, pw[i].ent);
+      pw[i].ent = Entry();  // now owned by the store
+    }
+  }
   // whatever did not make it into the store is released, old buffers in any case
   for (uint32_t i = 0; i < begun; ++i) {
     release_entry(pw[i].old);

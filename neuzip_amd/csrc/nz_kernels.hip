@@ -292,7 +292,7 @@ __device__ __forceinline__ uint32_t nz_block_max(uint32_t v, uint32_t* red) {
 
 template <int S>
 __device__ __forceinline__ void nz_split_hist_body(
-    const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms, uint32_t spc,
+    const uint64_t c, const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms, uint32_t spc,
     uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
     uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info,
     const NzNorm nm) {
@@ -307,7 +307,6 @@ __device__ __forceinline__ void nz_split_hist_body(
   __shared__ uint32_t cf[256];
 
   const uint32_t tid = threadIdx.x;
-  const uint64_t c = blockIdx.x;
   const uint64_t base = c * chunk_syms;
   const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
 
@@ -533,7 +532,7 @@ __device__ __forceinline__ void nz_chunk_finalize(uint64_t c, uint64_t n, uint32
 // that codes to more than its raw size is stored raw (decided at the end of this
 // kernel, once all segments of the chunk are coded).
 __device__ __forceinline__ void nz_rans_encode_body(
-    const uint8_t* __restrict__ exps, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
+    const uint64_t c, const uint8_t* __restrict__ exps, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
     uint32_t spc, const uint32_t* __restrict__ enc_tab, NzChunkInfo* __restrict__ info,
     const uint16_t* __restrict__ carry, uint16_t* __restrict__ slots,
     uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words,
@@ -542,7 +541,6 @@ __device__ __forceinline__ void nz_rans_encode_body(
   // per symbol: x = freq << 20 (renormalisation threshold), y = freq, z = cum,
   // w = bits of 1.0f / freq
   __shared__ uint4 tab[256];
-  const uint64_t c = blockIdx.x;
   for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) {
     const uint32_t fc = enc_tab[c * 256 + i];
     const uint32_t f = fc >> 16;
@@ -644,34 +642,72 @@ __device__ __forceinline__ void nz_rans_encode_body(
 // written.  Workgroups of different chunks are in different phases at any
 // time, so the two kinds of work overlap on the chip.
 // ----------------------------------------------------------------------------
+// The tensors of one encode call ride in the kernel argument block (as the
+// items of a decode batch do): the grid of the split/encode kernel is the
+// concatenation of their chunks, that of the scan kernel one workgroup per
+// tensor, that of the compaction the concatenation of their segments.
+#define NZ_ENC_BATCH_MAX 16
+struct NzEncItem {
+  const uint16_t* in;   // dense input
+  uint8_t* packed;      // stored sign|mantissa stream
+  uint8_t* ws;          // this tensor's slice of the scratch; the offsets below are into it
+  uint8_t* hdr;         // where header and directory are built (g.rec_off bytes)
+  uint8_t* comp;        // where the records go (header and directory are copied there unless comp == hdr)
+  uint64_t comp_cap;    // capacity the container size is checked against
+  uint64_t* d_total;    // container size
+  uint32_t* d_status;   // bit 0: the container does not fit
+  NzNorm nm;            // normalizer bytes (nullptr: none)
+  NzGeom g;
+  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units;
+  uint32_t chunk_end, seg_end;  // running totals over the batch
+};
+struct NzEncBatch {
+  uint32_t count, reserved;
+  NzEncItem item[NZ_ENC_BATCH_MAX];
+};
+
 template <int S>
-__global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_encode_kernel(
-    const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms, uint32_t spc,
-    uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
-    uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info,
-    const NzNorm nm, uint16_t* __restrict__ slots, uint32_t* __restrict__ states,
-    uint32_t* __restrict__ seg_words, uint32_t* __restrict__ seg_state_bytes,
-    uint32_t* __restrict__ seg_units) {
-  nz_split_hist_body<S>(in, n, chunk_syms, lane_syms * NZ_LANES, spc, packed, carry, exps, enc_tab, tab_ser,
-                        info, nm);
+__global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_encode_kernel(const NzEncBatch b) {
+  uint32_t t = 0, first = 0;
+  while (t + 1 < b.count && blockIdx.x >= b.item[t].chunk_end) {
+    first = b.item[t].chunk_end;
+    ++t;
+  }
+  const NzEncItem& it = b.item[t];
+  const uint64_t c = blockIdx.x - first;
+  const NzGeom& g = it.g;
+  uint8_t* carry = it.ws + it.carry;
+  uint8_t* exps = it.ws + it.exps;
+  uint32_t* enc_tab = reinterpret_cast<uint32_t*>(it.ws + it.enc_tab);
+  NzChunkInfo* info = reinterpret_cast<NzChunkInfo*>(it.ws + it.info);
+  nz_split_hist_body<S>(c, it.in, g.n, g.chunk_syms, g.seg_syms, g.spc, it.packed, carry, exps, enc_tab,
+                        it.ws + it.tab_ser, info, it.nm);
   // exponents, table, carried bytes and chunk info of this chunk are read back below
   __threadfence_block();
   __syncthreads();
-  nz_rans_encode_body(exps, n, chunk_syms, lane_syms, spc, enc_tab, info,
-                      reinterpret_cast<const uint16_t*>(carry), slots, states, seg_words, seg_state_bytes,
-                      seg_units);
+  nz_rans_encode_body(c, exps, g.n, g.chunk_syms, g.lane_syms, g.spc, enc_tab, info,
+                      reinterpret_cast<const uint16_t*>(carry), reinterpret_cast<uint16_t*>(it.ws + it.slots),
+                      reinterpret_cast<uint32_t*>(it.ws + it.states),
+                      reinterpret_cast<uint32_t*>(it.ws + it.seg_words),
+                      reinterpret_cast<uint32_t*>(it.ws + it.seg_sbytes),
+                      reinterpret_cast<uint32_t*>(it.ws + it.seg_units));
 }
 
 // ----------------------------------------------------------------------------
 // exclusive scan of the record sizes -> directory, header, total size
-// (single workgroup; a tensor has at most a few hundred thousand segments)
+// (a single workgroup per tensor; a tensor has at most a few hundred thousand segments)
 // ----------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void nz_scan_kernel(const uint32_t* __restrict__ seg_units,
-                                                       NzGeom g, uint8_t* __restrict__ comp,
-                                                       uint64_t cap, uint64_t* __restrict__ d_total,
-                                                       uint32_t* __restrict__ d_status) {
-  // `comp` only needs room for the header and directory (g.rec_off bytes); the
-  // records are placed by nz_compact_kernel, possibly in another buffer.
+__global__ __launch_bounds__(1024) void nz_scan_kernel(const NzEncBatch b) {
+  // one workgroup per tensor; header and directory go to `hdr` (g.rec_off
+  // bytes), the records are placed by nz_compact_kernel, possibly in another
+  // buffer
+  const NzEncItem& it = b.item[blockIdx.x];
+  const NzGeom& g = it.g;
+  const uint32_t* __restrict__ seg_units = reinterpret_cast<const uint32_t*>(it.ws + it.seg_units);
+  uint8_t* __restrict__ comp = it.hdr;
+  const uint64_t cap = it.comp_cap;
+  uint64_t* __restrict__ d_total = it.d_total;
+  uint32_t* __restrict__ d_status = it.d_status;
   __shared__ uint64_t wsum[16];
   __shared__ uint64_t carry_s;
   uint32_t* dir = reinterpret_cast<uint32_t*>(comp + g.dir_off);
@@ -726,13 +762,32 @@ __global__ __launch_bounds__(1024) void nz_scan_kernel(const uint32_t* __restric
 // ----------------------------------------------------------------------------
 // move every segment record to its final place: one workgroup per segment
 // ----------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void nz_compact_kernel(
-    const uint8_t* __restrict__ exps, NzGeom g, const NzChunkInfo* __restrict__ info,
-    const uint8_t* __restrict__ tab_ser, const uint8_t* __restrict__ carry,
-    const uint16_t* __restrict__ slots, const uint32_t* __restrict__ states,
-    const uint32_t* __restrict__ seg_words, const uint32_t* __restrict__ seg_state_bytes,
-    const uint32_t* __restrict__ dir, uint8_t* __restrict__ comp, uint64_t cap) {
-  const uint64_t seg = blockIdx.x;
+__global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
+  uint32_t t = 0, first = 0;
+  while (t + 1 < b.count && blockIdx.x >= b.item[t].seg_end) {
+    first = b.item[t].seg_end;
+    ++t;
+  }
+  const NzEncItem& it = b.item[t];
+  const NzGeom& g = it.g;
+  const uint8_t* __restrict__ exps = it.ws + it.exps;
+  const NzChunkInfo* __restrict__ info = reinterpret_cast<const NzChunkInfo*>(it.ws + it.info);
+  const uint8_t* __restrict__ tab_ser = it.ws + it.tab_ser;
+  const uint8_t* __restrict__ carry = it.ws + it.carry;
+  const uint16_t* __restrict__ slots = reinterpret_cast<const uint16_t*>(it.ws + it.slots);
+  const uint32_t* __restrict__ states = reinterpret_cast<const uint32_t*>(it.ws + it.states);
+  const uint32_t* __restrict__ seg_words = reinterpret_cast<const uint32_t*>(it.ws + it.seg_words);
+  const uint32_t* __restrict__ seg_state_bytes = reinterpret_cast<const uint32_t*>(it.ws + it.seg_sbytes);
+  const uint32_t* __restrict__ dir = reinterpret_cast<const uint32_t*>(it.hdr + g.dir_off);
+  uint8_t* __restrict__ comp = it.comp;
+  const uint64_t cap = it.comp_cap;
+  const uint64_t seg = blockIdx.x - first;
+  // header and directory were built elsewhere: every workgroup moves a share
+  if (it.hdr != it.comp && g.rec_off <= cap) {
+    const uint32_t* hs = reinterpret_cast<const uint32_t*>(it.hdr);
+    uint32_t* hd = reinterpret_cast<uint32_t*>(comp);
+    for (uint64_t i = seg * 256 + threadIdx.x; i < g.rec_off / 4; i += g.n_segs * 256) hd[i] = hs[i];
+  }
   const uint64_t c = seg / g.spc;
   const uint32_t k = (uint32_t)(seg - c * g.spc);
   const uint64_t o0 = dir[seg], o1 = dir[seg + 1];
