@@ -44,8 +44,7 @@ uint64_t norm_bytes_of(uint64_t n, uint32_t ns) { return ns ? (n + ns - 1) / ns 
 
 // Device scratch of one encode call.
 struct EncLayout {
-  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, hdr, total,
-      status, bytes;
+  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, hdr, bytes;
 };
 
 EncLayout enc_layout(const NzGeom& g) {
@@ -67,8 +66,6 @@ EncLayout enc_layout(const NzGeom& g) {
   L.seg_sbytes = take(g.n_segs * 4);
   L.seg_units = take((g.n_segs + 1) * 4);
   L.hdr = take(g.rec_off + NZ_TAIL_PAD);
-  L.total = take(8);
-  L.status = take(4);
   L.bytes = o;
   return L;
 }
