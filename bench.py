@@ -115,20 +115,25 @@ class Codec:
 
 
 def time_launches(torch, fn, steps, warmup):
-    """Wall time of `steps` back-to-back launches and the mean per-launch
-    duration from HIP events recorded on the launch stream around each one."""
+    """Wall time of `steps` back-to-back launches (nothing but the launches
+    between the two synchronisations), then, in a second pass over the same
+    launches, the per-launch duration from HIP events recorded on the launch
+    stream around each one.  -> wall seconds, mean and median launch seconds."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
     ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
     for a, b in ev:
         a.record()
         fn()
         b.record()
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
     per = [a.elapsed_time(b) * 1e-3 for a, b in ev]
     return wall, statistics.fmean(per), statistics.median(per)
 
