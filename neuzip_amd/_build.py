@@ -16,8 +16,9 @@ HIPCC_FLAGS = [
     "-shared",
     # packed-FP32 VALU forms are kept out of every code object built here
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    # the block-normalizer arithmetic must round like IEEE fp32 (exact division,
-    # gradual underflow), whatever the compiler's defaults are
+    # float arithmetic as written, whatever the compiler's defaults are: IEEE
+    # division where the code divides (the coder's reciprocal table), gradual
+    # underflow (the block normalizers scale bf16 subnormals), no contraction
     "-fhip-fp32-correctly-rounded-divide-sqrt",
     "-fno-gpu-flush-denormals-to-zero",
     "-ffp-contract=off",

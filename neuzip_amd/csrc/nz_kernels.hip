@@ -61,11 +61,16 @@ __device__ __forceinline__ uint32_t nz_merge_one(uint32_t exp, uint32_t repr) {
 }
 
 __device__ __forceinline__ float nz_bf16_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
-__device__ __forceinline__ uint32_t nz_f32_to_bf16(float f) {
-  const uint32_t u = __float_as_uint(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x0040u;  // NaN stays NaN
-  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;                      // round to nearest even
+// two floats -> two bf16 in one word, round to nearest even, NaN stays NaN: the
+// conversion instruction of gfx950 (v_cvt_pk_bf16_f32)
+typedef __bf16 nz_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float nz_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t nz_f32_to_bf16x2(float lo, float hi) {
+  const nz_f32x2 v = {lo, hi};
+  const nz_bf16x2 r = __builtin_convertvector(v, nz_bf16x2);
+  return __builtin_bit_cast(uint32_t, r);
 }
+__device__ __forceinline__ uint32_t nz_f32_to_bf16(float f) { return nz_f32_to_bf16x2(f, 0.0f) & 0xFFFFu; }
 
 // ----------------------------------------------------------------------------
 // block normalizers (cuda/kernels.cuh:94-118 on the split side, :208-216 on the
@@ -73,10 +78,14 @@ __device__ __forceinline__ uint32_t nz_f32_to_bf16(float f) {
 // 1.m, m = the 7 mantissa bits of the group's largest magnitude, before the
 // split, and multiplied by it again after the merge.  The group stores m << 1
 // (the top 8 of the 23 fraction bits of the float 1.m).  Division and product
-// run in fp32 and round to bf16, nearest even, exactly as the reference's
-// float expressions do (the quotient of two 8-bit significands never lies
-// close enough to a rounding boundary for the intermediate fp32 rounding to
-// matter).
+// run in fp32 and round to bf16, nearest even, and give what the reference's
+// float expressions give: the exact quotient A / B of two 8-bit significands
+// is never closer to a bf16 rounding boundary (odd / 2^k, k <= 8) than
+// 1 / (256 B) > 2^-16 of its value (256 A = odd * B has no solution with
+// B < 256), gradual underflow included, so an fp32 quotient that is off by a
+// few units in its last place rounds to the same bf16 as the correctly rounded
+// one.  The division is therefore a multiplication by the hardware reciprocal
+// of 1.m (one unit in the last place).
 // ----------------------------------------------------------------------------
 struct NzNorm {
   const uint8_t* bytes;  // one per group, null when the tensor is not normalized
@@ -87,16 +96,17 @@ __device__ __forceinline__ float nz_norm_base(uint32_t byte) {
   return __uint_as_float(0x3F800000u | (byte << 15));
 }
 __device__ __forceinline__ uint32_t nz_norm_div(uint32_t h, uint32_t byte) {
-  return nz_f32_to_bf16(nz_bf16_to_f32(h) / nz_norm_base(byte));
+  return nz_f32_to_bf16(nz_bf16_to_f32(h) * __builtin_amdgcn_rcpf(nz_norm_base(byte)));
 }
 __device__ __forceinline__ uint32_t nz_norm_mul(uint32_t h, uint32_t byte) {
   return nz_f32_to_bf16(nz_bf16_to_f32(h) * nz_norm_base(byte));
 }
 
 // The group bytes of the 8 consecutive elements that start at e0 (a multiple of
-// 8), one per element: byte j of the result belongs to element e0 + j.
+// 8), one per element: byte j of the result belongs to element e0 + j.  With
+// groups of 8 elements or more there is only one, in byte 0.
 __device__ __forceinline__ uint64_t nz_norm_load8(const NzNorm& nm, uint64_t e0) {
-  if (nm.log2n >= 3) return 0x0101010101010101ull * (uint64_t)nm.bytes[e0 >> nm.log2n];
+  if (nm.log2n >= 3) return nm.bytes[e0 >> nm.log2n];
   if (nm.log2n == 0) return *reinterpret_cast<const uint64_t*>(nm.bytes + e0);
   if (nm.log2n == 1) {
     const uint32_t w = *reinterpret_cast<const uint32_t*>(nm.bytes + (e0 >> 1));
@@ -107,24 +117,32 @@ __device__ __forceinline__ uint64_t nz_norm_load8(const NzNorm& nm, uint64_t e0)
   return (uint64_t)((w & 0xFFu) * 0x01010101u) | ((uint64_t)((w >> 8) * 0x01010101u) << 32);
 }
 
-// 8 bf16 values times their group factors
-__device__ __forceinline__ uint4 nz_denorm8(const uint4 v, const uint64_t nb) {
+// 8 bf16 values times (MUL) or divided by their group factors; `nb` holds the
+// group byte of every element (all the same when a group has 8 elements or more:
+// `same`, which saves seven of the eight factor set-ups)
+template <bool MUL>
+__device__ __forceinline__ uint4 nz_scale8(const uint4 v, const uint64_t nb, const bool same) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
   uint32_t o[4];
+  const auto factor = [](uint32_t byte) {
+    const float base = nz_norm_base(byte);
+    return MUL ? base : __builtin_amdgcn_rcpf(base);
+  };
+  if (same) {
+    const float f = factor((uint32_t)nb & 0xFFu);
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const uint32_t b0 = (uint32_t)(nb >> (16 * k)) & 0xFFu, b1 = (uint32_t)(nb >> (16 * k + 8)) & 0xFFu;
-    o[k] = nz_norm_mul(w[k] & 0xFFFFu, b0) | (nz_norm_mul(w[k] >> 16, b1) << 16);
-  }
-  return make_uint4(o[0], o[1], o[2], o[3]);
-}
-__device__ __forceinline__ uint4 nz_norm8(const uint4 v, const uint64_t nb) {
-  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-  uint32_t o[4];
+    for (int k = 0; k < 4; ++k) {
+      const float lo = __uint_as_float(w[k] << 16), hi = __uint_as_float(w[k] & 0xFFFF0000u);
+      o[k] = nz_f32_to_bf16x2(lo * f, hi * f);
+    }
+  } else {
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
-    const uint32_t b0 = (uint32_t)(nb >> (16 * k)) & 0xFFu, b1 = (uint32_t)(nb >> (16 * k + 8)) & 0xFFu;
-    o[k] = nz_norm_div(w[k] & 0xFFFFu, b0) | (nz_norm_div(w[k] >> 16, b1) << 16);
+    for (int k = 0; k < 4; ++k) {
+      const float f0 = factor((uint32_t)(nb >> (16 * k)) & 0xFFu);
+      const float f1 = factor((uint32_t)(nb >> (16 * k + 8)) & 0xFFu);
+      const float lo = __uint_as_float(w[k] << 16), hi = __uint_as_float(w[k] & 0xFFFF0000u);
+      o[k] = nz_f32_to_bf16x2(lo * f0, hi * f1);
+    }
   }
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
@@ -233,7 +251,7 @@ __global__ __launch_bounds__(256) void nz_split_unpacked_kernel(const uint16_t* 
   if (i0 >= n) return;
   if (i0 + 8 <= n) {
     uint4 v = *reinterpret_cast<const uint4*>(in + i0);
-    if (nm.bytes) v = nz_norm8(v, nz_norm_load8(nm, i0));
+    if (nm.bytes) v = nz_scale8<false>(v, nz_norm_load8(nm, i0), nm.log2n >= 3);
     uint32_t w[4] = {v.x, v.y, v.z, v.w};
     uint64_t e = 0, f = 0;
 #pragma unroll
@@ -335,7 +353,7 @@ __device__ __forceinline__ void nz_split_hist_body(
     const uint32_t rem = cn - i;
     if (rem >= 8) {
       uint4 v = *reinterpret_cast<const uint4*>(in + gi);
-      if (nm.bytes) v = nz_norm8(v, nz_norm_load8(nm, gi));
+      if (nm.bytes) v = nz_scale8<false>(v, nz_norm_load8(nm, gi), nm.log2n >= 3);
       uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
       for (int j = 0; j < 8; ++j) nz_split_one<S>((w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu, ex[j], rp[j]);
@@ -1441,7 +1459,7 @@ __device__ __forceinline__ void nz_decode_chunk(
 #pragma unroll
         for (int j = 0; j < 8; ++j) ew[j] = (uint32_t)((sy >> (8 * j)) & 0xFFu) << 24;
         uint4 mv = nz_merge_group<S>(sm, ew);
-        if constexpr (NORM) mv = nz_denorm8(mv, nz_norm_load8(nm, seg_base + idx0));
+        if constexpr (NORM) mv = nz_scale8<true>(mv, nz_norm_load8(nm, seg_base + idx0), nm.log2n >= 3);
         if constexpr (GEMV) walk.add(mv, walk.load(walk.col), lane);
         else *reinterpret_cast<uint4*>(dst + idx0) = mv;
       } else if constexpr (!GEMV) {
@@ -1497,7 +1515,7 @@ __device__ __forceinline__ void nz_decode_chunk(
     uint32_t sml = (uint32_t)sm, smh = (uint32_t)(sm >> 32);
     asm volatile("" : "+v"(sml), "+v"(smh), "+v"(ew[7]));
     uint4 mv = nz_merge_group<S>(((uint64_t)smh << 32) | sml, ew);
-    if constexpr (NORM) mv = nz_denorm8(mv, nb);
+    if constexpr (NORM) mv = nz_scale8<true>(mv, nb, nm.log2n >= 3);
     if constexpr (GEMV) walk.add(mv, xq, lane);
     else *reinterpret_cast<uint4*>(dst + (gq * NZ_LANES + lane) * NZ_GROUP) = mv;
   }
@@ -1542,7 +1560,7 @@ __device__ __forceinline__ void nz_decode_chunk(
         const uint32_t b = idx0 / 8 * (S + 1);
         const uint64_t sm = b >= keep ? nz_load_sm<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
         uint4 mv = nz_merge_group<S>(sm, ext[t]);
-        if constexpr (NORM) mv = nz_denorm8(mv, nz_norm_load8(nm, seg_base + idx0));
+        if constexpr (NORM) mv = nz_scale8<true>(mv, nz_norm_load8(nm, seg_base + idx0), nm.log2n >= 3);
         if constexpr (GEMV) walk.add(mv, walk.load(walk.col), lane);
         else *reinterpret_cast<uint4*>(dst + idx0) = mv;
       }
