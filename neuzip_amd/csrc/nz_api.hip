@@ -279,8 +279,8 @@ struct nz_manager {
   std::mutex mu;
   void* ws = nullptr;
   uint64_t ws_bytes = 0;
-  uint32_t* d_status = nullptr;
-  uint64_t* h_pin = nullptr;  // pinned: [0..15] container sizes of a write batch, [16] status
+  uint32_t* d_status = nullptr;  // 256 bytes: decode status | container sizes and status words of a write batch
+  uint64_t* h_pin = nullptr;     // pinned, 256 bytes: [0..15] those sizes, [16] decode status, [17..24] those status words
   long long* gemv_acc = nullptr;  // row accumulators of the matrix-vector product (all zero between calls)
   uint64_t gemv_rows = 0;         // rows the accumulator buffer can hold
 };
@@ -451,6 +451,7 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   if (e == hipSuccess && cus > 0) m->slots = 3u * (uint32_t)cus;
   if (e != hipSuccess) {
     if (m->d_status) (void)hipFree(m->d_status);
+    if (m->h_pin) (void)hipHostFree(m->h_pin);
     delete m;
     return fail(NZ_ERR_HIP, std::string("nz_manager_create: ") + hipGetErrorString(e));
   }
