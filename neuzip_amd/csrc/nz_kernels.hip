@@ -557,12 +557,13 @@ __device__ __forceinline__ void nz_rans_encode_body(
     uint32_t* __restrict__ seg_state_bytes, uint32_t* __restrict__ seg_units) {
   __shared__ uint32_t sbuf[NZ_MAX_SEGS_PER_CHUNK][NZ_STATE_MAX_BYTES / 4];
   // per symbol: x = freq << 20 (renormalisation threshold), y = freq, z = cum,
-  // w = bits of 1.0f / freq
+  // w = bits of a float just below 1 / freq (four units in the last place
+  // under the correctly rounded quotient)
   __shared__ uint4 tab[256];
   for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) {
     const uint32_t fc = enc_tab[c * 256 + i];
     const uint32_t f = fc >> 16;
-    tab[i] = make_uint4(f << 20, f, fc & 0xFFFFu, __float_as_uint(f ? 1.0f / (float)f : 0.0f));
+    tab[i] = make_uint4(f << 20, f, fc & 0xFFFFu, f ? __float_as_uint(1.0f / (float)f) - 4u : 0u);
   }
   __syncthreads();
 
@@ -608,17 +609,19 @@ __device__ __forceinline__ void nz_rans_encode_body(
       const bool need = x >= e[j].x;
       const uint64_t m = __ballot(need);
       pos -= (uint32_t)__popcll(m);
-      if (need) slot[pos + nz_rank_below(m)] = (uint16_t)(x & 0xFFFFu);
+      if (need)  // a 32-bit byte offset from the segment's slot: one add-shift for the address
+        *reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(slot) + ((pos + nz_rank_below(m)) << 1)) =
+            (uint16_t)(x & 0xFFFFu);
       x = need ? (x >> 16) : x;
-      // x < f << 20 here, so the quotient is below 2^20 and the float estimate
-      // x * (1/f) (three roundings of 2^-24 each) is off by less than one:
-      // truncate, then correct by the sign of the remainder.  With the exact
-      // quotient q the new state is (q << 12) + (x - q f) + cum
-      //                            = x + q (4096 - f) + cum.
+      // x < f << 20 here, so the quotient x / f is below 2^20.  The float estimate
+      // x * r with r four units in the last place under 1 / f (itself within half
+      // a unit) never exceeds the quotient - the roundings of x and of the product
+      // add at most one unit each - and falls short of it by less than
+      // 2^20 * 11 * 2^-24 < 1: truncated it is the exact quotient or one less,
+      // and the remainder tells which.  With the exact quotient q the new state
+      // is (q << 12) + (x - q f) + cum = x + q (4096 - f) + cum.
       uint32_t q = (uint32_t)((float)x * __uint_as_float(e[j].w));
-      const int32_t rem = (int32_t)(x - __umul24(q, f));
-      q += (rem >= (int32_t)f) ? 1u : 0u;
-      q -= (rem < 0) ? 1u : 0u;
+      q += (x - __umul24(q, f) >= f) ? 1u : 0u;
       x = __umul24(q, NZ_M - f) + (x + e[j].z);
     }
   }
