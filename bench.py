@@ -115,27 +115,24 @@ class Codec:
 
 
 def time_launches(torch, fn, steps, warmup):
-    """Wall time of `steps` back-to-back launches (nothing but the launches
-    between the two synchronisations), then, in a second pass over the same
-    launches, the per-launch duration from HIP events recorded on the launch
-    stream around each one.  -> wall seconds, mean and median launch seconds."""
+    """`steps` back-to-back launches between two synchronisations: wall time on
+    the host clock, and the time between two HIP events recorded on the launch
+    stream right before the first and right after the last launch (nothing else
+    is enqueued in between: an event record between two launches costs ~5 us
+    and lets the GPU idle, after which a launch runs ~5 % slower).
+    -> wall seconds, event seconds per launch."""
     for _ in range(warmup):
         fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    e0.record()
     for _ in range(steps):
         fn()
+    e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    torch.cuda.synchronize()
-    for a, b in ev:
-        a.record()
-        fn()
-        b.record()
-    torch.cuda.synchronize()
-    per = [a.elapsed_time(b) * 1e-3 for a, b in ev]
-    return wall, statistics.fmean(per), statistics.median(per)
+    return wall, e0.elapsed_time(e1) * 1e-3 / steps
 
 
 def _timed(torch, fn):
@@ -514,7 +511,7 @@ def main():
     headline_out = out.view(torch.int16).cpu().numpy().view(np.uint16).copy()
 
     # ---- the timed region: K decode launches ----
-    wall, mean_launch, med_launch = time_launches(torch, lambda: codec.decode(out), args.steps, args.warmup)
+    wall, mean_launch = time_launches(torch, lambda: codec.decode(out), args.steps, args.warmup)
     ms_per_step = wall / args.steps * 1e3
     dense_bytes = 2 * n
     value = dense_bytes * args.steps / wall / 1e9
@@ -570,7 +567,6 @@ def main():
             "kernel": f"nz_decode_kernel<{args.precision}>",
             "algorithmic_bytes_per_launch": algo_bytes,
             "mean_launch_us": round(mean_launch * 1e6, 2),
-            "median_launch_us": round(med_launch * 1e6, 2),
         },
     }
 
@@ -581,8 +577,8 @@ def main():
             c2 = codec if s == args.precision else Codec(torch, L, lib_mod, n, s, chunk, lane)
             c2.encode(dense)
             k = max(5, args.steps // 10)
-            w_d, m_d, _ = time_launches(torch, lambda: c2.decode(out), k, 3)
-            w_e, m_e, _ = time_launches(torch, lambda: c2.encode(dense, sync=False), k, 3)
+            w_d, m_d = time_launches(torch, lambda: c2.decode(out), k, 3)
+            w_e, m_e = time_launches(torch, lambda: c2.encode(dense, sync=False), k, 3)
             sweep[str(s)] = {
                 "decode_GBps": round(dense_bytes / m_d / 1e9, 1),
                 "decode_hbm_frac": round((c2.total + c2.packed_bytes + dense_bytes) / m_d / 1e9 / HBM_PEAK_GBPS, 4),
