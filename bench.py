@@ -511,6 +511,11 @@ def main():
     headline_out = out.view(torch.int16).cpu().numpy().view(np.uint16).copy()
 
     # ---- the timed region: K decode launches ----
+    # (the GPU's clocks take several milliseconds of load to settle: the first ~100
+    # launches after an idle period run up to 10 % slower than the steady state, so
+    # the device is kept busy for a while before the W warm-up steps)
+    for _ in range(600):
+        codec.decode(out)
     wall, mean_launch = time_launches(torch, lambda: codec.decode(out), args.steps, args.warmup)
     ms_per_step = wall / args.steps * 1e3
     dense_bytes = 2 * n
