@@ -150,9 +150,10 @@ void nz_manager_destroy(nz_manager* m);
 int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint64_t n,
                      int dtype, void* stream);
 
-/* Up to 16 writes with ONE host synchronisation: the device work of all tensors
-   is enqueued back to back, the container sizes come back together, then the
-   exact-size buffers are filled (an optimizer step that re-compresses the
+/* Up to 16 writes with THREE kernel launches and ONE host synchronisation: the
+   tensors ride in the kernel arguments, so split + coding of all of them is one
+   launch, the directories another, the container sizes come back together,
+   then one launch fills the exact-size buffers (an optimizer step that re-compresses the
    weights of a block pays one sync instead of one per weight,
    cuda/high_level.cu:114-115 per call).  Same semantics per entry as
    nz_manager_write; a name may appear only once. */
