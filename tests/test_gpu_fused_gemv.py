@@ -73,6 +73,27 @@ def test_gemv_matches_fp64_product(rows, cols, kind, lane, s):
     mgr._be.check()
 
 
+@pytest.mark.parametrize("rows,cols", [(14336, 4096), (4096, 4096), (2048, 14336)])
+def test_gemv_at_the_geometries_chosen_per_tensor(rows, cols):
+    """Per-tensor geometry: segments of 19 456 (rows straddle them), of 4096 (one
+    row each, stored directly) and of 8192 elements (a row spans two or three)."""
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=7, lane_symbols="auto")
+    bits = _weight(rows, cols, "normal", seed=rows)
+    w = torch.from_numpy(bits.view(np.int16).copy()).cuda().view(torch.bfloat16).view(rows, cols)
+    h = mgr.write(w)
+    g = torch.Generator(device="cuda").manual_seed(cols)
+    x = torch.randn(cols, device="cuda", generator=g).to(torch.bfloat16)
+    print(f"case gemv auto {rows}x{cols}", flush=True)
+    (y,) = _gemv(mgr, [h], x, None)
+    _check(y, bits, x, None, 7)
+    (y2,) = _gemv(mgr, [h], x, None)
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+    assert torch.equal(mgr.read(h), w)
+    mgr._be.check()
+
+
 def test_gemv_batch_equals_single_calls_and_rejects_bad_shapes():
     import neuzip_amd
 
