@@ -738,12 +738,9 @@ __global__ __launch_bounds__(1024) void nz_scan_kernel(const NzEncBatch b) {
   for (uint64_t start = 0; start < g.n_segs; start += 1024) {
     const uint64_t i = start + tid;
     const uint64_t v = i < g.n_segs ? seg_units[i] : 0;
-    uint64_t incl = v;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      uint64_t t = __shfl_up(incl, o, 64);
-      if ((tid & 63) >= (uint32_t)o) incl += t;
-    }
+    // a record has at most ~2^21 units (a segment has at most 2^22 symbols), so
+    // the sum over a wavefront fits 32 bits; across wavefronts it is kept in 64
+    const uint64_t incl = nz_wave_scan((uint32_t)v, tid & 63);
     if ((tid & 63) == 63) wsum[tid >> 6] = incl;
     __syncthreads();
     uint64_t woff = carry_s;
@@ -811,7 +808,11 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   }
   const uint64_t c = seg / g.spc;
   const uint32_t k = (uint32_t)(seg - c * g.spc);
+  // everything the move depends on is fetched at once: one round of memory latency
   const uint64_t o0 = dir[seg], o1 = dir[seg + 1];
+  const NzChunkInfo ci = info[c];
+  const uint32_t sbytes = seg_state_bytes[seg];
+  const uint32_t w = seg_words[seg];
   if (g.rec_off + 4 * o1 + NZ_TAIL_PAD > cap) return;  // flagged by the scan kernel
   uint8_t* dst = comp + g.rec_off + 4 * o0;
   if (seg + 1 == g.n_segs && threadIdx.x >= 256 - NZ_TAIL_PAD)  // closing zeros
@@ -819,7 +820,6 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   const uint64_t seg_base = c * g.chunk_syms + (uint64_t)k * g.seg_syms;
   const uint32_t nom = nz_seg_nominal(g.chunk_syms, g.seg_syms, g.spc, k);
   const uint32_t sn = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
-  const NzChunkInfo ci = info[c];
   const uint32_t tid = threadIdx.x;
   if (ci.raw) {
     uint32_t off = 0;
@@ -839,9 +839,7 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
     off = ci.tab_len;
   }
   uint32_t* sdst = reinterpret_cast<uint32_t*>(dst + off);
-  const uint32_t sbytes = seg_state_bytes[seg];
   if (tid < sbytes / 4) sdst[tid] = states[seg * (NZ_STATE_MAX_BYTES / 4) + tid];
-  const uint32_t w = seg_words[seg];
   const uint32_t cap_words = g.seg_syms;
   // the words sit at the end of the segment's slot, 2-byte aligned; they are moved
   // as dwords (two aligned loads and a funnel shift when the source is off by one
@@ -851,9 +849,24 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src - mis);
   uint32_t* wdst = reinterpret_cast<uint32_t*>(dst + off + sbytes);
   const uint32_t nd = (w + 1) / 2;
-  for (uint32_t i = tid; i < nd; i += 256) {
+  const uint32_t nd4 = nd & ~3u;  // four dwords per thread and turn, then the last one to three singly
+  for (uint32_t i = 4 * tid; i < nd4; i += 4 * 256) {
+    const uint32_t a0 = s32[i], a1 = s32[i + 1], a2 = s32[i + 2], a3 = s32[i + 3];
+    uint4 v = make_uint4(a0, a1, a2, a3);
+    if (mis) {
+      const uint32_t a4 = s32[i + 4];
+      v = make_uint4(__builtin_amdgcn_alignbit(a1, a0, 16), __builtin_amdgcn_alignbit(a2, a1, 16),
+                     __builtin_amdgcn_alignbit(a3, a2, 16), __builtin_amdgcn_alignbit(a4, a3, 16));
+    }
+    if ((w & 1) && i + 4 == nd) v.w &= 0xFFFFu;  // the padding word of an odd count is zero
+    wdst[i] = v.x;
+    wdst[i + 1] = v.y;
+    wdst[i + 2] = v.z;
+    wdst[i + 3] = v.w;
+  }
+  for (uint32_t i = nd4 + tid; i < nd; i += 256) {
     uint32_t v = mis ? __builtin_amdgcn_alignbit(s32[i + 1], s32[i], 16) : s32[i];
-    if ((w & 1) && i == nd - 1) v &= 0xFFFFu;  // the padding word of an odd count is zero
+    if ((w & 1) && i == nd - 1) v &= 0xFFFFu;
     wdst[i] = v;
   }
 }
