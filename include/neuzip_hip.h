@@ -213,6 +213,11 @@ int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype
    manager with normalizer_size > 0); 0 if unknown. */
 uint64_t nz_manager_size(nz_manager* m, const char* name);
 
+/* The same figure by the reference's formula, term by term: a manager without
+   normalizers also counts the ceil(numel / 1024)-byte buffer the reference
+   allocates and never uses (cuda/high_level.cu:89-93, summed at :208-221). */
+uint64_t nz_manager_size_reference(nz_manager* m, const char* name);
+
 /* Bytes of the exponent container alone / of the packed stream alone. */
 uint64_t nz_manager_exp_bytes(nz_manager* m, const char* name);
 uint64_t nz_manager_packed_bytes(nz_manager* m, const char* name);

@@ -202,8 +202,9 @@ class _HipBackend:
                                        _stream_ptr(self._device))
         _lib.raise_for(rc)
 
-    def size(self, handle: str) -> int:
-        return int(self._L.nz_manager_size(self._h, handle.encode()))
+    def size(self, handle: str, reference_accounting: bool = False) -> int:
+        fn = self._L.nz_manager_size_reference if reference_accounting else self._L.nz_manager_size
+        return int(fn(self._h, handle.encode()))
 
     def exp_bytes(self, handle: str) -> int:
         return int(self._L.nz_manager_exp_bytes(self._h, handle.encode()))
@@ -263,7 +264,7 @@ class _DenseBackend:
     def read(self, handle: str) -> torch.Tensor:
         return self._store[handle]
 
-    def size(self, handle: str) -> int:
+    def size(self, handle: str, reference_accounting: bool = False) -> int:
         t = self._store[handle]
         return t.numel() * t.element_size()
 
@@ -361,8 +362,14 @@ class Manager:
         drop it at once (the backward pass of a compressed Linear)."""
         return self.read(handle)
 
-    def size(self, handle: str) -> int:
-        return self._be.size(handle)
+    def size(self, handle: str, reference_accounting: bool = False) -> int:
+        """Bytes held for ``handle``: exponent container + stored sign|mantissa
+        bytes + normalizer bytes (0 for an unknown handle).  The reference also
+        counts a buffer of ``ceil(numel / 1024)`` bytes that it allocates and
+        never uses when normalizers are off (cuda/high_level.cu:89-93,208-221);
+        ``reference_accounting=True`` adds those bytes, so that the figure
+        follows the reference's formula term by term."""
+        return self._be.size(handle, reference_accounting)
 
     def linear(self, handle: str, inputs: torch.Tensor, bias=None) -> torch.Tensor:
         shape = self.meta_dict[handle]

@@ -911,6 +911,18 @@ uint64_t nz_manager_size(nz_manager* m, const char* name) {
   return it->second.comp_bytes + it->second.packed_bytes + it->second.norm_bytes;
 }
 
+uint64_t nz_manager_size_reference(nz_manager* m, const char* name) {
+  if (!m || !name) return 0;
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  if (it == m->entries.end()) return 0;
+  const Entry& e = it->second;
+  // cuda/high_level.cu:89-93: without normalizers the reference still allocates
+  // (and size() counts, :208-221) one byte per 1024 elements
+  const uint64_t idle_norm = m->normalizer ? 0 : (e.n + 1023) / 1024;
+  return e.comp_bytes + e.packed_bytes + e.norm_bytes + idle_norm;
+}
+
 uint64_t nz_manager_exp_bytes(nz_manager* m, const char* name) {
   if (!m || !name) return 0;
   std::lock_guard<std::mutex> lock(m->mu);
@@ -1034,10 +1046,7 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
   if (it != m->entries.end()) {
     // kernels reading the old buffers may still be in flight
     (void)hipDeviceSynchronize();
-    if (it->second.comp) (void)hipFree(it->second.comp);
-    if (it->second.packed) (void)hipFree(it->second.packed);
-  if (it->second.norm) (void)hipFree(it->second.norm);
-    if (it->second.norm) (void)hipFree(it->second.norm);
+    release_entry(it->second);
     m->entries.erase(it);
   }
   m->entries.emplace(name, ent);

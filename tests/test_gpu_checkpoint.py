@@ -118,3 +118,31 @@ def test_converted_model_resumes_from_checkpoint(tmp_path):
     model2.load_state_dict(torch.load(tmp_path / "m.pt", weights_only=True))
     with torch.no_grad():
         assert torch.equal(model2(x), want)
+
+
+def test_reload_over_live_normalized_entries(tmp_path, oracle):
+    """Loading a checkpoint over entries that already exist replaces container,
+    packed stream and normalizer bytes of each entry exactly once: every call
+    after the second load still succeeds (a stale HIP error left by a failed
+    release would surface in the next launch check)."""
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=3, normalizer_size=64)
+    shape = (200, 1024)
+    bits = stress_bits(*shape, seed=9)
+    bits = np.where((bits & 0x7F80) == 0x7F80, np.uint16(0x3F80), bits).astype(np.uint16)
+    hs = [mgr.write(_tensor(bits, shape)), mgr.write(_tensor(bits[: 64 * 1024], (64, 1024)))]
+    want = [oracle.reconstruct_normalized(bits, 3, 64), oracle.reconstruct_normalized(bits[: 64 * 1024], 3, 64)]
+    path = tmp_path / "n.pt"
+    mgr.save(path)
+    for _ in range(2):
+        mgr.load(path)
+        for h, w in zip(hs, want):
+            got = mgr.read(h).view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1)
+            assert np.array_equal(got, w)
+        mgr._be.check()
+    # a write after the reloads goes through the same error checks
+    h2 = mgr.write(_tensor(bits, shape), hs[0])
+    assert h2 == hs[0]
+    assert np.array_equal(mgr.read(h2).view(torch.int16).cpu().numpy().view(np.uint16).reshape(-1), want[0])
+    mgr._be.check()

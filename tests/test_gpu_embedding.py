@@ -9,10 +9,17 @@ pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
 
-def _table(rows, dim, seed, kind="normal"):
+def _table_bits(rows, dim, seed, kind="normal"):
     bits = bf16_bits_normal(rows * dim, seed) if kind == "normal" else stress_bits(rows, dim, seed)
-    bits = np.where((bits & 0x7F80) == 0x7F80, np.uint16(0x3F80), bits).astype(np.uint16)
+    return np.where((bits & 0x7F80) == 0x7F80, np.uint16(0x3F80), bits).astype(np.uint16)
+
+
+def _dev(bits, rows, dim):
     return torch.from_numpy(bits.view(np.int16).copy()).cuda().view(torch.bfloat16).view(rows, dim)
+
+
+def _table(rows, dim, seed, kind="normal"):
+    return _dev(_table_bits(rows, dim, seed, kind), rows, dim)
 
 
 @pytest.mark.parametrize("rows,dim,precision,norm,lane", [
@@ -22,12 +29,18 @@ def _table(rows, dim, seed, kind="normal"):
     (513, 768, 3, 512, "auto"),
     (129, 40, 0, 8, 128),       # odd row length: rows straddle groups of 8
 ])
-def test_gather_rows_equals_full_read(rows, dim, precision, norm, lane):
+def test_gather_rows_equals_oracle_rows(oracle, rows, dim, precision, norm, lane):
+    """Gathered rows against the CPU oracle's reconstruction of the same bits
+    (what the reference's Embedding.forward indexes after decompressing the
+    whole table, neuzip/nn/embedding.py:30-39), and against the full read."""
     import neuzip_amd
 
     mgr = neuzip_amd.Manager(precision=precision, normalizer_size=norm, lane_symbols=lane)
-    h = mgr.write(_table(rows, dim, seed=rows, kind="stress" if norm else "normal"))
-    full = mgr.read(h)
+    bits = _table_bits(rows, dim, seed=rows, kind="stress" if norm else "normal")
+    h = mgr.write(_dev(bits, rows, dim))
+    want = oracle.reconstruct_normalized(bits, precision, norm) if norm else oracle.reconstruct(bits, precision)
+    full = _dev(want, rows, dim)
+    assert torch.equal(mgr.read(h), full)
     g = torch.Generator().manual_seed(rows)
     for count in (1, 7, 200):
         idx = torch.randint(0, rows, (count,), generator=g)

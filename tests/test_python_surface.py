@@ -183,3 +183,39 @@ def test_manager_argument_errors():
         neuzip_amd.Manager(normalizer_size=3)
     with pytest.raises(RuntimeError, match="Unsupported algorithm"):
         neuzip_amd.Manager(algorithm=A.zstd)
+
+
+def test_reference_package_name_is_importable():
+    """``import neuzip`` exposes the reference's surface (neuzip/__init__.py:8-13)
+    and module paths, and its Manager keeps the reference's constructor
+    signature (neuzip/binding.py:56-62)."""
+    import inspect
+
+    import neuzip
+    import neuzip.binding
+    import neuzip.nn.embedding
+    import neuzip.nn.linear
+    import neuzip.nn.module
+    import neuzip.ops.linear
+    import neuzip.utils
+
+    assert neuzip.__all__ == ["ops", "nn", "Algorithm", "Manager"]
+    for name in neuzip.__all__ + ["lomo_hook", "compressed_lomo_hook"]:
+        assert hasattr(neuzip, name)
+    assert neuzip.nn is neuzip_amd.nn and neuzip.ops is neuzip_amd.ops
+    assert neuzip.nn.Linear is Linear and neuzip.nn.Parameter is Parameter
+    assert neuzip.nn.linear.Linear is Linear and neuzip.nn.module.Parameter is Parameter
+    assert neuzip.ops.CompressedLinear is neuzip_amd.ops.CompressedLinear
+    assert neuzip.ops.linear.CompressedLinear is neuzip_amd.ops.CompressedLinear
+    assert neuzip.utils._convert is _convert
+    assert neuzip.binding.Manager is neuzip.Manager and issubclass(neuzip.Manager, neuzip_amd.Manager)
+    assert [m.name for m in neuzip.Algorithm] == ["ans", "gdeflate", "zstd", "dummy"]  # neuzip/binding.py:23-27
+    params = inspect.signature(neuzip.Manager.__init__).parameters
+    assert list(params)[:5] == ["self", "algorithm", "precision", "normalizer_size", "chunk_size"]
+    assert params["algorithm"].default is neuzip.Algorithm.ans and params["precision"].default == 7
+    assert params["normalizer_size"].default is None and params["chunk_size"].default == 2 ** 16
+    # the dense pass-through needs no device: convert() runs as the reference words it
+    mgr = neuzip.Manager(algorithm=neuzip.Algorithm.dummy)
+    assert mgr.meta_dict == {} and callable(mgr.convert)
+    with pytest.raises(AttributeError, match="Manager_f5_n0"):
+        neuzip.Manager(precision=5)
