@@ -249,3 +249,112 @@ class CompressedAdamW:
             for p in batch:
                 p._gradient = None
                 p.grad = None
+
+
+def paired_parameters(dense: torch.nn.Module, comp: torch.nn.Module):
+    """``[(name, dense parameter, its counterpart in the converted twin)]``: for a
+    compressed Linear the counterpart of ``weight`` is the ``neuzip_amd.nn.Parameter``."""
+    from neuzip_amd.nn import Linear as CompressedLinearModule
+
+    dense_mods = dict(dense.named_modules())
+    pairs = []
+    for name, mod in comp.named_modules():
+        twin = dense_mods[name]
+        if isinstance(mod, CompressedLinearModule):
+            pairs.append((f"{name}.weight", twin.weight, mod._p))
+            if mod.bias is not None:
+                pairs.append((f"{name}.bias", twin.bias, mod.bias))
+            continue
+        for pname, p in mod.named_parameters(recurse=False):
+            pairs.append((f"{name}.{pname}" if name else pname, getattr(twin, pname), p))
+    return pairs
+
+
+def _same_bits(a: torch.Tensor, b: torch.Tensor) -> bool:
+    a, b = a.detach().reshape(-1), b.detach().reshape(-1)
+    if a.dtype == torch.bfloat16:
+        return bool(torch.equal(a.view(torch.int16), b.view(torch.int16)))
+    return bool(torch.equal(a, b))
+
+
+def lockstep_adamw(dense, comp, manager, ids_for_step, steps, group, lr=1e-4, probe_dense_twice=True):
+    """Train ``dense`` (torch.optim.AdamW) and ``comp`` (the same model converted
+    by ``manager``: CompressedAdamW re-compressing with ``write_many``) side by
+    side on the same token ids, and separate what the codec is responsible for
+    from what the GEMM / attention kernels are responsible for.
+
+    Per step both models run forward and backward; losses and gradients are
+    compared and the first tensor whose gradient differs is recorded (the
+    weights going in are identical, so such a difference belongs to the
+    forward / backward kernels, never to the codec).  Then the DENSE gradients
+    are handed to both optimizers, both step, and every weight of the
+    compressed model (decoded from its store) must equal the dense model's
+    weight bit for bit: that is the part the codec and the compressed
+    optimizer answer for.  With ``probe_dense_twice`` the dense model's
+    backward is run twice per step on the same input: if its own gradients
+    differ between the two runs, the kernels are not run-to-run deterministic
+    and no loss curve can be expected to repeat.
+
+    -> dict of findings; ``first_weight_mismatch`` must be None."""
+    import neuzip_amd
+
+    pairs = paired_parameters(dense, comp)
+    packed = [(n, d, c) for n, d, c in pairs if isinstance(c, neuzip_amd.nn.Parameter)]
+    plain = [(n, d, c) for n, d, c in pairs if not isinstance(c, neuzip_amd.nn.Parameter)]
+    opt_dense = torch.optim.AdamW([d for _, d, _ in pairs], lr=lr)
+    opt_packed = CompressedAdamW([c for _, _, c in packed], lr=lr, group=group)
+    opt_plain = torch.optim.AdamW([c for _, _, c in plain], lr=lr)
+
+    def loss_of(model, ids):
+        logits = model(ids[:, :-1])
+        return F.cross_entropy(logits.float().reshape(-1, logits.shape[-1]), ids[:, 1:].reshape(-1))
+
+    def grad_of(c):
+        return c._gradient if isinstance(c, neuzip_amd.nn.Parameter) else c.grad
+
+    out = {"steps": steps, "losses_equal": 0, "gradients_equal": 0, "first_loss_mismatch": None,
+           "first_gradient_mismatch": None, "first_weight_mismatch": None, "dense_repeats_itself": None,
+           "max_loss_gap": 0.0}
+    repeats = 0
+    for step in range(steps):
+        ids = ids_for_step(step)
+        if probe_dense_twice:
+            loss_of(dense, ids).backward()
+            first = [d.grad.clone() for _, d, _ in pairs]
+            opt_dense.zero_grad(set_to_none=True)
+        loss_d = loss_of(dense, ids)
+        loss_d.backward()
+        if probe_dense_twice:
+            repeats += all(_same_bits(g, d.grad) for g, (_, d, _) in zip(first, pairs))
+            del first
+        loss_c = loss_of(comp, ids)
+        loss_c.backward()
+        same_loss = bool(torch.equal(loss_d.detach(), loss_c.detach()))
+        out["losses_equal"] += same_loss
+        out["max_loss_gap"] = max(out["max_loss_gap"], abs(float(loss_d) - float(loss_c)))
+        if not same_loss and out["first_loss_mismatch"] is None:
+            out["first_loss_mismatch"] = step
+        differing = [n for n, d, c in pairs if not _same_bits(d.grad, grad_of(c).view_as(d.grad))]
+        out["gradients_equal"] += not differing
+        if differing and out["first_gradient_mismatch"] is None:
+            out["first_gradient_mismatch"] = {"step": step, "tensor": differing[0], "tensors": len(differing)}
+        # the same numbers into both optimizers
+        with torch.no_grad():
+            for _, d, c in packed:
+                c._gradient = d.grad.clone()
+            for _, d, c in plain:
+                c.grad = d.grad.clone()
+        opt_dense.step()
+        opt_packed.step()
+        opt_plain.step()
+        opt_dense.zero_grad(set_to_none=True)
+        opt_plain.zero_grad(set_to_none=True)
+        with torch.no_grad():
+            for n, d, c in pairs:
+                w = manager.read(c._handle) if isinstance(c, neuzip_amd.nn.Parameter) else c.data
+                if not _same_bits(d.data, w.view_as(d.data)):
+                    out["first_weight_mismatch"] = {"step": step, "tensor": n}
+                    return out
+    if probe_dense_twice:
+        out["dense_repeats_itself"] = f"{repeats} of {steps}"
+    return out
