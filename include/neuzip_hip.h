@@ -113,6 +113,24 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
               uint32_t* dev_status, uint64_t* host_total, uint32_t normalizer_size, void* dev_norm,
               void* stream);
 
+/* nz_encode for callers that cannot allocate or hand over a workspace (code
+   under HIP graph capture, tight serving loops, harnesses that forbid
+   hipMalloc).  No counterpart in the reference.  Same kernels, arguments and
+   results as nz_encode, but the scratch is a fixed array of
+   NZ_STATIC_SCRATCH_BYTES inside the library's code object (every GPU the
+   library runs on holds its own copy until the process ends), and the call
+   never allocates, frees or synchronises: the container size is delivered in
+   *dev_total only.  A tensor whose nz_encode_workspace_bytes() exceeds
+   NZ_STATIC_SCRATCH_BYTES is refused with NZ_ERR_CAPACITY (at the default
+   geometry: more than about 5.5 million elements).  All calls on one GPU share
+   that GPU's array: calls that overlap in time on one GPU (two streams, two
+   threads) race; order them on one stream or with events. */
+#define NZ_STATIC_SCRATCH_BYTES (16u << 20)
+int nz_encode_static(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
+                     uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
+                     uint64_t* dev_total, uint32_t* dev_status, uint32_t normalizer_size, void* dev_norm,
+                     void* stream);
+
 /* Manager::_decompress_and_merge, cuda/high_level.cu:169-206: entropy decode
    and merge in one kernel.  `dev_status` (device uint32, zeroed by the
    caller) is OR-ed with a non-zero value when the container fails validation

@@ -25,7 +25,7 @@ LANE_SYMS_AUTO = 0xFFFFFFFF
 
 EXPORTS = [
     "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",
-    "nz_encode_workspace_bytes", "nz_norm_bytes", "nz_split", "nz_encode", "nz_decode",
+    "nz_encode_workspace_bytes", "nz_norm_bytes", "nz_split", "nz_encode", "nz_encode_static", "nz_decode",
     "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_write_batch",
     "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
     "nz_manager_meta", "nz_manager_size", "nz_manager_size_reference", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
@@ -67,6 +67,8 @@ def load() -> ctypes.CDLL:
     L.nz_encode.restype = i32
     L.nz_encode.argtypes = [vp, u64, i32, u32, u32, vp, vp, u64, vp, u64, vp, vp,
                             ctypes.POINTER(u64), u32, vp, vp]
+    L.nz_encode_static.restype = i32
+    L.nz_encode_static.argtypes = [vp, u64, i32, u32, u32, vp, vp, u64, vp, vp, u32, vp, vp]
     L.nz_decode.restype = i32
     L.nz_decode.argtypes = [vp, u64, vp, u64, i32, u32, u32, vp, vp, i32, u32, vp, vp]
     L.nz_manager_create.restype = i32

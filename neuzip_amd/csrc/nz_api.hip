@@ -253,6 +253,59 @@ int make_geom(NzGeom* g, uint64_t n, uint32_t chunk, uint32_t lane_syms) {
   return NZ_OK;
 }
 
+// nz_encode and nz_encode_static behind their argument checks: the three encode
+// launches with `ws` as scratch.  Nothing here allocates or synchronises.
+int encode_stateless(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size, uint32_t lane_syms,
+                     void* dev_packed, void* dev_comp, uint64_t comp_cap, uint8_t* ws, uint64_t ws_bytes,
+                     const char* ws_error, uint64_t* dev_total, uint32_t* dev_status, uint32_t normalizer_size,
+                     void* dev_norm, hipStream_t st) {
+  if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
+  if (!normalizer_ok(normalizer_size))
+    return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
+  if (normalizer_size && n && (!dev_norm || ((uintptr_t)dev_norm & 7)))
+    return fail(NZ_ERR_ARG, "normalizer bytes: null or not 8-byte aligned");
+  NzGeom g;
+  if (int rc = make_geom(&g, n, chunk_size, lane_syms)) return rc;
+  if (!dev_comp || !dev_total || !dev_status || (n && (!dev_bf16 || !dev_packed)))
+    return fail(NZ_ERR_ARG, "null pointer");
+  if ((uintptr_t)dev_bf16 & 15) return fail(NZ_ERR_ALIGN, "dense input must be 16-byte aligned");
+  if (((uintptr_t)dev_packed & 7) || ((uintptr_t)dev_comp & 15))
+    return fail(NZ_ERR_ALIGN, "packed/comp buffers must be 8/16-byte aligned");
+  const EncLayout L = enc_layout(g);
+  if (ws_bytes < L.bytes) return fail(NZ_ERR_CAPACITY, ws_error);
+  if (comp_cap < nz_geom_bound(&g)) return fail(NZ_ERR_CAPACITY, "dev_comp smaller than nz_exp_bound_bytes");
+  NzEncBatch b{};
+  b.count = 1;
+  b.item[0] = enc_item(g, dev_bf16, (uint8_t*)dev_packed, ws, L, (uint8_t*)dev_comp, (uint8_t*)dev_comp, comp_cap,
+                       dev_total, dev_status, normalizer_size, (uint8_t*)dev_norm);
+  if (int rc = encode_phase1(&b, precision, normalizer_size, st)) return rc;
+  return encode_phase2(&b, st);
+}
+
+// Scratch of nz_encode_static: device memory that exists from the moment the
+// code object is loaded, one copy per GPU, so that the call allocates nothing.
+// In host code `nz_static_scratch` is only a handle for hipGetSymbolAddress;
+// the device address of each GPU's copy is looked up once and kept.
+static __device__ __align__(256) uint8_t nz_static_scratch[NZ_STATIC_SCRATCH_BYTES];
+#define NZ_MAX_DEVICES 64
+std::mutex g_static_mu;
+uint8_t* g_static_ptr[NZ_MAX_DEVICES];
+
+int static_scratch(uint8_t** out) {
+  int dev = 0;
+  NZ_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= NZ_MAX_DEVICES) return fail(NZ_ERR_ARG, "device index out of range");
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_ptr[dev]) {
+    void* p = nullptr;
+    NZ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(nz_static_scratch)));
+    if (!p) return fail(NZ_ERR_HIP, "hipGetSymbolAddress returned a null address");
+    g_static_ptr[dev] = (uint8_t*)p;
+  }
+  *out = g_static_ptr[dev];
+  return NZ_OK;
+}
+
 struct Entry {
   void* comp = nullptr;
   uint64_t comp_bytes = 0, comp_cap = 0;
@@ -342,30 +395,14 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
               void* dev_workspace, uint64_t workspace_bytes, uint64_t* dev_total,
               uint32_t* dev_status, uint64_t* host_total, uint32_t normalizer_size, void* dev_norm,
               void* stream) {
-  if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
-  if (!normalizer_ok(normalizer_size))
-    return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
-  if (normalizer_size && n && (!dev_norm || ((uintptr_t)dev_norm & 7)))
-    return fail(NZ_ERR_ARG, "normalizer bytes: null or not 8-byte aligned");
-  NzGeom g;
-  if (int rc = make_geom(&g, n, chunk_size, lane_syms)) return rc;
-  if (!dev_comp || !dev_workspace || !dev_total || !dev_status || (n && (!dev_bf16 || !dev_packed)))
-    return fail(NZ_ERR_ARG, "null pointer");
-  if ((uintptr_t)dev_bf16 & 15) return fail(NZ_ERR_ALIGN, "dense input must be 16-byte aligned");
-  if (((uintptr_t)dev_packed & 7) || ((uintptr_t)dev_comp & 15) || ((uintptr_t)dev_workspace & 255))
-    return fail(NZ_ERR_ALIGN, "packed/comp/workspace buffers must be 8/16/256-byte aligned");
-  const EncLayout L = enc_layout(g);
-  if (workspace_bytes < L.bytes) return fail(NZ_ERR_CAPACITY, "workspace too small");
-  if (comp_cap < nz_geom_bound(&g)) return fail(NZ_ERR_CAPACITY, "dev_comp smaller than nz_exp_bound_bytes");
-  hipStream_t st = (hipStream_t)stream;
-  uint8_t* ws = (uint8_t*)dev_workspace;
-  NzEncBatch b{};
-  b.count = 1;
-  b.item[0] = enc_item(g, dev_bf16, (uint8_t*)dev_packed, ws, L, (uint8_t*)dev_comp, (uint8_t*)dev_comp, comp_cap,
-                       dev_total, dev_status, normalizer_size, (uint8_t*)dev_norm);
-  if (int rc = encode_phase1(&b, precision, normalizer_size, st)) return rc;
-  if (int rc = encode_phase2(&b, st)) return rc;
+  if (!dev_workspace) return fail(NZ_ERR_ARG, "null pointer");
+  if ((uintptr_t)dev_workspace & 255) return fail(NZ_ERR_ALIGN, "workspace must be 256-byte aligned");
+  if (int rc = encode_stateless(dev_bf16, n, precision, chunk_size, lane_syms, dev_packed, dev_comp, comp_cap,
+                                (uint8_t*)dev_workspace, workspace_bytes, "workspace too small", dev_total,
+                                dev_status, normalizer_size, dev_norm, (hipStream_t)stream))
+    return rc;
   if (host_total) {
+    hipStream_t st = (hipStream_t)stream;
     uint32_t hs = 0;
     NZ_HIP(hipMemcpyAsync(host_total, dev_total, 8, hipMemcpyDeviceToHost, st));
     NZ_HIP(hipMemcpyAsync(&hs, dev_status, 4, hipMemcpyDeviceToHost, st));
@@ -373,6 +410,18 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
     if (hs & 1u) return fail(NZ_ERR_CAPACITY, "encoded container exceeds the output capacity");
   }
   return NZ_OK;
+}
+
+int nz_encode_static(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
+                     uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
+                     uint64_t* dev_total, uint32_t* dev_status, uint32_t normalizer_size, void* dev_norm,
+                     void* stream) {
+  uint8_t* ws = nullptr;
+  if (int rc = static_scratch(&ws)) return rc;
+  return encode_stateless(dev_bf16, n, precision, chunk_size, lane_syms, dev_packed, dev_comp, comp_cap, ws,
+                          NZ_STATIC_SCRATCH_BYTES,
+                          "tensor too large for nz_encode_static: its encode scratch exceeds NZ_STATIC_SCRATCH_BYTES",
+                          dev_total, dev_status, normalizer_size, dev_norm, (hipStream_t)stream);
 }
 
 int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed, uint64_t n,
