@@ -331,7 +331,7 @@ def lockstep_adamw(dense, comp, manager, ids_for_step, steps, group, lr=1e-4, pr
         loss_c.backward()
         same_loss = bool(torch.equal(loss_d.detach(), loss_c.detach()))
         out["losses_equal"] += same_loss
-        out["max_loss_gap"] = max(out["max_loss_gap"], abs(float(loss_d) - float(loss_c)))
+        out["max_loss_gap"] = max(out["max_loss_gap"], abs(float(loss_d.detach()) - float(loss_c.detach())))
         if not same_loss and out["first_loss_mismatch"] is None:
             out["first_loss_mismatch"] = step
         differing = [n for n, d, c in pairs if not _same_bits(d.grad, grad_of(c).view_as(d.grad))]
