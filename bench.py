@@ -212,10 +212,10 @@ class Workspace:
         """The three encode launches again, asynchronously, into the buffers of `st`."""
         self._encode(dense, s, st.packed, st.comp, st.comp.numel(), False)
 
-    def decode(self, st: Stored, out, check=False):
+    def decode(self, st: Stored, out, check=False, flags=0):
         stream = self.torch.cuda.current_stream().cuda_stream
         rc = self.L.nz_decode(st.comp.data_ptr(), st.total, st.packed.data_ptr(), st.n, st.s, self.chunk, self.lane,
-                              out.data_ptr(), self.status.data_ptr(), 1 if check else 0, 0, None, stream)
+                              out.data_ptr(), self.status.data_ptr(), (1 if check else 0) | flags, 0, None, stream)
         if rc != 0:
             raise RuntimeError(self.m.last_error())
 
@@ -666,9 +666,36 @@ def main():
     cold_launch = step_time / R
     cold = roofline_block(algo_bytes, cold_launch, args.precision,
                           working_set=int(R * algo_bytes), launches=args.steps * R,
-                          note=f"rotation over {R} independent stored tensors: out of the last-level cache")
+                          note=f"rotation over {R} independent (container, packed, output) sets: out of the "
+                               "last-level cache; default output policy (ordinary stores up to 128 MiB)")
     cold["traffic"], cold["traffic_source"] = recorded_traffic(
         f"nz_decode_kernel<{args.precision}>, {args.rows}x{args.cols}, chunk {chunk}, lane {lane}, rotating {R} sets")
+
+    # Two more views of the same cold inputs.  (1) The output goes to ONE buffer that every
+    # decode reuses, as in the library's read path (the weight is consumed by the GEMM that
+    # follows and the allocator or the per-block slot hands the same memory to the next
+    # decode): only compressed bytes come from HBM, the output lines are already cached.
+    # (2) Everything rotates as in the headline, but the output is written with streaming
+    # stores (NZ_DECODE_STREAM_OUT, the default only for tensors above 128 MiB): faster for
+    # a decode whose output nobody reads soon, slower for decode + GEMM.
+    extra = {}
+    if R > 1 and not args.no_hot:
+        def rotation_one_out():
+            for st in sets:
+                ws.decode(st, outs[0])
+
+        def rotation_streaming():
+            for st, o in zip(sets, outs):
+                ws.decode(st, o, flags=lib_mod.DECODE_STREAM_OUT)
+
+        for name, fn, note in (
+                ("roofline_cold_reused_output", rotation_one_out,
+                 f"{R} stored tensors in rotation, decoded into one reused output buffer"),
+                ("roofline_cold_streaming_stores", rotation_streaming,
+                 f"rotation over {R} independent stored tensors and outputs, streaming stores forced")):
+            _, t_step = time_launches(torch, fn, args.steps, args.warmup)
+            extra[name] = roofline_block(algo_bytes, t_step / R, args.precision, working_set=int(R * algo_bytes),
+                                         launches=args.steps * R, note=note)
 
     # the same kernel on ONE stored tensor over and over (what a single hot layer sees): its
     # 223 MB working set stays in the 256 MB last-level cache, so this is not an HBM figure
@@ -726,6 +753,7 @@ def main():
         "roofline": cold,
         "roofline_cold": cold,
     }
+    result.update(extra)
     if hot is not None:
         result["roofline_hot"] = hot
 

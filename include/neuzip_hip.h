@@ -134,12 +134,22 @@ int nz_encode_static(const void* dev_bf16, uint64_t n, int precision, uint32_t c
 /* Manager::_decompress_and_merge, cuda/high_level.cu:169-206: entropy decode
    and merge in one kernel.  `dev_status` (device uint32, zeroed by the
    caller) is OR-ed with a non-zero value when the container fails validation
-   (bit 4: the header does not name n / chunk_size / lane_syms as passed); with
-   `check` != 0 the call synchronises and returns NZ_ERR_CORRUPT in that
-   case.  chunk_size / lane_syms must be the ones used to encode. */
+   (bit 4: the header does not name n / chunk_size / lane_syms as passed).
+   `flags`: with NZ_DECODE_CHECK the call synchronises and returns
+   NZ_ERR_CORRUPT in that case.  The dense output is written with ordinary
+   stores when it is at most 128 MiB (half of the last-level cache: the GEMM
+   that consumes a just-decompressed weight then reads it from the cache) and
+   with streaming stores when it is larger (it cannot stay resident, and
+   streaming keeps it from churning the cache); NZ_DECODE_STREAM_OUT /
+   NZ_DECODE_RESIDENT_OUT force one or the other, for a caller who knows that
+   nothing will read the output soon / that its consumer runs next.
+   chunk_size / lane_syms must be the ones used to encode. */
+#define NZ_DECODE_CHECK 1
+#define NZ_DECODE_STREAM_OUT 2
+#define NZ_DECODE_RESIDENT_OUT 4
 int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed, uint64_t n,
               int precision, uint32_t chunk_size, uint32_t lane_syms, void* dev_bf16_out,
-              uint32_t* dev_status, int check, uint32_t normalizer_size, const void* dev_norm,
+              uint32_t* dev_status, int flags, uint32_t normalizer_size, const void* dev_norm,
               void* stream);
 
 /* ---- handle store: template struct Manager, cuda/high_level.cu:26-322 -- */

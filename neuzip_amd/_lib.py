@@ -22,6 +22,7 @@ DEFAULT_CHUNK = 131072
 DEFAULT_LANE_SYMS = 256
 LANE_SYMS_64K = 344
 LANE_SYMS_AUTO = 0xFFFFFFFF
+DECODE_CHECK, DECODE_STREAM_OUT, DECODE_RESIDENT_OUT = 1, 2, 4  # nz_decode flags
 
 EXPORTS = [
     "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",

@@ -162,50 +162,67 @@ int encode_phase2(NzEncBatch* b, hipStream_t st) {
 
 template <int S>
 void launch_decode(const NzGeom& g, const void* comp, uint64_t comp_bytes, const void* packed,
-                   void* out, uint32_t* d_status, const NzNorm& nm, hipStream_t st) {
+                   void* out, uint32_t* d_status, const NzNorm& nm, uint32_t stream_out, hipStream_t st) {
   const size_t lds = NZ_DEC_LDS_BYTES(g.spc);
   const dim3 gd((uint32_t)g.n_chunks), bd(64 * g.spc);
-  if (nm.bytes)
-    hipLaunchKernelGGL((nz_decode_kernel<S, true>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,
-                       (const uint8_t*)packed, (uint16_t*)out, g, d_status, nm);
-  else
-    hipLaunchKernelGGL((nz_decode_kernel<S, false>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,
-                       (const uint8_t*)packed, (uint16_t*)out, g, d_status, nm);
+#define NZ_DEC_LAUNCH(NORM, STREAM)                                                                            \
+  hipLaunchKernelGGL((nz_decode_kernel<S, NORM, STREAM>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes, \
+                     (const uint8_t*)packed, (uint16_t*)out, g, d_status, nm)
+  if (nm.bytes) {
+    if (stream_out) NZ_DEC_LAUNCH(true, true);
+    else NZ_DEC_LAUNCH(true, false);
+  } else {
+    if (stream_out) NZ_DEC_LAUNCH(false, true);
+    else NZ_DEC_LAUNCH(false, false);
+  }
+#undef NZ_DEC_LAUNCH
 }
 
+// `flags`: NZ_DECODE_STREAM_OUT / NZ_DECODE_RESIDENT_OUT override the output
+// policy that is otherwise chosen by the size of the dense tensor
 int decode_launch(const NzGeom& g, int precision, const void* comp, uint64_t comp_bytes,
                   const void* packed, void* out, uint32_t* d_status, uint32_t ns, const void* norm,
-                  hipStream_t st) {
+                  int flags, hipStream_t st) {
   if (g.n_chunks == 0) return NZ_OK;
   const NzNorm nm{ns ? (const uint8_t*)norm : nullptr, log2_of(ns ? ns : 1)};
+  const uint32_t so = (flags & NZ_DECODE_STREAM_OUT) ? 1u : (flags & NZ_DECODE_RESIDENT_OUT) ? 0u
+                                                                                              : (nz_stream_output(g.n) ? 1u : 0u);
   switch (precision) {
-    case 7: launch_decode<7>(g, comp, comp_bytes, packed, out, d_status, nm, st); break;
-    case 3: launch_decode<3>(g, comp, comp_bytes, packed, out, d_status, nm, st); break;
-    case 1: launch_decode<1>(g, comp, comp_bytes, packed, out, d_status, nm, st); break;
-    default: launch_decode<0>(g, comp, comp_bytes, packed, out, d_status, nm, st); break;
+    case 7: launch_decode<7>(g, comp, comp_bytes, packed, out, d_status, nm, so, st); break;
+    case 3: launch_decode<3>(g, comp, comp_bytes, packed, out, d_status, nm, so, st); break;
+    case 1: launch_decode<1>(g, comp, comp_bytes, packed, out, d_status, nm, so, st); break;
+    default: launch_decode<0>(g, comp, comp_bytes, packed, out, d_status, nm, so, st); break;
   }
   NZ_HIP(hipGetLastError());
   return NZ_OK;
 }
 
 template <int S>
-void launch_decode_batch(const NzBatch& b, uint32_t grid, uint32_t max_spc, uint32_t* d_status,
+void launch_decode_batch(const NzBatch& b, uint32_t grid, uint32_t max_spc, bool stream_out, uint32_t* d_status,
                          hipStream_t st) {
   const size_t lds = NZ_DEC_LDS_BYTES(max_spc);
-  if (b.item[0].norm)
-    hipLaunchKernelGGL((nz_decode_batch_kernel<S, true>), dim3(grid), dim3(64 * max_spc), lds, st, b, d_status);
-  else
-    hipLaunchKernelGGL((nz_decode_batch_kernel<S, false>), dim3(grid), dim3(64 * max_spc), lds, st, b, d_status);
+  const dim3 gd(grid), bd(64 * max_spc);
+#define NZ_BATCH_LAUNCH(NORM, STREAM) \
+  hipLaunchKernelGGL((nz_decode_batch_kernel<S, NORM, STREAM>), gd, bd, lds, st, b, d_status)
+  if (b.item[0].norm) {
+    if (stream_out) NZ_BATCH_LAUNCH(true, true);
+    else NZ_BATCH_LAUNCH(true, false);
+  } else {
+    if (stream_out) NZ_BATCH_LAUNCH(false, true);
+    else NZ_BATCH_LAUNCH(false, false);
+  }
+#undef NZ_BATCH_LAUNCH
 }
 
-int decode_batch_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int precision,
+// all items of one launch share the output policy (`stream_out`)
+int decode_batch_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int precision, bool stream_out,
                         uint32_t* d_status, hipStream_t st) {
   if (grid == 0) return NZ_OK;
   switch (precision) {
-    case 7: launch_decode_batch<7>(b, grid, max_spc, d_status, st); break;
-    case 3: launch_decode_batch<3>(b, grid, max_spc, d_status, st); break;
-    case 1: launch_decode_batch<1>(b, grid, max_spc, d_status, st); break;
-    default: launch_decode_batch<0>(b, grid, max_spc, d_status, st); break;
+    case 7: launch_decode_batch<7>(b, grid, max_spc, stream_out, d_status, st); break;
+    case 3: launch_decode_batch<3>(b, grid, max_spc, stream_out, d_status, st); break;
+    case 1: launch_decode_batch<1>(b, grid, max_spc, stream_out, d_status, st); break;
+    default: launch_decode_batch<0>(b, grid, max_spc, stream_out, d_status, st); break;
   }
   NZ_HIP(hipGetLastError());
   return NZ_OK;
@@ -426,8 +443,9 @@ int nz_encode_static(const void* dev_bf16, uint64_t n, int precision, uint32_t c
 
 int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed, uint64_t n,
               int precision, uint32_t chunk_size, uint32_t lane_syms, void* dev_bf16_out,
-              uint32_t* dev_status, int check, uint32_t normalizer_size, const void* dev_norm,
+              uint32_t* dev_status, int flags, uint32_t normalizer_size, const void* dev_norm,
               void* stream) {
+  const int check = flags & NZ_DECODE_CHECK;
   if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
   if (!normalizer_ok(normalizer_size))
     return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
@@ -443,8 +461,10 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
   if (!dev_status) return fail(NZ_ERR_ARG, "dev_status is required (the kernel reports there)");
   if (comp_bytes < g.rec_off + NZ_TAIL_PAD) return fail(NZ_ERR_CORRUPT, "container shorter than its directory");
   hipStream_t st = (hipStream_t)stream;
+  if ((flags & NZ_DECODE_STREAM_OUT) && (flags & NZ_DECODE_RESIDENT_OUT))
+    return fail(NZ_ERR_ARG, "NZ_DECODE_STREAM_OUT and NZ_DECODE_RESIDENT_OUT exclude each other");
   if (int rc = decode_launch(g, precision, dev_comp, comp_bytes, dev_packed, dev_bf16_out, dev_status,
-                             normalizer_size, dev_norm, st))
+                             normalizer_size, dev_norm, flags, st))
     return rc;
   if (check) {
     uint32_t hs = 0;
@@ -779,7 +799,7 @@ int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap
   NzGeom g;
   if (int rc = make_geom(&g, ent.n, ent.chunk_syms, ent.lane_syms)) return rc;
   return decode_launch(g, m->precision, ent.comp, ent.comp_bytes, ent.packed, dev_out, m->d_status,
-                       m->normalizer, ent.norm, (hipStream_t)stream);
+                       m->normalizer, ent.norm, 0, (hipStream_t)stream);
 }
 
 int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* dev_outs,
@@ -800,33 +820,41 @@ int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* 
   NzBatch b;
   std::memset(&b, 0, sizeof(b));
   uint32_t grid = 0, max_spc = 1;
+  bool streaming = false;
   auto flush = [&]() -> int {
-    int rc = decode_batch_launch(b, grid, max_spc, m->precision, m->d_status, (hipStream_t)stream);
+    int rc = decode_batch_launch(b, grid, max_spc, m->precision, streaming, m->d_status, (hipStream_t)stream);
     b.count = 0;
     grid = 0;
     max_spc = 1;
     return rc;
   };
-  for (uint32_t i = 0; i < count; ++i) {
-    const Entry& ent = m->entries.find(names[i])->second;
-    if (ent.n == 0) continue;
-    NzGeom g;
-    if (int rc = make_geom(&g, ent.n, ent.chunk_syms, ent.lane_syms)) return rc;
-    if (b.count == NZ_BATCH_MAX || (uint64_t)grid + g.n_chunks > 0x7FFFFFFFull)
+  // a launch has one output policy: the tensors small enough to stay in the
+  // last-level cache first, then (rarely any) the ones written with streaming stores
+  for (int pass = 0; pass < 2; ++pass) {
+    streaming = pass == 1;
+    for (uint32_t i = 0; i < count; ++i) {
+      const Entry& ent = m->entries.find(names[i])->second;
+      if (ent.n == 0 || nz_stream_output(ent.n) != streaming) continue;
+      NzGeom g;
+      if (int rc = make_geom(&g, ent.n, ent.chunk_syms, ent.lane_syms)) return rc;
+      if (b.count == NZ_BATCH_MAX || (uint64_t)grid + g.n_chunks > 0x7FFFFFFFull)
+        if (int rc = flush()) return rc;
+      NzBatchItem& it = b.item[b.count++];
+      it.comp = (const uint8_t*)ent.comp;
+      it.comp_bytes = ent.comp_bytes;
+      it.packed = (const uint8_t*)ent.packed;
+      it.out = (uint16_t*)dev_outs[i];
+      it.norm = (const uint8_t*)ent.norm;
+      b.log2n = log2_of(m->normalizer ? m->normalizer : 1);
+      it.g = g;
+      grid += (uint32_t)g.n_chunks;
+      it.chunk_end = grid;
+      if (g.spc > max_spc) max_spc = g.spc;
+    }
+    if (b.count)
       if (int rc = flush()) return rc;
-    NzBatchItem& it = b.item[b.count++];
-    it.comp = (const uint8_t*)ent.comp;
-    it.comp_bytes = ent.comp_bytes;
-    it.packed = (const uint8_t*)ent.packed;
-    it.out = (uint16_t*)dev_outs[i];
-    it.norm = (const uint8_t*)ent.norm;
-    b.log2n = log2_of(m->normalizer ? m->normalizer : 1);
-    it.g = g;
-    grid += (uint32_t)g.n_chunks;
-    it.chunk_end = grid;
-    if (g.spc > max_spc) max_spc = g.spc;
   }
-  return b.count ? flush() : NZ_OK;
+  return NZ_OK;
 }
 
 int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t count, const void* dev_x,

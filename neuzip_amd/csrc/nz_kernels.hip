@@ -888,9 +888,7 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
 // falls below 2^16 a 16-bit word taken at (words consumed so far by the wave +
 // rank of the lane among the lanes that need one).
 
-// a ring is followed by a copy of its first 64 words, so that the 64 words a
-// step may touch never wrap
-#define NZ_RING_ALLOC_DWORDS (NZ_RING_DWORDS + 32)
+#define NZ_RING_ALLOC_DWORDS NZ_RING_DWORDS
 // What the table parse leaves for the slot-table fill (runs, windows, flags)
 // lies in the last slots of the table itself; those are filled last, from
 // registers.
@@ -907,6 +905,38 @@ __device__ __forceinline__ uint64_t nz_load_sm(const uint8_t* p) {
   else if constexpr (S == 3) return *reinterpret_cast<const uint32_t*>(p);
   else if constexpr (S == 1) return *reinterpret_cast<const uint16_t*>(p);
   else return *p;
+}
+
+// 8 decoded values to the dense output as a streaming (non-temporal) 16-byte
+// store: for outputs too large to stay in the last-level cache until their
+// consumer runs (nz_stream_output).
+__device__ __forceinline__ void nz_stream_store(uint16_t* p, const uint4 v) {
+  typedef uint32_t nz_u32x4 __attribute__((ext_vector_type(4)));
+  const nz_u32x4 q = {v.x, v.y, v.z, v.w};
+  __builtin_nontemporal_store(q, reinterpret_cast<nz_u32x4*>(p));
+}
+
+// Output policy of a decode.  A tensor whose dense form is at most half of the
+// 256 MB last-level cache is written with ordinary stores: the GEMM that
+// consumes the weight right after finds it there (decode + matrix-vector
+// product of a 128 MiB weight: 66 us instead of 75), and a reused output buffer
+// costs nothing extra.  A larger tensor cannot stay resident anyway; writing it
+// with streaming stores keeps it from churning the cache (448 MiB: 145 us
+// instead of 167).
+#ifndef NZ_STREAM_OUT_BYTES
+#define NZ_STREAM_OUT_BYTES (128ull << 20)
+#endif
+NZ_HD static inline bool nz_stream_output(uint64_t n) { return 2 * n > NZ_STREAM_OUT_BYTES; }
+
+// S+1 packed bytes of one group from the stored stream in global memory,
+// which a decode reads exactly once: a streaming (non-temporal) load, so that
+// the bytes do not displace what the caches could keep.
+template <int S>
+__device__ __forceinline__ uint64_t nz_stream_sm(const uint8_t* p) {
+  if constexpr (S == 7) return __builtin_nontemporal_load(reinterpret_cast<const uint64_t*>(p));
+  else if constexpr (S == 3) return __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p));
+  else if constexpr (S == 1) return __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(p));
+  else return __builtin_nontemporal_load(p);
 }
 
 // Merge 8 exponents (byte 3 of ew[j]) with the group's packed bytes into 8
@@ -1109,12 +1139,13 @@ struct NzWaveDec {
   uint32_t* ring32;       // 512 dwords = 1024 words: a window of the record
   const uint8_t* words;   // start of the record (uniform); word indices count from here
   uint32_t lim;           // largest byte offset from `words` that may be loaded: container end - 16 (uniform)
-  uint32_t ring_addr;     // LDS byte address of the ring (uniform)
+  uint32_t ring_lds;      // LDS byte address of the ring (the same in all lanes, kept in a vector register)
   uint32_t nwords;        // 16-bit units the record holds, table and states included
   uint32_t lane;
   uint32_t x;             // this lane's rANS state
-  uint32_t base;          // words consumed by the wave
-  uint32_t filled;        // dwords staged into the ring (multiple of 256)
+  uint32_t base;          // words consumed by the wave (the same in all lanes, kept in a vector register)
+  uint32_t filled;        // dwords staged into the ring (multiple of 256; uniform)
+  uint32_t sel_keep, sel_shift;  // byte selectors of the renormalisation (vector registers)
   uint4 r;                // 8 words per lane fetched during the previous group
 
   // 16 bytes of the word stream at dword index d (multiple of 4 per lane).
@@ -1128,16 +1159,14 @@ struct NzWaveDec {
   }
 
   __device__ __forceinline__ void commit(uint32_t d, const uint4& v) {
-    const uint32_t i = d & (NZ_RING_DWORDS - 1);
-    *reinterpret_cast<uint4*>(ring32 + i) = v;
-    if (i < 32) *reinterpret_cast<uint4*>(ring32 + NZ_RING_DWORDS + i) = v;  // the copy behind the end
+    *reinterpret_cast<uint4*>(ring32 + (d & (NZ_RING_DWORDS - 1))) = v;
   }
 
   // record at comp + pos of a container of comp_bytes (pos + 16 <= comp_bytes)
   __device__ __forceinline__ void attach(const uint8_t* comp, uint64_t comp_bytes, uint64_t pos, uint32_t* ring) {
     typedef __attribute__((address_space(3))) uint32_t lds_u32;
     ring32 = ring;
-    ring_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)((lds_u32*)ring));
+    ring_lds = (uint32_t)(uintptr_t)((lds_u32*)ring);
     words = comp + pos;
     const uint64_t room = comp_bytes - NZ_TAIL_PAD - pos;
     lim = room < 0xFFFFFFF0ull ? (uint32_t)room : 0xFFFFFFF0u;
@@ -1158,29 +1187,43 @@ struct NzWaveDec {
   // into the record (at most 348, so at least 676 words are staged ahead).
   __device__ __forceinline__ void start(uint32_t x0, uint32_t first_word) {
     x = x0;
-    base = __builtin_amdgcn_readfirstlane(first_word);  // the same in all lanes: keep it scalar
+    base = first_word;
     filled = __builtin_amdgcn_readfirstlane(filled);
-    r = make_uint4(0, 0, 0, 0);
+    r = fetch(filled + 4 * lane);  // the 512 words behind the staged window
+    // keep the three per-lane constants in vector registers of their own (an
+    // instruction can name only one scalar register or literal)
+    sel_keep = 0x07060504u;
+    sel_shift = 0x05040100u;
+    asm volatile("" : "+v"(sel_keep), "+v"(sel_shift), "+v"(ring_lds), "+v"(base));
   }
 
   // Decode the next 8 symbols of every lane into byte 3 of ew[0..7].
   //
-  // Ring upkeep is software-pipelined over two groups so that no load is
-  // waited for in the group that issued it: every group fetches the 512 words
-  // that follow the staged ones into registers (clamped addresses, mostly
-  // cache hits); at the start of the next group they are committed to the
-  // ring if no more than 512 words are still ahead of `base`.  A group
-  // consumes at most 8 * 64 = 512 words, so at least 512 words are ahead at
-  // every group start and the window [base, filled) never exceeds the 1024
-  // ring words.
+  // Ring upkeep: the 512 words that follow the staged window wait in
+  // registers (`r`, fetched right after the previous commit, addresses clamped
+  // to the container); at the start of a group they are committed to the ring
+  // if no more than 512 words are still ahead of `base`, and the next 512 are
+  // fetched.  A group consumes at most 8 * 64 = 512 words, so at least 512
+  // words are ahead at every group start, the window [base, filled) never
+  // exceeds the 1024 ring words, and a fetch has at least one group (for
+  // exponent data about six) to arrive before its commit.
+  //
+  // A step issues: slot read, multiply-add, compare, the lane's word index
+  // (words consumed by the wave + its rank among the lanes that renormalise:
+  // the two mbcnt instructions add the rank to `base`), the index wrapped into
+  // the ring, the word read, and one byte permute whose selector either keeps
+  // the state or shifts the word in; `base` advances by the ballot's
+  // popcount.  No execution-mask changes and three scalar instructions per
+  // step (popcount and the two waits).
   __device__ __forceinline__ void group(uint32_t (&ew)[8]) {
-    if ((2 * filled - base) <= 512u) {
+    const uint32_t ahead = __builtin_amdgcn_readfirstlane(base);
+    if ((2 * filled - ahead) <= 512u) {
       commit(filled + 4 * lane, r);
       filled += 256;
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
+      r = fetch(filled + 4 * lane);
     }
-    r = fetch(filled + 4 * lane);
     typedef __attribute__((address_space(3))) const uint16_t lds_cu16;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -1189,23 +1232,16 @@ struct NzWaveDec {
       ew[j] = e.x;
       const bool need = x < NZ_L;
       const uint64_t m = __ballot(need);
-      const uint32_t rank = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
-                                                      __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
-      // word base + rank of the record: the ring position of `base` is scalar
-      // arithmetic, the lane adds its rank (never past the copy behind the end)
-      const uint32_t at = ring_addr + 2u * (base & (NZ_RING_WORDS - 1)) + 2u * rank;
+      const uint32_t widx = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                                      __builtin_amdgcn_mbcnt_lo((uint32_t)m, base));
+      uint32_t ring_word = widx & (NZ_RING_WORDS - 1);
+      asm volatile("" : "+v"(ring_word));  // mask, then one shift-add (not shift, mask, add)
+      const uint32_t at = (ring_word << 1) + ring_lds;
       uint32_t w = *(lds_cu16*)(uintptr_t)at;
       // keep the word read unconditional: straight-line code, no exec-mask branch
       asm volatile("" : "+v"(w));
-      // renormalise: x = x << 16 | w in the lanes that need it.  One byte permute
-      // under the ballot as exec mask (every lane of the wave is active here, so
-      // exec is all ones before and after); cheaper than select + permute.
-      asm volatile(
-          "s_mov_b64 exec, %[m]\n\t"
-          "v_perm_b32 %[x], %[x], %[w], %[sel]\n\t"
-          "s_mov_b64 exec, -1"
-          : [x] "+v"(x)
-          : [w] "v"(w), [m] "s"(m), [sel] "s"(0x05040100u));
+      const uint32_t sel = need ? sel_shift : sel_keep;
+      x = __builtin_amdgcn_perm(x, w, sel);  // x << 16 | w where the state fell below 2^16
       base += (uint32_t)__popcll(m);
     }
   }
@@ -1220,7 +1256,7 @@ struct NzWaveDec {
 // ragged and no group straddles two rows).
 // With NORM every merged value is multiplied by its group's factor (`nm`)
 // before it is stored or used.
-template <int S, bool GEMV, bool NORM>
+template <int S, bool GEMV, bool NORM, bool STREAM>
 __device__ __forceinline__ void nz_decode_chunk(
     const uint8_t* __restrict__ comp, const uint64_t comp_bytes, const uint8_t* __restrict__ packed,
     uint16_t* __restrict__ out, const NzGeom& g, uint32_t* __restrict__ d_status, const uint64_t c,
@@ -1305,7 +1341,7 @@ __device__ __forceinline__ void nz_decode_chunk(
       xq_next = walk.load(walk.col);
     }
     if (whole) {
-      sm_next = nz_load_sm<S>(pk + lane_off);
+      sm_next = nz_stream_sm<S>(pk + lane_off);
       if constexpr (NORM) nb_next = nz_norm_load8(nm, seg_base + lane * NZ_GROUP);
     }
   }
@@ -1514,27 +1550,49 @@ __device__ __forceinline__ void nz_decode_chunk(
   const uint32_t x0 = (uint32_t)(win >> (8 * (fb & 3) + 4 * (at & 1))) & (0xFFFFFFFFu >> (32 - 4 * nn));
   w.start(x0, (rec_skip + sbytes) / 2);
 
-  for (uint32_t gq = 0; gq < whole; ++gq) {
-    const uint64_t sm = sm_next;
-    const uint32_t noff = (gq + 1) * NZ_LANES * (S + 1) + lane_off;
-    sm_next = nz_load_sm<S>(pk + (noff < last_off ? noff : last_off));
+  // Groups in which every lane has 8 elements.  Packed bytes (and normalizer
+  // bytes) are fetched TWO groups before their use, alternately into two
+  // registers, so that the wait in front of a merge is for a load issued two
+  // groups (about two microseconds) earlier and for nothing younger: neither
+  // the latency of a load that misses every cache nor the previous group's
+  // store is waited for.
+  const auto sm_at = [&](uint32_t gq) {
+    const uint32_t off = gq * NZ_LANES * (S + 1) + lane_off;
+    return nz_stream_sm<S>(pk + (off < last_off ? off : last_off));
+  };
+  const auto nb_at = [&](uint32_t gq) {
+    return nz_norm_load8(nm, seg_base + ((gq < whole ? gq : whole - 1) * NZ_LANES + lane) * NZ_GROUP);
+  };
+  const auto full_group = [&](uint32_t gq, const uint64_t sm, const uint64_t nb) {
     const uint4 xq = xq_next;
     if constexpr (GEMV) xq_next = walk.load(walk.next_col());  // always inside x
-    const uint64_t nb = nb_next;
-    if constexpr (NORM)
-      nb_next = nz_norm_load8(nm, seg_base + ((gq + 1 < whole ? gq + 1 : gq) * NZ_LANES + lane) * NZ_GROUP);
     uint32_t ew[8];
     w.group(ew);
-    // the merge starts only here: its wait for the packed bytes (fetched a group
-    // ago) must not be hoisted in front of the rANS steps, where it would also
-    // wait for the previous group's store
+    // the merge starts only here: its wait for the packed bytes must not be
+    // hoisted in front of the rANS steps
     uint32_t sml = (uint32_t)sm, smh = (uint32_t)(sm >> 32);
     asm volatile("" : "+v"(sml), "+v"(smh), "+v"(ew[7]));
     uint4 mv = nz_merge_group<S>(((uint64_t)smh << 32) | sml, ew);
     if constexpr (NORM) mv = nz_scale8<true>(mv, nb, nm.log2n >= 3);
     if constexpr (GEMV) walk.add(mv, xq, lane);
+    else if constexpr (STREAM) nz_stream_store(dst + (gq * NZ_LANES + lane) * NZ_GROUP, mv);
     else *reinterpret_cast<uint4*>(dst + (gq * NZ_LANES + lane) * NZ_GROUP) = mv;
+  };
+  uint64_t sm_a = sm_next, sm_b = 0, nb_a = nb_next, nb_b = 0;
+  if (whole > 1) {
+    sm_b = sm_at(1);
+    if constexpr (NORM) nb_b = nb_at(1);
   }
+  uint32_t gq = 0;
+  for (; gq + 1 < whole; gq += 2) {
+    full_group(gq, sm_a, nb_a);
+    sm_a = sm_at(gq + 2);
+    if constexpr (NORM) nb_a = nb_at(gq + 2);
+    full_group(gq + 1, sm_b, nb_b);
+    sm_b = sm_at(gq + 3);
+    if constexpr (NORM) nb_b = nb_at(gq + 3);
+  }
+  if (gq < whole) full_group(gq, sm_a, nb_a);
   if (!GEMV && whole < body) {  // the ragged last group of the tensor
     const uint32_t idx0 = (whole * NZ_LANES + lane) * NZ_GROUP;
     uint32_t ew[8];
@@ -1586,11 +1644,11 @@ __device__ __forceinline__ void nz_decode_chunk(
     if (walk.pending) walk.flush(lane);
 }
 
-template <int S, bool NORM>
+template <int S, bool NORM, bool STREAM>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
     uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status, const NzNorm nm) {
-  nz_decode_chunk<S, false, NORM>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x, NzGemv{}, nm);
+  nz_decode_chunk<S, false, NORM, STREAM>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x, NzGemv{}, nm);
 }
 
 // Several tensors in one launch: the grid is the concatenation of their
@@ -1619,7 +1677,7 @@ struct NzBatch {
   NzBatchItem item[NZ_BATCH_MAX];
 };
 
-template <int S, bool NORM>
+template <int S, bool NORM, bool STREAM>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_batch_kernel(
     const NzBatch b, uint32_t* __restrict__ d_status) {
   uint32_t t = 0, first = 0;
@@ -1628,8 +1686,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_batch_ke
     ++t;
   }
   const NzBatchItem& it = b.item[t];
-  nz_decode_chunk<S, false, NORM>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status,
-                                  blockIdx.x - first, NzGemv{}, NzNorm{it.norm, b.log2n});
+  nz_decode_chunk<S, false, NORM, STREAM>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status,
+                                          blockIdx.x - first, NzGemv{}, NzNorm{it.norm, b.log2n});
 }
 
 // The same walk over several matrices that multiply one activation row.
@@ -1643,8 +1701,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_gemv_ker
   }
   const NzBatchItem& it = b.item[t];
   const NzGemv gv{b.x, it.acc, it.y, it.bias, b.in_features};
-  nz_decode_chunk<S, true, NORM>(it.comp, it.comp_bytes, it.packed, nullptr, it.g, d_status,
-                                 blockIdx.x - first, gv, NzNorm{it.norm, b.log2n});
+  nz_decode_chunk<S, true, NORM, false>(it.comp, it.comp_bytes, it.packed, nullptr, it.g, d_status,
+                                        blockIdx.x - first, gv, NzNorm{it.norm, b.log2n});
 }
 
 // ----------------------------------------------------------------------------
@@ -1671,7 +1729,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_rows_ker
   // the chunk function writes element e of the tensor to out[e]: shift `out` so
   // that the chunk's first element lands at the start of this workgroup's slot
   uint16_t* out = scratch + ((int64_t)blockIdx.x - (int64_t)c) * (int64_t)g.chunk_syms;
-  nz_decode_chunk<S, false, NORM>(comp, comp_bytes, packed, out, g, d_status, c, NzGemv{}, nm);
+  // (the slots are read back by the copy kernel right away: ordinary stores)
+  nz_decode_chunk<S, false, NORM, false>(comp, comp_bytes, packed, out, g, d_status, c, NzGemv{}, nm);
 }
 
 __global__ __launch_bounds__(256) void nz_copy_rows_kernel(const uint16_t* __restrict__ scratch,

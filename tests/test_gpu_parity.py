@@ -207,3 +207,26 @@ def test_split_api(oracle):
         oe, of = oracle.split(bits, 7)
         assert np.array_equal(e[:n].cpu().numpy(), oe)
         assert np.array_equal(f[:n].cpu().numpy(), of)
+
+
+def test_decode_output_policy_flags(oracle):
+    """nz_decode writes the same values whether the output is written with
+    ordinary or with streaming stores; asking for both is an argument error."""
+    L, m = _lib()
+    for s in (7, 1):
+        bits = stress_bits(64, 4099, seed=40 + s)
+        comp, packed = gpu_encode(bits, s)
+        want = oracle.reconstruct(bits, s)
+        for flags in (0, m.DECODE_STREAM_OUT, m.DECODE_RESIDENT_OUT, m.DECODE_CHECK | m.DECODE_STREAM_OUT):
+            out = torch.zeros(bits.size, dtype=torch.int16, device="cuda")
+            status = torch.zeros(2, dtype=torch.int32, device="cuda")
+            rc = L.nz_decode(comp.data_ptr(), comp.numel(), packed.data_ptr(), bits.size, s, 131072, 256,
+                             out.data_ptr(), status.data_ptr(), flags, 0, None, torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, m.last_error()
+            torch.cuda.synchronize()
+            assert int(status[0]) == 0
+            assert np.array_equal(out.cpu().numpy().view(np.uint16), want)
+        rc = L.nz_decode(comp.data_ptr(), comp.numel(), packed.data_ptr(), bits.size, s, 131072, 256,
+                         out.data_ptr(), status.data_ptr(), m.DECODE_STREAM_OUT | m.DECODE_RESIDENT_OUT, 0, None,
+                         torch.cuda.current_stream().cuda_stream)
+        assert rc == m.ERR_ARG and "exclude" in m.last_error()
