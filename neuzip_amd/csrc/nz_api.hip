@@ -574,37 +574,45 @@ void release_entry(Entry& e) {
 int pick_geometry(const nz_manager* m, uint64_t n, NzGeom* g, uint32_t* chunk_out, uint32_t* lane_out) {
   uint32_t lane_syms = m->lane_syms, chunk_syms = m->chunk_syms;
   if (m->auto_lanes && m->own_chunk && chunk_syms == NZ_DEFAULT_CHUNK && lane_syms == NZ_DEFAULT_LANE_SYMS) {
-    // The device holds `slots` decode workgroups at once; a launch is fastest as
-    // ONE round of them, and while they do not fill the device the time of the
-    // round goes with the length of a segment.  So, by size:
-    //   more chunks than slots          the default geometry
-    //   more than half the slots        segments stretched until the chunks fit
-    //                                   into half the slots: two such tensors
-    //                                   decoded by one launch (gate and up
-    //                                   projection of a block, say) are one round
-    //                                   instead of one and a badly filled second
-    //   fewer                           64 Ki chunks of eight 8 Ki segments, or
-    //                                   32 Ki chunks of eight 4 Ki segments when
-    //                                   those still fit into the slots
-    // (shorter segments cost compression: 1.8 % and 3.6 % of the exponent bytes
-    // instead of 1 %).
-    const uint64_t slots = m->slots, half = slots / 2;
+    // The device holds `slots` decode workgroups (three per compute unit) at
+    // once, and a launch is fastest when every compute unit has the same number
+    // of them: 378 workgroups on 256 units run as long as 512 would (measured on
+    // a 4096 x 14336 matrix: 51 us with 378 chunks, 38 us with 512).  A tensor
+    // with more default-sized chunks than slots keeps the default geometry.  A
+    // smaller one is cut into one, two or three workgroups per compute unit
+    // (more of them only where the model below promises 10 % or more), with
+    // segments of 64 to 512
+    // symbols per lane (shorter segments cost compression: ~4.5 bits per lane
+    // and segment); a tensor too small for that gets 32 Ki chunks of eight
+    // 4 Ki segments.  Time of a round ~ symbols per lane x time of a step, which
+    // grows with the wavefronts that share a SIMD unit (2, 4, 6 of them: about
+    // 107, 147, 215 ns per step).
+    const uint64_t slots = m->slots, cus = slots / 3;
     const uint64_t chunks = (n + chunk_syms - 1) / chunk_syms;
-    if (chunks > slots || half == 0) {
+    if (chunks > slots || cus == 0) {
       // default
-    } else if (chunks > half) {
-      const uint64_t per_seg = (n + half * NZ_MAX_SEGS_PER_CHUNK - 1) / (half * NZ_MAX_SEGS_PER_CHUNK);
-      const uint32_t lane = (uint32_t)((per_seg + NZ_LANES * 8 - 1) / (NZ_LANES * 8)) * 8;
-      if (lane <= 2 * NZ_DEFAULT_LANE_SYMS && nz_geom_check(lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK, lane) == 0) {
-        lane_syms = lane;
-        chunk_syms = lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK;
-      }
-    } else if (n > slots * 32768) {
-      chunk_syms = 65536;
-      lane_syms = 128;
     } else {
-      chunk_syms = 32768;
-      lane_syms = 64;
+      static const uint32_t step_ns[3] = {107, 147, 215};
+      uint64_t best_t = ~0ull;
+      uint32_t best_lane = 0;
+      for (uint32_t k = 1; k <= 3; ++k) {
+        const uint64_t per_lane = (n + k * cus * 512 - 1) / (k * cus * 512);  // a chunk is 8 x 64 lanes
+        const uint32_t lane = (uint32_t)((per_lane + 7) / 8) * 8;
+        if (lane < 64 || lane > 2 * NZ_DEFAULT_LANE_SYMS) continue;
+        if (nz_geom_check(lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK, lane)) continue;
+        const uint64_t t = (uint64_t)lane * step_ns[k - 1];
+        if (best_lane == 0 || 10 * t < 9 * best_t) {  // more, shorter segments only for a gain above 10 %
+          best_t = t;
+          best_lane = lane;
+        }
+      }
+      if (best_lane) {
+        lane_syms = best_lane;
+        chunk_syms = best_lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK;
+      } else {
+        chunk_syms = 32768;
+        lane_syms = 64;
+      }
     }
   } else if (m->auto_lanes) {
     // a chunk size given by the caller: shorter segments while that is a valid

@@ -75,8 +75,8 @@ def test_gemv_matches_fp64_product(rows, cols, kind, lane, s):
 
 @pytest.mark.parametrize("rows,cols", [(14336, 4096), (4096, 4096), (2048, 14336)])
 def test_gemv_at_the_geometries_chosen_per_tensor(rows, cols):
-    """Per-tensor geometry: segments of 19 456 (rows straddle them), of 4096 (one
-    row each, stored directly) and of 8192 elements (a row spans two or three)."""
+    """Per-tensor geometry: segments of 14 336 elements (rows straddle them), of
+    4096 (one row each, stored directly) and of 7168 (a row spans two or three)."""
     import neuzip_amd
 
     mgr = neuzip_amd.Manager(precision=7, lane_symbols="auto")

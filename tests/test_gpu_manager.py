@@ -405,17 +405,36 @@ def test_read_batch_equals_single_reads(oracle):
         assert all(int(o.view(torch.int16).abs().max()) == 0 for o in outs2)
 
 
+def _auto_geometry(n, cus=256):
+    """The per-tensor rule of nz_manager_create(lane_syms = NZ_LANE_SYMS_AUTO) with
+    the library's own chunk: k = 1, 2 or 3 workgroups per compute unit, segments
+    of 64..512 symbols per lane, more workgroups only for a modelled gain above 10 %."""
+    if -(-n // 131072) > 3 * cus:
+        return 131072, 256
+    best = None
+    for k, step_ns in ((1, 107), (2, 147), (3, 215)):
+        lane = -(-(-(-n // (k * cus * 512))) // 8) * 8
+        if lane < 64 or lane > 512:
+            continue
+        t = lane * step_ns
+        if best is None or 10 * t < 9 * best[0]:
+            best = (t, lane)
+    return (512 * best[1], best[1]) if best else (32768, 64)
+
+
 def test_auto_lane_symbols(oracle):
-    """Per-tensor geometry: small tensors get shorter segments (32 Ki or 64 Ki
-    chunks of eight segments), tensors whose chunks would take between half and
-    all of the device's 768 workgroup slots get longer ones (at most 384
-    chunks), the stored bytes are those of the oracle at that geometry, and
-    reads are exact."""
+    """Per-tensor geometry: a tensor that does not fill the device's 768
+    workgroup slots at the default geometry is cut into 256, 512 or 768 chunks
+    (the same number of workgroups on every compute unit) of eight segments, a
+    very small one into 32 Ki chunks; the stored bytes are those of the oracle
+    at that geometry, and reads are exact."""
     import neuzip_amd
 
+    assert _auto_geometry(14336 * 4096) == (114688, 224) and _auto_geometry(4096 * 4096) == (32768, 64)
+    assert _auto_geometry(16384 * 4096) == (131072, 256) and _auto_geometry(110_000_000) == (131072, 256)
     for chunk_arg, cases in (
-        (None, ((1000, 32768, 64), (40_001, 32768, 64), (1 << 20, 32768, 64), (25_165_824, 32768, 64), (40_000_000, 65536, 128), (14336 * 4096, 155648, 304),
-                (70_000_000, 184320, 360), (110_000_000, 131072, 256))),
+        (None, tuple((n,) + _auto_geometry(n) for n in (1000, 40_001, 1 << 20, 25_165_824, 40_000_000, 14336 * 4096,
+                                                        70_000_000, 110_000_000))),
         (65536, ((1 << 20, 65536, 176), (40_000_000, 65536, 176), (70_000_000, 65536, 344))),
     ):
         mgr = neuzip_amd.Manager(chunk_size=chunk_arg, lane_symbols="auto")
