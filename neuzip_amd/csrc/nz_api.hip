@@ -44,8 +44,11 @@ uint64_t norm_bytes_of(uint64_t n, uint32_t ns) { return ns ? (n + ns - 1) / ns 
 
 // Device scratch of one encode call.
 struct EncLayout {
-  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, hdr, bytes;
+  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units, bytes;
 };
+
+// segments short enough for the kernel that keeps the exponents in registers
+bool enc_in_registers(const NzGeom& g) { return g.lane_syms <= NZ_ENC_MAX_LANE_SYMS; }
 
 EncLayout enc_layout(const NzGeom& g) {
   EncLayout L;
@@ -55,17 +58,16 @@ EncLayout enc_layout(const NzGeom& g) {
     o = align_up(o + b, 256);
     return at;
   };
-  L.exps = take(g.n + 16);
-  L.enc_tab = take(g.n_chunks * 256 * 4);
+  L.exps = take(enc_in_registers(g) ? 0 : g.n + 16);  // only long segments park their exponents in memory
   L.tab_ser = take(g.n_chunks * NZ_TABLE_MAX_BYTES);
   L.info = take(g.n_chunks * sizeof(NzChunkInfo));
   L.carry = take(g.n_segs * NZ_CARRY_BYTES);
-  L.slots = take(g.n_segs * 2 * (uint64_t)g.seg_syms);  // one 2-byte word per symbol: the worst case
+  L.slots = take(g.n_segs * 2 * (uint64_t)g.seg_syms + 16);  // one 2-byte word per symbol: the worst case
   L.states = take(g.n_segs * NZ_STATE_MAX_BYTES);
   L.seg_words = take(g.n_segs * 4);
   L.seg_sbytes = take(g.n_segs * 4);
   L.seg_units = take((g.n_segs + 1) * 4);
-  L.hdr = take(g.rec_off + NZ_TAIL_PAD);
+  L.chunk_units = take((g.n_chunks + 1) * 4);
   L.bytes = o;
   return L;
 }
@@ -79,17 +81,15 @@ int launch_absmax(const void* in, uint64_t n, uint32_t ns, uint8_t* norm, hipStr
   return NZ_OK;
 }
 
-// One tensor of an encode call, as the kernels see it.  `hdr` is where header
-// and directory are built, `comp`/`comp_cap` where the records go (known only
-// after phase 1 when the buffer is sized to fit).
+// One tensor of an encode call, as the kernels see it.  `comp`/`comp_cap`: where
+// the container goes (known only after phase 1 when the buffer is sized to fit).
 NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws, const EncLayout& L,
-                   uint8_t* hdr, uint8_t* comp, uint64_t comp_cap, uint64_t* d_total, uint32_t* d_status,
+                   uint8_t* comp, uint64_t comp_cap, uint64_t* d_total, uint32_t* d_status,
                    uint32_t ns, uint8_t* norm) {
   NzEncItem it{};
   it.in = (const uint16_t*)in;
   it.packed = packed;
   it.ws = ws;
-  it.hdr = hdr;
   it.comp = comp;
   it.comp_cap = comp_cap;
   it.d_total = d_total;
@@ -97,7 +97,6 @@ NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws
   it.nm = NzNorm{ns ? norm : nullptr, log2_of(ns ? ns : 1)};
   it.g = g;
   it.exps = L.exps;
-  it.enc_tab = L.enc_tab;
   it.tab_ser = L.tab_ser;
   it.info = L.info;
   it.carry = L.carry;
@@ -106,6 +105,7 @@ NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws
   it.seg_words = L.seg_words;
   it.seg_sbytes = L.seg_sbytes;
   it.seg_units = L.seg_units;
+  it.chunk_units = L.chunk_units;
   return it;
 }
 
@@ -122,6 +122,23 @@ bool enc_batch_close(NzEncBatch* b) {
   return true;
 }
 
+// One encode launch for the tensors of `b` whose segments are of class `cls`
+// (0..2: up to 64 / 128 / 256 symbols per lane, coded from registers; 3: longer).
+template <int S>
+void launch_encode_class(const NzEncBatch& b, int cls, uint32_t chunks, uint32_t max_spc, hipStream_t st) {
+  const dim3 grid(chunks), block(64 * (max_spc < 4 ? 4 : max_spc));
+  switch (cls) {
+    case 0: hipLaunchKernelGGL((nz_encode_kernel<S, 8>), grid, block, 0, st, b); break;
+    case 1: hipLaunchKernelGGL((nz_encode_kernel<S, 16>), grid, block, 0, st, b); break;
+    case 2: hipLaunchKernelGGL((nz_encode_kernel<S, 32>), grid, block, 0, st, b); break;
+    default: hipLaunchKernelGGL((nz_encode_long_kernel<S>), grid, dim3(NZ_ENC_LONG_THREADS), 0, st, b); break;
+  }
+}
+
+int enc_class(const NzGeom& g) {
+  return g.lane_syms <= 64 ? 0 : g.lane_syms <= 128 ? 1 : g.lane_syms <= NZ_ENC_MAX_LANE_SYMS ? 2 : 3;
+}
+
 // Phase 1 for all tensors of the batch: everything up to the directory.  Header
 // + directory land in each item's `hdr`, the container size in its *d_total.
 int encode_phase1(NzEncBatch* b, int precision, uint32_t ns, hipStream_t st) {
@@ -129,30 +146,48 @@ int encode_phase1(NzEncBatch* b, int precision, uint32_t ns, hipStream_t st) {
   for (uint32_t i = 0; i < b->count; ++i)
     if (int rc = launch_absmax(b->item[i].in, b->item[i].g.n, ns, const_cast<uint8_t*>(b->item[i].nm.bytes), st))
       return rc;
-  const uint32_t chunks = b->count ? b->item[b->count - 1].chunk_end : 0;
-  if (chunks) {
-    const dim3 grid(chunks), block(NZ_SPLIT_THREADS);
+  // the tensors of the batch, by segment-length class: one launch per class in use
+  for (int cls = 0; cls < 4; ++cls) {
+    NzEncBatch sub{};
+    uint32_t chunks = 0, max_spc = 1;
+    for (uint32_t i = 0; i < b->count; ++i) {
+      const NzEncItem& it = b->item[i];
+      if (it.g.n_chunks == 0 || enc_class(it.g) != cls) continue;
+      NzEncItem& d = sub.item[sub.count++];
+      d = it;
+      chunks += (uint32_t)it.g.n_chunks;
+      d.chunk_end = chunks;
+      if (it.g.spc > max_spc) max_spc = it.g.spc;
+    }
+    if (!sub.count) continue;
     switch (precision) {
-      case 7: hipLaunchKernelGGL(nz_split_encode_kernel<7>, grid, block, 0, st, *b); break;
-      case 3: hipLaunchKernelGGL(nz_split_encode_kernel<3>, grid, block, 0, st, *b); break;
-      case 1: hipLaunchKernelGGL(nz_split_encode_kernel<1>, grid, block, 0, st, *b); break;
-      default: hipLaunchKernelGGL(nz_split_encode_kernel<0>, grid, block, 0, st, *b); break;
+      case 7: launch_encode_class<7>(sub, cls, chunks, max_spc, st); break;
+      case 3: launch_encode_class<3>(sub, cls, chunks, max_spc, st); break;
+      case 1: launch_encode_class<1>(sub, cls, chunks, max_spc, st); break;
+      default: launch_encode_class<0>(sub, cls, chunks, max_spc, st); break;
     }
   }
-  if (b->count) hipLaunchKernelGGL(nz_scan_kernel, dim3(b->count), dim3(1024), 0, st, *b);
   NZ_HIP(hipGetLastError());
   return NZ_OK;
 }
 
-// Phase 2: the records (and, where it was built elsewhere, header and directory)
-// go to each item's `comp`.
+// Container sizes (and status) of the batch on the device, before the records
+// are placed: for a caller that sizes the container's memory to fit.  Also
+// writes the header-only container of a tensor without elements.
+int encode_totals(NzEncBatch* b, hipStream_t st) {
+  if (b->count) hipLaunchKernelGGL(nz_total_kernel, dim3(b->count), dim3(256), 0, st, *b);
+  NZ_HIP(hipGetLastError());
+  return NZ_OK;
+}
+
+// Phase 2: header, directory and records go to each item's `comp`; the
+// container size lands in *d_total, bit 0 of *d_status is set when it does not fit.
 int encode_phase2(NzEncBatch* b, hipStream_t st) {
   const uint32_t segs = b->count ? b->item[b->count - 1].seg_end : 0;
-  for (uint32_t i = 0; i < b->count; ++i) {  // a tensor without segments has no workgroup to move its header
-    const NzEncItem& it = b->item[i];
-    if (it.g.n_segs == 0 && it.hdr != it.comp)
-      NZ_HIP(hipMemcpyAsync(it.comp, it.hdr, it.g.rec_off + NZ_TAIL_PAD, hipMemcpyDeviceToDevice, st));
-  }
+  bool empty = false;  // a tensor without segments has no workgroup to write its header
+  for (uint32_t i = 0; i < b->count; ++i) empty = empty || b->item[i].g.n_segs == 0;
+  if (empty)
+    if (int rc = encode_totals(b, st)) return rc;
   if (segs) {
     hipLaunchKernelGGL(nz_compact_kernel, dim3(segs), dim3(256), 0, st, *b);
     NZ_HIP(hipGetLastError());
@@ -293,8 +328,8 @@ int encode_stateless(const void* dev_bf16, uint64_t n, int precision, uint32_t c
   if (comp_cap < nz_geom_bound(&g)) return fail(NZ_ERR_CAPACITY, "dev_comp smaller than nz_exp_bound_bytes");
   NzEncBatch b{};
   b.count = 1;
-  b.item[0] = enc_item(g, dev_bf16, (uint8_t*)dev_packed, ws, L, (uint8_t*)dev_comp, (uint8_t*)dev_comp, comp_cap,
-                       dev_total, dev_status, normalizer_size, (uint8_t*)dev_norm);
+  b.item[0] = enc_item(g, dev_bf16, (uint8_t*)dev_packed, ws, L, (uint8_t*)dev_comp, comp_cap, dev_total, dev_status,
+                       normalizer_size, (uint8_t*)dev_norm);
   if (int rc = encode_phase1(&b, precision, normalizer_size, st)) return rc;
   return encode_phase2(&b, st);
 }
@@ -678,10 +713,9 @@ int write_begin(nz_manager* m, const char* name, const void* dev_data, uint64_t 
     }
   }
   if (e != hipSuccess) return fail(NZ_ERR_HIP, std::string("write: ") + hipGetErrorString(e));
-  // header and directory are built in the scratch; where the records go is decided
-  // once the size is known
-  *item = enc_item(g, dev_data, (uint8_t*)ent.packed, ws, pw->L, ws + pw->L.hdr, nullptr, ~0ull,
-                   write_totals(m) + slot, write_status(m) + slot, m->normalizer, (uint8_t*)ent.norm);
+  // where the container goes is decided once its size is known
+  *item = enc_item(g, dev_data, (uint8_t*)ent.packed, ws, pw->L, nullptr, ~0ull, write_totals(m) + slot,
+                   write_status(m) + slot, m->normalizer, (uint8_t*)ent.norm);
   return NZ_OK;
 }
 
@@ -761,6 +795,7 @@ int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* 
     hipError_t e = hipMemsetAsync(write_status(m), 0, 64, st);
     if (e != hipSuccess) rc = fail(NZ_ERR_HIP, std::string("write: ") + hipGetErrorString(e));
     if (rc == NZ_OK) rc = encode_phase1(&b, m->precision, m->normalizer, st);
+    if (rc == NZ_OK) rc = encode_totals(&b, st);
     if (rc == NZ_OK) {
       e = hipMemcpyAsync(h_totals, write_totals(m), 8 * count, hipMemcpyDeviceToHost, st);
       if (e == hipSuccess) e = hipMemcpyAsync(h_status, write_status(m), 4 * count, hipMemcpyDeviceToHost, st);

@@ -1,12 +1,12 @@
 // gfx950 (CDNA4, wave64) kernels of the NeuZip bf16 codec.
 //
 //   nz_split_unpacked_kernel   Manager::split            cuda/high_level.cu:265-321
-//   nz_split_encode_kernel     kernel_aligned_split      cuda/kernels.cuh:62-156
-//                              + per-chunk exponent histogram, 12-bit frequency
+//   nz_encode_kernel           kernel_aligned_split      cuda/kernels.cuh:62-156
+//   nz_encode_long_kernel      + per-chunk exponent histogram, 12-bit frequency
 //                              table and its serialized form, then
 //                              nvcomp ANS compress       cuda/high_level.cu:103-115
-//   nz_scan_kernel             \ exact-size compaction    cuda/high_level.cu:117-124
-//   nz_compact_kernel          / (done on the device, no host round trip between the kernels)
+//   nz_compact_kernel          exact-size compaction     cuda/high_level.cu:117-124
+//                              (on the device: every record finds its own place)
 //   nz_decode_kernel           nvcomp ANS decompress + kernel_aligned_merge fused:
 //                              cuda/high_level.cu:184-201, cuda/kernels.cuh:167-217
 //
@@ -275,12 +275,37 @@ __global__ __launch_bounds__(256) void nz_split_unpacked_kernel(const uint16_t* 
 }
 
 // ----------------------------------------------------------------------------
-// split + histogram + table: one workgroup per chunk
+// encode: one workgroup per chunk
 // ----------------------------------------------------------------------------
+//
+// Two kernels share the pieces below.  nz_encode_kernel (segments of up to
+// NZ_ENC_MAX_LANE_SYMS symbols per lane, which covers every geometry the
+// library picks by itself): wavefront k of the workgroup splits segment k of
+// the chunk, keeps the exponent bytes of its lanes in registers, and codes
+// them from there once the chunk's table exists: the exponents never reach
+// memory.  nz_encode_long_kernel (longer segments): all wavefronts split the
+// chunk and park the exponents in scratch, then one wavefront per segment
+// codes them from there.
 
-#define NZ_SPLIT_THREADS 1024u
-#define NZ_SPLIT_WAVES (NZ_SPLIT_THREADS / 64u)
+#define NZ_ENC_MAX_LANE_SYMS 256u
+#define NZ_ENC_LONG_THREADS 1024u
 
+// f(constant I) for I = FROM, FROM + STEP, ... while I < TO (or, with a negative
+// step, while I >= TO): straight-line code with compile-time indices, so that
+// a register array indexed by I never needs an address
+template <int I>
+struct NzConst {
+  static constexpr int value = I;
+};
+template <int FROM, int TO, int STEP, class F>
+__device__ __forceinline__ void nz_static_for(F&& f) {
+  if constexpr ((STEP > 0 && FROM < TO) || (STEP < 0 && FROM >= TO)) {
+    f(NzConst<FROM>{});
+    nz_static_for<FROM + STEP, TO, STEP>(f);
+  }
+}
+
+// sums / maxima over the workgroup (at most 16 wavefronts)
 __device__ __forceinline__ uint32_t nz_block_sum(uint32_t v, uint32_t* red) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
@@ -288,8 +313,7 @@ __device__ __forceinline__ uint32_t nz_block_sum(uint32_t v, uint32_t* red) {
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
   __syncthreads();
   uint32_t t = 0;
-#pragma unroll
-  for (uint32_t w = 0; w < NZ_SPLIT_WAVES; ++w) t += red[w];
+  for (uint32_t w = 0; w < blockDim.x / 64; ++w) t += red[w];
   return t;
 }
 
@@ -303,107 +327,91 @@ __device__ __forceinline__ uint32_t nz_block_max(uint32_t v, uint32_t* red) {
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
   __syncthreads();
   uint32_t t = 0;
-#pragma unroll
-  for (uint32_t w = 0; w < NZ_SPLIT_WAVES; ++w) t = red[w] > t ? red[w] : t;
+  for (uint32_t w = 0; w < blockDim.x / 64; ++w) t = red[w] > t ? red[w] : t;
   return t;
 }
 
+// LDS of an encode workgroup.  8 histogram copies (one per lane & 7) at a
+// stride of 257 words: exponents of weights cluster on a few values, so a
+// single copy would serialise most of a wavefront's atomics on one address;
+// the odd stride keeps the copies of a bin in different banks.
+struct NzEncLds {
+  uint32_t hist[NZ_HIST_COPIES * NZ_HIST_STRIDE];
+  uint32_t red[16];
+  uint32_t scan_s[4];
+  uint64_t mw[4];
+  uint32_t cf[256];
+  // per symbol: x = freq << 20 (renormalisation threshold), y = freq, z = cum,
+  // w = bits of a float just below 1 / freq (four units in the last place
+  // under the correctly rounded quotient)
+  uint4 tab[256];
+  uint32_t sbuf[NZ_MAX_SEGS_PER_CHUNK][NZ_STATE_MAX_BYTES / 4];
+  uint32_t pad_sym, raw;
+};
+
+// Split one element group: 8 bf16 values -> 8 exponent bytes and the S+1 packed bytes.
 template <int S>
-__device__ __forceinline__ void nz_split_hist_body(
-    const uint64_t c, const uint16_t* __restrict__ in, uint64_t n, uint32_t chunk_syms, uint32_t seg_syms, uint32_t spc,
-    uint8_t* __restrict__ packed, uint8_t* __restrict__ carry, uint8_t* __restrict__ exps,
-    uint32_t* __restrict__ enc_tab, uint8_t* __restrict__ tab_ser, NzChunkInfo* __restrict__ info,
-    const NzNorm nm) {
-  // 8 histogram copies (one per lane & 7) at a stride of 257 words: exponents of
-  // weights cluster on a few values, so a single copy would serialise most of
-  // a wavefront's atomics on one address; the odd stride keeps the copies of a
-  // bin in different banks
-  __shared__ uint32_t hist[NZ_HIST_COPIES * NZ_HIST_STRIDE];
-  __shared__ uint32_t red[NZ_SPLIT_WAVES];
-  __shared__ uint32_t scan_s[4];
-  __shared__ uint64_t mw[4];
-  __shared__ uint32_t cf[256];
-
-  const uint32_t tid = threadIdx.x;
-  const uint64_t base = c * chunk_syms;
-  const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
-
-  for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += NZ_SPLIT_THREADS) hist[i] = 0;
-  __syncthreads();
-  uint32_t* myhist = hist + (tid & (NZ_HIST_COPIES - 1)) * NZ_HIST_STRIDE;
-
-  // Packed bytes go to the stored layout: segment k starts at k * keep, and the
-  // last NZ_CARRY_BYTES of a full segment go to carry[k] instead (they ride in
-  // the rANS start states).
-  const uint32_t seg_keep = seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES;     // of a segment of nominal length
-  const uint64_t chunk_keep = (uint64_t)chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * spc;
-  const uint64_t seg0 = c * spc;
-
-  for (uint32_t i = tid * 8; i < cn; i += NZ_SPLIT_THREADS * 8) {
-    const uint64_t gi = base + i;
-    const uint32_t sk = i / seg_syms;                    // segment inside the chunk
-    const uint32_t sb = (i - sk * seg_syms) / 8 * (S + 1);  // byte inside the segment
-    const uint64_t seg = seg0 + sk;
-    const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, sk);
-    const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
-    const bool seg_full = base + (uint64_t)sk * seg_syms + nom <= n;
-    uint8_t* pp = (seg_full && sb >= keep) ? carry + seg * NZ_CARRY_BYTES + (sb - keep)
-                                           : packed + c * chunk_keep + (uint64_t)sk * seg_keep + sb;
-    uint32_t ex[8], rp[8];
-    const uint32_t rem = cn - i;
-    if (rem >= 8) {
-      uint4 v = *reinterpret_cast<const uint4*>(in + gi);
-      if (nm.bytes) v = nz_scale8<false>(v, nz_norm_load8(nm, gi), nm.log2n >= 3);
-      uint32_t w[4] = {v.x, v.y, v.z, v.w};
+__device__ __forceinline__ void nz_split_group(const uint4 v, uint64_t& e, uint64_t& f) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  e = 0;
+  f = 0;
 #pragma unroll
-      for (int j = 0; j < 8; ++j) nz_split_one<S>((w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu, ex[j], rp[j]);
-      uint64_t e = 0, f = 0;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        e |= (uint64_t)ex[j] << (8 * j);
-        f |= (uint64_t)rp[j] << nz_field_shift<S>(j);
-      }
-      *reinterpret_cast<uint64_t*>(exps + gi) = e;
-      if constexpr (S == 7) *reinterpret_cast<uint64_t*>(pp) = f;
-      else if constexpr (S == 3) *reinterpret_cast<uint32_t*>(pp) = (uint32_t)f;
-      else if constexpr (S == 1) *reinterpret_cast<uint16_t*>(pp) = (uint16_t)f;
-      else *pp = (uint8_t)f;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) atomicAdd(&myhist[ex[j]], 1u);
-    } else {
-      // last elements of the tensor: missing ones contribute zero bits
-      // (cuda/kernels.cuh:92), and only ceil(rem*(S+1)/8) packed bytes exist.
-      uint64_t f = 0;
-      for (uint32_t j = 0; j < rem; ++j) {
-        uint32_t h = in[gi + j];
-        if (nm.bytes) h = nz_norm_div(h, nm.bytes[(gi + j) >> nm.log2n]);
-        nz_split_one<S>(h, ex[0], rp[0]);
-        exps[gi + j] = (uint8_t)ex[0];
-        uint32_t bit = j * (S + 1);
-        f |= (uint64_t)rp[0] << (8u * (bit >> 3) + (7u - S - (bit & 7u)));
-        atomicAdd(&myhist[ex[0]], 1u);
-      }
-      uint32_t nb = (rem * (S + 1) + 7) / 8;
-      for (uint32_t b = 0; b < nb; ++b) pp[b] = (uint8_t)(f >> (8 * b));
-    }
+  for (int j = 0; j < 8; ++j) {
+    uint32_t ex, rp;
+    nz_split_one<S>((w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu, ex, rp);
+    e |= (uint64_t)ex << (8 * j);
+    f |= (uint64_t)rp << nz_field_shift<S>(j);
   }
-  __syncthreads();
+}
 
-  // ---- quantise the histogram to 12-bit frequencies (sum exactly 4096) ----
+template <int S>
+__device__ __forceinline__ void nz_store_packed(uint8_t* pp, uint64_t f) {
+  if constexpr (S == 7) __builtin_nontemporal_store(f, reinterpret_cast<uint64_t*>(pp));
+  else if constexpr (S == 3) __builtin_nontemporal_store((uint32_t)f, reinterpret_cast<uint32_t*>(pp));
+  else if constexpr (S == 1) __builtin_nontemporal_store((uint16_t)f, reinterpret_cast<uint16_t*>(pp));
+  else __builtin_nontemporal_store((uint8_t)f, pp);
+}
+
+// The last elements of the tensor (fewer than 8 in this lane's group): missing
+// ones contribute zero bits (cuda/kernels.cuh:92), and only ceil(rem*(S+1)/8)
+// packed bytes exist.  -> the exponent bytes, zero above `rem`.
+template <int S>
+__device__ __forceinline__ uint64_t nz_split_tail(const uint16_t* __restrict__ in, uint64_t gi, uint32_t rem,
+                                                  uint8_t* pp, const NzNorm& nm) {
+  uint64_t e = 0, f = 0;
+  for (uint32_t j = 0; j < rem; ++j) {
+    uint32_t h = in[gi + j], ex, rp;
+    if (nm.bytes) h = nz_norm_div(h, nm.bytes[(gi + j) >> nm.log2n]);
+    nz_split_one<S>(h, ex, rp);
+    e |= (uint64_t)ex << (8 * j);
+    const uint32_t bit = j * (S + 1);
+    f |= (uint64_t)rp << (8u * (bit >> 3) + (7u - S - (bit & 7u)));
+  }
+  const uint32_t nb = (rem * (S + 1) + 7) / 8;
+  for (uint32_t b = 0; b < nb; ++b) pp[b] = (uint8_t)(f >> (8 * b));
+  return e;
+}
+
+// From the chunk's histogram (cn symbols): the 12-bit frequency table (sum
+// exactly 4096), the encoder's per-symbol entries in LDS, the serialized table
+// and the chunk record.  Run by the whole workgroup (at least 256 threads).
+__device__ __forceinline__ void nz_build_table(NzEncLds& L, const uint32_t cn, uint8_t* __restrict__ out,
+                                               NzChunkInfo* __restrict__ info_c) {
+  const uint32_t tid = threadIdx.x;
   // threads 0..255 own one symbol each; the others take part in the reductions
   // with neutral values
   const bool own = tid < 256;
   uint32_t cnt = 0;
   if (own) {
 #pragma unroll
-    for (uint32_t k = 0; k < NZ_HIST_COPIES; ++k) cnt += hist[k * NZ_HIST_STRIDE + tid];
+    for (uint32_t k = 0; k < NZ_HIST_COPIES; ++k) cnt += L.hist[k * NZ_HIST_STRIDE + tid];
   }
   const uint32_t live = cnt > 0;
-  const uint32_t k = nz_block_sum(live, red);
+  const uint32_t k = nz_block_sum(live, L.red);
   uint32_t f = live ? 1u + (uint32_t)(((uint64_t)cnt * (NZ_M - k)) / cn) : 0u;
-  const uint32_t sum = nz_block_sum(f, red);
+  const uint32_t sum = nz_block_sum(f, L.red);
   // most frequent symbol, lowest index on ties (cnt <= 2^24 fits above the index byte)
-  const uint32_t key = nz_block_max(own ? ((cnt << 8) | (255u - tid)) : 0u, red);
+  const uint32_t key = nz_block_max(own ? ((cnt << 8) | (255u - tid)) : 0u, L.red);
   const uint32_t imax = 255u - (key & 0xFFu);
   if (tid == imax) f += NZ_M - sum;
   if (k == 1) f = (tid == imax) ? (NZ_M - 1) : ((tid == (imax ^ 1u)) ? 1u : 0u);
@@ -415,29 +423,29 @@ __device__ __forceinline__ void nz_split_hist_body(
     uint32_t t = __shfl_up(incl, o, 64);
     if ((tid & 63) >= (uint32_t)o) incl += t;
   }
-  if (own && (tid & 63) == 63) scan_s[tid >> 6] = incl;
+  if (own && (tid & 63) == 63) L.scan_s[tid >> 6] = incl;
   __syncthreads();
   if (own) {
     uint32_t woff = 0;
-    for (uint32_t w = 0; w < (tid >> 6); ++w) woff += scan_s[w];
+    for (uint32_t w = 0; w < (tid >> 6); ++w) woff += L.scan_s[w];
     const uint32_t cum = woff + incl - f;
-    enc_tab[c * 256 + tid] = (f << 16) | cum;
+    L.tab[tid] = make_uint4(f << 20, f, cum, f ? __float_as_uint(1.0f / (float)f) - 4u : 0u);
   }
 
   // ---- serialise the table, in parallel ----
   // 256-bit live mask from the ballots of the four owning waves; the rank of a
   // live symbol is the number of live symbols below it.
   const uint64_t bal = __ballot(own && f != 0);
-  if (own && (tid & 63) == 0) mw[tid >> 6] = bal;
+  if (own && (tid & 63) == 0) L.mw[tid >> 6] = bal;
   __syncthreads();
-  const uint64_t m0 = mw[0], m1 = mw[1], m2 = mw[2], m3 = mw[3];
+  const uint64_t m0 = L.mw[0], m1 = L.mw[1], m2 = L.mw[2], m3 = L.mw[3];
   const uint32_t kk = (uint32_t)(__popcll(m0) + __popcll(m1) + __popcll(m2) + __popcll(m3));
   if (own && f != 0) {
     const uint32_t w = tid >> 6;
     const uint32_t below = (w > 0 ? (uint32_t)__popcll(m0) : 0u) + (w > 1 ? (uint32_t)__popcll(m1) : 0u) +
                            (w > 2 ? (uint32_t)__popcll(m2) : 0u) +
                            (uint32_t)__popcll(bal & ((1ull << (tid & 63)) - 1ull));
-    cf[below] = f;
+    L.cf[below] = f;
   }
   // a run starts at a live symbol whose predecessor is not live
   const uint64_t s0 = m0 & ~(m0 << 1);
@@ -447,13 +455,12 @@ __device__ __forceinline__ void nz_split_hist_body(
   const uint32_t runs = (uint32_t)(__popcll(s0) + __popcll(s1) + __popcll(s2) + __popcll(s3));
   const bool run_form = runs >= 1 && runs <= NZ_MAX_RUNS;
   const uint32_t head = run_form ? 1u + 2u * runs : 33u;
-  uint8_t* out = tab_ser + c * NZ_TABLE_MAX_BYTES;
   __syncthreads();
   // 12-bit fields, two per three bytes
-  for (uint32_t pj = tid; 2 * pj < kk; pj += NZ_SPLIT_THREADS) {
-    const uint32_t a = cf[2 * pj];
+  for (uint32_t pj = tid; 2 * pj < kk; pj += blockDim.x) {
+    const uint32_t a = L.cf[2 * pj];
     const bool two = 2 * pj + 1 < kk;
-    const uint32_t b = two ? cf[2 * pj + 1] : 0u;
+    const uint32_t b = two ? L.cf[2 * pj + 1] : 0u;
     uint8_t* fp = out + head + 3 * pj;
     fp[0] = (uint8_t)(a & 0xFF);
     fp[1] = (uint8_t)((a >> 8) | ((b & 0xF) << 4));
@@ -501,18 +508,20 @@ __device__ __forceinline__ void nz_split_hist_body(
     ci.pad_sym = imax;
     ci.raw = 0;
     ci.reserved = 0;
-    info[c] = ci;
+    *info_c = ci;
+    L.pad_sym = imax;
   }
+  __syncthreads();
 }
 
 // ----------------------------------------------------------------------------
 // per chunk: coded or raw, and the record size of each of its segments (run by one
 // thread of the encode kernel once all segments of the chunk are coded)
 // ----------------------------------------------------------------------------
-__device__ __forceinline__ void nz_chunk_finalize(uint64_t c, uint64_t n, uint32_t chunk_syms,
+__device__ __forceinline__ bool nz_chunk_finalize(uint64_t c, uint64_t n, uint32_t chunk_syms,
                                                   uint32_t seg_syms, uint32_t spc, NzChunkInfo* info,
                                                   const uint32_t* seg_words, const uint32_t* seg_state_bytes,
-                                                  uint32_t* seg_units) {
+                                                  uint32_t* seg_units, uint32_t* chunk_units) {
   const uint64_t base = c * chunk_syms;
   const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
   const uint32_t nseg = (cn + seg_syms - 1) / seg_syms;
@@ -526,6 +535,7 @@ __device__ __forceinline__ void nz_chunk_finalize(uint64_t c, uint64_t n, uint32
   }
   const bool raw = rans_total >= raw_total;
   info[c].raw = raw ? 1u : 0u;
+  uint32_t chunk_total = 0;  // a record has at most ~2^21 units, a chunk eight records
   for (uint32_t k = 0; k < nseg; ++k) {
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
     const uint32_t w = seg_words[c * spc + k];
@@ -535,11 +545,14 @@ __device__ __forceinline__ void nz_chunk_finalize(uint64_t c, uint64_t n, uint32
               (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
     else bytes = (k == 0 ? tab_len : 0u) + seg_state_bytes[c * spc + k] + 2u * ((w + 1) & ~1u);
     seg_units[c * spc + k] = bytes / 4;
+    chunk_total += bytes / 4;
   }
+  chunk_units[c] = chunk_total;
+  return raw;
 }
 
 // ----------------------------------------------------------------------------
-// rANS encode: one workgroup per chunk, one wavefront per segment
+// rANS encode of one segment by one wavefront
 // ----------------------------------------------------------------------------
 //
 // The 64 lanes run backwards over their symbols.  Per symbol: emit the low 16
@@ -547,94 +560,55 @@ __device__ __forceinline__ void nz_chunk_finalize(uint64_t c, uint64_t n, uint32
 // slot back to front, so that the decoder reads front to back), then
 // x = (x / f) << 12 | (x % f) + cum.  A segment's slot holds one word per
 // symbol, the most any input can emit, so there is no overflow path; a chunk
-// that codes to more than its raw size is stored raw (decided at the end of this
+// that codes to more than its raw size is stored raw (decided at the end of the
 // kernel, once all segments of the chunk are coded).
-__device__ __forceinline__ void nz_rans_encode_body(
-    const uint64_t c, const uint8_t* __restrict__ exps, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
-    uint32_t spc, const uint32_t* __restrict__ enc_tab, NzChunkInfo* __restrict__ info,
-    const uint16_t* __restrict__ carry, uint16_t* __restrict__ slots,
-    uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words,
-    uint32_t* __restrict__ seg_state_bytes, uint32_t* __restrict__ seg_units) {
-  __shared__ uint32_t sbuf[NZ_MAX_SEGS_PER_CHUNK][NZ_STATE_MAX_BYTES / 4];
-  // per symbol: x = freq << 20 (renormalisation threshold), y = freq, z = cum,
-  // w = bits of a float just below 1 / freq (four units in the last place
-  // under the correctly rounded quotient)
-  __shared__ uint4 tab[256];
-  for (uint32_t i = threadIdx.x; i < 256; i += blockDim.x) {
-    const uint32_t fc = enc_tab[c * 256 + i];
-    const uint32_t f = fc >> 16;
-    tab[i] = make_uint4(f << 20, f, fc & 0xFFFFu, f ? __float_as_uint(1.0f / (float)f) - 4u : 0u);
-  }
-  __syncthreads();
 
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t seg_syms = lane_syms * NZ_LANES;
-  const uint64_t seg = c * spc + wave;
-  const uint64_t seg_base = c * chunk_syms + (uint64_t)wave * seg_syms;
-  // wavefronts without a segment leave: their slots go to the next chunk's
-  // split phase, which then overlaps this chunk's coding
-  if (wave >= spc) return;
-  if (seg_base < n) {  // a wavefront beyond the tensor's end only takes part in the barrier below
-  const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, wave);
-  const uint32_t seg_n = (uint32_t)((n - seg_base) < nom ? (n - seg_base) : nom);
-  const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
-  const uint32_t cap_words = seg_syms;
-  const uint32_t pad = info[c].pad_sym;
-  uint16_t* slot = slots + seg * cap_words;
-  const uint8_t* src = exps + seg_base;
-
-  // a full segment starts from 2^16 | 16 carried bits of the packed stream
-  uint32_t x = NZ_L | (seg_n == nom ? (uint32_t)carry[seg * NZ_LANES + lane] : 0u);
-  uint32_t pos = cap_words;
-  for (uint32_t g = ngroups; g-- > 0;) {
-    const uint32_t idx0 = (g * NZ_LANES + lane) * NZ_GROUP;
-    uint64_t sy;
-    if (idx0 + 8 <= seg_n) {
-      sy = *reinterpret_cast<const uint64_t*>(src + idx0);
-    } else {
-      sy = 0;
-      for (int j = 0; j < 8; ++j) {
-        uint32_t b = (idx0 + j < seg_n) ? src[idx0 + j] : pad;
-        sy |= (uint64_t)b << (8 * j);
-      }
-    }
-    // the table entries do not depend on the state: fetch all eight up front
-    uint4 e[8];
+// the 8 symbols of one group (byte j of `sy` = symbol j), last symbol first
+__device__ __forceinline__ void nz_enc_group(uint32_t& x, uint32_t& pos, const uint64_t sy,
+                                             const uint4* __restrict__ tab, uint16_t* __restrict__ slot) {
+  // the table entries do not depend on the state: fetch four at a time, up front
 #pragma unroll
-    for (int j = 0; j < 8; ++j) e[j] = tab[(uint32_t)(sy >> (8 * j)) & 0xFFu];
+  for (int h = 1; h >= 0; --h) {
+  uint4 e[8];
 #pragma unroll
-    for (int j = 7; j >= 0; --j) {
-      const uint32_t f = e[j].y;
-      const bool need = x >= e[j].x;
-      const uint64_t m = __ballot(need);
-      pos -= (uint32_t)__popcll(m);
-      if (need)  // a 32-bit byte offset from the segment's slot: one add-shift for the address
-        *reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(slot) + ((pos + nz_rank_below(m)) << 1)) =
-            (uint16_t)(x & 0xFFFFu);
-      x = need ? (x >> 16) : x;
-      // x < f << 20 here, so the quotient x / f is below 2^20.  The float estimate
-      // x * r with r four units in the last place under 1 / f (itself within half
-      // a unit) never exceeds the quotient - the roundings of x and of the product
-      // add at most one unit each - and falls short of it by less than
-      // 2^20 * 11 * 2^-24 < 1: truncated it is the exact quotient or one less,
-      // and the remainder tells which.  With the exact quotient q the new state
-      // is (q << 12) + (x - q f) + cum = x + q (4096 - f) + cum.
-      uint32_t q = (uint32_t)((float)x * __uint_as_float(e[j].w));
-      q += (x - __umul24(q, f) >= f) ? 1u : 0u;
-      x = __umul24(q, NZ_M - f) + (x + e[j].z);
-    }
+  for (int j = 4 * h; j < 4 * h + 4; ++j) e[j] = tab[(uint32_t)(sy >> (8 * j)) & 0xFFu];
+#pragma unroll
+  for (int j = 4 * h + 3; j >= 4 * h; --j) {
+    const uint32_t f = e[j].y;
+    const bool need = x >= e[j].x;
+    const uint64_t m = __ballot(need);
+    pos -= (uint32_t)__popcll(m);
+    if (need)  // a 32-bit byte offset from the segment's slot: one add-shift for the address
+      *reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(slot) + ((pos + nz_rank_below(m)) << 1)) =
+          (uint16_t)(x & 0xFFFFu);
+    x = need ? (x >> 16) : x;
+    // x < f << 20 here, so the quotient x / f is below 2^20.  The float estimate
+    // x * r with r four units in the last place under 1 / f (itself within half
+    // a unit) never exceeds the quotient - the roundings of x and of the product
+    // add at most one unit each - and falls short of it by less than
+    // 2^20 * 11 * 2^-24 < 1: truncated it is the exact quotient or one less,
+    // and the remainder tells which.  With the exact quotient q the new state
+    // is (q << 12) + (x - q f) + cum = x + q (4096 - f) + cum.
+    uint32_t q = (uint32_t)((float)x * __uint_as_float(e[j].w));
+    q += (x - __umul24(q, f) >= f) ? 1u : 0u;
+    x = __umul24(q, NZ_M - f) + (x + e[j].z);
   }
-  // Final states, variable length: 64 two-bit codes (code c = 5 + c nibbles),
-  // then the states as a little-endian nibble stream in lane order.  A state
-  // is >= 2^16, so it takes 20..32 bits; a flat 32 would waste ~4 more per lane.
+  }
+}
+
+// Final states, variable length: 64 two-bit codes (code c = 5 + c nibbles),
+// then the states as a little-endian nibble stream in lane order.  A state
+// is >= 2^16, so it takes 20..32 bits; a flat 32 would waste ~4 more per lane.
+__device__ __forceinline__ void nz_enc_finish(const uint32_t x, const uint32_t words, const uint64_t seg,
+                                              uint32_t* __restrict__ sb, const uint32_t lane,
+                                              uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words,
+                                              uint32_t* __restrict__ seg_state_bytes) {
   const uint32_t code = (x >> 20 ? 1u : 0u) + (x >> 24 ? 1u : 0u) + (x >> 28 ? 1u : 0u);
   const uint32_t nn = 5u + code;
   const uint32_t incl = nz_wave_scan(nn, lane);
   const uint32_t at = incl - nn;  // nibble offset of this lane's field
   const uint32_t total = __builtin_amdgcn_readlane(incl, 63);
   const uint32_t sbytes = 16u + ((((total + 1u) >> 1) + 3u) & ~3u);
-  uint32_t* sb = sbuf[wave];
   for (uint32_t i = lane; i < NZ_STATE_MAX_BYTES / 4; i += 64) sb[i] = 0;
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
@@ -647,24 +621,13 @@ __device__ __forceinline__ void nz_rans_encode_body(
   uint32_t* sdst = states + seg * (NZ_STATE_MAX_BYTES / 4);
   for (uint32_t i = lane; i < sbytes / 4; i += 64) sdst[i] = sb[i];
   if (lane == 0) {
-    seg_words[seg] = cap_words - pos;
+    seg_words[seg] = words;
     seg_state_bytes[seg] = sbytes;
   }
-  }
-  // every segment of the chunk is coded: decide coded-or-raw and size the records
-  __syncthreads();
-  if (threadIdx.x == 0) nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units);
 }
 
-// ----------------------------------------------------------------------------
-// One workgroup of 1024 threads per chunk: split + histogram + table with all
-// sixteen wavefronts (bandwidth-bound), then the chunk's segments are coded by
-// one wavefront each (latency-bound) from the exponents the workgroup has just
-// written.  Workgroups of different chunks are in different phases at any
-// time, so the two kinds of work overlap on the chip.
-// ----------------------------------------------------------------------------
 // The tensors of one encode call ride in the kernel argument block (as the
-// items of a decode batch do): the grid of the split/encode kernel is the
+// items of a decode batch do): the grid of an encode kernel is the
 // concatenation of their chunks, that of the scan kernel one workgroup per
 // tensor, that of the compaction the concatenation of their segments.
 #define NZ_ENC_BATCH_MAX 16
@@ -672,14 +635,13 @@ struct NzEncItem {
   const uint16_t* in;   // dense input
   uint8_t* packed;      // stored sign|mantissa stream
   uint8_t* ws;          // this tensor's slice of the scratch; the offsets below are into it
-  uint8_t* hdr;         // where header and directory are built (g.rec_off bytes)
-  uint8_t* comp;        // where the records go (header and directory are copied there unless comp == hdr)
+  uint8_t* comp;        // the container: header, directory, records
   uint64_t comp_cap;    // capacity the container size is checked against
   uint64_t* d_total;    // container size
   uint32_t* d_status;   // bit 0: the container does not fit
   NzNorm nm;            // normalizer bytes (nullptr: none)
   NzGeom g;
-  uint64_t exps, enc_tab, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units;
+  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units;
   uint32_t chunk_end, seg_end;  // running totals over the batch
 };
 struct NzEncBatch {
@@ -687,100 +649,350 @@ struct NzEncBatch {
   NzEncItem item[NZ_ENC_BATCH_MAX];
 };
 
-template <int S>
-__global__ __launch_bounds__(NZ_SPLIT_THREADS) void nz_split_encode_kernel(const NzEncBatch b) {
+// Segments of up to 8 * NG symbols per lane: the exponents stay in registers.
+// Workgroup = max(4, segments per chunk) wavefronts; wavefront k owns segment k.
+template <int S, int NG>
+__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kernel(const NzEncBatch b) {
+  __shared__ NzEncLds L;
   uint32_t t = 0, first = 0;
   while (t + 1 < b.count && blockIdx.x >= b.item[t].chunk_end) {
     first = b.item[t].chunk_end;
     ++t;
   }
   const NzEncItem& it = b.item[t];
-  const uint64_t c = blockIdx.x - first;
   const NzGeom& g = it.g;
-  uint8_t* carry = it.ws + it.carry;
-  uint8_t* exps = it.ws + it.exps;
-  uint32_t* enc_tab = reinterpret_cast<uint32_t*>(it.ws + it.enc_tab);
+  const uint64_t c = blockIdx.x - first;
+  const uint64_t n = g.n;
+  const uint32_t chunk_syms = g.chunk_syms, seg_syms = g.seg_syms, spc = g.spc;
+  const uint16_t* __restrict__ in = it.in;
+  const NzNorm nm = it.nm;
   NzChunkInfo* info = reinterpret_cast<NzChunkInfo*>(it.ws + it.info);
-  nz_split_hist_body<S>(c, it.in, g.n, g.chunk_syms, g.seg_syms, g.spc, it.packed, carry, exps, enc_tab,
-                        it.ws + it.tab_ser, info, it.nm);
-  // exponents, table, carried bytes and chunk info of this chunk are read back below
+  uint32_t* seg_words = reinterpret_cast<uint32_t*>(it.ws + it.seg_words);
+  uint32_t* seg_state_bytes = reinterpret_cast<uint32_t*>(it.ws + it.seg_sbytes);
+  uint32_t* seg_units = reinterpret_cast<uint32_t*>(it.ws + it.seg_units);
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t lane = tid & 63;
+  const uint64_t base = c * chunk_syms;
+  const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
+  const uint64_t seg = c * spc + wave;
+  const uint64_t seg_base = base + (uint64_t)wave * seg_syms;
+  const bool has_seg = wave < spc && seg_base < n;
+  const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, wave < spc ? wave : 0u);
+  const uint32_t seg_n = has_seg ? (uint32_t)((n - seg_base) < nom ? (n - seg_base) : nom) : 0u;
+  const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;  // at most NG
+  const bool seg_full = has_seg && seg_n == nom;
+
+  for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += blockDim.x) L.hist[i] = 0;
+  __syncthreads();
+  uint32_t* myhist = L.hist + (lane & (NZ_HIST_COPIES - 1)) * NZ_HIST_STRIDE;
+
+  // ---- phase 1: split.  Packed bytes go to the stored layout: segment k of a
+  // chunk starts at k * seg_keep, and the last NZ_CARRY_BYTES of a full segment
+  // go to carry[seg] instead (they ride in the rANS start states).
+  const uint32_t seg_keep = seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES;  // of a segment of nominal length
+  const uint64_t chunk_keep = (uint64_t)chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * spc;
+  const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
+  uint8_t* pk = it.packed + c * chunk_keep + (uint64_t)wave * seg_keep;
+  uint8_t* carry_seg = it.ws + it.carry + seg * NZ_CARRY_BYTES;
+  const uint32_t whole = seg_n / NZ_GROUP_SYMS;  // groups in which every lane has 8 elements
+  uint64_t ex[NG];
+  const auto dest = [&](uint32_t g8) {  // where the packed bytes of this lane's group g8 go
+    const uint32_t sb = (g8 * NZ_LANES + lane) * (S + 1);
+    return (seg_full && sb >= keep) ? carry_seg + (sb - keep) : pk + sb;
+  };
+  const auto count8 = [&](uint64_t e) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) atomicAdd(&myhist[(uint32_t)(e >> (8 * j)) & 0xFFu], 1u);
+  };
+  typedef uint32_t nz_u32x4 __attribute__((ext_vector_type(4)));
+  nz_static_for<0, NG, 4>([&](auto g4c) {
+    constexpr int g4 = decltype(g4c)::value;
+    // the group number as a run-time value for all address arithmetic: with
+    // constants the compiler precomputes the addresses of all groups up front
+    // and runs out of registers; ex[] keeps its compile-time index
+    uint32_t gv = (uint32_t)g4;
+    asm volatile("" : "+s"(gv));
+    if (gv + 4 <= whole) {
+      // four groups at a time: their loads are in flight together
+      const uint16_t* src = in + seg_base + (gv * NZ_LANES + lane) * NZ_GROUP;
+      uint4 v[4];
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const nz_u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const nz_u32x4*>(src + q * NZ_GROUP_SYMS));
+        v[q] = make_uint4(r.x, r.y, r.z, r.w);
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (nm.bytes)
+          v[q] = nz_scale8<false>(v[q], nz_norm_load8(nm, seg_base + ((gv + q) * NZ_LANES + lane) * NZ_GROUP),
+                                  nm.log2n >= 3);
+        uint64_t f;
+        nz_split_group<S>(v[q], ex[g4 + q], f);
+        nz_store_packed<S>(dest(gv + q), f);
+        count8(ex[g4 + q]);
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t g8 = gv + q;
+        ex[g4 + q] = 0;
+        if (g8 < ngroups) {
+          const uint32_t idx0 = (g8 * NZ_LANES + lane) * NZ_GROUP;
+          const uint64_t gi = seg_base + idx0;
+          if (idx0 + 8 <= seg_n) {
+            uint4 v = *reinterpret_cast<const uint4*>(in + gi);
+            if (nm.bytes) v = nz_scale8<false>(v, nz_norm_load8(nm, gi), nm.log2n >= 3);
+            uint64_t f;
+            nz_split_group<S>(v, ex[g4 + q], f);
+            nz_store_packed<S>(dest(g8), f);
+            count8(ex[g4 + q]);
+          } else if (idx0 < seg_n) {
+            const uint32_t rem = seg_n - idx0;
+            ex[g4 + q] = nz_split_tail<S>(in, gi, rem, dest(g8), nm);
+            for (uint32_t j = 0; j < rem; ++j) atomicAdd(&myhist[(uint32_t)(ex[g4 + q] >> (8 * j)) & 0xFFu], 1u);
+          }
+        }
+      }
+    }
+  });
+  __threadfence_block();  // the carried bytes are read back below
+  __syncthreads();
+
+  // ---- the chunk's table ----
+  nz_build_table(L, cn, it.ws + it.tab_ser + c * NZ_TABLE_MAX_BYTES, info + c);
+
+  // ---- phase 2: code the segment from the registers, last group first ----
+  const uint32_t cap_words = seg_syms;
+  uint16_t* slot = reinterpret_cast<uint16_t*>(it.ws + it.slots) + seg * cap_words;
+  if (has_seg) {
+    const uint32_t pad = L.pad_sym;
+    // a full segment starts from 2^16 | 16 carried bits of the packed stream
+    uint32_t x = NZ_L | (seg_full ? (uint32_t)reinterpret_cast<const uint16_t*>(carry_seg)[lane] : 0u);
+    uint32_t pos = cap_words;
+    nz_static_for<NG - 1, 0, -1>([&](auto g8c) {
+      constexpr int g8 = decltype(g8c)::value;
+      uint32_t gv = (uint32_t)g8;
+      asm volatile("" : "+s"(gv));
+      if (gv < ngroups) {
+        uint64_t sy = ex[g8];
+        if (gv >= whole) {  // the tensor ends inside this group: the most frequent symbol stands in
+          const uint32_t idx0 = (gv * NZ_LANES + lane) * NZ_GROUP;
+          const uint32_t have = idx0 < seg_n ? seg_n - idx0 : 0u;  // < 8 in some lane
+          if (have < 8) {
+            const uint64_t keepm = have ? (~0ull >> (64 - 8 * have)) : 0ull;
+            sy = (sy & keepm) | ((0x0101010101010101ull * pad) & ~keepm);
+          }
+        }
+        nz_enc_group(x, pos, sy, L.tab, slot);
+      }
+    });
+    nz_enc_finish(x, cap_words - pos, seg, L.sbuf[wave], lane, reinterpret_cast<uint32_t*>(it.ws + it.states),
+                  seg_words, seg_state_bytes);
+  }
+  // every segment of the chunk is coded: decide coded-or-raw and size the records
   __threadfence_block();
   __syncthreads();
-  nz_rans_encode_body(c, exps, g.n, g.chunk_syms, g.lane_syms, g.spc, enc_tab, info,
-                      reinterpret_cast<const uint16_t*>(carry), reinterpret_cast<uint16_t*>(it.ws + it.slots),
-                      reinterpret_cast<uint32_t*>(it.ws + it.states),
-                      reinterpret_cast<uint32_t*>(it.ws + it.seg_words),
-                      reinterpret_cast<uint32_t*>(it.ws + it.seg_sbytes),
-                      reinterpret_cast<uint32_t*>(it.ws + it.seg_units));
+  if (tid == 0) L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
+                                          reinterpret_cast<uint32_t*>(it.ws + it.chunk_units));
+  __syncthreads();
+  if (L.raw && has_seg) {
+    // a chunk that does not compress: its exponent bytes take the place of the words
+    uint8_t* rawp = reinterpret_cast<uint8_t*>(slot);
+    nz_static_for<0, NG, 1>([&](auto g8c) {
+      constexpr int g8 = decltype(g8c)::value;
+      uint32_t gv = (uint32_t)g8;
+      asm volatile("" : "+s"(gv));
+      const uint32_t idx0 = (gv * NZ_LANES + lane) * NZ_GROUP;
+      if (idx0 < seg_n) *reinterpret_cast<uint64_t*>(rawp + idx0) = ex[g8];
+    });
+  }
+}
+
+// Longer segments: all wavefronts split the chunk into scratch, then one
+// wavefront per segment codes from there.
+template <int S>
+__global__ __launch_bounds__(NZ_ENC_LONG_THREADS) void nz_encode_long_kernel(const NzEncBatch b) {
+  __shared__ NzEncLds L;
+  uint32_t t = 0, first = 0;
+  while (t + 1 < b.count && blockIdx.x >= b.item[t].chunk_end) {
+    first = b.item[t].chunk_end;
+    ++t;
+  }
+  const NzEncItem& it = b.item[t];
+  const NzGeom& g = it.g;
+  const uint64_t c = blockIdx.x - first;
+  const uint64_t n = g.n;
+  const uint32_t chunk_syms = g.chunk_syms, seg_syms = g.seg_syms, spc = g.spc;
+  const uint16_t* __restrict__ in = it.in;
+  const NzNorm nm = it.nm;
+  uint8_t* carry = it.ws + it.carry;
+  uint8_t* exps = it.ws + it.exps;
+  NzChunkInfo* info = reinterpret_cast<NzChunkInfo*>(it.ws + it.info);
+  uint32_t* seg_words = reinterpret_cast<uint32_t*>(it.ws + it.seg_words);
+  uint32_t* seg_state_bytes = reinterpret_cast<uint32_t*>(it.ws + it.seg_sbytes);
+  uint32_t* seg_units = reinterpret_cast<uint32_t*>(it.ws + it.seg_units);
+
+  const uint32_t tid = threadIdx.x;
+  const uint64_t base = c * chunk_syms;
+  const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
+
+  for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += blockDim.x) L.hist[i] = 0;
+  __syncthreads();
+  uint32_t* myhist = L.hist + (tid & (NZ_HIST_COPIES - 1)) * NZ_HIST_STRIDE;
+
+  const uint32_t seg_keep = seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES;     // of a segment of nominal length
+  const uint64_t chunk_keep = (uint64_t)chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * spc;
+  const uint64_t seg0 = c * spc;
+  for (uint32_t i = tid * 8; i < cn; i += blockDim.x * 8) {
+    const uint64_t gi = base + i;
+    const uint32_t sk = i / seg_syms;                       // segment inside the chunk
+    const uint32_t sb = (i - sk * seg_syms) / 8 * (S + 1);  // byte inside the segment
+    const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, sk);
+    const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
+    const bool seg_full = base + (uint64_t)sk * seg_syms + nom <= n;
+    uint8_t* pp = (seg_full && sb >= keep) ? carry + (seg0 + sk) * NZ_CARRY_BYTES + (sb - keep)
+                                           : it.packed + c * chunk_keep + (uint64_t)sk * seg_keep + sb;
+    const uint32_t rem = cn - i;
+    uint64_t e;
+    if (rem >= 8) {
+      uint4 v = *reinterpret_cast<const uint4*>(in + gi);
+      if (nm.bytes) v = nz_scale8<false>(v, nz_norm_load8(nm, gi), nm.log2n >= 3);
+      uint64_t f;
+      nz_split_group<S>(v, e, f);
+      nz_store_packed<S>(pp, f);
+      *reinterpret_cast<uint64_t*>(exps + gi) = e;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) atomicAdd(&myhist[(uint32_t)(e >> (8 * j)) & 0xFFu], 1u);
+    } else {
+      e = nz_split_tail<S>(in, gi, rem, pp, nm);
+      for (uint32_t j = 0; j < rem; ++j) {
+        exps[gi + j] = (uint8_t)(e >> (8 * j));
+        atomicAdd(&myhist[(uint32_t)(e >> (8 * j)) & 0xFFu], 1u);
+      }
+    }
+  }
+  __syncthreads();
+  nz_build_table(L, cn, it.ws + it.tab_ser + c * NZ_TABLE_MAX_BYTES, info + c);
+  // exponents and carried bytes of this chunk are read back below
+  __threadfence_block();
+  __syncthreads();
+
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t lane = tid & 63;
+  const uint64_t seg = seg0 + wave;
+  const uint64_t seg_base = base + (uint64_t)wave * seg_syms;
+  const uint32_t cap_words = seg_syms;
+  uint16_t* slot = reinterpret_cast<uint16_t*>(it.ws + it.slots) + seg * cap_words;
+  const bool has_seg = wave < spc && seg_base < n;
+  uint32_t seg_n = 0;
+  if (has_seg) {
+    const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, wave);
+    seg_n = (uint32_t)((n - seg_base) < nom ? (n - seg_base) : nom);
+    const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
+    const uint32_t pad = L.pad_sym;
+    const uint8_t* src = exps + seg_base;
+    uint32_t x = NZ_L | (seg_n == nom ? (uint32_t)reinterpret_cast<const uint16_t*>(carry)[seg * NZ_LANES + lane] : 0u);
+    uint32_t pos = cap_words;
+    for (uint32_t gq = ngroups; gq-- > 0;) {
+      const uint32_t idx0 = (gq * NZ_LANES + lane) * NZ_GROUP;
+      uint64_t sy;
+      if (idx0 + 8 <= seg_n) {
+        sy = *reinterpret_cast<const uint64_t*>(src + idx0);
+      } else {
+        sy = 0;
+        for (int j = 0; j < 8; ++j) {
+          uint32_t bb = (idx0 + j < seg_n) ? src[idx0 + j] : pad;
+          sy |= (uint64_t)bb << (8 * j);
+        }
+      }
+      nz_enc_group(x, pos, sy, L.tab, slot);
+    }
+    nz_enc_finish(x, cap_words - pos, seg, L.sbuf[wave], lane, reinterpret_cast<uint32_t*>(it.ws + it.states),
+                  seg_words, seg_state_bytes);
+  }
+  __threadfence_block();
+  __syncthreads();
+  if (tid == 0) L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
+                                          reinterpret_cast<uint32_t*>(it.ws + it.chunk_units));
+  __syncthreads();
+  if (L.raw && has_seg) {
+    // a chunk that does not compress: its exponent bytes take the place of the words
+    uint8_t* rawp = reinterpret_cast<uint8_t*>(slot);
+    const uint8_t* src = exps + seg_base;
+    for (uint32_t i = lane; i < seg_n; i += 64) rawp[i] = src[i];
+  }
 }
 
 // ----------------------------------------------------------------------------
-// exclusive scan of the record sizes -> directory, header, total size
-// (a single workgroup per tensor; a tensor has at most a few hundred thousand segments)
+// container size, header
 // ----------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void nz_scan_kernel(const NzEncBatch b) {
-  // one workgroup per tensor; header and directory go to `hdr` (g.rec_off
-  // bytes), the records are placed by nz_compact_kernel, possibly in another
-  // buffer
+
+// sum of v over the 256 threads of the workgroup, in every thread
+__device__ __forceinline__ uint64_t nz_block_sum64(uint64_t v, uint64_t* red4) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor((unsigned long long)v, o, 64);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red4[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return red4[0] + red4[1] + red4[2] + red4[3];
+}
+
+__device__ __forceinline__ void nz_write_header(uint8_t* comp, const NzGeom& g, uint64_t total) {
+  uint32_t* h = reinterpret_cast<uint32_t*>(comp);
+  h[0] = NZ_MAGIC;
+  h[1] = NZ_FORMAT_VERSION;
+  h[2] = (uint32_t)(g.n & 0xFFFFFFFFu);
+  h[3] = (uint32_t)(g.n >> 32);
+  h[4] = g.chunk_syms;
+  h[5] = g.lane_syms;
+  h[6] = (uint32_t)g.n_chunks;
+  h[7] = (uint32_t)g.n_segs;
+  h[8] = (uint32_t)g.dir_off;
+  h[9] = (uint32_t)g.rec_off;
+  h[10] = (uint32_t)(total & 0xFFFFFFFFu);
+  h[11] = (uint32_t)(total >> 32);
+  h[12] = h[13] = h[14] = h[15] = 0;
+  // the alignment gap between directory and records
+  for (uint64_t b = g.dir_off + 4 * (g.n_segs + 1); b < g.rec_off; ++b) comp[b] = 0;
+}
+
+// Container size of every tensor of the batch from the record sizes of its
+// chunks (one workgroup of 256 threads per tensor): for a caller that wants the
+// size before it provides the container's memory.  A tensor without elements
+// has no compaction workgroup: its (header-only) container is written here
+// when `comp` is known.
+__global__ __launch_bounds__(256) void nz_total_kernel(const NzEncBatch b) {
+  __shared__ uint64_t red4[4];
   const NzEncItem& it = b.item[blockIdx.x];
   const NzGeom& g = it.g;
-  const uint32_t* __restrict__ seg_units = reinterpret_cast<const uint32_t*>(it.ws + it.seg_units);
-  uint8_t* __restrict__ comp = it.hdr;
-  const uint64_t cap = it.comp_cap;
-  uint64_t* __restrict__ d_total = it.d_total;
-  uint32_t* __restrict__ d_status = it.d_status;
-  __shared__ uint64_t wsum[16];
-  __shared__ uint64_t carry_s;
-  uint32_t* dir = reinterpret_cast<uint32_t*>(comp + g.dir_off);
-  const uint32_t tid = threadIdx.x;
-  if (tid == 0) carry_s = 0;
-  __syncthreads();
-  for (uint64_t start = 0; start < g.n_segs; start += 1024) {
-    const uint64_t i = start + tid;
-    const uint64_t v = i < g.n_segs ? seg_units[i] : 0;
-    // a record has at most ~2^21 units (a segment has at most 2^22 symbols), so
-    // the sum over a wavefront fits 32 bits; across wavefronts it is kept in 64
-    const uint64_t incl = nz_wave_scan((uint32_t)v, tid & 63);
-    if ((tid & 63) == 63) wsum[tid >> 6] = incl;
-    __syncthreads();
-    uint64_t woff = carry_s;
-    for (uint32_t w = 0; w < (tid >> 6); ++w) woff += wsum[w];
-    if (i < g.n_segs) dir[i] = (uint32_t)(woff + incl - v);
-    __syncthreads();
-    if (tid == 1023) carry_s = woff + incl;
-    __syncthreads();
-  }
-  if (tid == 0) {
-    const uint64_t units = carry_s;
-    dir[g.n_segs] = (uint32_t)units;
-    // zero the alignment gap between directory and records
-    for (uint64_t b = g.dir_off + 4 * (g.n_segs + 1); b < g.rec_off; ++b) comp[b] = 0;
+  const uint32_t* __restrict__ chunk_units = reinterpret_cast<const uint32_t*>(it.ws + it.chunk_units);
+  uint64_t part = 0;
+  for (uint64_t i = threadIdx.x; i < g.n_chunks; i += 256) part += chunk_units[i];
+  const uint64_t units = nz_block_sum64(part, red4);
+  if (threadIdx.x == 0) {
     const uint64_t total = g.rec_off + 4 * units + NZ_TAIL_PAD;
-    if (g.n_segs == 0)  // otherwise the last segment's compaction writes the closing zeros
-      for (uint32_t b = 0; b < NZ_TAIL_PAD; ++b) comp[g.rec_off + b] = 0;
-    uint32_t* h = reinterpret_cast<uint32_t*>(comp);
-    h[0] = NZ_MAGIC;
-    h[1] = NZ_FORMAT_VERSION;
-    h[2] = (uint32_t)(g.n & 0xFFFFFFFFu);
-    h[3] = (uint32_t)(g.n >> 32);
-    h[4] = g.chunk_syms;
-    h[5] = g.lane_syms;
-    h[6] = (uint32_t)g.n_chunks;
-    h[7] = (uint32_t)g.n_segs;
-    h[8] = (uint32_t)g.dir_off;
-    h[9] = (uint32_t)g.rec_off;
-    h[10] = (uint32_t)(total & 0xFFFFFFFFu);
-    h[11] = (uint32_t)(total >> 32);
-    h[12] = h[13] = h[14] = h[15] = 0;
-    *d_total = total;
-    if (total > cap || units > 0xFFFFFFFFull) atomicOr(d_status, 1u);
+    *it.d_total = total;
+    if (total > it.comp_cap || units > 0xFFFFFFFFull) atomicOr(it.d_status, 1u);
+    if (g.n_segs == 0 && it.comp && total <= it.comp_cap) {
+      nz_write_header(it.comp, g, total);
+      reinterpret_cast<uint32_t*>(it.comp + g.dir_off)[0] = 0;
+      for (uint32_t q = 0; q < NZ_TAIL_PAD; ++q) it.comp[g.rec_off + q] = 0;
+    }
   }
 }
 
 // ----------------------------------------------------------------------------
 // move every segment record to its final place: one workgroup per segment
 // ----------------------------------------------------------------------------
+// The workgroup of segment k of chunk c finds where its record goes by itself:
+// the record sizes of all chunks before c (one number per chunk, left by the
+// encode kernel) plus those of the segments before k in c.  It writes its own
+// directory entry; the workgroup of the last segment adds the closing entry,
+// the header, the container size and the overflow flag.
 __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
+  __shared__ uint64_t red4[4];
   uint32_t t = 0, first = 0;
   while (t + 1 < b.count && blockIdx.x >= b.item[t].seg_end) {
     first = b.item[t].seg_end;
@@ -788,7 +1000,6 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   }
   const NzEncItem& it = b.item[t];
   const NzGeom& g = it.g;
-  const uint8_t* __restrict__ exps = it.ws + it.exps;
   const NzChunkInfo* __restrict__ info = reinterpret_cast<const NzChunkInfo*>(it.ws + it.info);
   const uint8_t* __restrict__ tab_ser = it.ws + it.tab_ser;
   const uint8_t* __restrict__ carry = it.ws + it.carry;
@@ -796,31 +1007,43 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   const uint32_t* __restrict__ states = reinterpret_cast<const uint32_t*>(it.ws + it.states);
   const uint32_t* __restrict__ seg_words = reinterpret_cast<const uint32_t*>(it.ws + it.seg_words);
   const uint32_t* __restrict__ seg_state_bytes = reinterpret_cast<const uint32_t*>(it.ws + it.seg_sbytes);
-  const uint32_t* __restrict__ dir = reinterpret_cast<const uint32_t*>(it.hdr + g.dir_off);
+  const uint32_t* __restrict__ seg_units = reinterpret_cast<const uint32_t*>(it.ws + it.seg_units);
+  const uint32_t* __restrict__ chunk_units = reinterpret_cast<const uint32_t*>(it.ws + it.chunk_units);
   uint8_t* __restrict__ comp = it.comp;
   const uint64_t cap = it.comp_cap;
   const uint64_t seg = blockIdx.x - first;
-  // header and directory were built elsewhere: every workgroup moves a share
-  if (it.hdr != it.comp && g.rec_off <= cap) {
-    const uint32_t* hs = reinterpret_cast<const uint32_t*>(it.hdr);
-    uint32_t* hd = reinterpret_cast<uint32_t*>(comp);
-    for (uint64_t i = seg * 256 + threadIdx.x; i < g.rec_off / 4; i += g.n_segs * 256) hd[i] = hs[i];
-  }
   const uint64_t c = seg / g.spc;
   const uint32_t k = (uint32_t)(seg - c * g.spc);
+  const uint32_t tid = threadIdx.x;
   // everything the move depends on is fetched at once: one round of memory latency
-  const uint64_t o0 = dir[seg], o1 = dir[seg + 1];
+  uint64_t part = 0;
+  for (uint64_t i = tid; i < c; i += 256) part += chunk_units[i];
+  if (tid < k) part += seg_units[c * g.spc + tid];
+  const uint32_t mine = seg_units[seg];
   const NzChunkInfo ci = info[c];
   const uint32_t sbytes = seg_state_bytes[seg];
   const uint32_t w = seg_words[seg];
-  if (g.rec_off + 4 * o1 + NZ_TAIL_PAD > cap) return;  // flagged by the scan kernel
+  const uint64_t o0 = nz_block_sum64(part, red4), o1 = o0 + mine;
+  const bool fits = o1 <= 0xFFFFFFFFull && g.rec_off + 4 * o1 + NZ_TAIL_PAD <= cap;
+  if (seg + 1 == g.n_segs && tid == 0) {
+    const uint64_t total = g.rec_off + 4 * o1 + NZ_TAIL_PAD;
+    *it.d_total = total;
+    if (!fits) atomicOr(it.d_status, 1u);
+  }
+  if (!fits) return;  // (a record before this one may still fit and be written: harmless)
+  uint32_t* dir = reinterpret_cast<uint32_t*>(comp + g.dir_off);
+  if (tid == 0) dir[seg] = (uint32_t)o0;
   uint8_t* dst = comp + g.rec_off + 4 * o0;
-  if (seg + 1 == g.n_segs && threadIdx.x >= 256 - NZ_TAIL_PAD)  // closing zeros
-    comp[g.rec_off + 4 * o1 + (threadIdx.x - (256 - NZ_TAIL_PAD))] = 0;
+  if (seg + 1 == g.n_segs) {
+    if (tid == 0) {
+      dir[g.n_segs] = (uint32_t)o1;
+      nz_write_header(comp, g, g.rec_off + 4 * o1 + NZ_TAIL_PAD);
+    }
+    if (tid >= 256 - NZ_TAIL_PAD) comp[g.rec_off + 4 * o1 + (tid - (256 - NZ_TAIL_PAD))] = 0;  // closing zeros
+  }
   const uint64_t seg_base = c * g.chunk_syms + (uint64_t)k * g.seg_syms;
   const uint32_t nom = nz_seg_nominal(g.chunk_syms, g.seg_syms, g.spc, k);
   const uint32_t sn = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
-  const uint32_t tid = threadIdx.x;
   if (ci.raw) {
     uint32_t off = 0;
     if (k == 0) {
@@ -828,7 +1051,8 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
       off = 4;
     }
     const uint32_t padded = (sn + 3) & ~3u;
-    for (uint32_t i = tid; i < padded; i += 256) dst[off + i] = i < sn ? exps[seg_base + i] : 0;
+    const uint8_t* rawp = reinterpret_cast<const uint8_t*>(slots + seg * g.seg_syms);  // left there by the encode kernel
+    for (uint32_t i = tid; i < padded; i += 256) dst[off + i] = i < sn ? rawp[i] : 0;
     if (sn == nom && tid < NZ_CARRY_BYTES) dst[off + padded + tid] = carry[seg * NZ_CARRY_BYTES + tid];
     return;
   }
