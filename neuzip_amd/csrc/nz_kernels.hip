@@ -349,18 +349,39 @@ struct NzEncLds {
   uint32_t pad_sym, raw;
 };
 
-// Split one element group: 8 bf16 values -> 8 exponent bytes and the S+1 packed bytes.
+// Split one element group: 8 bf16 values -> 8 exponent bytes (byte j of `e` =
+// element j) and the S+1 packed bytes (`f`, little-endian).  Two elements at a
+// time, both halves of a dword in parallel: the rounding add cannot carry
+// from the low half into the high one (0x7FFF + 2^(6-S) < 2^16), so the closed
+// form of nz_split_one holds for both halves at once.
 template <int S>
 __device__ __forceinline__ void nz_split_group(const uint4 v, uint64_t& e, uint64_t& f) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-  e = 0;
-  f = 0;
+  uint32_t t[4], p[4];  // per dword: exponents in bytes 0 and 2 | the two (S+1)-bit fields, first element on top
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    uint32_t ex, rp;
-    nz_split_one<S>((w[j >> 1] >> (16 * (j & 1))) & 0xFFFFu, ex, rp);
-    e |= (uint64_t)ex << (8 * j);
-    f |= (uint64_t)rp << nz_field_shift<S>(j);
+  for (int k = 0; k < 4; ++k) {
+    if constexpr (S == 7) {
+      t[k] = (w[k] >> 7) & 0x00FF00FFu;
+      p[k] = ((w[k] >> 8) & 0x00800080u) | (w[k] & 0x007F007Fu);  // sign | mantissa in bytes 0 and 2
+    } else {
+      const uint32_t a = ((w[k] & 0x7FFF7FFFu) + (0x00010001u << (6 - S))) & 0x7FFF7FFFu;
+      t[k] = (a >> 7) & 0x00FF00FFu;
+      const uint32_t fld = ((w[k] >> (15 - S)) & (0x00010001u << S)) | ((a >> (7 - S)) & (0x00010001u * ((1u << S) - 1u)));
+      p[k] = ((fld << (S + 1)) | (fld >> 16)) & ((1u << (2 * S + 2)) - 1u);
+    }
+  }
+  // bytes 0 and 2 of two dwords -> four consecutive bytes
+  const uint32_t e_lo = __builtin_amdgcn_perm(t[1], t[0], 0x06040200u), e_hi = __builtin_amdgcn_perm(t[3], t[2], 0x06040200u);
+  e = ((uint64_t)e_hi << 32) | e_lo;
+  if constexpr (S == 7) {
+    const uint32_t f_lo = __builtin_amdgcn_perm(p[1], p[0], 0x06040200u), f_hi = __builtin_amdgcn_perm(p[3], p[2], 0x06040200u);
+    f = ((uint64_t)f_hi << 32) | f_lo;
+  } else if constexpr (S == 3) {
+    f = p[0] | (p[1] << 8) | (p[2] << 16) | (p[3] << 24);  // one byte per pair of elements
+  } else if constexpr (S == 1) {
+    f = ((p[0] << 4) | p[1]) | (((p[2] << 4) | p[3]) << 8);  // one nibble per pair
+  } else {
+    f = (p[0] << 6) | (p[1] << 4) | (p[2] << 2) | p[3];      // two bits per pair, element 0 on top
   }
 }
 
