@@ -728,6 +728,18 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     for (int j = 0; j < 8; ++j) atomicAdd(&myhist[(uint32_t)(e >> (8 * j)) & 0xFFu], 1u);
   };
   typedef uint32_t nz_u32x4 __attribute__((ext_vector_type(4)));
+  // Four groups at a time, and the loads of the next four are issued before the
+  // current four are split: eight 16-byte loads per lane in flight.
+  uint4 vn[4];  // the block after the current one
+  const auto load4 = [&](uint32_t gv) {
+    const uint16_t* src = in + seg_base + (gv * NZ_LANES + lane) * NZ_GROUP;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const nz_u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const nz_u32x4*>(src + q * NZ_GROUP_SYMS));
+      vn[q] = make_uint4(r.x, r.y, r.z, r.w);
+    }
+  };
+  if (4 <= whole) load4(0);
   nz_static_for<0, NG, 4>([&](auto g4c) {
     constexpr int g4 = decltype(g4c)::value;
     // the group number as a run-time value for all address arithmetic: with
@@ -736,14 +748,10 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     uint32_t gv = (uint32_t)g4;
     asm volatile("" : "+s"(gv));
     if (gv + 4 <= whole) {
-      // four groups at a time: their loads are in flight together
-      const uint16_t* src = in + seg_base + (gv * NZ_LANES + lane) * NZ_GROUP;
       uint4 v[4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const nz_u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const nz_u32x4*>(src + q * NZ_GROUP_SYMS));
-        v[q] = make_uint4(r.x, r.y, r.z, r.w);
-      }
+      for (int q = 0; q < 4; ++q) v[q] = vn[q];
+      if (gv + 8 <= whole) load4(gv + 4);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         if (nm.bytes)
