@@ -47,10 +47,10 @@ extern "C" {
 /* The library's own geometry (chunk_size 0): tables shared by 128 Ki elements,
    eight wavefronts of 256 symbols per lane each.  The reference hands nvcomp
    chunks of 64 Ki (cuda/neuzip.cu:31); that size is honoured when asked for,
-   its best segment length being 344 (22016 + 22016 + 21504 elements). */
+   cut into four segments of 256 symbols per lane. */
 #define NZ_DEFAULT_CHUNK 131072u
 #define NZ_DEFAULT_LANE_SYMS 256u
-#define NZ_LANE_SYMS_64K 344u
+#define NZ_LANE_SYMS_64K 256u
 #define NZ_LANE_SYMS_AUTO 0xFFFFFFFFu /* nz_manager_create: choose per tensor */
 
 typedef struct nz_manager nz_manager;
@@ -174,19 +174,32 @@ void nz_manager_destroy(nz_manager* m);
 
 /* Manager::write(name, tensor), cuda/high_level.cu:132-162.  Replaces an
    existing entry of the same name (:137-140).  Synchronises the stream once
-   to learn the compressed size (as the reference does, :114-115). */
+   to learn the compressed size (as the reference does, :114-115), unless the
+   handle already holds a tensor of the same element count (see
+   nz_manager_rewrite_stats). */
 int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint64_t n,
                      int dtype, void* stream);
 
-/* Up to 16 writes with THREE kernel launches and ONE host synchronisation: the
-   tensors ride in the kernel arguments, so split + coding of all of them is one
-   launch, the directories another, the container sizes come back together,
-   then one launch fills the exact-size buffers (an optimizer step that re-compresses the
-   weights of a block pays one sync instead of one per weight,
+/* Up to 16 writes together: the tensors ride in the kernel arguments, so split +
+   coding of all of them is one launch (one per segment-length class in use),
+   their container sizes come back with ONE host synchronisation, then one
+   launch fills the exact-size buffers (an optimizer step that re-compresses
+   the weights of a block pays one sync instead of one per weight,
    cuda/high_level.cu:114-115 per call).  Same semantics per entry as
    nz_manager_write; a name may appear only once. */
 int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* const* dev_data,
                            const uint64_t* ns, uint32_t count, int dtype, void* stream);
+
+/* A write (single or batch) whose handles all hold a tensor of the same element
+   count already - the re-compress after an optimizer step,
+   neuzip/__init__.py:25-35 - encodes straight into the buffers those entries
+   have: no allocation, no free and no wait for the container size, which
+   comes back through pinned memory and is looked at when the entry is used
+   next (an entry whose container outgrew its buffer, which has ~1.5 % of
+   headroom, is then given a larger one and re-compacted from scratch memory
+   that is kept until then).  Counters for tests and tuning: batches written in
+   place so far, entries that outgrew their buffer.  Settles what is pending. */
+int nz_manager_rewrite_stats(nz_manager* m, uint64_t* in_place_batches, uint64_t* outgrown_entries);
 
 /* Manager::read(name), cuda/high_level.cu:223-250, into caller-owned memory of
    at least `cap_elems` elements.  Asynchronous on `stream` (the reference

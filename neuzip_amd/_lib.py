@@ -20,7 +20,7 @@ DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 ALGO_ANS = 0
 DEFAULT_CHUNK = 131072
 DEFAULT_LANE_SYMS = 256
-LANE_SYMS_64K = 344
+LANE_SYMS_64K = 256
 LANE_SYMS_AUTO = 0xFFFFFFFF
 DECODE_CHECK, DECODE_STREAM_OUT, DECODE_RESIDENT_OUT = 1, 2, 4  # nz_decode flags
 
@@ -31,7 +31,7 @@ EXPORTS = [
     "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
     "nz_manager_meta", "nz_manager_size", "nz_manager_size_reference", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
     "nz_manager_norm_bytes", "nz_manager_buffers", "nz_manager_erase", "nz_manager_check",
-    "nz_manager_export", "nz_manager_import", "nz_manager_trim",
+    "nz_manager_export", "nz_manager_import", "nz_manager_trim", "nz_manager_rewrite_stats",
 ]
 
 _lib = None
@@ -83,6 +83,8 @@ def load() -> ctypes.CDLL:
                                          u32, i32, vp]
     L.nz_manager_read.restype = i32
     L.nz_manager_read.argtypes = [vp, ctypes.c_char_p, vp, u64, vp]
+    L.nz_manager_rewrite_stats.restype = i32
+    L.nz_manager_rewrite_stats.argtypes = [vp, ctypes.POINTER(u64), ctypes.POINTER(u64)]
     L.nz_manager_trim.restype = i32
     L.nz_manager_trim.argtypes = [vp]
     L.nz_manager_export.restype = i32

@@ -215,6 +215,12 @@ class _HipBackend:
     def trim(self) -> None:
         _lib.raise_for(self._L.nz_manager_trim(self._h))
 
+    def rewrite_stats(self):
+        """(write batches encoded in place, entries that outgrew their buffer and were re-placed)"""
+        a, b = ctypes.c_uint64(), ctypes.c_uint64()
+        _lib.raise_for(self._L.nz_manager_rewrite_stats(self._h, ctypes.byref(a), ctypes.byref(b)))
+        return int(a.value), int(b.value)
+
     def check(self) -> None:
         _lib.raise_for(self._L.nz_manager_check(self._h, _stream_ptr(self._device)))
 

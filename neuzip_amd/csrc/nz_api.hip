@@ -369,6 +369,25 @@ struct Entry {
   uint32_t chunk_syms = 0;
   void* norm = nullptr;    // one byte per normalizer group (managers with normalizer_size > 0)
   uint64_t norm_bytes = 0, norm_cap = 0;
+  int pending = -1;        // rewrite slot whose result (container size) the host has not looked at yet
+};
+
+// One batch of in-place rewrites in flight: tensors written again under handles
+// that already hold a tensor of the same size are encoded straight into the
+// buffers they have, without allocation and without waiting for the container
+// size.  The size comes back through pinned memory behind an event and is
+// looked at when the entry is used next (or when the slot is needed again).
+struct RewriteSlot {
+  bool busy = false;
+  hipEvent_t ev = nullptr;
+  hipStream_t stream = nullptr;
+  void* ws = nullptr;
+  uint64_t ws_bytes = 0;
+  uint64_t* d_totals = nullptr;  // device, 16 sizes
+  uint64_t* h_totals = nullptr;  // pinned, 16 sizes
+  uint32_t count = 0;
+  std::string names[NZ_ENC_BATCH_MAX];
+  NzEncBatch b;
 };
 
 }  // namespace
@@ -388,6 +407,9 @@ struct nz_manager {
   uint64_t* h_pin = nullptr;     // pinned, 256 bytes: [0..15] those sizes, [16] decode status, [17..24] those status words
   long long* gemv_acc = nullptr;  // row accumulators of the matrix-vector product (all zero between calls)
   uint64_t gemv_rows = 0;         // rows the accumulator buffer can hold
+  RewriteSlot rw[2];              // in-place rewrites in flight (two batches: the host runs one ahead)
+  uint32_t rw_next = 0;
+  uint64_t rewrites = 0, rewrites_replaced = 0;  // statistics: batches rewritten in place / entries that outgrew their buffer
 };
 
 extern "C" {
@@ -532,7 +554,7 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   }
   if (lane_syms == 0 || auto_lanes) {
     // the best measured segment length for the chunk: 8 segments of 256 per lane
-    // in a 128 Ki chunk, three ragged segments (344 per lane) in a 64 Ki chunk
+    // in a 128 Ki chunk, four of them in a 64 Ki chunk
     lane_syms = chunk_size == NZ_DEFAULT_CHUNK ? NZ_DEFAULT_LANE_SYMS : NZ_LANE_SYMS_64K;
     while (lane_syms > 8 && (uint64_t)lane_syms * NZ_LANES > chunk_size) lane_syms /= 2;
     while ((uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size) lane_syms *= 2;
@@ -546,14 +568,23 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   m->own_chunk = own_chunk;
   m->lane_syms = lane_syms;
   m->auto_lanes = auto_lanes;
-  hipError_t e = hipMalloc((void**)&m->d_status, 256);
-  if (e == hipSuccess) e = hipMemset(m->d_status, 0, 256);
-  if (e == hipSuccess) e = hipHostMalloc((void**)&m->h_pin, 256, hipHostMallocDefault);
+  // device block and its pinned mirror, 1 KiB each: [0, 256) as described at the members;
+  // [256 + 256 k, ...) the 16 container sizes of rewrite slot k; the last word a status sink
+  hipError_t e = hipMalloc((void**)&m->d_status, 1024);
+  if (e == hipSuccess) e = hipMemset(m->d_status, 0, 1024);
+  if (e == hipSuccess) e = hipHostMalloc((void**)&m->h_pin, 1024, hipHostMallocDefault);
+  for (int k = 0; k < 2 && e == hipSuccess; ++k) {
+    m->rw[k].d_totals = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(m->d_status) + 256 + 256 * k);
+    m->rw[k].h_totals = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(m->h_pin) + 256 + 256 * k);
+    e = hipEventCreateWithFlags(&m->rw[k].ev, hipEventDisableTiming);
+  }
   int dev = 0, cus = 0;
   if (e == hipSuccess) e = hipGetDevice(&dev);
   if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
   if (e == hipSuccess && cus > 0) m->slots = 3u * (uint32_t)cus;
   if (e != hipSuccess) {
+    for (int k = 0; k < 2; ++k)
+      if (m->rw[k].ev) (void)hipEventDestroy(m->rw[k].ev);
     if (m->d_status) (void)hipFree(m->d_status);
     if (m->h_pin) (void)hipHostFree(m->h_pin);
     delete m;
@@ -571,6 +602,10 @@ void nz_manager_destroy(nz_manager* m) {
     if (kv.second.norm) (void)hipFree(kv.second.norm);
   }
   if (m->ws) (void)hipFree(m->ws);
+  for (int k = 0; k < 2; ++k) {
+    if (m->rw[k].ws) (void)hipFree(m->rw[k].ws);
+    if (m->rw[k].ev) (void)hipEventDestroy(m->rw[k].ev);
+  }
   if (m->gemv_acc) (void)hipFree(m->gemv_acc);
   if (m->d_status) (void)hipFree(m->d_status);
   if (m->h_pin) (void)hipHostFree(m->h_pin);
@@ -741,6 +776,54 @@ int write_place(PendingWrite* pw, uint64_t total, NzEncItem* item) {
   return NZ_OK;
 }
 
+// Look at the outcome of rewrite slot k (waiting for it only if it is still
+// running): the container sizes become known, and an entry whose new container
+// did not fit the buffer it had gets a larger one, filled by a second
+// compaction from the slot's scratch, which nothing has touched since.
+int settle_slot(nz_manager* m, int k) {
+  RewriteSlot& s = m->rw[k];
+  if (!s.busy) return NZ_OK;
+  if (hipEventQuery(s.ev) != hipSuccess) NZ_HIP(hipEventSynchronize(s.ev));
+  s.busy = false;
+  for (uint32_t j = 0; j < s.count; ++j) {
+    auto it = m->entries.find(s.names[j]);
+    if (it == m->entries.end() || it->second.pending != k) continue;
+    Entry& ent = it->second;
+    ent.pending = -1;
+    const uint64_t total = s.h_totals[j];
+    if (total <= ent.comp_cap) {
+      ent.comp_bytes = total;
+      continue;
+    }
+    // outgrown: a buffer that fits, the records moved again
+    ++m->rewrites_replaced;
+    void* bigger = nullptr;
+    const uint64_t cap = total + total / 32 + 4096;
+    NZ_HIP(hipMalloc(&bigger, cap));
+    NzEncBatch one{};
+    one.count = 1;
+    one.item[0] = s.b.item[j];
+    one.item[0].comp = (uint8_t*)bigger;
+    one.item[0].comp_cap = cap;
+    if (!enc_batch_close(&one)) return fail(NZ_ERR_ARG, "too many chunks for one launch");
+    if (int rc = encode_phase2(&one, s.stream)) return rc;
+    NZ_HIP(hipStreamSynchronize(s.stream));
+    (void)hipFree(ent.comp);
+    ent.comp = bigger;
+    ent.comp_cap = cap;
+    ent.comp_bytes = total;
+  }
+  return NZ_OK;
+}
+
+int settle_entry(nz_manager* m, const Entry& ent) { return ent.pending >= 0 ? settle_slot(m, ent.pending) : NZ_OK; }
+
+int settle_all(nz_manager* m) {
+  for (int k = 0; k < 2; ++k)
+    if (int rc = settle_slot(m, k)) return rc;
+  return NZ_OK;
+}
+
 int grow_workspace(nz_manager* m, uint64_t bytes, hipStream_t st) {
   if (m->ws_bytes >= bytes) return NZ_OK;
   // the previous scratch may still be in use by kernels on the stream
@@ -778,6 +861,63 @@ int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* 
     at[i + 1] = at[i] + enc_layout(g[i]).bytes;
   }
   std::lock_guard<std::mutex> lock(m->mu);
+  // ---- in place: every handle already holds a tensor of this size and geometry.  The new
+  // streams go straight into the buffers the entries have (an optimizer step changes the
+  // container size by a few bytes; a buffer has ~1.5 % of headroom): no allocation, no free,
+  // no wait.  The sizes are looked at later (settle_slot), where an entry that has outgrown
+  // its buffer is given a larger one.
+  bool in_place = count > 0;
+  for (uint32_t i = 0; i < count && in_place; ++i) {
+    auto it = m->entries.find(names[i]);
+    in_place = it != m->entries.end() && ns[i] != 0 && it->second.n == ns[i] && it->second.dtype == dtype &&
+               it->second.chunk_syms == chunk[i] && it->second.lane_syms == lane[i] && it->second.comp != nullptr;
+  }
+  if (in_place) {
+    // the slot is free once its previous batch has been looked at; an entry written
+    // again while its last rewrite is still unseen is settled first
+    const int k = (int)m->rw_next;
+    if (int rc = settle_slot(m, k)) return rc;
+    for (uint32_t i = 0; i < count; ++i)
+      if (int rc = settle_entry(m, m->entries.find(names[i])->second)) return rc;
+    RewriteSlot& s = m->rw[k];
+    if (s.ws_bytes < at[count]) {
+      if (s.ws) {
+        NZ_HIP(hipStreamSynchronize(st));
+        NZ_HIP(hipFree(s.ws));
+      }
+      s.ws = nullptr;
+      s.ws_bytes = 0;
+      NZ_HIP(hipMalloc(&s.ws, at[count]));
+      s.ws_bytes = at[count];
+    }
+    s.b = NzEncBatch{};
+    s.b.count = count;
+    s.count = count;
+    s.stream = st;
+    uint32_t* status_sink = m->d_status + 255;  // the sizes tell the host everything it needs
+    for (uint32_t i = 0; i < count; ++i) {
+      Entry& ent = m->entries.find(names[i])->second;
+      s.names[i] = names[i];
+      s.b.item[i] = enc_item(g[i], dev_data[i], (uint8_t*)ent.packed, (uint8_t*)s.ws + at[i], enc_layout(g[i]),
+                             (uint8_t*)ent.comp, ent.comp_cap, s.d_totals + i, status_sink, m->normalizer,
+                             (uint8_t*)ent.norm);
+    }
+    if (int rc = encode_phase1(&s.b, m->precision, m->normalizer, st)) return rc;
+    if (int rc = encode_phase2(&s.b, st)) return rc;
+    NZ_HIP(hipMemcpyAsync(s.h_totals, s.d_totals, 8 * count, hipMemcpyDeviceToHost, st));
+    NZ_HIP(hipEventRecord(s.ev, st));
+    for (uint32_t i = 0; i < count; ++i) {
+      Entry& ent = m->entries.find(names[i])->second;
+      ent.pending = k;
+      ent.comp_bytes = ent.comp_cap;  // an upper bound that keeps every access inside the buffer until the size is known
+    }
+    s.busy = true;
+    m->rw_next ^= 1u;
+    ++m->rewrites;
+    return NZ_OK;
+  }
+  // ---- otherwise: new entries (or entries of another size), buffers sized to fit
+  if (int rc = settle_all(m)) return rc;
   if (int rc = grow_workspace(m, at[count], st)) return rc;
   PendingWrite pw[NZ_WRITE_BATCH_MAX];
   int rc = NZ_OK;
@@ -834,6 +974,7 @@ int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  if (int rc = settle_entry(m, it->second)) return rc;
   const Entry& ent = it->second;
   if (cap_elems < ent.n) return fail(NZ_ERR_CAPACITY, "output smaller than the stored tensor");
   if (ent.n == 0) return NZ_OK;
@@ -855,6 +996,7 @@ int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* 
     if (!names[i]) return fail(NZ_ERR_ARG, "null name");
     auto it = m->entries.find(names[i]);
     if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+    if (int rc = settle_entry(m, it->second)) return rc;
     const Entry& ent = it->second;
     if (cap_elems[i] < ent.n) return fail(NZ_ERR_CAPACITY, "output smaller than the stored tensor");
     if (ent.n && !dev_outs[i]) return fail(NZ_ERR_ARG, "null output pointer");
@@ -921,6 +1063,7 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
     if (!names[i]) return fail(NZ_ERR_ARG, "null name");
     auto it = m->entries.find(names[i]);
     if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+    if (int rc = settle_entry(m, it->second)) return rc;
     const Entry& ent = it->second;
     if (ent.n == 0 || ent.n % in_features)
       return fail(NZ_ERR_ARG, "stored tensor is not a matrix with rows of in_features elements");
@@ -973,6 +1116,7 @@ int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indi
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  if (int rc = settle_entry(m, it->second)) return rc;
   const Entry& ent = it->second;
   if (row_len == 0 || ent.n == 0 || ent.n % row_len)
     return fail(NZ_ERR_ARG, "stored tensor is not a table with rows of row_len elements");
@@ -1028,6 +1172,7 @@ uint64_t nz_manager_size(nz_manager* m, const char* name) {
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return 0;  // cuda/high_level.cu:209-211
+  (void)settle_entry(m, it->second);
   return it->second.comp_bytes + it->second.packed_bytes + it->second.norm_bytes;
 }
 
@@ -1036,6 +1181,7 @@ uint64_t nz_manager_size_reference(nz_manager* m, const char* name) {
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return 0;
+  (void)settle_entry(m, it->second);
   const Entry& e = it->second;
   // cuda/high_level.cu:89-93: without normalizers the reference still allocates
   // (and size() counts, :208-221) one byte per 1024 elements
@@ -1047,7 +1193,9 @@ uint64_t nz_manager_exp_bytes(nz_manager* m, const char* name) {
   if (!m || !name) return 0;
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
-  return it == m->entries.end() ? 0 : it->second.comp_bytes;
+  if (it == m->entries.end()) return 0;
+  (void)settle_entry(m, it->second);
+  return it->second.comp_bytes;
 }
 
 uint64_t nz_manager_packed_bytes(nz_manager* m, const char* name) {
@@ -1063,6 +1211,7 @@ int nz_manager_buffers(nz_manager* m, const char* name, const void** dev_comp, u
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  if (int rc = settle_entry(m, it->second)) return rc;
   if (dev_comp) *dev_comp = it->second.comp;
   if (comp_bytes) *comp_bytes = it->second.comp_bytes;
   if (dev_packed) *dev_packed = it->second.packed;
@@ -1085,6 +1234,7 @@ int nz_manager_export(nz_manager* m, const char* name, void* host_comp, uint64_t
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  if (int rc = settle_entry(m, it->second)) return rc;
   const Entry& ent = it->second;
   if (comp_cap < ent.comp_bytes || packed_cap < ent.packed_bytes || norm_cap < ent.norm_bytes)
     return fail(NZ_ERR_CAPACITY, "host buffers smaller than the stored streams");
@@ -1166,6 +1316,7 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
   if (it != m->entries.end()) {
     // kernels reading the old buffers may still be in flight
     (void)hipDeviceSynchronize();
+    (void)settle_entry(m, it->second);
     release_entry(it->second);
     m->entries.erase(it);
   }
@@ -1180,6 +1331,7 @@ int nz_manager_erase(nz_manager* m, const char* name) {
   if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
   // kernels reading these buffers may still be in flight
   NZ_HIP(hipDeviceSynchronize());
+  if (int rc = settle_entry(m, it->second)) return rc;
   if (it->second.comp) (void)hipFree(it->second.comp);
   if (it->second.packed) (void)hipFree(it->second.packed);
   if (it->second.norm) (void)hipFree(it->second.norm);
@@ -1192,12 +1344,27 @@ int nz_manager_trim(nz_manager* m) {
   std::lock_guard<std::mutex> lock(m->mu);
   // kernels of earlier writes, gathers or products may still use the scratch
   NZ_HIP(hipDeviceSynchronize());
+  if (int rc = settle_all(m)) return rc;
   if (m->ws) NZ_HIP(hipFree(m->ws));
   m->ws = nullptr;
   m->ws_bytes = 0;
+  for (int k = 0; k < 2; ++k) {
+    if (m->rw[k].ws) NZ_HIP(hipFree(m->rw[k].ws));
+    m->rw[k].ws = nullptr;
+    m->rw[k].ws_bytes = 0;
+  }
   if (m->gemv_acc) NZ_HIP(hipFree(m->gemv_acc));
   m->gemv_acc = nullptr;
   m->gemv_rows = 0;
+  return NZ_OK;
+}
+
+int nz_manager_rewrite_stats(nz_manager* m, uint64_t* in_place_batches, uint64_t* outgrown_entries) {
+  if (!m) return fail(NZ_ERR_ARG, "null manager");
+  std::lock_guard<std::mutex> lock(m->mu);
+  if (int rc = settle_all(m)) return rc;
+  if (in_place_batches) *in_place_batches = m->rewrites;
+  if (outgrown_entries) *outgrown_entries = m->rewrites_replaced;
   return NZ_OK;
 }
 

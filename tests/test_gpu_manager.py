@@ -435,7 +435,7 @@ def test_auto_lane_symbols(oracle):
     for chunk_arg, cases in (
         (None, tuple((n,) + _auto_geometry(n) for n in (1000, 40_001, 1 << 20, 25_165_824, 40_000_000, 14336 * 4096,
                                                         70_000_000, 110_000_000))),
-        (65536, ((1 << 20, 65536, 176), (40_000_000, 65536, 176), (70_000_000, 65536, 344))),
+        (65536, ((1 << 20, 65536, 128), (40_000_000, 65536, 256), (70_000_000, 65536, 256))),
     ):
         mgr = neuzip_amd.Manager(chunk_size=chunk_arg, lane_symbols="auto")
         for n, chunk, lane in cases:
@@ -492,3 +492,52 @@ def test_write_many_equals_single_writes(oracle):
         with pytest.raises(ValueError):
             many.write_many(ws[:2], ["same", "same"])
         many._be.check()
+
+
+def test_rewrite_in_place_needs_no_size_round_trip(oracle):
+    """Writing again under handles that hold tensors of the same size (the
+    re-compress after an optimizer step, neuzip/__init__.py:25-35) goes straight
+    into the entries' buffers; the stored bytes are still the oracle's, and an
+    entry whose container outgrows its buffer is re-placed without losing data."""
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager()
+    shapes = [(300, 1000), (257, 513), (64, 4096)]
+    ws = [from_bits(bf16_bits_normal(int(np.prod(s)), seed=i), s) for i, s in enumerate(shapes)]
+    hs = [mgr.write(w) for w in ws]
+    assert mgr._be.rewrite_stats() == (0, 0)
+    # three optimizer-like steps over all tensors (slots alternate), single writes and batches
+    for step in range(3):
+        ws = [(w.float() * (1.0 + 0.001 * (step + 1))).to(torch.bfloat16) for w in ws]
+        if step == 1:
+            for w, h in zip(ws, hs):
+                mgr.write(w, h)
+        else:
+            mgr.write_many(ws, hs)
+        for w, h in zip(ws, hs):
+            assert torch.equal(mgr.read(h), w)
+            o_comp, o_packed = oracle.compress_bf16(bits_of(w), 7, 131072, 256)
+            assert mgr.size(h) == o_comp.size + o_packed.size
+            comp, packed, _ = mgr._be.export(h)
+            assert np.array_equal(comp.numpy(), o_comp) and np.array_equal(packed.numpy(), o_packed)
+    batches, outgrown = mgr._be.rewrite_stats()
+    assert batches == 2 + len(hs) and outgrown == 0
+    # a handle whose new content compresses far worse than the old: the container
+    # outgrows the buffer it has and moves to a larger one
+    n = 1 << 20
+    flat = torch.full((n,), 0.5, dtype=torch.bfloat16, device="cuda")     # one exponent value: a tiny container
+    h = mgr.write(flat)
+    small, small_container = mgr.size(h), mgr._be.exp_bytes(h)
+    noisy = from_bits(stress_bits(1024, 1024, seed=3), (n,))
+    mgr.write(noisy, h)
+    assert torch.equal(mgr.read(h).view(torch.int16), noisy.view(torch.int16))
+    assert mgr._be.exp_bytes(h) > 20 * small_container
+    assert mgr._be.rewrite_stats() == (batches + 1, 1)
+    mgr.write(flat, h)                                                    # and back: fits the larger buffer
+    assert torch.equal(mgr.read(h), flat) and mgr.size(h) == small
+    assert mgr._be.rewrite_stats() == (batches + 2, 1)
+    # a different element count under the same handle takes the sized-to-fit route
+    mgr.write(flat[: n // 2], h)
+    assert torch.equal(mgr.read(h), flat[: n // 2])
+    assert mgr._be.rewrite_stats() == (batches + 2, 1)
+    mgr._be.check()
