@@ -241,10 +241,18 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
    `name`, read as rows of row_len elements, goes to dev_out[i * row_len ...];
    only the chunks that hold the requested rows are decoded.  An index outside
    the table gives a row of zeros and makes the next nz_manager_check fail.
-   Uses the manager's write scratch (grown when needed: calls must be ordered on
-   one stream with the writes).  Asynchronous on `stream`. */
+   Every (row, chunk) pair is decoded on its own, so a call that asks for about
+   as many rows as the table has chunks is better served by nz_manager_read
+   (neuzip_amd.Manager.gather_rows makes that choice).  Uses the manager's write
+   scratch, at most a quarter GiB of it: larger requests are served in slices
+   (calls must be ordered on one stream with the writes).  Asynchronous on
+   `stream`. */
 int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indices, uint64_t count,
                            uint32_t row_len, void* dev_out, void* stream);
+
+/* Geometry an entry was written with (it travels in the container's header):
+   elements per frequency table and symbols per rANS lane and segment. */
+int nz_manager_geometry(nz_manager* m, const char* name, uint32_t* chunk_size, uint32_t* lane_syms);
 
 /* meta_cache lookup, cuda/high_level.cu:42-43,228-230. */
 int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype);

@@ -120,6 +120,12 @@ class _HipBackend:
         _lib.raise_for(self._L.nz_manager_meta(self._h, handle.encode(), ctypes.byref(n), None))
         return int(n.value)
 
+    def geometry(self, handle: str):
+        """(elements per frequency table, symbols per rANS lane and segment) the entry was written with"""
+        c, l = ctypes.c_uint32(), ctypes.c_uint32()
+        _lib.raise_for(self._L.nz_manager_geometry(self._h, handle.encode(), ctypes.byref(c), ctypes.byref(l)))
+        return int(c.value), int(l.value)
+
     def read_into(self, handle: str, out: torch.Tensor) -> torch.Tensor:
         """Decompress into caller-provided bf16 storage (no allocation), on the current stream."""
         if out.dtype != torch.bfloat16 or not out.is_contiguous():
@@ -222,7 +228,15 @@ class _HipBackend:
         return int(a.value), int(b.value)
 
     def check(self) -> None:
+        outside, self._outside = getattr(self, "_outside", None), None
         _lib.raise_for(self._L.nz_manager_check(self._h, _stream_ptr(self._device)))
+        if outside is not None and bool(outside):
+            raise RuntimeError("a row gather was given an index outside the table")
+
+    def note_outside(self, flag: torch.Tensor) -> None:
+        """Keeps a device-side flag (no synchronisation) for the next check()."""
+        prev = getattr(self, "_outside", None)
+        self._outside = flag if prev is None else prev | flag
 
     def linear(self, handle: str, inputs: torch.Tensor, shape, bias: torch.Tensor) -> torch.Tensor:
         # cuda/high_level.cu:252-257: addmm(bias, input, W^T).  The reference only
@@ -392,7 +406,20 @@ class Manager:
             raise ValueError("gather_rows needs a stored 2-D table")
         if isinstance(self._be, _DenseBackend):
             return self._be.read(handle).reshape(shape)[indices.reshape(-1)]
-        return self._be.gather_rows(handle, indices, int(shape[1]))
+        # Every requested row decodes the chunk(s) it lies in.  Once that is as much
+        # work as decoding the table, do what the reference does: the whole table
+        # once, then an ordinary index (neuzip/nn/embedding.py:30-39).
+        rows, row_len = int(shape[0]), int(shape[1])
+        chunk, _ = self._be.geometry(handle)
+        per_row = 1 if (row_len <= chunk and chunk % row_len == 0) else (row_len + chunk - 2) // chunk + 1
+        n_chunks = -(-rows * row_len // chunk)
+        if indices.numel() * per_row >= n_chunks:
+            idx = indices.reshape(-1).to(device=self._be._device, dtype=torch.int64)
+            outside = (idx < 0) | (idx >= rows)  # as in the row gather: a row of zeros
+            out = self.read(handle).index_select(0, idx.clamp(0, rows - 1))
+            self._be.note_outside(outside.any())     # reported by check(), as the row gather's are
+            return out.masked_fill_(outside.unsqueeze(1), 0)
+        return self._be.gather_rows(handle, indices, row_len)
 
     # -- checkpointing (no counterpart in the reference, whose compressed tensors
     #    live only inside the process: neuzip/nn/module.py:13) ------------------

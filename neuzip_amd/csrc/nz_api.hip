@@ -1122,14 +1122,27 @@ int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indi
     return fail(NZ_ERR_ARG, "stored tensor is not a table with rows of row_len elements");
   NzGeom g;
   if (int rc = make_geom(&g, ent.n, ent.chunk_syms, ent.lane_syms)) return rc;
-  // chunks a row can touch, wherever it starts
-  const uint32_t cpr = (uint32_t)(((uint64_t)row_len + g.chunk_syms - 2) / g.chunk_syms + 1);
-  if (count * (uint64_t)cpr > 0x7FFFFFFFull || count > 0xFFFFull * 0xFFFFull)
-    return fail(NZ_ERR_ARG, "too many rows for one call");
-  // one chunk-sized slot per (row, touched chunk): taken from the encode scratch of this manager
-  const uint64_t need = count * (uint64_t)cpr * g.chunk_syms * 2;
+  // chunks a row can touch: one when rows never straddle a chunk boundary, else
+  // as many as a row can reach wherever it starts
+  const uint32_t cpr = (row_len <= g.chunk_syms && g.chunk_syms % row_len == 0)
+                           ? 1u
+                           : (uint32_t)(((uint64_t)row_len + g.chunk_syms - 2) / g.chunk_syms + 1);
+  // One chunk-sized slot per (row, touched chunk), taken from the encode scratch
+  // of this manager.  The rows are served in slices, so that the slots of a
+  // slice stay below a quarter GiB and its grid inside the launch limits,
+  // whatever the number of rows; everything is validated before the first launch.
+  const uint64_t slot_bytes = (uint64_t)cpr * g.chunk_syms * 2;
+  const uint64_t cap_bytes = 256ull << 20;
+  uint64_t per_slice = cap_bytes / slot_bytes;
+  if (per_slice == 0) per_slice = 1;
+  if (per_slice > count) per_slice = count;
+  const uint32_t bx = (row_len + 255) / 256 < 64 ? (row_len + 255) / 256 : 64;
+  if (per_slice * cpr > 0x7FFFFFFFull || per_slice * bx > 0x7FFFFFFFull)
+    per_slice = 0x7FFFFFFFull / (cpr > bx ? cpr : bx);
+  const uint64_t need = per_slice * slot_bytes;
   if (m->ws_bytes < need) {
     NZ_HIP(hipStreamSynchronize(st));
+    if (int rc = settle_all(m)) return rc;
     if (m->ws) NZ_HIP(hipFree(m->ws));
     m->ws = nullptr;
     m->ws_bytes = 0;
@@ -1137,23 +1150,35 @@ int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indi
     m->ws_bytes = need;
   }
   const NzNorm nm{m->normalizer ? (const uint8_t*)ent.norm : nullptr, log2_of(m->normalizer ? m->normalizer : 1)};
-  const long long* idx = (const long long*)dev_indices;
   uint16_t* scratch = (uint16_t*)m->ws;
+  for (uint64_t at = 0; at < count; at += per_slice) {
+    const uint32_t rows_now = (uint32_t)(count - at < per_slice ? count - at : per_slice);
+    const long long* idx = (const long long*)dev_indices + at;
 #define NZ_ROWS_CASE(S)                                                                              \
   launch_decode_rows<S>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx,     \
-                        (uint32_t)count, row_len, cpr, st)
-  switch (m->precision) {
-    case 7: NZ_ROWS_CASE(7); break;
-    case 3: NZ_ROWS_CASE(3); break;
-    case 1: NZ_ROWS_CASE(1); break;
-    default: NZ_ROWS_CASE(0); break;
-  }
+                        rows_now, row_len, cpr, st)
+    switch (m->precision) {
+      case 7: NZ_ROWS_CASE(7); break;
+      case 3: NZ_ROWS_CASE(3); break;
+      case 1: NZ_ROWS_CASE(1); break;
+      default: NZ_ROWS_CASE(0); break;
+    }
 #undef NZ_ROWS_CASE
-  NZ_HIP(hipGetLastError());
-  const uint32_t bx = (row_len + 255) / 256 < 64 ? (row_len + 255) / 256 : 64;
-  hipLaunchKernelGGL(nz_copy_rows_kernel, dim3(bx, (uint32_t)count), dim3(256), 0, st, (const uint16_t*)scratch,
-                     idx, ent.n / row_len, row_len, g.chunk_syms, cpr, (uint16_t*)dev_out);
-  NZ_HIP(hipGetLastError());
+    NZ_HIP(hipGetLastError());
+    hipLaunchKernelGGL(nz_copy_rows_kernel, dim3(bx * rows_now), dim3(256), 0, st, (const uint16_t*)scratch, idx,
+                       ent.n / row_len, row_len, g.chunk_syms, cpr, bx, (uint16_t*)dev_out + at * (uint64_t)row_len);
+    NZ_HIP(hipGetLastError());
+  }
+  return NZ_OK;
+}
+
+int nz_manager_geometry(nz_manager* m, const char* name, uint32_t* chunk_size, uint32_t* lane_syms) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  std::lock_guard<std::mutex> lock(m->mu);
+  auto it = m->entries.find(name);
+  if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  if (chunk_size) *chunk_size = it->second.chunk_syms;
+  if (lane_syms) *lane_syms = it->second.lane_syms;
   return NZ_OK;
 }
 

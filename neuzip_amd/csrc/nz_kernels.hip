@@ -1986,17 +1986,19 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_rows_ker
   nz_decode_chunk<S, false, NORM, false>(comp, comp_bytes, packed, out, g, d_status, c, NzGemv{}, nm);
 }
 
+// `bx` workgroups per row, rows along the same grid dimension (no limit of
+// 65535 rows); `i` counts from the start of the slice the scratch holds.
 __global__ __launch_bounds__(256) void nz_copy_rows_kernel(const uint16_t* __restrict__ scratch,
                                                            const long long* __restrict__ indices,
                                                            uint64_t rows, uint32_t row_len,
-                                                           uint32_t chunk_syms, uint32_t cpr,
+                                                           uint32_t chunk_syms, uint32_t cpr, uint32_t bx,
                                                            uint16_t* __restrict__ out) {
-  const uint32_t i = blockIdx.y;
+  const uint32_t i = blockIdx.x / bx, part = blockIdx.x - i * bx;
   const long long idx = indices[i];
   const bool ok = idx >= 0 && (uint64_t)idx < rows;
   const uint64_t first = ok ? (uint64_t)idx * row_len : 0;
   const uint64_t c0 = first / chunk_syms;
-  for (uint32_t e = blockIdx.x * 256 + threadIdx.x; e < row_len; e += gridDim.x * 256) {
+  for (uint32_t e = part * 256 + threadIdx.x; e < row_len; e += bx * 256) {
     const uint64_t ge = first + e;
     const uint64_t c = ge / chunk_syms;
     const uint16_t v = ok ? scratch[((uint64_t)i * cpr + (c - c0)) * chunk_syms + (ge - c * chunk_syms)] : 0;

@@ -103,3 +103,41 @@ def test_embedding_module_and_unroll_convert():
     de = neuzip_amd.nn.Embedding(dm, torch.nn.Embedding(20, 8).to(torch.bfloat16).cuda())
     assert de(torch.tensor([[1, 2]]).cuda()).shape == (1, 2, 8)
     mgr._be.check()
+
+
+def test_large_lookups_are_bounded(oracle):
+    """A lookup of more rows than the table has chunks goes through one full
+    read; a lookup whose slots would exceed the scratch cap is served in slices;
+    more than 65535 rows are fine; all equal the oracle's rows."""
+    import neuzip_amd
+
+    rows, dim = 3000, 4096          # 94 chunks of 131072 elements, 32 rows per chunk
+    bits = _table_bits(rows, dim, seed=5)
+    mgr = neuzip_amd.Manager()
+    h = mgr.write(_dev(bits, rows, dim))
+    full = _dev(oracle.reconstruct(bits, 7), rows, dim)
+    g = torch.Generator().manual_seed(1)
+    assert mgr._be.geometry(h) == (131072, 256)
+    for count in (50, 93, 94, 5000):                      # below / at / above the number of chunks
+        idx = torch.randint(0, rows, (count,), generator=g).cuda()
+        print(f"case lookup count={count}", flush=True)
+        assert torch.equal(mgr.gather_rows(h, idx), full[idx])
+    idx = torch.tensor([0, rows, -1, rows - 1] * 40).cuda()  # the full-read route zeroes rows outside the table too
+    got = mgr.gather_rows(h, idx)
+    assert torch.equal(got[0], full[0]) and torch.equal(got[3], full[rows - 1])
+    assert int(got[1].view(torch.int16).abs().max()) == 0 and int(got[2].view(torch.int16).abs().max()) == 0
+    with pytest.raises(RuntimeError, match="outside the table"):
+        mgr._be.check()
+    mgr._be.check()                 # reported once
+    # the native gather in slices: 2500 rows of 2 chunk-sized slots each are 1.3 GB of slots, the cap a quarter GiB
+    rows2, dim2 = 70_000, 24        # rows straddle chunk boundaries (131072 is not a multiple of 24)
+    bits2 = _table_bits(rows2, dim2, seed=6)
+    h2 = mgr.write(_dev(bits2, rows2, dim2))
+    full2 = _dev(oracle.reconstruct(bits2, 7), rows2, dim2)
+    idx = torch.randint(0, rows2, (2500,), generator=g).cuda()
+    got = mgr._be.gather_rows(h2, idx, dim2)
+    assert torch.equal(got, full2[idx])
+    many = torch.randint(0, rows2, (66_000,), generator=g).cuda()   # more rows than a grid dimension of 65535 holds
+    assert torch.equal(mgr.gather_rows(h2, many), full2[many])
+    assert torch.equal(mgr._be.gather_rows(h2, many[:66_000], dim2), full2[many])
+    mgr._be.check()
