@@ -330,7 +330,8 @@ class Manager:
         once per step)."""
         normalizer_size = 0 if normalizer_size is None else normalizer_size
         self.meta_dict = {}  # handle -> original shape
-        self._writes = 0     # bumped by every write: lets caches of decoded weights notice
+        self._stamps = {}    # handle -> number of writes: lets caches of decoded weights notice
+        self._on_write = None  # called with the handle before a write is enqueued (decode-ahead hooks in here)
         if algorithm == Algorithm.dummy:
             self._be = _DenseBackend()
             return
@@ -348,10 +349,15 @@ class Manager:
         self._settings = {"precision": int(precision), "normalizer_size": int(normalizer_size)}
 
     # -- store ---------------------------------------------------------------
+    def _note_write(self, handle: str) -> None:
+        self._stamps[handle] = self._stamps.get(handle, 0) + 1
+        if self._on_write is not None:
+            self._on_write(handle)
+
     def write(self, tensor: torch.Tensor, handle: Optional[str] = None) -> str:
         key = str(len(self.meta_dict)) if handle is None else handle
         self.meta_dict[key] = tensor.shape
-        self._writes += 1
+        self._note_write(key)
         self._be.write(key, tensor)  # note the argument order of the backend
         return key
 
@@ -364,7 +370,7 @@ class Manager:
             raise ValueError("one distinct handle per tensor")
         for t, h in zip(tensors, handles):
             self.meta_dict[h] = t.shape
-        self._writes += 1
+            self._note_write(h)
         if hasattr(self._be, "write_batch"):
             self._be.write_batch(handles, tensors)
         else:
@@ -448,7 +454,7 @@ class Manager:
                 raise RuntimeError(f"checkpoint has {key}={state.get(key)}, this manager {key}={mine}")
         for handle, ent in state["entries"].items():
             shape = torch.Size(ent["shape"])
-            self._writes += 1
+            self._note_write(handle)
             self._be.import_(handle, ent["container"], ent["packed"], ent.get("normalizers"))
             if self._be.numel(handle) != shape.numel():
                 raise RuntimeError(f"entry {handle!r}: shape {tuple(shape)} does not match the stored element count")

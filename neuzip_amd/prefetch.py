@@ -46,13 +46,13 @@ def _default_blocks(model: torch.nn.Module):
 class _Slot:
     """One static dense buffer able to hold the weights of any block."""
 
-    __slots__ = ("buf", "ready", "block", "stamp")
+    __slots__ = ("buf", "ready", "block", "stamps")
 
     def __init__(self, numel: int, device):
         self.buf = torch.empty(numel, dtype=torch.bfloat16, device=device)
         self.ready = None  # event of a side-stream decode the consumer has not waited for yet
         self.block = -1    # index of the block whose weights the buffer holds (or will hold)
-        self.stamp = -1    # the manager's write counter when the block was decoded
+        self.stamps = []   # per tensor of that block: the handle's write count when it was decoded
 
 
 class DecompressAhead:
@@ -72,6 +72,7 @@ class DecompressAhead:
             for k, h in enumerate(hs):
                 self._where[h] = (bi, k)
         self._plans = [be.batch_plan(hs) for hs in self._handles]
+        self._single = {}  # (block, k) -> plan that decodes that one tensor again after a write
         # element offsets of the block's tensors in a slot buffer, 16-byte aligned
         self._offsets, need = [], 0
         for hs in self._handles:
@@ -95,12 +96,14 @@ class DecompressAhead:
         if not self._enabled:
             self.manager.linear = self._linear  # instance attributes shadow the methods
             self.manager.read_shared = self._read_shared
+            self.manager._on_write = self._before_write
             self._enabled = True
 
     def disable(self):
         if self._enabled:
             del self.manager.linear
             del self.manager.read_shared
+            self.manager._on_write = None
             self.join()
             self._enabled = False
 
@@ -115,15 +118,16 @@ class DecompressAhead:
     def join(self):
         """Make the current stream wait for any decode still running on the side
         stream and forget what the buffers hold (call before ending a stream
-        capture).  Writes through the manager need no call: a decoded block is
-        used only while the manager's write counter is what it was at decode time."""
+        capture).  Writes through the manager need no call: a decoded tensor is
+        used only while its handle's write count is what it was at decode time,
+        and only that tensor is decoded again."""
         cur = torch.cuda.current_stream()
         for s in self._slots:
             if s.ready is not None:
                 cur.wait_event(s.ready)
             s.ready = None
             s.block = -1
-            s.stamp = -1
+            s.stamps = []
         self._last, self._step = -1, 1
 
     # -- the hook ---------------------------------------------------------------
@@ -138,7 +142,7 @@ class DecompressAhead:
             slot.ready = None
         self.manager._be.read_batch(self._plans[bi], self._views[slot_i][bi])
         slot.block = bi
-        slot.stamp = self.manager._writes
+        slot.stamps = self._stamps_now(bi)
 
     def _decode_ahead(self, bi: int, slot_i: int, cur) -> None:
         slot = self._slots[slot_i]
@@ -150,21 +154,33 @@ class DecompressAhead:
             slot.ready = torch.cuda.Event()
             slot.ready.record(self.stream)
         slot.block = bi
-        slot.stamp = self.manager._writes
+        slot.stamps = self._stamps_now(bi)
+
+    def _stamps_now(self, bi: int):
+        stamps = self.manager._stamps
+        return [stamps.get(h, 0) for h in self._handles[bi]]
+
+    def _before_write(self, handle: str) -> None:
+        """A write may encode in place, over the container a decode-ahead on the
+        side stream is still reading: the writing stream waits for that decode."""
+        where = self._where.get(handle)
+        if where is None:
+            return
+        for s in self._slots:
+            if s.block == where[0] and s.ready is not None:
+                torch.cuda.current_stream().wait_event(s.ready)
 
     def _weight(self, handle: str):
         bi, k = self._where[handle]
-        now = self.manager._writes
         slot_i = next((i for i, s in enumerate(self._slots) if s.block == bi), None)
-        if slot_i is not None and self._slots[slot_i].stamp != now:
-            self._slots[slot_i].block = -1  # decoded before a later write: decode again
-            slot_i = None
         entering = bi != self._last
         if entering:
-            self._step = -1 if bi < self._last else 1  # backward passes walk the blocks in reverse
+            # backward passes walk the blocks in reverse; the step from the last block
+            # to the first one is the start of the next forward pass
+            self._step = -1 if bi == self._last - 1 else 1
             self._last = bi
+        cur = torch.cuda.current_stream()
         if entering or slot_i is None:
-            cur = torch.cuda.current_stream()
             if slot_i is None:
                 slot_i = next((i for i, s in enumerate(self._slots) if s.block < 0), 0)
                 self._decode_here(bi, slot_i, cur)
@@ -176,14 +192,22 @@ class DecompressAhead:
             if self.ahead and entering and (self.wrap or 0 <= nxt < len(self._handles)):
                 nxt %= len(self._handles)
                 other = 1 - slot_i
-                if self._slots[other].block != nxt or self._slots[other].stamp != now:
+                if self._slots[other].block != nxt:
                     if self._slots[other].ready is not None:  # never consumed: keep the streams joined
                         cur.wait_event(self._slots[other].ready)
                         self._slots[other].ready = None
                     self._decode_ahead(nxt, other, cur)
         elif self._slots[slot_i].ready is not None:
-            torch.cuda.current_stream().wait_event(self._slots[slot_i].ready)
+            cur.wait_event(self._slots[slot_i].ready)
             self._slots[slot_i].ready = None
+        slot = self._slots[slot_i]
+        now = self.manager._stamps.get(handle, 0)
+        if slot.stamps[k] != now:  # written since the block was decoded: this tensor again, the others stay
+            plan = self._single.get((bi, k))
+            if plan is None:
+                plan = self._single[(bi, k)] = self.manager._be.batch_plan([handle])
+            self.manager._be.read_batch(plan, [self._views[slot_i][bi][k]])
+            slot.stamps[k] = now
         return self._views[slot_i][bi][k]
 
     def _read_shared(self, handle: str) -> torch.Tensor:

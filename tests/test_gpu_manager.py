@@ -277,11 +277,54 @@ def test_decompress_ahead_sees_rewritten_weights():
     with torch.no_grad(), neuzip_amd.DecompressAhead(mgr, model) as da:
         y0 = model(x)
         lin = model.blocks[0].a
-        mgr.write(lin.weight() * 2, lin.weight._handle)  # bumps the manager's write counter
+        mgr.write(lin.weight() * 2, lin.weight._handle)  # bumps the handle's write count
         y1 = model(x)
     with torch.no_grad():
         assert torch.equal(y1, model(x))
     assert not torch.equal(y0, y1)
+
+
+def test_decompress_ahead_decodes_only_the_rewritten_tensor_again():
+    """One write per parameter while the blocks are walked (the reference's
+    in-backward update idiom, neuzip/utils.py:36-50): each write makes only that
+    tensor decode again, the block's other tensors and the decode-ahead of the
+    neighbouring block stay valid."""
+    import neuzip_amd
+
+    torch.manual_seed(8)
+    model = _Stack(128, 3).to(torch.bfloat16)
+    mgr = neuzip_amd.Manager()
+    mgr.convert(model)
+    model = model.cuda()
+    x = torch.randn(2, 128, device="cuda", dtype=torch.bfloat16)
+    calls = []
+    real = mgr._be.read_batch
+
+    def counting(plan, outs):
+        calls.append(plan[2])
+        return real(plan, outs)
+
+    mgr._be.read_batch = counting
+    try:
+        with torch.no_grad(), neuzip_amd.DecompressAhead(mgr, model) as da:
+            model(x)
+            calls.clear()
+            model(x)
+            assert calls == [3, 3, 3]                   # steady state: one decode-ahead of three tensors per block
+            halves = [(lin.weight._handle, lin.weight() * 0.5) for lin in
+                      (model.blocks[0].a, model.blocks[0].b, model.blocks[0].c)]
+            model(x)                                    # leaves block 0 decoded ahead for the next pass
+            calls.clear()
+            for h, t in halves:                         # one write per parameter of that block
+                mgr.write(t, h)
+            y = model(x)
+            # its three tensors again, one at a time as each is used; the other blocks' decode-aheads as before
+            assert sorted(calls) == [1, 1, 1, 3, 3, 3]
+        with torch.no_grad():
+            assert torch.equal(y, model(x))
+    finally:
+        del mgr._be.read_batch
+    mgr._be.check()
 
 
 def test_decode_under_graph_capture_replays_exactly():
