@@ -473,9 +473,11 @@ def run_gpt2m(args, torch):
     # time every codec call with events on the stream it runs on
     be = mgr._be
     spans = []
+    n_calls = {"decode": 0, "encode": 0}
 
     def timed(fn, kind):
         def wrapper(*a, **k):
+            n_calls[kind] += 1
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             r = fn(*a, **k)
@@ -530,6 +532,10 @@ def run_gpt2m(args, torch):
     per_block["dense_last_loss"] = round(float(dense_losses[-1]), 4)
     per_linear, _, _ = run(1)
     mgr._be.check()
+    # writes that went into the entries' existing buffers (no allocation, no wait for the size)
+    in_place, outgrown = be.rewrite_stats()
+    rewrites = {"write_batches_in_place": in_place, "entries_that_outgrew_their_buffer": outgrown,
+                "write_calls": n_calls["encode"]}
     n_comp = len(comp_params)
     stored_ratio = round(sum(mgr.size(p._handle) for p in comp_params) /
                          sum(2 * int(np.prod(p._shape)) for p in comp_params), 5)
@@ -541,28 +547,30 @@ def run_gpt2m(args, torch):
     # both optimizers, every decoded weight compared with the dense weight after every step
     # (bench_models.lockstep_adamw).  The losses above compare two separate runs and so also
     # see whatever the GEMM and attention kernels do differently from run to run.
-    from bench_models import lockstep_adamw
+    lockstep = None
+    if args.verify_steps > 0:
+        from bench_models import lockstep_adamw
 
-    def twin():
-        torch.manual_seed(args.seed)
-        with torch.device("cuda"):
-            torch.set_default_dtype(torch.bfloat16)
-            try:
-                return GPT2Shaped(layers=layers, ctx=args.seq_len)
-            finally:
-                torch.set_default_dtype(torch.float32)
+        def twin():
+            torch.manual_seed(args.seed)
+            with torch.device("cuda"):
+                torch.set_default_dtype(torch.bfloat16)
+                try:
+                    return GPT2Shaped(layers=layers, ctx=args.seq_len)
+                finally:
+                    torch.set_default_dtype(torch.float32)
 
-    dense_twin, comp_twin = twin(), twin()
-    mgr2 = neuzip_amd.Manager(precision=7, chunk_size=args.chunk_size or None,
-                              lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
-    mgr2.convert(comp_twin)
-    g = torch.Generator(device="cuda").manual_seed(args.seed + 2)
-    with neuzip_amd.DecompressAhead(mgr2, comp_twin, ahead=False):
-        lockstep = lockstep_adamw(
-            dense_twin, comp_twin, mgr2,
-            lambda i: torch.randint(0, 50257, (args.batch, args.seq_len), device="cuda", generator=g),
-            steps=args.verify_steps, group=per_block_linears)
-    mgr2._be.check()
+        dense_twin, comp_twin = twin(), twin()
+        mgr2 = neuzip_amd.Manager(precision=7, chunk_size=args.chunk_size or None,
+                                  lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
+        mgr2.convert(comp_twin)
+        g = torch.Generator(device="cuda").manual_seed(args.seed + 2)
+        with neuzip_amd.DecompressAhead(mgr2, comp_twin, ahead=False):
+            lockstep = lockstep_adamw(
+                dense_twin, comp_twin, mgr2,
+                lambda i: torch.randint(0, 50257, (args.batch, args.seq_len), device="cuda", generator=g),
+                steps=args.verify_steps, group=per_block_linears)
+        mgr2._be.check()
     tokens = args.batch * (args.seq_len - 1) * args.steps
     out = {
         "metric": "gpt2m_shape_compressed_training_tok_s",
@@ -578,6 +586,7 @@ def run_gpt2m(args, torch):
             "decode_per_block": per_block,
             "decode_per_linear": per_linear,
             "lockstep_check_lossless": lockstep,
+            "rewrites": rewrites,
             "compressed_tensors": n_comp,
             "lane_symbols": "auto" if args.lane_symbols < 0 else (args.lane_symbols or "default"),
             "stored_over_dense": stored_ratio,
