@@ -1813,10 +1813,16 @@ __device__ __forceinline__ void nz_decode_chunk(
     const uint32_t off = gq * NZ_LANES * (S + 1) + lane_off;
     return nz_stream_sm<S>(pk + (off < last_off ? off : last_off));
   };
-  const auto nb_at = [&](uint32_t gq) {
-    return nz_norm_load8(nm, seg_base + ((gq < whole ? gq : whole - 1) * NZ_LANES + lane) * NZ_GROUP);
+  // `wide`: groups of 8 elements or more, one byte per lane and group.  The
+  // walk over the full groups exists once per case, so that the common one has
+  // no branch between the byte's load and its use two groups later (a load
+  // behind a branch is waited for at the join, with every store before it).
+  const auto nb_at = [&](uint32_t gq, auto wide) -> uint64_t {
+    const uint64_t e0 = seg_base + ((gq < whole ? gq : whole - 1) * NZ_LANES + lane) * NZ_GROUP;
+    if constexpr (decltype(wide)::value) return nm.bytes[e0 >> nm.log2n];
+    else return nz_norm_load8(nm, e0);
   };
-  const auto full_group = [&](uint32_t gq, const uint64_t sm, const uint64_t nb) {
+  const auto full_group = [&](uint32_t gq, const uint64_t sm, const uint64_t nb, auto wide) {
     const uint4 xq = xq_next;
     if constexpr (GEMV) xq_next = walk.load(walk.next_col());  // always inside x
     uint32_t ew[8];
@@ -1826,26 +1832,30 @@ __device__ __forceinline__ void nz_decode_chunk(
     uint32_t sml = (uint32_t)sm, smh = (uint32_t)(sm >> 32);
     asm volatile("" : "+v"(sml), "+v"(smh), "+v"(ew[7]));
     uint4 mv = nz_merge_group<S>(((uint64_t)smh << 32) | sml, ew);
-    if constexpr (NORM) mv = nz_scale8<true>(mv, nb, nm.log2n >= 3);
+    if constexpr (NORM) mv = nz_scale8<true>(mv, nb, decltype(wide)::value);
     if constexpr (GEMV) walk.add(mv, xq, lane);
     else if constexpr (STREAM) nz_stream_store(dst + (gq * NZ_LANES + lane) * NZ_GROUP, mv);
     else *reinterpret_cast<uint4*>(dst + (gq * NZ_LANES + lane) * NZ_GROUP) = mv;
   };
-  uint64_t sm_a = sm_next, sm_b = 0, nb_a = nb_next, nb_b = 0;
-  if (whole > 1) {
-    sm_b = sm_at(1);
-    if constexpr (NORM) nb_b = nb_at(1);
-  }
-  uint32_t gq = 0;
-  for (; gq + 1 < whole; gq += 2) {
-    full_group(gq, sm_a, nb_a);
-    sm_a = sm_at(gq + 2);
-    if constexpr (NORM) nb_a = nb_at(gq + 2);
-    full_group(gq + 1, sm_b, nb_b);
-    sm_b = sm_at(gq + 3);
-    if constexpr (NORM) nb_b = nb_at(gq + 3);
-  }
-  if (gq < whole) full_group(gq, sm_a, nb_a);
+  const auto full_groups = [&](auto wide) {
+    uint64_t sm_a = sm_next, sm_b = 0, nb_a = nb_next, nb_b = 0;
+    if (whole > 1) {
+      sm_b = sm_at(1);
+      if constexpr (NORM) nb_b = nb_at(1, wide);
+    }
+    uint32_t gq = 0;
+    for (; gq + 1 < whole; gq += 2) {
+      full_group(gq, sm_a, nb_a, wide);
+      sm_a = sm_at(gq + 2);
+      if constexpr (NORM) nb_a = nb_at(gq + 2, wide);
+      full_group(gq + 1, sm_b, nb_b, wide);
+      sm_b = sm_at(gq + 3);
+      if constexpr (NORM) nb_b = nb_at(gq + 3, wide);
+    }
+    if (gq < whole) full_group(gq, sm_a, nb_a, wide);
+  };
+  if (!NORM || nm.log2n >= 3) full_groups(NzConst<1>{});
+  else full_groups(NzConst<0>{});
   if (!GEMV && whole < body) {  // the ragged last group of the tensor
     const uint32_t idx0 = (whole * NZ_LANES + lane) * NZ_GROUP;
     uint32_t ew[8];
