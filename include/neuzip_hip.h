@@ -161,13 +161,14 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
    for the chunk (NZ_DEFAULT_LANE_SYMS, NZ_LANE_SYMS_64K, or the chunk cut in 1..8);
    NZ_LANE_SYMS_AUTO picks the geometry per tensor from its size and the
    number of decode workgroups the device holds at once (three per compute
-   unit): with chunk_size 0, tensors with fewer chunks than that get 64 Ki or
-   32 Ki chunks of eight short segments (more wavefronts; ~4.5 bits of
-   container per extra lane), tensors between half and all of it get segments
-   stretched until their chunks fit into half, so that two of them decoded by
-   one launch are a single round of workgroups; with a given chunk_size only
-   the segments are shortened.  Every entry records the geometry it was written
-   with. */
+   unit): with chunk_size 0, a tensor with fewer default-sized chunks than that
+   is cut into one, two or three chunks per compute unit (eight segments of 64
+   to 512 symbols per lane each), so that every compute unit holds the same
+   number of workgroups, and a tensor too small for that into 32 Ki chunks of
+   eight 4 Ki segments (shorter segments cost ~4.5 bits of container per lane
+   and segment); with a given chunk_size only the segments are shortened.
+   Every entry records the geometry it was written with
+   (nz_manager_geometry). */
 int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_t chunk_size,
                       uint32_t lane_syms, nz_manager** out);
 void nz_manager_destroy(nz_manager* m);
