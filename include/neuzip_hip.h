@@ -104,9 +104,13 @@ int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fr
    code the exponents.  `dev_packed` receives nz_packed_stored_bytes() bytes,
    `dev_comp` (capacity comp_cap >= nz_exp_bound_bytes) the container.
    `dev_total` (device uint64) receives the container size, `dev_status`
-   (device uint32, OR-ed into) is non-zero on overflow.  If `host_total` is
-   not NULL the call synchronises the stream and returns the size and status
-   on the host (the reference's get_compressed_output_size sync, :114-115). */
+   (device uint32, OR-ed into) stays zero when the container is complete: bit 0
+   = it did not fit, bit 2 = a workgroup gave up waiting for the record sizes
+   of the chunks before its own (see nz_set_lookback_spins; the container is
+   then incomplete and the call has to be made again).  If `host_total` is not
+   NULL the call synchronises the stream, returns the size and status on the
+   host (the reference's get_compressed_output_size sync, :114-115) and deals
+   with bit 2 itself. */
 int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
               uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
               void* dev_workspace, uint64_t workspace_bytes, uint64_t* dev_total,
@@ -130,6 +134,17 @@ int nz_encode_static(const void* dev_bf16, uint64_t n, int precision, uint32_t c
                      uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
                      uint64_t* dev_total, uint32_t* dev_status, uint32_t normalizer_size, void* dev_norm,
                      void* stream);
+
+/* No counterpart in the reference.  The encode kernel of the calls above (and
+   of the manager's writes into existing buffers) places its records itself:
+   every workgroup waits until the workgroups of the chunks before its own have
+   announced their record sizes.  The wait is bounded: after `spins` looks at an
+   announcement (about a microsecond each; default 2^21) a workgroup gives up,
+   and the records are placed by a second kernel once the host has seen that
+   (at once in nz_encode with host_total; when the entry is used next in a
+   manager).  For tests and tuning; 0 makes every workgroup give up whose
+   predecessors are not done at its first look. */
+void nz_set_lookback_spins(uint32_t spins);
 
 /* Manager::_decompress_and_merge, cuda/high_level.cu:169-206: entropy decode
    and merge in one kernel.  `dev_status` (device uint32, zeroed by the
@@ -199,8 +214,10 @@ int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* 
    next (an entry whose container outgrew its buffer, which has ~1.5 % of
    headroom, is then given a larger one and re-compacted from scratch memory
    that is kept until then).  Counters for tests and tuning: batches written in
-   place so far, entries that outgrew their buffer.  Settles what is pending. */
-int nz_manager_rewrite_stats(nz_manager* m, uint64_t* in_place_batches, uint64_t* outgrown_entries);
+   place so far, entries that outgrew their buffer, entries whose records were
+   placed a second time (see nz_set_lookback_spins).  Settles what is pending. */
+int nz_manager_rewrite_stats(nz_manager* m, uint64_t* in_place_batches, uint64_t* outgrown_entries,
+                             uint64_t* placed_again);
 
 /* Manager::read(name), cuda/high_level.cu:223-250, into caller-owned memory of
    at least `cap_elems` elements.  Asynchronous on `stream` (the reference

@@ -224,8 +224,15 @@ class _HipBackend:
     def rewrite_stats(self):
         """(write batches encoded in place, entries that outgrew their buffer and were re-placed)"""
         a, b = ctypes.c_uint64(), ctypes.c_uint64()
-        _lib.raise_for(self._L.nz_manager_rewrite_stats(self._h, ctypes.byref(a), ctypes.byref(b)))
+        _lib.raise_for(self._L.nz_manager_rewrite_stats(self._h, ctypes.byref(a), ctypes.byref(b), None))
         return int(a.value), int(b.value)
+
+    def placed_again(self) -> int:
+        """Entries written in place whose records a second kernel had to place
+        (a workgroup of the encode kernel gave up waiting for its predecessors)."""
+        c = ctypes.c_uint64()
+        _lib.raise_for(self._L.nz_manager_rewrite_stats(self._h, None, None, ctypes.byref(c)))
+        return int(c.value)
 
     def check(self) -> None:
         outside, self._outside = getattr(self, "_outside", None), None

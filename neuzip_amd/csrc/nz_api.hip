@@ -5,6 +5,8 @@
 // No torch types, no private streams: every kernel goes to the caller's stream.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <chrono>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -44,7 +46,7 @@ uint64_t norm_bytes_of(uint64_t n, uint32_t ns) { return ns ? (n + ns - 1) / ns 
 
 // Device scratch of one encode call.
 struct EncLayout {
-  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units, bytes;
+  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units, pub, bytes;
 };
 
 // segments short enough for the kernel that keeps the exponents in registers
@@ -68,6 +70,7 @@ EncLayout enc_layout(const NzGeom& g) {
   L.seg_sbytes = take(g.n_segs * 4);
   L.seg_units = take((g.n_segs + 1) * 4);
   L.chunk_units = take((g.n_chunks + 1) * 4);
+  L.pub = take(g.n_chunks * 16);  // size announcements of the chunks (records placed by the encode kernel)
   L.bytes = o;
   return L;
 }
@@ -81,8 +84,25 @@ int launch_absmax(const void* in, uint64_t n, uint32_t ns, uint8_t* norm, hipStr
   return NZ_OK;
 }
 
+// A number no earlier call of this process has used and nothing in memory is
+// likely to show: it marks the size announcements of one encode call.
+uint64_t next_nonce() {
+  static std::atomic<uint64_t> ctr{(uint64_t)std::chrono::steady_clock::now().time_since_epoch().count() *
+                                   0x9E3779B97F4A7C15ull};
+  uint64_t z = ctr.fetch_add(0x9E3779B97F4A7C15ull) + 0x9E3779B97F4A7C15ull;  // splitmix64
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+// How often a chunk of a direct encode looks for an announcement it waits for
+// (about a microsecond per look) before it gives up.
+std::atomic<uint32_t> g_lookback_spins{1u << 21};
+
 // One tensor of an encode call, as the kernels see it.  `comp`/`comp_cap`: where
 // the container goes (known only after phase 1 when the buffer is sized to fit).
+// With `comp` known and segments short enough for the register kernel the
+// records are placed by the encode kernel itself (`direct`).
 NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws, const EncLayout& L,
                    uint8_t* comp, uint64_t comp_cap, uint64_t* d_total, uint32_t* d_status,
                    uint32_t ns, uint8_t* norm) {
@@ -106,6 +126,11 @@ NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws
   it.seg_sbytes = L.seg_sbytes;
   it.seg_units = L.seg_units;
   it.chunk_units = L.chunk_units;
+  it.pub = L.pub;
+  it.nonce = next_nonce();
+  it.d_gave_up = nullptr;
+  it.direct = (comp != nullptr && g.n_segs != 0 && enc_in_registers(g)) ? 1u : 0u;
+  it.spin_limit = g_lookback_spins.load(std::memory_order_relaxed);
   return it;
 }
 
@@ -183,16 +208,31 @@ int encode_totals(NzEncBatch* b, hipStream_t st) {
 // Phase 2: header, directory and records go to each item's `comp`; the
 // container size lands in *d_total, bit 0 of *d_status is set when it does not fit.
 int encode_phase2(NzEncBatch* b, hipStream_t st) {
-  const uint32_t segs = b->count ? b->item[b->count - 1].seg_end : 0;
+  NzEncBatch rest{};  // what the encode kernel has not placed itself
   bool empty = false;  // a tensor without segments has no workgroup to write its header
-  for (uint32_t i = 0; i < b->count; ++i) empty = empty || b->item[i].g.n_segs == 0;
+  for (uint32_t i = 0; i < b->count; ++i) {
+    empty = empty || b->item[i].g.n_segs == 0;
+    if (!b->item[i].direct) rest.item[rest.count++] = b->item[i];
+  }
   if (empty)
     if (int rc = encode_totals(b, st)) return rc;
+  if (!enc_batch_close(&rest)) return fail(NZ_ERR_ARG, "too many chunks for one launch");
+  const uint32_t segs = rest.count ? rest.item[rest.count - 1].seg_end : 0;
   if (segs) {
-    hipLaunchKernelGGL(nz_compact_kernel, dim3(segs), dim3(256), 0, st, *b);
+    hipLaunchKernelGGL(nz_compact_kernel, dim3(segs), dim3(256), 0, st, rest);
     NZ_HIP(hipGetLastError());
   }
   return NZ_OK;
+}
+
+// The records of item i again, by nz_compact_kernel from what the encode kernel
+// left in the scratch (into another buffer, or after a chunk gave up waiting).
+int encode_replace(const NzEncItem& item, hipStream_t st) {
+  NzEncBatch one{};
+  one.count = 1;
+  one.item[0] = item;
+  one.item[0].direct = 0;
+  return encode_phase2(&one, st);
 }
 
 template <int S>
@@ -310,7 +350,7 @@ int make_geom(NzGeom* g, uint64_t n, uint32_t chunk, uint32_t lane_syms) {
 int encode_stateless(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size, uint32_t lane_syms,
                      void* dev_packed, void* dev_comp, uint64_t comp_cap, uint8_t* ws, uint64_t ws_bytes,
                      const char* ws_error, uint64_t* dev_total, uint32_t* dev_status, uint32_t normalizer_size,
-                     void* dev_norm, hipStream_t st) {
+                     void* dev_norm, hipStream_t st, NzEncItem* item_out = nullptr) {
   if (!precision_ok(precision)) return fail(NZ_ERR_ARG, "precision must be one of 0, 1, 3, 7");
   if (!normalizer_ok(normalizer_size))
     return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
@@ -330,6 +370,7 @@ int encode_stateless(const void* dev_bf16, uint64_t n, int precision, uint32_t c
   b.count = 1;
   b.item[0] = enc_item(g, dev_bf16, (uint8_t*)dev_packed, ws, L, (uint8_t*)dev_comp, comp_cap, dev_total, dev_status,
                        normalizer_size, (uint8_t*)dev_norm);
+  if (item_out) *item_out = b.item[0];
   if (int rc = encode_phase1(&b, precision, normalizer_size, st)) return rc;
   return encode_phase2(&b, st);
 }
@@ -383,8 +424,8 @@ struct RewriteSlot {
   hipStream_t stream = nullptr;
   void* ws = nullptr;
   uint64_t ws_bytes = 0;
-  uint64_t* d_totals = nullptr;  // device, 16 sizes
-  uint64_t* h_totals = nullptr;  // pinned, 16 sizes
+  uint64_t* d_totals = nullptr;  // device: 16 sizes, then 16 give-up marks (the nonce of the item that gave up)
+  uint64_t* h_totals = nullptr;  // pinned, the same
   uint32_t count = 0;
   std::string names[NZ_ENC_BATCH_MAX];
   NzEncBatch b;
@@ -409,7 +450,9 @@ struct nz_manager {
   uint64_t gemv_rows = 0;         // rows the accumulator buffer can hold
   RewriteSlot rw[2];              // in-place rewrites in flight (two batches: the host runs one ahead)
   uint32_t rw_next = 0;
-  uint64_t rewrites = 0, rewrites_replaced = 0;  // statistics: batches rewritten in place / entries that outgrew their buffer
+  // statistics: batches rewritten in place / entries that outgrew their buffer / entries whose records were
+  // placed a second time because a chunk gave up waiting
+  uint64_t rewrites = 0, rewrites_replaced = 0, rewrites_redone = 0;
 };
 
 extern "C" {
@@ -471,9 +514,10 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
               void* stream) {
   if (!dev_workspace) return fail(NZ_ERR_ARG, "null pointer");
   if ((uintptr_t)dev_workspace & 255) return fail(NZ_ERR_ALIGN, "workspace must be 256-byte aligned");
+  NzEncItem item;
   if (int rc = encode_stateless(dev_bf16, n, precision, chunk_size, lane_syms, dev_packed, dev_comp, comp_cap,
                                 (uint8_t*)dev_workspace, workspace_bytes, "workspace too small", dev_total,
-                                dev_status, normalizer_size, dev_norm, (hipStream_t)stream))
+                                dev_status, normalizer_size, dev_norm, (hipStream_t)stream, &item))
     return rc;
   if (host_total) {
     hipStream_t st = (hipStream_t)stream;
@@ -481,10 +525,19 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
     NZ_HIP(hipMemcpyAsync(host_total, dev_total, 8, hipMemcpyDeviceToHost, st));
     NZ_HIP(hipMemcpyAsync(&hs, dev_status, 4, hipMemcpyDeviceToHost, st));
     NZ_HIP(hipStreamSynchronize(st));
+    if (hs & 4u) {
+      // a chunk gave up waiting for the sizes before it: the records once more, by the compaction
+      if (int rc = encode_replace(item, st)) return rc;
+      NZ_HIP(hipMemcpyAsync(host_total, dev_total, 8, hipMemcpyDeviceToHost, st));
+      NZ_HIP(hipMemcpyAsync(&hs, dev_status, 4, hipMemcpyDeviceToHost, st));
+      NZ_HIP(hipStreamSynchronize(st));
+    }
     if (hs & 1u) return fail(NZ_ERR_CAPACITY, "encoded container exceeds the output capacity");
   }
   return NZ_OK;
 }
+
+void nz_set_lookback_spins(uint32_t spins) { g_lookback_spins.store(spins, std::memory_order_relaxed); }
 
 int nz_encode_static(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
                      uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
@@ -790,7 +843,15 @@ int settle_slot(nz_manager* m, int k) {
     if (it == m->entries.end() || it->second.pending != k) continue;
     Entry& ent = it->second;
     ent.pending = -1;
-    const uint64_t total = s.h_totals[j];
+    uint64_t total = s.h_totals[j];
+    if (s.h_totals[16 + j] == s.b.item[j].nonce) {
+      // a chunk gave up waiting for the sizes before it: the records once more, by the compaction
+      ++m->rewrites_redone;
+      if (int rc = encode_replace(s.b.item[j], s.stream)) return rc;
+      NZ_HIP(hipMemcpyAsync(s.h_totals + j, s.d_totals + j, 8, hipMemcpyDeviceToHost, s.stream));
+      NZ_HIP(hipStreamSynchronize(s.stream));
+      total = s.h_totals[j];
+    }
     if (total <= ent.comp_cap) {
       ent.comp_bytes = total;
       continue;
@@ -800,13 +861,10 @@ int settle_slot(nz_manager* m, int k) {
     void* bigger = nullptr;
     const uint64_t cap = total + total / 32 + 4096;
     NZ_HIP(hipMalloc(&bigger, cap));
-    NzEncBatch one{};
-    one.count = 1;
-    one.item[0] = s.b.item[j];
-    one.item[0].comp = (uint8_t*)bigger;
-    one.item[0].comp_cap = cap;
-    if (!enc_batch_close(&one)) return fail(NZ_ERR_ARG, "too many chunks for one launch");
-    if (int rc = encode_phase2(&one, s.stream)) return rc;
+    NzEncItem again = s.b.item[j];
+    again.comp = (uint8_t*)bigger;
+    again.comp_cap = cap;
+    if (int rc = encode_replace(again, s.stream)) return rc;
     NZ_HIP(hipStreamSynchronize(s.stream));
     (void)hipFree(ent.comp);
     ent.comp = bigger;
@@ -901,10 +959,11 @@ int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* 
       s.b.item[i] = enc_item(g[i], dev_data[i], (uint8_t*)ent.packed, (uint8_t*)s.ws + at[i], enc_layout(g[i]),
                              (uint8_t*)ent.comp, ent.comp_cap, s.d_totals + i, status_sink, m->normalizer,
                              (uint8_t*)ent.norm);
+      s.b.item[i].d_gave_up = s.d_totals + 16 + i;
     }
     if (int rc = encode_phase1(&s.b, m->precision, m->normalizer, st)) return rc;
     if (int rc = encode_phase2(&s.b, st)) return rc;
-    NZ_HIP(hipMemcpyAsync(s.h_totals, s.d_totals, 8 * count, hipMemcpyDeviceToHost, st));
+    NZ_HIP(hipMemcpyAsync(s.h_totals, s.d_totals, 256, hipMemcpyDeviceToHost, st));  // sizes, then give-up marks
     NZ_HIP(hipEventRecord(s.ev, st));
     for (uint32_t i = 0; i < count; ++i) {
       Entry& ent = m->entries.find(names[i])->second;
@@ -1384,12 +1443,14 @@ int nz_manager_trim(nz_manager* m) {
   return NZ_OK;
 }
 
-int nz_manager_rewrite_stats(nz_manager* m, uint64_t* in_place_batches, uint64_t* outgrown_entries) {
+int nz_manager_rewrite_stats(nz_manager* m, uint64_t* in_place_batches, uint64_t* outgrown_entries,
+                             uint64_t* placed_again) {
   if (!m) return fail(NZ_ERR_ARG, "null manager");
   std::lock_guard<std::mutex> lock(m->mu);
   if (int rc = settle_all(m)) return rc;
   if (in_place_batches) *in_place_batches = m->rewrites;
   if (outgrown_entries) *outgrown_entries = m->rewrites_replaced;
+  if (placed_again) *placed_again = m->rewrites_redone;
   return NZ_OK;
 }
 

@@ -347,6 +347,11 @@ struct NzEncLds {
   uint4 tab[256];
   uint32_t sbuf[NZ_MAX_SEGS_PER_CHUNK][NZ_STATE_MAX_BYTES / 4];
   uint32_t pad_sym, raw;
+  // for records that go straight to their place: the chunk's record sizes, the
+  // sum over the chunks before it, whether the wait for those was given up
+  uint32_t seg_units[NZ_MAX_SEGS_PER_CHUNK];
+  uint32_t chunk_total, gave_up;
+  uint64_t red64[NZ_ENC_LONG_THREADS / 64];
 };
 
 // Split one element group: 8 bf16 values -> 8 exponent bytes (byte j of `e` =
@@ -542,7 +547,8 @@ __device__ __forceinline__ void nz_build_table(NzEncLds& L, const uint32_t cn, u
 __device__ __forceinline__ bool nz_chunk_finalize(uint64_t c, uint64_t n, uint32_t chunk_syms,
                                                   uint32_t seg_syms, uint32_t spc, NzChunkInfo* info,
                                                   const uint32_t* seg_words, const uint32_t* seg_state_bytes,
-                                                  uint32_t* seg_units, uint32_t* chunk_units) {
+                                                  uint32_t* seg_units, uint32_t* chunk_units,
+                                                  uint32_t* lds_seg_units, uint32_t* lds_chunk_total) {
   const uint64_t base = c * chunk_syms;
   const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
   const uint32_t nseg = (cn + seg_syms - 1) / seg_syms;
@@ -566,9 +572,11 @@ __device__ __forceinline__ bool nz_chunk_finalize(uint64_t c, uint64_t n, uint32
               (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
     else bytes = (k == 0 ? tab_len : 0u) + seg_state_bytes[c * spc + k] + 2u * ((w + 1) & ~1u);
     seg_units[c * spc + k] = bytes / 4;
+    lds_seg_units[k] = bytes / 4;
     chunk_total += bytes / 4;
   }
   chunk_units[c] = chunk_total;
+  *lds_chunk_total = chunk_total;
   return raw;
 }
 
@@ -664,11 +672,132 @@ struct NzEncItem {
   NzGeom g;
   uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units;
   uint32_t chunk_end, seg_end;  // running totals over the batch
+  // records straight to their place (nz_encode_kernel, `direct` != 0): where the
+  // chunks announce their sizes (two words per chunk, offset into ws), the
+  // number that marks this call's announcements, how often a chunk looks for
+  // an announcement before it gives up, and where it says so (may be null)
+  uint64_t pub, nonce;
+  uint64_t* d_gave_up;
+  uint32_t direct, spin_limit;
 };
 struct NzEncBatch {
   uint32_t count, reserved;
   NzEncItem item[NZ_ENC_BATCH_MAX];
 };
+
+__device__ __forceinline__ void nz_write_header(uint8_t* comp, const NzGeom& g, uint64_t total) {
+  uint32_t* h = reinterpret_cast<uint32_t*>(comp);
+  h[0] = NZ_MAGIC;
+  h[1] = NZ_FORMAT_VERSION;
+  h[2] = (uint32_t)(g.n & 0xFFFFFFFFu);
+  h[3] = (uint32_t)(g.n >> 32);
+  h[4] = g.chunk_syms;
+  h[5] = g.lane_syms;
+  h[6] = (uint32_t)g.n_chunks;
+  h[7] = (uint32_t)g.n_segs;
+  h[8] = (uint32_t)g.dir_off;
+  h[9] = (uint32_t)g.rec_off;
+  h[10] = (uint32_t)(total & 0xFFFFFFFFu);
+  h[11] = (uint32_t)(total >> 32);
+  h[12] = h[13] = h[14] = h[15] = 0;
+  // the alignment gap between directory and records
+  for (uint64_t b = g.dir_off + 4 * (g.n_segs + 1); b < g.rec_off; ++b) comp[b] = 0;
+}
+
+
+// ----------------------------------------------------------------------------
+// move a segment record to its final place
+// ----------------------------------------------------------------------------
+// NT threads (t = 0 .. NT-1) move the record of segment `seg` = segment k of
+// chunk c to o0, counted in 4-byte units from the start of the record area
+// (`mine` = its size in the same units; ci, sbytes, w: the chunk's info, the
+// size of the coder states, the number of words).  They write the segment's
+// directory entry; those of the last segment add the closing entry, the
+// header, the container size and the overflow flag.
+template <uint32_t NT>
+__device__ __forceinline__ void nz_move_record(const NzEncItem& it, const uint64_t seg, const uint64_t c,
+                                               const uint32_t k, const uint64_t o0, const uint32_t mine,
+                                               const NzChunkInfo ci, const uint32_t sbytes, const uint32_t w,
+                                               const uint32_t t) {
+  static_assert(NT >= NZ_TAIL_PAD, "too few threads for the closing zeros");
+  const NzGeom& g = it.g;
+  const uint8_t* __restrict__ tab_ser = it.ws + it.tab_ser;
+  const uint8_t* __restrict__ carry = it.ws + it.carry;
+  const uint16_t* __restrict__ slots = reinterpret_cast<const uint16_t*>(it.ws + it.slots);
+  const uint32_t* __restrict__ states = reinterpret_cast<const uint32_t*>(it.ws + it.states);
+  uint8_t* __restrict__ comp = it.comp;
+  const uint64_t o1 = o0 + mine;
+  const bool fits = o1 <= 0xFFFFFFFFull && g.rec_off + 4 * o1 + NZ_TAIL_PAD <= it.comp_cap;
+  if (seg + 1 == g.n_segs && t == 0) {
+    const uint64_t total = g.rec_off + 4 * o1 + NZ_TAIL_PAD;
+    *it.d_total = total;
+    if (!fits) atomicOr(it.d_status, 1u);
+  }
+  if (!fits) return;  // (a record before this one may still fit and be written: harmless)
+  uint32_t* dir = reinterpret_cast<uint32_t*>(comp + g.dir_off);
+  if (t == 0) dir[seg] = (uint32_t)o0;
+  uint8_t* dst = comp + g.rec_off + 4 * o0;
+  if (seg + 1 == g.n_segs) {
+    if (t == 0) {
+      dir[g.n_segs] = (uint32_t)o1;
+      nz_write_header(comp, g, g.rec_off + 4 * o1 + NZ_TAIL_PAD);
+    }
+    if (t < NZ_TAIL_PAD) comp[g.rec_off + 4 * o1 + t] = 0;  // closing zeros
+  }
+  const uint64_t seg_base = c * g.chunk_syms + (uint64_t)k * g.seg_syms;
+  const uint32_t nom = nz_seg_nominal(g.chunk_syms, g.seg_syms, g.spc, k);
+  const uint32_t sn = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
+  if (ci.raw) {
+    uint32_t off = 0;
+    if (k == 0) {
+      if (t < 4) dst[t] = t == 0 ? NZ_MODE_RAW : 0;
+      off = 4;
+    }
+    const uint32_t padded = (sn + 3) & ~3u;
+    const uint8_t* rawp = reinterpret_cast<const uint8_t*>(slots + seg * g.seg_syms);  // left there by the encode kernel
+    for (uint32_t i = t; i < padded; i += NT) dst[off + i] = i < sn ? rawp[i] : 0;
+    if (sn == nom)
+      for (uint32_t i = t; i < NZ_CARRY_BYTES; i += NT) dst[off + padded + i] = carry[seg * NZ_CARRY_BYTES + i];
+    return;
+  }
+  uint32_t off = 0;
+  if (k == 0) {
+    const uint8_t* tb = tab_ser + c * NZ_TABLE_MAX_BYTES;
+    for (uint32_t i = t; i < ci.tab_len; i += NT) dst[i] = tb[i];
+    off = ci.tab_len;
+  }
+  uint32_t* sdst = reinterpret_cast<uint32_t*>(dst + off);
+  for (uint32_t i = t; i < sbytes / 4; i += NT) sdst[i] = states[seg * (NZ_STATE_MAX_BYTES / 4) + i];
+  const uint32_t cap_words = g.seg_syms;
+  // the words sit at the end of the segment's slot, 2-byte aligned; they are moved
+  // as dwords (two aligned loads and a funnel shift when the source is off by one
+  // word; the load past the last word stays inside the scratch buffer)
+  const uint16_t* src = slots + seg * cap_words + (cap_words - w);
+  const uint32_t mis = (uint32_t)((reinterpret_cast<uintptr_t>(src) >> 1) & 1u);
+  const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src - mis);
+  uint32_t* wdst = reinterpret_cast<uint32_t*>(dst + off + sbytes);
+  const uint32_t nd = (w + 1) / 2;
+  const uint32_t nd4 = nd & ~3u;  // four dwords per thread and turn, then the last one to three singly
+  for (uint32_t i = 4 * t; i < nd4; i += 4 * NT) {
+    const uint32_t a0 = s32[i], a1 = s32[i + 1], a2 = s32[i + 2], a3 = s32[i + 3];
+    uint4 v = make_uint4(a0, a1, a2, a3);
+    if (mis) {
+      const uint32_t a4 = s32[i + 4];
+      v = make_uint4(__builtin_amdgcn_alignbit(a1, a0, 16), __builtin_amdgcn_alignbit(a2, a1, 16),
+                     __builtin_amdgcn_alignbit(a3, a2, 16), __builtin_amdgcn_alignbit(a4, a3, 16));
+    }
+    if ((w & 1) && i + 4 == nd) v.w &= 0xFFFFu;  // the padding word of an odd count is zero
+    wdst[i] = v.x;
+    wdst[i + 1] = v.y;
+    wdst[i + 2] = v.z;
+    wdst[i + 3] = v.w;
+  }
+  for (uint32_t i = nd4 + t; i < nd; i += NT) {
+    uint32_t v = mis ? __builtin_amdgcn_alignbit(s32[i + 1], s32[i], 16) : s32[i];
+    if ((w & 1) && i == nd - 1) v &= 0xFFFFu;
+    wdst[i] = v;
+  }
+}
 
 // Segments of up to 8 * NG symbols per lane: the exponents stay in registers.
 // Workgroup = max(4, segments per chunk) wavefronts; wavefront k owns segment k.
@@ -823,8 +952,11 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   // every segment of the chunk is coded: decide coded-or-raw and size the records
   __threadfence_block();
   __syncthreads();
-  if (tid == 0) L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
-                                          reinterpret_cast<uint32_t*>(it.ws + it.chunk_units));
+  if (tid == 0) {
+    L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
+                              reinterpret_cast<uint32_t*>(it.ws + it.chunk_units), L.seg_units, &L.chunk_total);
+    L.gave_up = 0;
+  }
   __syncthreads();
   if (L.raw && has_seg) {
     // a chunk that does not compress: its exponent bytes take the place of the words
@@ -836,6 +968,65 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
       const uint32_t idx0 = (gv * NZ_LANES + lane) * NZ_GROUP;
       if (idx0 < seg_n) *reinterpret_cast<uint64_t*>(rawp + idx0) = ex[g8];
     });
+  }
+  if (!it.direct) return;  // the records are placed by nz_compact_kernel
+
+  // ---- the records go straight to their place ----
+  // The chunk announces the size of its records: two words, each with half of
+  // the call's 64-bit mark on top and the size (or its complement) below, so
+  // that whatever the scratch memory held before cannot pass for an
+  // announcement.  Then it adds up the announcements of the chunks before it,
+  // waiting for those that are not there yet.  Workgroups start in the order of
+  // their numbers, so every chunk waited for is running or done, and none of
+  // them waits before it has announced; the wait is bounded all the same
+  // (`spin_limit` looks per announcement): a chunk that gives up says so and
+  // leaves its records where they are, for nz_compact_kernel.  Nothing but
+  // the announcements passes between workgroups: relaxed device-scope
+  // accesses, no fences.
+  typedef unsigned long long nz_u64;
+  nz_u64* pub = reinterpret_cast<nz_u64*>(it.ws + it.pub);
+  const uint32_t mark_a = (uint32_t)(it.nonce >> 32), mark_b = (uint32_t)it.nonce;
+  if (tid == 0) {
+    const uint32_t u = L.chunk_total;
+    __hip_atomic_store(pub + 2 * c, ((nz_u64)mark_a << 32) | u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(pub + 2 * c + 1, ((nz_u64)mark_b << 32) | (uint32_t)~u, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+  }
+  uint64_t part = 0;
+  bool lost = false;
+  for (uint64_t i = tid; i < c && !lost; i += blockDim.x) {
+    for (uint32_t tries = 0;; ++tries) {
+      const nz_u64 a = __hip_atomic_load(pub + 2 * i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const nz_u64 q = __hip_atomic_load(pub + 2 * i + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if ((uint32_t)(a >> 32) == mark_a && (uint32_t)(q >> 32) == mark_b && (uint32_t)a == (uint32_t)~(uint32_t)q) {
+        part += (uint32_t)a;
+        break;
+      }
+      if (tries >= it.spin_limit) {
+        lost = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
+    }
+  }
+  if (lost) L.gave_up = 1;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) part += __shfl_xor((nz_u64)part, o, 64);
+  if (lane == 0) L.red64[wave] = part;
+  __threadfence_block();  // also: the raw bytes above are read back by the move
+  __syncthreads();
+  if (L.gave_up) {
+    if (tid == 0) {
+      atomicOr(it.d_status, 4u);
+      if (it.d_gave_up) *it.d_gave_up = it.nonce;
+    }
+    return;
+  }
+  if (has_seg) {
+    uint64_t o0 = 0;
+    for (uint32_t q = 0; q < blockDim.x / 64; ++q) o0 += L.red64[q];
+    for (uint32_t q = 0; q < wave; ++q) o0 += L.seg_units[q];
+    nz_move_record<64>(it, seg, c, wave, o0, L.seg_units[wave], info[c], seg_state_bytes[seg], seg_words[seg], lane);
   }
 }
 
@@ -944,7 +1135,8 @@ __global__ __launch_bounds__(NZ_ENC_LONG_THREADS) void nz_encode_long_kernel(con
   __threadfence_block();
   __syncthreads();
   if (tid == 0) L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
-                                          reinterpret_cast<uint32_t*>(it.ws + it.chunk_units));
+                                          reinterpret_cast<uint32_t*>(it.ws + it.chunk_units), L.seg_units,
+                                          &L.chunk_total);
   __syncthreads();
   if (L.raw && has_seg) {
     // a chunk that does not compress: its exponent bytes take the place of the words
@@ -966,25 +1158,6 @@ __device__ __forceinline__ uint64_t nz_block_sum64(uint64_t v, uint64_t* red4) {
   if ((threadIdx.x & 63) == 0) red4[threadIdx.x >> 6] = v;
   __syncthreads();
   return red4[0] + red4[1] + red4[2] + red4[3];
-}
-
-__device__ __forceinline__ void nz_write_header(uint8_t* comp, const NzGeom& g, uint64_t total) {
-  uint32_t* h = reinterpret_cast<uint32_t*>(comp);
-  h[0] = NZ_MAGIC;
-  h[1] = NZ_FORMAT_VERSION;
-  h[2] = (uint32_t)(g.n & 0xFFFFFFFFu);
-  h[3] = (uint32_t)(g.n >> 32);
-  h[4] = g.chunk_syms;
-  h[5] = g.lane_syms;
-  h[6] = (uint32_t)g.n_chunks;
-  h[7] = (uint32_t)g.n_segs;
-  h[8] = (uint32_t)g.dir_off;
-  h[9] = (uint32_t)g.rec_off;
-  h[10] = (uint32_t)(total & 0xFFFFFFFFu);
-  h[11] = (uint32_t)(total >> 32);
-  h[12] = h[13] = h[14] = h[15] = 0;
-  // the alignment gap between directory and records
-  for (uint64_t b = g.dir_off + 4 * (g.n_segs + 1); b < g.rec_off; ++b) comp[b] = 0;
 }
 
 // Container size of every tensor of the batch from the record sizes of its
@@ -1017,9 +1190,7 @@ __global__ __launch_bounds__(256) void nz_total_kernel(const NzEncBatch b) {
 // ----------------------------------------------------------------------------
 // The workgroup of segment k of chunk c finds where its record goes by itself:
 // the record sizes of all chunks before c (one number per chunk, left by the
-// encode kernel) plus those of the segments before k in c.  It writes its own
-// directory entry; the workgroup of the last segment adds the closing entry,
-// the header, the container size and the overflow flag.
+// encode kernel) plus those of the segments before k in c.
 __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   __shared__ uint64_t red4[4];
   uint32_t t = 0, first = 0;
@@ -1030,16 +1201,10 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   const NzEncItem& it = b.item[t];
   const NzGeom& g = it.g;
   const NzChunkInfo* __restrict__ info = reinterpret_cast<const NzChunkInfo*>(it.ws + it.info);
-  const uint8_t* __restrict__ tab_ser = it.ws + it.tab_ser;
-  const uint8_t* __restrict__ carry = it.ws + it.carry;
-  const uint16_t* __restrict__ slots = reinterpret_cast<const uint16_t*>(it.ws + it.slots);
-  const uint32_t* __restrict__ states = reinterpret_cast<const uint32_t*>(it.ws + it.states);
   const uint32_t* __restrict__ seg_words = reinterpret_cast<const uint32_t*>(it.ws + it.seg_words);
   const uint32_t* __restrict__ seg_state_bytes = reinterpret_cast<const uint32_t*>(it.ws + it.seg_sbytes);
   const uint32_t* __restrict__ seg_units = reinterpret_cast<const uint32_t*>(it.ws + it.seg_units);
   const uint32_t* __restrict__ chunk_units = reinterpret_cast<const uint32_t*>(it.ws + it.chunk_units);
-  uint8_t* __restrict__ comp = it.comp;
-  const uint64_t cap = it.comp_cap;
   const uint64_t seg = blockIdx.x - first;
   const uint64_t c = seg / g.spc;
   const uint32_t k = (uint32_t)(seg - c * g.spc);
@@ -1052,76 +1217,8 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   const NzChunkInfo ci = info[c];
   const uint32_t sbytes = seg_state_bytes[seg];
   const uint32_t w = seg_words[seg];
-  const uint64_t o0 = nz_block_sum64(part, red4), o1 = o0 + mine;
-  const bool fits = o1 <= 0xFFFFFFFFull && g.rec_off + 4 * o1 + NZ_TAIL_PAD <= cap;
-  if (seg + 1 == g.n_segs && tid == 0) {
-    const uint64_t total = g.rec_off + 4 * o1 + NZ_TAIL_PAD;
-    *it.d_total = total;
-    if (!fits) atomicOr(it.d_status, 1u);
-  }
-  if (!fits) return;  // (a record before this one may still fit and be written: harmless)
-  uint32_t* dir = reinterpret_cast<uint32_t*>(comp + g.dir_off);
-  if (tid == 0) dir[seg] = (uint32_t)o0;
-  uint8_t* dst = comp + g.rec_off + 4 * o0;
-  if (seg + 1 == g.n_segs) {
-    if (tid == 0) {
-      dir[g.n_segs] = (uint32_t)o1;
-      nz_write_header(comp, g, g.rec_off + 4 * o1 + NZ_TAIL_PAD);
-    }
-    if (tid >= 256 - NZ_TAIL_PAD) comp[g.rec_off + 4 * o1 + (tid - (256 - NZ_TAIL_PAD))] = 0;  // closing zeros
-  }
-  const uint64_t seg_base = c * g.chunk_syms + (uint64_t)k * g.seg_syms;
-  const uint32_t nom = nz_seg_nominal(g.chunk_syms, g.seg_syms, g.spc, k);
-  const uint32_t sn = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
-  if (ci.raw) {
-    uint32_t off = 0;
-    if (k == 0) {
-      if (tid < 4) dst[tid] = tid == 0 ? NZ_MODE_RAW : 0;
-      off = 4;
-    }
-    const uint32_t padded = (sn + 3) & ~3u;
-    const uint8_t* rawp = reinterpret_cast<const uint8_t*>(slots + seg * g.seg_syms);  // left there by the encode kernel
-    for (uint32_t i = tid; i < padded; i += 256) dst[off + i] = i < sn ? rawp[i] : 0;
-    if (sn == nom && tid < NZ_CARRY_BYTES) dst[off + padded + tid] = carry[seg * NZ_CARRY_BYTES + tid];
-    return;
-  }
-  uint32_t off = 0;
-  if (k == 0) {
-    const uint8_t* t = tab_ser + c * NZ_TABLE_MAX_BYTES;
-    for (uint32_t i = tid; i < ci.tab_len; i += 256) dst[i] = t[i];
-    off = ci.tab_len;
-  }
-  uint32_t* sdst = reinterpret_cast<uint32_t*>(dst + off);
-  if (tid < sbytes / 4) sdst[tid] = states[seg * (NZ_STATE_MAX_BYTES / 4) + tid];
-  const uint32_t cap_words = g.seg_syms;
-  // the words sit at the end of the segment's slot, 2-byte aligned; they are moved
-  // as dwords (two aligned loads and a funnel shift when the source is off by one
-  // word; the load past the last word stays inside the scratch buffer)
-  const uint16_t* src = slots + seg * cap_words + (cap_words - w);
-  const uint32_t mis = (uint32_t)((reinterpret_cast<uintptr_t>(src) >> 1) & 1u);
-  const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src - mis);
-  uint32_t* wdst = reinterpret_cast<uint32_t*>(dst + off + sbytes);
-  const uint32_t nd = (w + 1) / 2;
-  const uint32_t nd4 = nd & ~3u;  // four dwords per thread and turn, then the last one to three singly
-  for (uint32_t i = 4 * tid; i < nd4; i += 4 * 256) {
-    const uint32_t a0 = s32[i], a1 = s32[i + 1], a2 = s32[i + 2], a3 = s32[i + 3];
-    uint4 v = make_uint4(a0, a1, a2, a3);
-    if (mis) {
-      const uint32_t a4 = s32[i + 4];
-      v = make_uint4(__builtin_amdgcn_alignbit(a1, a0, 16), __builtin_amdgcn_alignbit(a2, a1, 16),
-                     __builtin_amdgcn_alignbit(a3, a2, 16), __builtin_amdgcn_alignbit(a4, a3, 16));
-    }
-    if ((w & 1) && i + 4 == nd) v.w &= 0xFFFFu;  // the padding word of an odd count is zero
-    wdst[i] = v.x;
-    wdst[i + 1] = v.y;
-    wdst[i + 2] = v.z;
-    wdst[i + 3] = v.w;
-  }
-  for (uint32_t i = nd4 + tid; i < nd; i += 256) {
-    uint32_t v = mis ? __builtin_amdgcn_alignbit(s32[i + 1], s32[i], 16) : s32[i];
-    if ((w & 1) && i == nd - 1) v &= 0xFFFFu;
-    wdst[i] = v;
-  }
+  const uint64_t o0 = nz_block_sum64(part, red4);
+  nz_move_record<256>(it, seg, c, k, o0, mine, ci, sbytes, w, tid);
 }
 
 // ----------------------------------------------------------------------------

@@ -584,3 +584,48 @@ def test_rewrite_in_place_needs_no_size_round_trip(oracle):
     assert torch.equal(mgr.read(h), flat[: n // 2])
     assert mgr._be.rewrite_stats() == (batches + 2, 1)
     mgr._be.check()
+
+
+def test_records_are_placed_again_when_a_workgroup_gives_up_waiting(oracle):
+    """The encode kernel places its records itself; a workgroup waits for the
+    record sizes of the chunks before its own, and gives up after a bounded
+    number of looks.  With that number forced to zero from the host, workgroups
+    whose predecessors are not done at their first look give up (every kernel
+    still runs to its end): the records are then placed by the second kernel,
+    at once in nz_encode, at the next use in a manager, and the stored bytes
+    are the oracle's either way."""
+    import neuzip_amd
+    from neuzip_amd import _lib
+    from test_gpu_parity import gpu_encode
+
+    L = _lib.load()
+    n = 40 * 131072 + 777                       # 41 chunks
+    bits = bf16_bits_normal(n, seed=21)
+    o_comp, o_packed = oracle.compress_bf16(bits, 7, 131072, 256)
+    mgr = neuzip_amd.Manager()
+    w = from_bits(bits, (n,))
+    h = mgr.write(w)                            # sized to fit: the two-kernel route
+    try:
+        L.nz_set_lookback_spins(0)
+        print("case stateless encode, spin limit 0", flush=True)
+        comp, packed = gpu_encode(bits, 7)
+        assert np.array_equal(comp.cpu().numpy(), o_comp) and np.array_equal(packed.cpu().numpy(), o_packed)
+        print("case in-place rewrites, spin limit 0", flush=True)
+        w2 = (w.float() * 1.001).to(torch.bfloat16)
+        o2_comp, o2_packed = oracle.compress_bf16(bits_of(w2), 7, 131072, 256)
+        for _ in range(3):
+            mgr.write(w2, h)
+            assert torch.equal(mgr.read(h), w2)
+            comp, packed, _ = mgr._be.export(h)
+            assert np.array_equal(comp.numpy(), o2_comp) and np.array_equal(packed.numpy(), o2_packed)
+        again = mgr._be.placed_again()
+        print(f"placed again: {again} of 3", flush=True)
+    finally:
+        L.nz_set_lookback_spins(1 << 21)
+    before = mgr._be.placed_again()
+    mgr.write(w, h)                             # with the usual bound nothing gives up
+    assert torch.equal(mgr.read(h), w)
+    comp, packed, _ = mgr._be.export(h)
+    assert np.array_equal(comp.numpy(), o_comp) and np.array_equal(packed.numpy(), o_packed)
+    assert mgr._be.placed_again() == before
+    mgr._be.check()
