@@ -46,7 +46,7 @@ uint64_t norm_bytes_of(uint64_t n, uint32_t ns) { return ns ? (n + ns - 1) / ns 
 
 // Device scratch of one encode call.
 struct EncLayout {
-  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units, pub, bytes;
+  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units, pub, placed, bytes;
 };
 
 // segments short enough for the kernel that keeps the exponents in registers
@@ -71,6 +71,7 @@ EncLayout enc_layout(const NzGeom& g) {
   L.seg_units = take((g.n_segs + 1) * 4);
   L.chunk_units = take((g.n_chunks + 1) * 4);
   L.pub = take(g.n_chunks * 16);  // size announcements of the chunks (records placed by the encode kernel)
+  L.placed = take(g.n_segs);      // per segment: its record is in the container only
   L.bytes = o;
   return L;
 }
@@ -127,6 +128,9 @@ NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws
   it.seg_units = L.seg_units;
   it.chunk_units = L.chunk_units;
   it.pub = L.pub;
+  it.placed = L.placed;
+  it.old_comp = nullptr;
+  it.use_placed = 0;
   it.nonce = next_nonce();
   it.d_gave_up = nullptr;
   it.direct = (comp != nullptr && g.n_segs != 0 && enc_in_registers(g)) ? 1u : 0u;
@@ -149,15 +153,52 @@ bool enc_batch_close(NzEncBatch* b) {
 
 // One encode launch for the tensors of `b` whose segments are of class `cls`
 // (0..2: up to 64 / 128 / 256 symbols per lane, coded from registers; 3: longer).
+// nz_encode_kernel<S, NG> with `lds` bytes of dynamic LDS (word staging).  More
+// than 64 KiB of LDS per workgroup has to be allowed once per kernel and device.
+template <int S, int NG>
+int launch_encode_reg(const NzEncBatch& b, dim3 grid, dim3 block, uint32_t lds, hipStream_t st) {
+  static std::atomic<uint64_t> allowed{0};  // bit d: done on device d
+  int dev = 0;
+  NZ_HIP(hipGetDevice(&dev));
+  if (lds && dev >= 0 && dev < 64 && !((allowed.load(std::memory_order_relaxed) >> dev) & 1ull)) {
+    NZ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&nz_encode_kernel<S, NG>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    allowed.fetch_or(1ull << dev, std::memory_order_relaxed);
+  }
+  hipLaunchKernelGGL((nz_encode_kernel<S, NG>), grid, block, lds, st, b);
+  return NZ_OK;
+}
+
+// Words of LDS staging per wavefront for a direct encode of class `cls` with
+// workgroups of `waves` wavefronts: what a workgroup can have without lowering
+// the number of workgroups that the registers allow per compute unit (4, 6, 8
+// wavefronts per SIMD unit for 256, 128, 64 symbols per lane), less the
+// kernel's own 17 KiB.
+uint32_t stage_words_for(int cls, uint32_t waves) {
+  const uint32_t waves_per_cu = cls == 2 ? 16u : cls == 1 ? 24u : 32u;
+  const uint32_t groups = waves_per_cu / waves ? waves_per_cu / waves : 1u;
+  const uint32_t per_group = 160u * 1024u / groups;
+  const uint32_t fixed = 17u * 1024u;
+  if (per_group <= fixed + 1024u) return 0;
+  const uint32_t per_wave = ((per_group - fixed - 64u) / waves) & ~511u;  // bytes
+  return per_wave / 2;
+}
+
 template <int S>
-void launch_encode_class(const NzEncBatch& b, int cls, uint32_t chunks, uint32_t max_spc, hipStream_t st) {
-  const dim3 grid(chunks), block(64 * (max_spc < 4 ? 4 : max_spc));
+int launch_encode_class(NzEncBatch& b, int cls, uint32_t chunks, uint32_t max_spc, hipStream_t st) {
+  const uint32_t waves = max_spc < 4 ? 4 : max_spc;
+  const dim3 grid(chunks), block(64 * waves);
+  bool direct = false;
+  for (uint32_t i = 0; i < b.count; ++i) direct = direct || b.item[i].direct;
+  b.stage_words = (direct && cls < 3) ? stage_words_for(cls, waves) : 0u;
+  const uint32_t lds = b.stage_words ? waves * b.stage_words * 2u + 16u : 0u;
   switch (cls) {
-    case 0: hipLaunchKernelGGL((nz_encode_kernel<S, 8>), grid, block, 0, st, b); break;
-    case 1: hipLaunchKernelGGL((nz_encode_kernel<S, 16>), grid, block, 0, st, b); break;
-    case 2: hipLaunchKernelGGL((nz_encode_kernel<S, 32>), grid, block, 0, st, b); break;
+    case 0: return launch_encode_reg<S, 8>(b, grid, block, lds, st);
+    case 1: return launch_encode_reg<S, 16>(b, grid, block, lds, st);
+    case 2: return launch_encode_reg<S, 32>(b, grid, block, lds, st);
     default: hipLaunchKernelGGL((nz_encode_long_kernel<S>), grid, dim3(NZ_ENC_LONG_THREADS), 0, st, b); break;
   }
+  return NZ_OK;
 }
 
 int enc_class(const NzGeom& g) {
@@ -185,12 +226,14 @@ int encode_phase1(NzEncBatch* b, int precision, uint32_t ns, hipStream_t st) {
       if (it.g.spc > max_spc) max_spc = it.g.spc;
     }
     if (!sub.count) continue;
+    int rc;
     switch (precision) {
-      case 7: launch_encode_class<7>(sub, cls, chunks, max_spc, st); break;
-      case 3: launch_encode_class<3>(sub, cls, chunks, max_spc, st); break;
-      case 1: launch_encode_class<1>(sub, cls, chunks, max_spc, st); break;
-      default: launch_encode_class<0>(sub, cls, chunks, max_spc, st); break;
+      case 7: rc = launch_encode_class<7>(sub, cls, chunks, max_spc, st); break;
+      case 3: rc = launch_encode_class<3>(sub, cls, chunks, max_spc, st); break;
+      case 1: rc = launch_encode_class<1>(sub, cls, chunks, max_spc, st); break;
+      default: rc = launch_encode_class<0>(sub, cls, chunks, max_spc, st); break;
     }
+    if (rc) return rc;
   }
   NZ_HIP(hipGetLastError());
   return NZ_OK;
@@ -227,10 +270,14 @@ int encode_phase2(NzEncBatch* b, hipStream_t st) {
 
 // The records of item i again, by nz_compact_kernel from what the encode kernel
 // left in the scratch (into another buffer, or after a chunk gave up waiting).
-int encode_replace(const NzEncItem& item, hipStream_t st) {
+// `placed_in`: the container the direct encode wrote to (records that went there
+// from LDS exist nowhere else and are copied from it).
+int encode_replace(const NzEncItem& item, const uint8_t* placed_in, hipStream_t st) {
   NzEncBatch one{};
   one.count = 1;
   one.item[0] = item;
+  one.item[0].use_placed = item.direct;
+  one.item[0].old_comp = placed_in;
   one.item[0].direct = 0;
   return encode_phase2(&one, st);
 }
@@ -527,7 +574,7 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
     NZ_HIP(hipStreamSynchronize(st));
     if (hs & 4u) {
       // a chunk gave up waiting for the sizes before it: the records once more, by the compaction
-      if (int rc = encode_replace(item, st)) return rc;
+      if (int rc = encode_replace(item, item.comp, st)) return rc;
       NZ_HIP(hipMemcpyAsync(host_total, dev_total, 8, hipMemcpyDeviceToHost, st));
       NZ_HIP(hipMemcpyAsync(&hs, dev_status, 4, hipMemcpyDeviceToHost, st));
       NZ_HIP(hipStreamSynchronize(st));
@@ -847,7 +894,7 @@ int settle_slot(nz_manager* m, int k) {
     if (s.h_totals[16 + j] == s.b.item[j].nonce) {
       // a chunk gave up waiting for the sizes before it: the records once more, by the compaction
       ++m->rewrites_redone;
-      if (int rc = encode_replace(s.b.item[j], s.stream)) return rc;
+      if (int rc = encode_replace(s.b.item[j], s.b.item[j].comp, s.stream)) return rc;
       NZ_HIP(hipMemcpyAsync(s.h_totals + j, s.d_totals + j, 8, hipMemcpyDeviceToHost, s.stream));
       NZ_HIP(hipStreamSynchronize(s.stream));
       total = s.h_totals[j];
@@ -864,7 +911,7 @@ int settle_slot(nz_manager* m, int k) {
     NzEncItem again = s.b.item[j];
     again.comp = (uint8_t*)bigger;
     again.comp_cap = cap;
-    if (int rc = encode_replace(again, s.stream)) return rc;
+    if (int rc = encode_replace(again, s.b.item[j].comp, s.stream)) return rc;
     NZ_HIP(hipStreamSynchronize(s.stream));
     (void)hipFree(ent.comp);
     ent.comp = bigger;

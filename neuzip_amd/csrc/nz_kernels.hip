@@ -351,6 +351,7 @@ struct NzEncLds {
   // sum over the chunks before it, whether the wait for those was given up
   uint32_t seg_units[NZ_MAX_SEGS_PER_CHUNK];
   uint32_t chunk_total, gave_up;
+  uint32_t redo;  // a wavefront ran out of staging room: the chunk is coded again, into the slots
   uint64_t red64[NZ_ENC_LONG_THREADS / 64];
 };
 
@@ -421,8 +422,10 @@ __device__ __forceinline__ uint64_t nz_split_tail(const uint16_t* __restrict__ i
 // From the chunk's histogram (cn symbols): the 12-bit frequency table (sum
 // exactly 4096), the encoder's per-symbol entries in LDS, the serialized table
 // and the chunk record.  Run by the whole workgroup (at least 256 threads).
-__device__ __forceinline__ void nz_build_table(NzEncLds& L, const uint32_t cn, uint8_t* __restrict__ out,
-                                               NzChunkInfo* __restrict__ info_c) {
+// -> an estimate of the chunk's coded length in bits (sum of count x -log2 of
+// the quantised probability), the same in every thread.
+__device__ __forceinline__ uint32_t nz_build_table(NzEncLds& L, const uint32_t cn, uint8_t* __restrict__ out,
+                                                   NzChunkInfo* __restrict__ info_c) {
   const uint32_t tid = threadIdx.x;
   // threads 0..255 own one symbol each; the others take part in the reductions
   // with neutral values
@@ -441,6 +444,7 @@ __device__ __forceinline__ void nz_build_table(NzEncLds& L, const uint32_t cn, u
   const uint32_t imax = 255u - (key & 0xFFu);
   if (tid == imax) f += NZ_M - sum;
   if (k == 1) f = (tid == imax) ? (NZ_M - 1) : ((tid == (imax ^ 1u)) ? 1u : 0u);
+  const uint32_t est_bits = nz_block_sum(live ? (uint32_t)((float)cnt * (12.0f - __log2f((float)f))) + 1u : 0u, L.red);
 
   // exclusive prefix sum over the 256 symbols
   uint32_t incl = f;
@@ -538,6 +542,7 @@ __device__ __forceinline__ void nz_build_table(NzEncLds& L, const uint32_t cn, u
     L.pad_sym = imax;
   }
   __syncthreads();
+  return est_bits;
 }
 
 // ----------------------------------------------------------------------------
@@ -593,8 +598,13 @@ __device__ __forceinline__ bool nz_chunk_finalize(uint64_t c, uint64_t n, uint32
 // kernel, once all segments of the chunk are coded).
 
 // the 8 symbols of one group (byte j of `sy` = symbol j), last symbol first
+// (words go to the segment's slot in scratch memory, or with LDS to the
+// wavefront's staging area: word p of the slot at LDS byte address lds0 + 2 p)
+template <bool LDS>
 __device__ __forceinline__ void nz_enc_group(uint32_t& x, uint32_t& pos, const uint64_t sy,
-                                             const uint4* __restrict__ tab, uint16_t* __restrict__ slot) {
+                                             const uint4* __restrict__ tab, uint16_t* __restrict__ slot,
+                                             const uint32_t lds0) {
+  typedef __attribute__((address_space(3))) uint16_t lds_u16;
   // the table entries do not depend on the state: fetch four at a time, up front
 #pragma unroll
   for (int h = 1; h >= 0; --h) {
@@ -607,9 +617,13 @@ __device__ __forceinline__ void nz_enc_group(uint32_t& x, uint32_t& pos, const u
     const bool need = x >= e[j].x;
     const uint64_t m = __ballot(need);
     pos -= (uint32_t)__popcll(m);
-    if (need)  // a 32-bit byte offset from the segment's slot: one add-shift for the address
-      *reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(slot) + ((pos + nz_rank_below(m)) << 1)) =
-          (uint16_t)(x & 0xFFFFu);
+    if (need) {  // a 32-bit byte offset from the segment's slot: one add-shift for the address
+      if constexpr (LDS)
+        *(lds_u16*)(uintptr_t)(lds0 + ((pos + nz_rank_below(m)) << 1)) = (uint16_t)(x & 0xFFFFu);
+      else
+        *reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(slot) + ((pos + nz_rank_below(m)) << 1)) =
+            (uint16_t)(x & 0xFFFFu);
+    }
     x = need ? (x >> 16) : x;
     // x < f << 20 here, so the quotient x / f is below 2^20.  The float estimate
     // x * r with r four units in the last place under 1 / f (itself within half
@@ -679,9 +693,17 @@ struct NzEncItem {
   uint64_t pub, nonce;
   uint64_t* d_gave_up;
   uint32_t direct, spin_limit;
+  // `placed`: one byte per segment (offset into ws), left by a direct encode: 1 =
+  // the record is in the container and not in the scratch (its words went there
+  // from LDS).  nz_compact_kernel with `use_placed` takes such records from
+  // `old_comp`, where they lie at the offsets they keep.
+  uint64_t placed;
+  const uint8_t* old_comp;
+  uint32_t use_placed, reserved;
 };
 struct NzEncBatch {
-  uint32_t count, reserved;
+  uint32_t count;
+  uint32_t stage_words;  // nz_encode_kernel: 16-bit words of LDS staging per wavefront (dynamic LDS), 0 = none
   NzEncItem item[NZ_ENC_BATCH_MAX];
 };
 
@@ -711,14 +733,18 @@ __device__ __forceinline__ void nz_write_header(uint8_t* comp, const NzGeom& g, 
 // NT threads (t = 0 .. NT-1) move the record of segment `seg` = segment k of
 // chunk c to o0, counted in 4-byte units from the start of the record area
 // (`mine` = its size in the same units; ci, sbytes, w: the chunk's info, the
-// size of the coder states, the number of words).  They write the segment's
-// directory entry; those of the last segment add the closing entry, the
-// header, the container size and the overflow flag.
+// size of the coder states, the number of words; `words`: where the words are,
+// the end of the segment's slot or a staging area in LDS).  With `whole` the
+// record is not assembled from its parts but copied from there (the same record
+// in another container).  They write the segment's directory entry; those of
+// the last segment add the closing entry, the header, the container size and
+// the overflow flag.  -> whether the record fits the container (if not, nothing
+// of it is written).
 template <uint32_t NT>
-__device__ __forceinline__ void nz_move_record(const NzEncItem& it, const uint64_t seg, const uint64_t c,
+__device__ __forceinline__ bool nz_move_record(const NzEncItem& it, const uint64_t seg, const uint64_t c,
                                                const uint32_t k, const uint64_t o0, const uint32_t mine,
                                                const NzChunkInfo ci, const uint32_t sbytes, const uint32_t w,
-                                               const uint32_t t) {
+                                               const uint16_t* words, const uint8_t* whole, const uint32_t t) {
   static_assert(NT >= NZ_TAIL_PAD, "too few threads for the closing zeros");
   const NzGeom& g = it.g;
   const uint8_t* __restrict__ tab_ser = it.ws + it.tab_ser;
@@ -733,7 +759,7 @@ __device__ __forceinline__ void nz_move_record(const NzEncItem& it, const uint64
     *it.d_total = total;
     if (!fits) atomicOr(it.d_status, 1u);
   }
-  if (!fits) return;  // (a record before this one may still fit and be written: harmless)
+  if (!fits) return false;  // (a record before this one may still fit and be written: harmless)
   uint32_t* dir = reinterpret_cast<uint32_t*>(comp + g.dir_off);
   if (t == 0) dir[seg] = (uint32_t)o0;
   uint8_t* dst = comp + g.rec_off + 4 * o0;
@@ -743,6 +769,12 @@ __device__ __forceinline__ void nz_move_record(const NzEncItem& it, const uint64
       nz_write_header(comp, g, g.rec_off + 4 * o1 + NZ_TAIL_PAD);
     }
     if (t < NZ_TAIL_PAD) comp[g.rec_off + 4 * o1 + t] = 0;  // closing zeros
+  }
+  if (whole) {
+    if (whole != dst)
+      for (uint32_t i = t; i < mine; i += NT)
+        reinterpret_cast<uint32_t*>(dst)[i] = reinterpret_cast<const uint32_t*>(whole)[i];
+    return true;
   }
   const uint64_t seg_base = c * g.chunk_syms + (uint64_t)k * g.seg_syms;
   const uint32_t nom = nz_seg_nominal(g.chunk_syms, g.seg_syms, g.spc, k);
@@ -758,7 +790,7 @@ __device__ __forceinline__ void nz_move_record(const NzEncItem& it, const uint64
     for (uint32_t i = t; i < padded; i += NT) dst[off + i] = i < sn ? rawp[i] : 0;
     if (sn == nom)
       for (uint32_t i = t; i < NZ_CARRY_BYTES; i += NT) dst[off + padded + i] = carry[seg * NZ_CARRY_BYTES + i];
-    return;
+    return true;
   }
   uint32_t off = 0;
   if (k == 0) {
@@ -768,11 +800,10 @@ __device__ __forceinline__ void nz_move_record(const NzEncItem& it, const uint64
   }
   uint32_t* sdst = reinterpret_cast<uint32_t*>(dst + off);
   for (uint32_t i = t; i < sbytes / 4; i += NT) sdst[i] = states[seg * (NZ_STATE_MAX_BYTES / 4) + i];
-  const uint32_t cap_words = g.seg_syms;
-  // the words sit at the end of the segment's slot, 2-byte aligned; they are moved
-  // as dwords (two aligned loads and a funnel shift when the source is off by one
-  // word; the load past the last word stays inside the scratch buffer)
-  const uint16_t* src = slots + seg * cap_words + (cap_words - w);
+  // the words are 2-byte aligned; they are moved as dwords (two aligned loads and a
+  // funnel shift when the source is off by one word; the load past the last word
+  // stays inside the scratch buffer or the staging area)
+  const uint16_t* src = words;
   const uint32_t mis = (uint32_t)((reinterpret_cast<uintptr_t>(src) >> 1) & 1u);
   const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src - mis);
   uint32_t* wdst = reinterpret_cast<uint32_t*>(dst + off + sbytes);
@@ -797,10 +828,12 @@ __device__ __forceinline__ void nz_move_record(const NzEncItem& it, const uint64
     if ((w & 1) && i == nd - 1) v &= 0xFFFFu;
     wdst[i] = v;
   }
+  return true;
 }
 
 // Segments of up to 8 * NG symbols per lane: the exponents stay in registers.
 // Workgroup = max(4, segments per chunk) wavefronts; wavefront k owns segment k.
+extern __shared__ uint32_t nz_enc_stage[];  // word staging of nz_encode_kernel: stage_words / 2 dwords per wavefront + 4
 template <int S, int NG>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kernel(const NzEncBatch b) {
   __shared__ NzEncLds L;
@@ -835,6 +868,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   const bool seg_full = has_seg && seg_n == nom;
 
   for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += blockDim.x) L.hist[i] = 0;
+  if (tid == 0) L.redo = 0;
   __syncthreads();
   uint32_t* myhist = L.hist + (lane & (NZ_HIST_COPIES - 1)) * NZ_HIST_STRIDE;
 
@@ -919,39 +953,75 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   __syncthreads();
 
   // ---- the chunk's table ----
-  nz_build_table(L, cn, it.ws + it.tab_ser + c * NZ_TABLE_MAX_BYTES, info + c);
+  const uint32_t est_bits = nz_build_table(L, cn, it.ws + it.tab_ser + c * NZ_TABLE_MAX_BYTES, info + c);
 
   // ---- phase 2: code the segment from the registers, last group first ----
+  // The words go to the segment's slot in scratch memory, or, when the records
+  // are placed by this kernel and the estimate says they fit, to the wavefront's
+  // staging area in LDS (the last `stage_w` words of the slot), from where they
+  // are written once, to their final place.  A wavefront that would run out of
+  // staging stops; the chunk is then coded again into the slots (the exponents
+  // are still in registers).
   const uint32_t cap_words = seg_syms;
   uint16_t* slot = reinterpret_cast<uint16_t*>(it.ws + it.slots) + seg * cap_words;
-  if (has_seg) {
+  const uint32_t stage_w = b.stage_words < cap_words ? b.stage_words : cap_words;
+  const uint32_t stage_lo = cap_words - stage_w;  // first word of the slot that has a place in the staging area
+  const uint32_t est_seg_words = (uint32_t)(((uint64_t)est_bits * seg_syms / cn) >> 4);
+  bool staged = it.direct && stage_w >= 1024 && est_seg_words + (est_seg_words >> 4) + 64 <= stage_w;
+  typedef __attribute__((address_space(3))) uint32_t lds_u32;
+  uint32_t* stage = nz_enc_stage + wave * (b.stage_words / 2);
+  const uint32_t stage_lds = (uint32_t)(uintptr_t)((lds_u32*)stage);
+  uint32_t pos_end = cap_words;  // where the segment's words begin in its slot
+  const auto code_segment = [&](auto lds_tag) -> bool {
+    constexpr bool LDS = decltype(lds_tag)::value != 0;
     const uint32_t pad = L.pad_sym;
     // a full segment starts from 2^16 | 16 carried bits of the packed stream
     uint32_t x = NZ_L | (seg_full ? (uint32_t)reinterpret_cast<const uint16_t*>(carry_seg)[lane] : 0u);
     uint32_t pos = cap_words;
+    bool out_of_room = false;
     nz_static_for<NG - 1, 0, -1>([&](auto g8c) {
       constexpr int g8 = decltype(g8c)::value;
       uint32_t gv = (uint32_t)g8;
       asm volatile("" : "+s"(gv));
-      if (gv < ngroups) {
-        uint64_t sy = ex[g8];
-        if (gv >= whole) {  // the tensor ends inside this group: the most frequent symbol stands in
-          const uint32_t idx0 = (gv * NZ_LANES + lane) * NZ_GROUP;
-          const uint32_t have = idx0 < seg_n ? seg_n - idx0 : 0u;  // < 8 in some lane
-          if (have < 8) {
-            const uint64_t keepm = have ? (~0ull >> (64 - 8 * have)) : 0ull;
-            sy = (sy & keepm) | ((0x0101010101010101ull * pad) & ~keepm);
+      if (gv < ngroups && !out_of_room) {
+        if (LDS && pos - stage_lo < NZ_GROUP * NZ_LANES) {  // a group emits at most 512 words
+          out_of_room = true;
+        } else {
+          uint64_t sy = ex[g8];
+          if (gv >= whole) {  // the tensor ends inside this group: the most frequent symbol stands in
+            const uint32_t idx0 = (gv * NZ_LANES + lane) * NZ_GROUP;
+            const uint32_t have = idx0 < seg_n ? seg_n - idx0 : 0u;  // < 8 in some lane
+            if (have < 8) {
+              const uint64_t keepm = have ? (~0ull >> (64 - 8 * have)) : 0ull;
+              sy = (sy & keepm) | ((0x0101010101010101ull * pad) & ~keepm);
+            }
           }
+          nz_enc_group<LDS>(x, pos, sy, L.tab, slot, stage_lds - 2u * stage_lo);
         }
-        nz_enc_group(x, pos, sy, L.tab, slot);
       }
     });
+    if (out_of_room) return true;
     nz_enc_finish(x, cap_words - pos, seg, L.sbuf[wave], lane, reinterpret_cast<uint32_t*>(it.ws + it.states),
                   seg_words, seg_state_bytes);
+    pos_end = pos;
+    return false;
+  };
+#pragma nounroll
+  for (int pass = 0; pass < 2; ++pass) {
+    if (has_seg) {
+      if (staged) {
+        if (code_segment(NzConst<1>{})) L.redo = 1;
+      } else {
+        code_segment(NzConst<0>{});
+      }
+    }
+    // every segment of the chunk is coded (or one has run out of staging)
+    __threadfence_block();
+    __syncthreads();
+    if (!(staged && L.redo)) break;
+    staged = false;
   }
-  // every segment of the chunk is coded: decide coded-or-raw and size the records
-  __threadfence_block();
-  __syncthreads();
+  // decide coded-or-raw and size the records
   if (tid == 0) {
     L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
                               reinterpret_cast<uint32_t*>(it.ws + it.chunk_units), L.seg_units, &L.chunk_total);
@@ -1015,10 +1085,20 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   if (lane == 0) L.red64[wave] = part;
   __threadfence_block();  // also: the raw bytes above are read back by the move
   __syncthreads();
+  // staged words of this wavefront to their slot, for the kernel that places records afterwards
+  const auto unstage = [&]() {
+    const uint16_t* sw = reinterpret_cast<const uint16_t*>(stage);
+    for (uint32_t p = pos_end + lane; p < cap_words; p += NZ_LANES) slot[p] = sw[p - stage_lo];
+  };
+  uint8_t* placed = it.ws + it.placed;  // per segment: its record is in the container and nowhere else
   if (L.gave_up) {
     if (tid == 0) {
       atomicOr(it.d_status, 4u);
       if (it.d_gave_up) *it.d_gave_up = it.nonce;
+    }
+    if (has_seg) {
+      if (staged && !L.raw) unstage();
+      if (lane == 0) placed[seg] = 0;
     }
     return;
   }
@@ -1026,7 +1106,12 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     uint64_t o0 = 0;
     for (uint32_t q = 0; q < blockDim.x / 64; ++q) o0 += L.red64[q];
     for (uint32_t q = 0; q < wave; ++q) o0 += L.seg_units[q];
-    nz_move_record<64>(it, seg, c, wave, o0, L.seg_units[wave], info[c], seg_state_bytes[seg], seg_words[seg], lane);
+    const bool from_stage = staged && !L.raw;
+    const uint16_t* words = from_stage ? reinterpret_cast<const uint16_t*>(stage) + (pos_end - stage_lo) : slot + pos_end;
+    const bool fits = nz_move_record<64>(it, seg, c, wave, o0, L.seg_units[wave], info[c], seg_state_bytes[seg],
+                                         cap_words - pos_end, words, nullptr, lane);
+    if (from_stage && !fits) unstage();
+    if (lane == 0) placed[seg] = (from_stage && fits) ? 1 : 0;
   }
 }
 
@@ -1127,7 +1212,7 @@ __global__ __launch_bounds__(NZ_ENC_LONG_THREADS) void nz_encode_long_kernel(con
           sy |= (uint64_t)bb << (8 * j);
         }
       }
-      nz_enc_group(x, pos, sy, L.tab, slot);
+      nz_enc_group<false>(x, pos, sy, L.tab, slot, 0u);
     }
     nz_enc_finish(x, cap_words - pos, seg, L.sbuf[wave], lane, reinterpret_cast<uint32_t*>(it.ws + it.states),
                   seg_words, seg_state_bytes);
@@ -1217,8 +1302,11 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   const NzChunkInfo ci = info[c];
   const uint32_t sbytes = seg_state_bytes[seg];
   const uint32_t w = seg_words[seg];
+  const bool in_old = it.use_placed && (it.ws + it.placed)[seg] != 0;
   const uint64_t o0 = nz_block_sum64(part, red4);
-  nz_move_record<256>(it, seg, c, k, o0, mine, ci, sbytes, w, tid);
+  const uint16_t* words = reinterpret_cast<const uint16_t*>(it.ws + it.slots) + seg * g.seg_syms + (g.seg_syms - w);
+  nz_move_record<256>(it, seg, c, k, o0, mine, ci, sbytes, w, words,
+                      in_old ? it.old_comp + g.rec_off + 4 * o0 : nullptr, tid);
 }
 
 // ----------------------------------------------------------------------------

@@ -230,3 +230,30 @@ def test_decode_output_policy_flags(oracle):
                          out.data_ptr(), status.data_ptr(), m.DECODE_STREAM_OUT | m.DECODE_RESIDENT_OUT, 0, None,
                          torch.cuda.current_stream().cuda_stream)
         assert rc == m.ERR_ARG and "exclude" in m.last_error()
+
+
+@pytest.mark.parametrize("lane,chunk", [(256, 131072), (128, 65536), (64, 32768)])
+def test_segment_that_outgrows_its_word_staging(oracle, lane, chunk):
+    """The encode kernel keeps a segment's words in LDS when the chunk's histogram
+    says they fit.  A chunk whose exponents are constant except for one segment of
+    uniformly random ones has a small estimate and one segment that emits several
+    times the staging room: that chunk is coded a second time, through scratch
+    memory, and the bytes are the oracle's all the same (as are those of its
+    ordinary neighbours)."""
+    rng = np.random.default_rng(lane)
+    n = 5 * chunk + 999
+    seg = 64 * lane
+    bits = bf16_bits_normal(n, seed=lane + 1)
+    odd = slice(2 * chunk, 3 * chunk)                    # chunk 2: exponent 120 everywhere ...
+    b = bits[odd]
+    b = (b & 0x807F) | (120 << 7)
+    hot = slice(3 * seg, 4 * seg)                        # ... but in its fourth segment any exponent
+    b[hot] = (b[hot] & 0x807F) | (rng.integers(0, 255, seg).astype(np.uint16) << 7)
+    bits[odd] = b
+    print(f"case lane={lane} chunk={chunk}", flush=True)
+    comp, packed = gpu_encode(bits, 7, chunk, lane)
+    o_comp, o_packed = oracle.compress_bf16(bits, 7, chunk, lane)
+    assert np.array_equal(packed.cpu().numpy(), o_packed)
+    assert np.array_equal(comp.cpu().numpy(), o_comp)
+    rc, out = gpu_decode(comp, packed, n, 7, chunk, lane)
+    assert rc == 0 and np.array_equal(out, bits)
