@@ -209,7 +209,7 @@ class Workspace:
         return st
 
     def encode_into(self, dense, s, st: Stored) -> None:
-        """The three encode launches again, asynchronously, into the buffers of `st`."""
+        """The encode again, asynchronously, into the buffers of `st`."""
         self._encode(dense, s, st.packed, st.comp, st.comp.numel(), False)
 
     def decode(self, st: Stored, out, check=False, flags=0):
