@@ -153,18 +153,37 @@ bool enc_batch_close(NzEncBatch* b) {
 
 // One encode launch for the tensors of `b` whose segments are of class `cls`
 // (0..2: up to 64 / 128 / 256 symbols per lane, coded from registers; 3: longer).
-// nz_encode_kernel<S, NG> with `lds` bytes of dynamic LDS (word staging).  More
-// than 64 KiB of LDS per workgroup has to be allowed once per kernel and device.
+// The register encode kernels may use more than 64 KiB of LDS per workgroup
+// (word staging): that has to be allowed once per kernel and device, and is
+// done for all of them before the first encode on a device.
 template <int S, int NG>
-int launch_encode_reg(const NzEncBatch& b, dim3 grid, dim3 block, uint32_t lds, hipStream_t st) {
+hipError_t allow_encode_lds_one() {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(&nz_encode_kernel<S, NG>),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+}
+template <int S>
+hipError_t allow_encode_lds_s() {
+  hipError_t e = allow_encode_lds_one<S, 8>();
+  if (e == hipSuccess) e = allow_encode_lds_one<S, 16>();
+  if (e == hipSuccess) e = allow_encode_lds_one<S, 32>();
+  return e;
+}
+int allow_encode_lds() {
   static std::atomic<uint64_t> allowed{0};  // bit d: done on device d
   int dev = 0;
   NZ_HIP(hipGetDevice(&dev));
-  if (lds && dev >= 0 && dev < 64 && !((allowed.load(std::memory_order_relaxed) >> dev) & 1ull)) {
-    NZ_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(&nz_encode_kernel<S, NG>),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-    allowed.fetch_or(1ull << dev, std::memory_order_relaxed);
-  }
+  if (dev < 0 || dev >= 64) return fail(NZ_ERR_ARG, "device index out of range");
+  if ((allowed.load(std::memory_order_acquire) >> dev) & 1ull) return NZ_OK;
+  NZ_HIP(allow_encode_lds_s<7>());
+  NZ_HIP(allow_encode_lds_s<3>());
+  NZ_HIP(allow_encode_lds_s<1>());
+  NZ_HIP(allow_encode_lds_s<0>());
+  allowed.fetch_or(1ull << dev, std::memory_order_release);
+  return NZ_OK;
+}
+
+template <int S, int NG>
+int launch_encode_reg(const NzEncBatch& b, dim3 grid, dim3 block, uint32_t lds, hipStream_t st) {
   hipLaunchKernelGGL((nz_encode_kernel<S, NG>), grid, block, lds, st, b);
   return NZ_OK;
 }
@@ -209,6 +228,7 @@ int enc_class(const NzGeom& g) {
 // + directory land in each item's `hdr`, the container size in its *d_total.
 int encode_phase1(NzEncBatch* b, int precision, uint32_t ns, hipStream_t st) {
   if (!enc_batch_close(b)) return fail(NZ_ERR_ARG, "too many chunks for one launch");
+  if (int rc = allow_encode_lds()) return rc;
   for (uint32_t i = 0; i < b->count; ++i)
     if (int rc = launch_absmax(b->item[i].in, b->item[i].g.n, ns, const_cast<uint8_t*>(b->item[i].nm.bytes), st))
       return rc;
