@@ -629,3 +629,32 @@ def test_records_are_placed_again_when_a_workgroup_gives_up_waiting(oracle):
     assert np.array_equal(comp.numpy(), o_comp) and np.array_equal(packed.numpy(), o_packed)
     assert mgr._be.placed_again() == before
     mgr._be.check()
+
+
+def test_in_place_rewrites_of_two_managers_on_two_streams(oracle):
+    """Two managers re-compress their tensors at the same time on streams of
+    their own (encode kernels of both are resident together; each places its own
+    records): every read returns what was written last."""
+    import neuzip_amd
+
+    n = 24 * 131072 + 5
+    mgrs = [neuzip_amd.Manager(), neuzip_amd.Manager(precision=3)]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]  # default priority
+    base = [from_bits(bf16_bits_normal(n, seed=40 + i), (n,)) for i in range(2)]
+    hs = [m.write(w) for m, w in zip(mgrs, base)]
+    torch.cuda.synchronize()
+    last = [None, None]
+    for it in range(12):
+        for i in (0, 1):
+            with torch.cuda.stream(streams[i]):
+                w = (base[i].float() * (1.0 + 0.002 * (it + 1))).to(torch.bfloat16)
+                mgrs[i].write(w, hs[i])
+                last[i] = w
+    for i in (0, 1):
+        with torch.cuda.stream(streams[i]):
+            got = mgrs[i].read(hs[i])
+            want = from_bits(oracle.reconstruct(bits_of(last[i]), 7 if i == 0 else 3), (n,))
+        streams[i].synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+        assert mgrs[i]._be.placed_again() == 0
+        mgrs[i]._be.check()
