@@ -272,6 +272,16 @@ int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indi
    elements per frequency table and symbols per rANS lane and segment. */
 int nz_manager_geometry(nz_manager* m, const char* name, uint32_t* chunk_size, uint32_t* lane_syms);
 
+/* No counterpart in the reference (its chunk size is one constructor argument,
+   neuzip/binding.py:56-62).  The next writes under `name` use this geometry
+   instead of the manager's own choice; (0, 0) takes the hint back.  For tensors
+   that are always decoded together by one launch (nz_manager_gemv_batch,
+   nz_manager_read_batch): the launch is fastest when the chunks of all of them
+   together are a whole number of workgroups per compute unit, which no choice
+   per tensor can know (neuzip_amd.FusedGemv.trace uses it).  The write under
+   `name` must be serialised with this call by the caller. */
+int nz_manager_geometry_hint(nz_manager* m, const char* name, uint32_t chunk_size, uint32_t lane_syms);
+
 /* meta_cache lookup, cuda/high_level.cu:42-43,228-230. */
 int nz_manager_meta(nz_manager* m, const char* name, uint64_t* numel, int* dtype);
 

@@ -31,7 +31,7 @@ EXPORTS = [
     "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
     "nz_manager_meta", "nz_manager_geometry", "nz_manager_size", "nz_manager_size_reference", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
     "nz_manager_norm_bytes", "nz_manager_buffers", "nz_manager_erase", "nz_manager_check",
-    "nz_manager_export", "nz_manager_import", "nz_manager_trim", "nz_manager_rewrite_stats", "nz_set_lookback_spins",
+    "nz_manager_export", "nz_manager_import", "nz_manager_trim", "nz_manager_rewrite_stats", "nz_set_lookback_spins", "nz_manager_geometry_hint",
 ]
 
 _lib = None
@@ -85,6 +85,8 @@ def load() -> ctypes.CDLL:
     L.nz_manager_read.argtypes = [vp, ctypes.c_char_p, vp, u64, vp]
     L.nz_manager_rewrite_stats.restype = i32
     L.nz_manager_rewrite_stats.argtypes = [vp, ctypes.POINTER(u64), ctypes.POINTER(u64), ctypes.POINTER(u64)]
+    L.nz_manager_geometry_hint.restype = i32
+    L.nz_manager_geometry_hint.argtypes = [vp, ctypes.c_char_p, ctypes.c_uint32, ctypes.c_uint32]
     L.nz_set_lookback_spins.restype = None
     L.nz_set_lookback_spins.argtypes = [ctypes.c_uint32]
     L.nz_manager_trim.restype = i32

@@ -41,6 +41,7 @@ class _HipBackend:
     def __init__(self, precision: int, normalizer_size: int, chunk_size: int, lane_symbols: int):
         self._L = _lib.load()
         self._h = ctypes.c_void_p()
+        self.auto_geometry = lane_symbols == "auto" and not chunk_size
         if lane_symbols == "auto":
             lane_symbols = _lib.LANE_SYMS_AUTO
         rc = self._L.nz_manager_create(_lib.ALGO_ANS, precision, normalizer_size, chunk_size,
@@ -125,6 +126,10 @@ class _HipBackend:
         c, l = ctypes.c_uint32(), ctypes.c_uint32()
         _lib.raise_for(self._L.nz_manager_geometry(self._h, handle.encode(), ctypes.byref(c), ctypes.byref(l)))
         return int(c.value), int(l.value)
+
+    def geometry_hint(self, handle: str, chunk_size: int, lane_symbols: int) -> None:
+        """The next writes under ``handle`` use this geometry; (0, 0) takes the hint back."""
+        _lib.raise_for(self._L.nz_manager_geometry_hint(self._h, handle.encode(), chunk_size, lane_symbols))
 
     def read_into(self, handle: str, out: torch.Tensor) -> torch.Tensor:
         """Decompress into caller-provided bf16 storage (no allocation), on the current stream."""

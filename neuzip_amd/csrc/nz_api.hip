@@ -508,6 +508,7 @@ struct nz_manager {
   bool auto_lanes = false;  // pick the geometry per tensor so that small tensors still fill the GPU
   uint32_t slots = 768;     // decode workgroups of eight wavefronts the device holds at once (3 per CU)
   std::unordered_map<std::string, Entry> entries;  // compress_cache + meta_cache
+  std::unordered_map<std::string, std::pair<uint32_t, uint32_t>> hints;  // name -> (chunk, lane) for its next writes
   std::mutex mu;
   void* ws = nullptr;
   uint64_t ws_bytes = 0;
@@ -761,8 +762,15 @@ void release_entry(Entry& e) {
 // In auto mode a tensor too small to give every SIMD two wavefronts at the
 // default gets shorter segments (and, with the library's own chunk, the smaller
 // 64 Ki table scope that allows them), at ~4.5 bits per extra lane.
-int pick_geometry(const nz_manager* m, uint64_t n, NzGeom* g, uint32_t* chunk_out, uint32_t* lane_out) {
+int pick_geometry(const nz_manager* m, const char* name, uint64_t n, NzGeom* g, uint32_t* chunk_out,
+                  uint32_t* lane_out) {
   uint32_t lane_syms = m->lane_syms, chunk_syms = m->chunk_syms;
+  const auto hint = m->hints.find(name);
+  if (hint != m->hints.end()) {  // nz_manager_geometry_hint
+    *chunk_out = hint->second.first;
+    *lane_out = hint->second.second;
+    return make_geom(g, n, *chunk_out, *lane_out);
+  }
   if (m->auto_lanes && m->own_chunk && chunk_syms == NZ_DEFAULT_CHUNK && lane_syms == NZ_DEFAULT_LANE_SYMS) {
     // The device holds `slots` decode workgroups (three per compute unit) at
     // once, and a launch is fastest when every compute unit has the same number
@@ -982,7 +990,7 @@ int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* 
       if (std::strcmp(names[i], names[j]) == 0) return fail(NZ_ERR_ARG, "a name appears twice in the batch");
     if (ns[i] && !dev_data[i]) return fail(NZ_ERR_ARG, "null data pointer");
     if ((uintptr_t)dev_data[i] & 15) return fail(NZ_ERR_ALIGN, "dense input must be 16-byte aligned");
-    if (int rc = pick_geometry(m, ns[i], &g[i], &chunk[i], &lane[i])) return rc;
+    if (int rc = pick_geometry(m, names[i], ns[i], &g[i], &chunk[i], &lane[i])) return rc;
     at[i + 1] = at[i] + enc_layout(g[i]).bytes;
   }
   std::lock_guard<std::mutex> lock(m->mu);
@@ -1305,6 +1313,21 @@ int nz_manager_geometry(nz_manager* m, const char* name, uint32_t* chunk_size, u
   if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
   if (chunk_size) *chunk_size = it->second.chunk_syms;
   if (lane_syms) *lane_syms = it->second.lane_syms;
+  return NZ_OK;
+}
+
+int nz_manager_geometry_hint(nz_manager* m, const char* name, uint32_t chunk_size, uint32_t lane_syms) {
+  if (!m || !name) return fail(NZ_ERR_ARG, "null manager or name");
+  std::lock_guard<std::mutex> lock(m->mu);
+  if (chunk_size == 0 && lane_syms == 0) {
+    m->hints.erase(name);
+    return NZ_OK;
+  }
+  if (nz_geom_check(chunk_size, lane_syms))
+    return fail(NZ_ERR_ARG,
+                "unsupported geometry: lane_syms must be a multiple of 8 (>= 16), chunk_size a multiple "
+                "of 512 cut into 1..8 segments of 64*lane_syms, the last one at least 1024 long");
+  m->hints[name] = std::make_pair(chunk_size, lane_syms);
   return NZ_OK;
 }
 

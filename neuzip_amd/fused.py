@@ -68,9 +68,11 @@ class FusedGemv:
         for k, h in enumerate(handles):
             self._where[h] = (g, k)
 
-    def trace(self, fn) -> None:
+    def trace(self, fn, regroup: bool = True) -> None:
         """Run ``fn()`` once on the ordinary path and group the Linears that were
-        called back to back with the very same single-row input tensor."""
+        called back to back with the very same single-row input tensor.  With a
+        manager that chooses the geometry per tensor, the matrices of a group
+        are then stored again with a geometry chosen for the group (``regroup``)."""
         self._recording = []
         was = self._enabled
         self.enable()
@@ -93,6 +95,44 @@ class FusedGemv:
         for h in self._layers:
             if h not in self._where:
                 self._add_group([h])
+        if regroup and getattr(self.manager._be, "auto_geometry", False):
+            for g in self._groups:
+                if len(g.handles) > 1:
+                    self._fit_geometry(g)
+
+    # Step time of a wavefront (ns) with one, two, three 8-wavefront workgroups per
+    # compute unit, measured on MI355X; the same figures choose a tensor's geometry
+    # when it is written on its own.
+    _STEP_NS = (107, 147, 215)
+
+    def _fit_geometry(self, g) -> None:
+        """Matrices that one launch decodes together are stored again with ONE
+        geometry under which their chunks are a whole number of workgroups per
+        compute unit (at most three, what a unit holds): chosen per tensor, two
+        512-chunk matrices are a round of 768 workgroups and a poorly filled second."""
+        be = self.manager._be
+        cus = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+        sizes = [be.numel(h) for h in g.handles]
+        best = None
+        for k in (1, 2, 3):
+            lane = -(-sum(sizes) // (k * cus * 512 * 8)) * 8
+            while lane <= 512 and sum(-(-n // (lane * 512)) for n in sizes) > k * cus:
+                lane += 8  # every tensor's last chunk is rounded up
+            if not 64 <= lane <= 512:
+                continue
+            t = lane * self._STEP_NS[k - 1]
+            if best is None or t <= best[0]:  # measured on gate/up of an 8B model: 2 x 512 chunks 73-76 us, 2 x 256 71.5, 2 x 378 69.4
+                best = (t, lane)
+        if best is None:
+            return
+        lane = best[1]
+        chunk = lane * 512
+        if all(be.geometry(h) == (chunk, lane) for h in g.handles):
+            return
+        for h in g.handles:
+            dense = self.manager.read(h)
+            be.geometry_hint(h, chunk, lane)
+            self.manager.write(dense, h)
 
     # -- context management ---------------------------------------------------
     def enable(self):

@@ -233,3 +233,45 @@ def test_raw_chunks_through_product_gather_and_normalizers():
         # the sums are resolved to 2^-40; the bf16 result to half a unit in the last place
         assert bool(((y.double() - ref).abs() <= 2.0 ** -8 * ref.abs() + 2.0 ** -40).all())
         mgr._be.check()
+
+
+def test_group_geometry_is_refitted_and_results_stay_the_same():
+    """FusedGemv.trace stores the matrices of a group again with one geometry
+    chosen for the group (manager with per-tensor geometry); later writes under
+    those handles keep it; the stored values do not change."""
+    import neuzip_amd
+
+    class Pair(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = torch.nn.Linear(2048, 6144, bias=False)
+            self.b = torch.nn.Linear(2048, 6144, bias=True)
+
+        def forward(self, x):
+            return self.a(x) + self.b(x)
+
+    torch.manual_seed(11)
+    model = Pair().to(torch.bfloat16)
+    for p in model.parameters():
+        p.data.normal_(0, 0.02)
+    mgr = neuzip_amd.Manager(lane_symbols="auto")
+    mgr.convert(model)
+    model = model.cuda()
+    ha, hb = model.a.weight._handle, model.b.weight._handle
+    wa, wb = mgr.read(ha).clone(), mgr.read(hb).clone()
+    before = mgr._be.geometry(ha)
+    x = torch.randn(1, 2048, device="cuda", dtype=torch.bfloat16)
+    fused = neuzip_amd.FusedGemv(mgr, model)
+    with torch.no_grad():
+        want = model(x)
+        fused.trace(lambda: model(x))
+        after = mgr._be.geometry(ha)
+        print(f"geometry {before} -> {after}", flush=True)
+        assert after == mgr._be.geometry(hb) and after[0] == 512 * after[1]
+        assert torch.equal(mgr.read(ha), wa) and torch.equal(mgr.read(hb), wb)
+        with fused:
+            got = model(x)
+        assert torch.allclose(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+        mgr.write(wa * 2, ha)                      # a later write keeps the group's geometry
+        assert mgr._be.geometry(ha) == after and torch.equal(mgr.read(ha), wa * 2)
+    mgr._be.check()
