@@ -46,7 +46,7 @@ uint64_t norm_bytes_of(uint64_t n, uint32_t ns) { return ns ? (n + ns - 1) / ns 
 
 // Device scratch of one encode call.
 struct EncLayout {
-  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units, pub, placed, bytes;
+  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units, pub, placed, lb_state, bytes;
 };
 
 // segments short enough for the kernel that keeps the exponents in registers
@@ -72,6 +72,7 @@ EncLayout enc_layout(const NzGeom& g) {
   L.chunk_units = take((g.n_chunks + 1) * 4);
   L.pub = take(g.n_chunks * 16);  // size announcements of the chunks (records placed by the encode kernel)
   L.placed = take(g.n_segs);      // per segment: its record is in the container only
+  L.lb_state = take(8);           // run count and abort mark of the announcements
   L.bytes = o;
   return L;
 }
@@ -129,6 +130,7 @@ NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws
   it.chunk_units = L.chunk_units;
   it.pub = L.pub;
   it.placed = L.placed;
+  it.lb_state = L.lb_state;
   it.old_comp = nullptr;
   it.use_placed = 0;
   it.nonce = next_nonce();

@@ -674,6 +674,7 @@ __device__ __forceinline__ void nz_enc_finish(const uint32_t x, const uint32_t w
 // concatenation of their chunks, that of the scan kernel one workgroup per
 // tensor, that of the compaction the concatenation of their segments.
 #define NZ_ENC_BATCH_MAX 16
+#define NZ_LOOKBACK_ABORT 0xAB0F7EDDu
 struct NzEncItem {
   const uint16_t* in;   // dense input
   uint8_t* packed;      // stored sign|mantissa stream
@@ -693,6 +694,15 @@ struct NzEncItem {
   uint64_t pub, nonce;
   uint64_t* d_gave_up;
   uint32_t direct, spin_limit;
+  // two words in ws (offset): [0] counts the direct encodes that have used this
+  // scratch, advanced by the workgroup of the last chunk - the announcements'
+  // mark is made of it and the nonce, so those of an earlier run of the very
+  // same call (a replayed graph) do not pass for this run's; [1] holds
+  // NZ_LOOKBACK_ABORT after a run in which a workgroup gave up: the next run
+  // then leaves the placing to nz_compact_kernel as well (and says so through
+  // the same flags) and takes the mark away.  Whatever the memory held
+  // before its first use is as good a start as any.
+  uint64_t lb_state;
   // `placed`: one byte per segment (offset into ws), left by a direct encode: 1 =
   // the record is in the container and not in the scratch (its words went there
   // from LDS).  nz_compact_kernel with `use_placed` takes such records from
@@ -867,6 +877,15 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;  // at most NG
   const bool seg_full = has_seg && seg_n == nom;
 
+  // state of the scratch's size announcements (see NzEncItem::lb_state), read
+  // long before it is needed
+  uint32_t* lb_state = reinterpret_cast<uint32_t*>(it.ws + it.lb_state);
+  uint32_t lb_gen = 0;
+  bool direct = false;  // this run places its records itself
+  if (it.direct) {
+    lb_gen = __hip_atomic_load(lb_state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    direct = __hip_atomic_load(lb_state + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != NZ_LOOKBACK_ABORT;
+  }
   for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += blockDim.x) L.hist[i] = 0;
   if (tid == 0) L.redo = 0;
   __syncthreads();
@@ -967,7 +986,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   const uint32_t stage_w = b.stage_words < cap_words ? b.stage_words : cap_words;
   const uint32_t stage_lo = cap_words - stage_w;  // first word of the slot that has a place in the staging area
   const uint32_t est_seg_words = (uint32_t)(((uint64_t)est_bits * seg_syms / cn) >> 4);
-  bool staged = it.direct && stage_w >= 1024 && est_seg_words + (est_seg_words >> 4) + 64 <= stage_w;
+  bool staged = direct && stage_w >= 1024 && est_seg_words + (est_seg_words >> 4) + 64 <= stage_w;
   typedef __attribute__((address_space(3))) uint32_t lds_u32;
   uint32_t* stage = nz_enc_stage + wave * (b.stage_words / 2);
   const uint32_t stage_lds = (uint32_t)(uintptr_t)((lds_u32*)stage);
@@ -1040,10 +1059,26 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     });
   }
   if (!it.direct) return;  // the records are placed by nz_compact_kernel
+  uint8_t* placed = it.ws + it.placed;  // per segment: its record is in the container and nowhere else
+  const bool last_chunk = c + 1 == g.n_chunks;
+  if (!direct) {
+    // the run before this one ended with a workgroup giving up: nothing is
+    // placed, the caller is told, and the mark is taken away for the next run
+    if (tid == 0) {
+      atomicOr(it.d_status, 4u);
+      if (it.d_gave_up) *it.d_gave_up = it.nonce;
+      if (last_chunk) {
+        __hip_atomic_store(lb_state, lb_gen + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(lb_state + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    if (has_seg && lane == 0) placed[seg] = 0;
+    return;
+  }
 
   // ---- the records go straight to their place ----
   // The chunk announces the size of its records: two words, each with half of
-  // the call's 64-bit mark on top and the size (or its complement) below, so
+  // the run's 64-bit mark on top and the size (or its complement) below, so
   // that whatever the scratch memory held before cannot pass for an
   // announcement.  Then it adds up the announcements of the chunks before it,
   // waiting for those that are not there yet.  Workgroups start in the order of
@@ -1055,7 +1090,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   // accesses, no fences.
   typedef unsigned long long nz_u64;
   nz_u64* pub = reinterpret_cast<nz_u64*>(it.ws + it.pub);
-  const uint32_t mark_a = (uint32_t)(it.nonce >> 32), mark_b = (uint32_t)it.nonce;
+  const uint32_t mark_a = (uint32_t)(it.nonce >> 32) ^ lb_gen, mark_b = (uint32_t)it.nonce ^ (lb_gen * 0x9E3779B1u);
   if (tid == 0) {
     const uint32_t u = L.chunk_total;
     __hip_atomic_store(pub + 2 * c, ((nz_u64)mark_a << 32) | u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1090,11 +1125,14 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     const uint16_t* sw = reinterpret_cast<const uint16_t*>(stage);
     for (uint32_t p = pos_end + lane; p < cap_words; p += NZ_LANES) slot[p] = sw[p - stage_lo];
   };
-  uint8_t* placed = it.ws + it.placed;  // per segment: its record is in the container and nowhere else
+  // the workgroup of the last chunk has seen every other announce (or has given
+  // up): all of them have read the count, which can now move on
   if (L.gave_up) {
     if (tid == 0) {
+      __hip_atomic_store(lb_state + 1, NZ_LOOKBACK_ABORT, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       atomicOr(it.d_status, 4u);
       if (it.d_gave_up) *it.d_gave_up = it.nonce;
+      if (last_chunk) __hip_atomic_store(lb_state, lb_gen + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (has_seg) {
       if (staged && !L.raw) unstage();
@@ -1102,6 +1140,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     }
     return;
   }
+  if (last_chunk && tid == 0)
+    __hip_atomic_store(lb_state, lb_gen + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   if (has_seg) {
     uint64_t o0 = 0;
     for (uint32_t q = 0; q < blockDim.x / 64; ++q) o0 += L.red64[q];

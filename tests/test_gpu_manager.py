@@ -622,6 +622,9 @@ def test_records_are_placed_again_when_a_workgroup_gives_up_waiting(oracle):
         print(f"placed again: {again} of 3", flush=True)
     finally:
         L.nz_set_lookback_spins(1 << 21)
+    for _ in range(2):                          # a scratch in which a workgroup gave up is marked: the next encode
+        mgr.write(w2, h)                        # that uses it (one per rewrite slot) leaves the placing to the second
+        assert torch.equal(mgr.read(h), w2)     # kernel once more and takes the mark away
     before = mgr._be.placed_again()
     mgr.write(w, h)                             # with the usual bound nothing gives up
     assert torch.equal(mgr.read(h), w)

@@ -257,3 +257,46 @@ def test_segment_that_outgrows_its_word_staging(oracle, lane, chunk):
     assert np.array_equal(comp.cpu().numpy(), o_comp)
     rc, out = gpu_decode(comp, packed, n, 7, chunk, lane)
     assert rc == 0 and np.array_equal(out, bits)
+
+
+def test_encode_replayed_from_a_graph(oracle):
+    """nz_encode captured into a HIP graph and replayed on new contents of the same
+    buffers: every replay runs the very same call (same arguments, same scratch),
+    so the size announcements of the replay before carry this call's mark; the
+    run count kept in the scratch tells them apart.  Every replay's bytes are the
+    oracle's."""
+    L, m = _lib()
+    n, s, chunk, lane = 9 * 131072 + 4321, 7, 131072, 256
+    d_in = torch.zeros(n, dtype=torch.int16, device="cuda")
+    cap = L.nz_exp_bound_bytes(n, chunk, lane)
+    ws_bytes = L.nz_encode_workspace_bytes(n, chunk, lane)
+    comp = torch.zeros(cap, dtype=torch.uint8, device="cuda")
+    stored = L.nz_packed_stored_bytes(n, s, chunk, lane)
+    packed = torch.zeros(stored, dtype=torch.uint8, device="cuda")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+    aux = torch.zeros(4, dtype=torch.int64, device="cuda")
+
+    def encode():
+        rc = L.nz_encode(d_in.data_ptr(), n, s, chunk, lane, packed.data_ptr(), comp.data_ptr(), cap,
+                         ws.data_ptr(), ws_bytes, aux.data_ptr(), aux.data_ptr() + 8, None, 0, None,
+                         torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, m.last_error()
+
+    encode()                                     # outside the capture first (one-time set-up of the kernels)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        encode()
+    for rep in range(4):
+        # different data every time, sizes of the chunks included (the exponent spread changes)
+        bits = bf16_bits_normal(n, seed=100 + rep) if rep % 2 == 0 else stress_bits(n // 1024 + 1, 1024, seed=rep)[:n]
+        d_in.copy_(_to_dev(bits))
+        print(f"case graph replay {rep}", flush=True)
+        g.replay()
+        torch.cuda.synchronize()
+        assert int(aux[1].item()) & 0xFFFFFFFF == 0
+        total = int(aux[0].item())
+        o_comp, o_packed = oracle.compress_bf16(bits, s, chunk, lane)
+        assert total == o_comp.size
+        assert np.array_equal(comp[:total].cpu().numpy(), o_comp)
+        assert np.array_equal(packed.cpu().numpy(), o_packed)
