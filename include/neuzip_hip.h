@@ -107,7 +107,10 @@ int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fr
    (device uint32, OR-ed into) stays zero when the container is complete: bit 0
    = it did not fit, bit 2 = a workgroup gave up waiting for the record sizes
    of the chunks before its own (see nz_set_lookback_spins; the container is
-   then incomplete and the call has to be made again).  If `host_total` is not
+   then incomplete and the call has to be made again; the workspace is marked,
+   and the next call that uses it sets bit 2 once more and takes the mark
+   away).  The call may be captured into a HIP graph and replayed: the
+   workspace keeps a count of the runs that have used it.  If `host_total` is not
    NULL the call synchronises the stream, returns the size and status on the
    host (the reference's get_compressed_output_size sync, :114-115) and deals
    with bit 2 itself. */
