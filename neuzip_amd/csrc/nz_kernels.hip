@@ -180,17 +180,20 @@ __global__ __launch_bounds__(256) void nz_absmax_kernel(const uint16_t* __restri
   uint32_t m8 = 0;
 #pragma unroll
   for (int j = 0; j < 8; ++j) m8 = mag[j] > m8 ? mag[j] : m8;
-  smax[tid] = m8;
-  __syncthreads();
-  const uint32_t per = 1u << (log2n - 3);  // threads per group
-  if (tid < (256u >> (log2n - 3))) {
-    const uint64_t g0 = blk0 + ((uint64_t)tid << log2n);
-    if (g0 < n) {
-      uint32_t m = 0;
-      for (uint32_t q = 0; q < per; ++q) m = smax[tid * per + q] > m ? smax[tid * per + q] : m;
-      norm[g0 >> log2n] = (uint8_t)((m & 0x7Fu) << 1);
-    }
+  // a group is `per` consecutive threads: butterfly inside the wavefront, then
+  // (groups of 1024 elements: two wavefronts) through LDS
+  const uint32_t per = 1u << (log2n - 3);
+  for (uint32_t o = 1; o < per && o < 64; o <<= 1) {
+    const uint32_t other = (uint32_t)__shfl_xor((int)m8, (int)o, 64);
+    m8 = other > m8 ? other : m8;
   }
+  if (per > 64) {
+    if ((tid & 63) == 0) smax[tid >> 6] = m8;
+    __syncthreads();
+    const uint32_t other = smax[(tid >> 6) ^ 1u];
+    m8 = other > m8 ? other : m8;
+  }
+  if ((tid & (per - 1)) == 0 && e0 < n) norm[e0 >> log2n] = (uint8_t)((m8 & 0x7Fu) << 1);
 }
 
 __device__ __forceinline__ uint32_t nz_lane_id() {
