@@ -493,8 +493,9 @@ struct RewriteSlot {
   hipStream_t stream = nullptr;
   void* ws = nullptr;
   uint64_t ws_bytes = 0;
-  uint64_t* d_totals = nullptr;  // device: 16 sizes, then 16 give-up marks (the nonce of the item that gave up)
-  uint64_t* h_totals = nullptr;  // pinned, the same
+  uint64_t* d_totals = nullptr;  // 16 sizes, then 16 give-up marks (the nonce of the item that gave up): pinned host
+                                 // memory, this is its address on the device ...
+  uint64_t* h_totals = nullptr;  // ... and this the one on the host
   uint32_t count = 0;
   std::string names[NZ_ENC_BATCH_MAX];
   NzEncBatch b;
@@ -696,8 +697,13 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   hipError_t e = hipMalloc((void**)&m->d_status, 1024);
   if (e == hipSuccess) e = hipMemset(m->d_status, 0, 1024);
   if (e == hipSuccess) e = hipHostMalloc((void**)&m->h_pin, 1024, hipHostMallocDefault);
+  // the sizes of a rewrite are written by the kernel straight into the pinned block (it is
+  // mapped into the device's address space): no copy has to be enqueued to bring them back
+  void* pin_dev = nullptr;
+  if (e == hipSuccess) e = hipHostGetDevicePointer(&pin_dev, m->h_pin, 0);
+  if (e == hipSuccess) std::memset(m->h_pin, 0, 1024);
   for (int k = 0; k < 2 && e == hipSuccess; ++k) {
-    m->rw[k].d_totals = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(m->d_status) + 256 + 256 * k);
+    m->rw[k].d_totals = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(pin_dev) + 256 + 256 * k);
     m->rw[k].h_totals = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(m->h_pin) + 256 + 256 * k);
     e = hipEventCreateWithFlags(&m->rw[k].ev, hipEventDisableTiming);
   }
@@ -925,7 +931,6 @@ int settle_slot(nz_manager* m, int k) {
       // a chunk gave up waiting for the sizes before it: the records once more, by the compaction
       ++m->rewrites_redone;
       if (int rc = encode_replace(s.b.item[j], s.b.item[j].comp, s.stream)) return rc;
-      NZ_HIP(hipMemcpyAsync(s.h_totals + j, s.d_totals + j, 8, hipMemcpyDeviceToHost, s.stream));
       NZ_HIP(hipStreamSynchronize(s.stream));
       total = s.h_totals[j];
     }
@@ -1040,8 +1045,7 @@ int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* 
     }
     if (int rc = encode_phase1(&s.b, m->precision, m->normalizer, st)) return rc;
     if (int rc = encode_phase2(&s.b, st)) return rc;
-    NZ_HIP(hipMemcpyAsync(s.h_totals, s.d_totals, 256, hipMemcpyDeviceToHost, st));  // sizes, then give-up marks
-    NZ_HIP(hipEventRecord(s.ev, st));
+    NZ_HIP(hipEventRecord(s.ev, st));  // behind it the sizes and give-up marks are in the pinned block
     for (uint32_t i = 0; i < count; ++i) {
       Entry& ent = m->entries.find(names[i])->second;
       ent.pending = k;
