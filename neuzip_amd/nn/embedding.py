@@ -25,6 +25,18 @@ class Embedding(torch.nn.Module):
         self.scale_grad_by_freq = embedding.scale_grad_by_freq
         self.sparse = embedding.sparse
         self._p = Parameter(self.manager, embedding.weight.data)
+        # A lookup decodes whole chunks.  With a manager that chooses the geometry
+        # per tensor, the table is stored with the shortest segments there are
+        # (32 Ki chunks of eight 4 Ki segments): one row of a 128256 x 4096 table
+        # then takes 18 us instead of 39, 512 rows 27 us instead of 55, for 0.6 %
+        # more stored bytes and a slower read of the whole table (424 against 344 us).
+        be = getattr(self.manager, "_be", None)
+        if getattr(be, "auto_geometry", False):
+            h = self._p._handle
+            if be.geometry(h) != (32768, 64):
+                dense = self.manager.read(h)
+                be.geometry_hint(h, 32768, 64)
+                self.manager.write(dense, h)
 
     @property
     def weight(self) -> Parameter:

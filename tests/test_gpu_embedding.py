@@ -141,3 +141,24 @@ def test_large_lookups_are_bounded(oracle):
     assert torch.equal(mgr.gather_rows(h2, many), full2[many])
     assert torch.equal(mgr._be.gather_rows(h2, many[:66_000], dim2), full2[many])
     mgr._be.check()
+
+
+def test_embedding_table_gets_short_segments_under_per_tensor_geometry(oracle):
+    """With a manager that chooses the geometry per tensor, a converted Embedding
+    stores its table in 32 Ki chunks of eight 4 Ki segments (a lookup decodes whole
+    chunks); the rows are the oracle's."""
+    import neuzip_amd
+
+    rows, dim = 5000, 1024          # 5.1 M elements: on its own the table would get longer segments
+    bits = _table_bits(rows, dim, seed=9)
+    emb = torch.nn.Embedding(rows, dim).to(torch.bfloat16)
+    emb.weight.data = _dev(bits, rows, dim).cpu()
+    mgr = neuzip_amd.Manager(lane_symbols="auto")
+    conv = neuzip_amd.nn.Embedding(mgr, emb)
+    h = conv.weight._handle
+    assert mgr._be.geometry(h) == (32768, 64)
+    full = _dev(oracle.reconstruct(bits, 7), rows, dim)
+    idx = torch.randint(0, rows, (3, 17), generator=torch.Generator().manual_seed(2)).cuda()
+    assert torch.equal(conv(idx), full[idx])
+    assert torch.equal(mgr.read(h).view(rows, dim), full)
+    mgr._be.check()
