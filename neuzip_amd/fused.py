@@ -105,13 +105,14 @@ class FusedGemv:
     # when it is written on its own.
     _STEP_NS = (107, 147, 215)
 
-    def _fit_geometry(self, g) -> None:
+    def _fit_geometry(self, g, cus=None) -> None:
         """Matrices that one launch decodes together are stored again with ONE
         geometry under which their chunks are a whole number of workgroups per
         compute unit (at most three, what a unit holds): chosen per tensor, two
         512-chunk matrices are a round of 768 workgroups and a poorly filled second."""
         be = self.manager._be
-        cus = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+        if cus is None:
+            cus = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
         sizes = [be.numel(h) for h in g.handles]
         best = None
         for k in (1, 2, 3):

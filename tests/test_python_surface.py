@@ -219,3 +219,66 @@ def test_reference_package_name_is_importable():
     assert mgr.meta_dict == {} and callable(mgr.convert)
     with pytest.raises(AttributeError, match="Manager_f5_n0"):
         neuzip.Manager(precision=5)
+
+
+def test_group_geometry_choice_is_one_round_of_workgroups():
+    """FusedGemv picks, for matrices that one launch decodes together, a geometry
+    under which their chunks are at most three per compute unit in total, and
+    stores them again only when that differs from what they have (host logic,
+    no GPU: a stand-in backend records the calls)."""
+    from neuzip_amd.fused import FusedGemv, _Group
+
+    class Be:
+        auto_geometry = True
+
+        def __init__(self, sizes, geo):
+            self.sizes, self.geo, self.hints = sizes, dict(geo), {}
+
+        def numel(self, h):
+            return self.sizes[h]
+
+        def geometry(self, h):
+            return self.geo[h]
+
+        def geometry_hint(self, h, chunk, lane):
+            self.hints[h] = (chunk, lane)
+
+    class Mgr:
+        def __init__(self, be):
+            self._be, self.written = be, []
+
+        def read(self, h):
+            return h
+
+        def write(self, dense, h):
+            self.written.append(h)
+            self._be.geo[h] = self._be.hints[h]
+
+    def group_of(handles):
+        g = _Group.__new__(_Group)
+        g.handles = handles
+        return g
+
+    cus = 256
+    for sizes in ({"gate": 14336 * 4096, "up": 14336 * 4096},            # 8B-shaped gate / up
+                  {"q": 4096 * 4096, "k": 1024 * 4096, "v": 1024 * 4096},  # q / k / v
+                  {"a": 3_000_000, "b": 5_000_001}):
+        be = Be(sizes, {h: (131072, 256) for h in sizes})
+        f = FusedGemv.__new__(FusedGemv)
+        f.manager = Mgr(be)
+        f._fit_geometry(group_of(list(sizes)), cus=cus)
+        geos = {be.geo[h] for h in sizes}
+        assert len(geos) == 1
+        chunk, lane = geos.pop()
+        assert chunk == 512 * lane and 64 <= lane <= 512 and lane % 8 == 0
+        chunks = sum(-(-n // chunk) for n in sizes.values())
+        assert chunks <= 3 * cus
+        assert sorted(f.manager.written) == sorted(sizes)
+        f._fit_geometry(group_of(list(sizes)), cus=cus)            # already fitted: nothing is stored again
+        assert sorted(f.manager.written) == sorted(sizes)
+    # gate / up of the 8B shape: 2 x 378 chunks of 304 symbols per lane
+    be = Be({"gate": 14336 * 4096, "up": 14336 * 4096}, {"gate": (114688, 224), "up": (114688, 224)})
+    f = FusedGemv.__new__(FusedGemv)
+    f.manager = Mgr(be)
+    f._fit_geometry(group_of(["gate", "up"]), cus=cus)
+    assert be.geo["gate"] == (304 * 512, 304)
