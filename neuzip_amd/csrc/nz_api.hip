@@ -194,14 +194,14 @@ int launch_encode_reg(const NzEncBatch& b, dim3 grid, dim3 block, uint32_t lds, 
 // workgroups of `waves` wavefronts: what a workgroup can have without lowering
 // the number of workgroups that the registers allow per compute unit (4, 6, 8
 // wavefronts per SIMD unit for 256, 128, 64 symbols per lane), less the
-// kernel's own 17 KiB.
+// kernel's own LDS.
 uint32_t stage_words_for(int cls, uint32_t waves) {
   const uint32_t waves_per_cu = cls == 2 ? 16u : cls == 1 ? 24u : 32u;
   const uint32_t groups = waves_per_cu / waves ? waves_per_cu / waves : 1u;
   const uint32_t per_group = 160u * 1024u / groups;
-  const uint32_t fixed = 17u * 1024u;
+  const uint32_t fixed = ((uint32_t)sizeof(NzEncLds) + 511u) & ~511u;  // the kernel's own LDS
   if (per_group <= fixed + 1024u) return 0;
-  const uint32_t per_wave = ((per_group - fixed - 64u) / waves) & ~511u;  // bytes
+  const uint32_t per_wave = ((per_group - fixed - 512u) / waves) & ~127u;  // bytes (512: the closing slack, rounding)
   return per_wave / 2;
 }
 
