@@ -1,39 +1,77 @@
-"""Compile libneuzip_hip.so for gfx950 with hipcc (cross-compiles without a GPU)."""
+"""Compile libneuzip_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
+
+Five translation units: nz_launch.hip once per precision (the kernels that
+exist per kept-mantissa setting) and nz_api.hip (the C ABI and the kernels all
+precisions share); they compile side by side and are linked into one library.
+"""
 from __future__ import annotations
 
 import os
 import subprocess
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(_HERE, "csrc")
 LIB_PATH = os.path.join(_HERE, "libneuzip_hip.so")
+PRECISIONS = (7, 3, 1, 0)
 
 HIPCC_FLAGS = [
     "-O3",
     "--offload-arch=gfx950",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     # no packed-FP32 VALU forms (v_pk_add/mul/fma_f32) in the gfx950 code object:
     # the device pass honours the feature; the x86 host pass of the same command
-    # does not know it and prints "not a recognized feature for this target
-    # (ignoring feature)" once per pass, which is harmless
+    # does not know it and says so once ("not a recognized feature for this
+    # target"), which run() below leaves out of what it prints
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # float arithmetic as written, whatever the compiler's defaults are: IEEE
-    # division where the code divides (the coder's reciprocal table), gradual
-    # underflow (the block normalizers scale bf16 subnormals), no contraction
+    # division where the code divides, gradual underflow (the block normalizers
+    # scale bf16 subnormals), no contraction
     "-fhip-fp32-correctly-rounded-divide-sqrt",
     "-fno-gpu-flush-denormals-to-zero",
     "-ffp-contract=off",
 ]
 
 
-def build(verbose: bool = False) -> str:
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *HIPCC_FLAGS, os.path.join(CSRC, "nz_api.hip"), "-o", LIB_PATH]
+def units(objdir: str):
+    """(source, extra flags, object file) of every translation unit."""
+    out = [(os.path.join(CSRC, "nz_api.hip"), [], os.path.join(objdir, "nz_api.o"))]
+    for s in PRECISIONS:
+        out.append((os.path.join(CSRC, "nz_launch.hip"), [f"-DNZ_S={s}"], os.path.join(objdir, f"nz_launch_s{s}.o")))
+    return out
+
+
+def run(cmd, verbose: bool) -> None:
+    """Run a compiler command; its messages are passed on, the host pass's note
+    about the device-only feature aside."""
     if verbose:
         print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd, cwd=CSRC)
+    res = subprocess.run(cmd, cwd=CSRC, capture_output=True, text=True)
+    lines = (res.stdout + res.stderr).splitlines()
+    # the note is one line, or two with the count of warnings it caused
+    keep = [ln for ln in lines if "-packed-fp32-ops' is not a recognized feature" not in ln
+            and ln.strip() != "1 warning generated when compiling for host."]
+    if keep:
+        print("\n".join(keep), flush=True)
+    if res.returncode != 0:
+        raise subprocess.CalledProcessError(res.returncode, cmd)
+
+
+def build(verbose: bool = False) -> str:
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    with tempfile.TemporaryDirectory(prefix="nz_build_") as objdir:
+        tus = units(objdir)
+
+        def compile_one(tu):
+            src, extra, obj = tu
+            run([hipcc, *HIPCC_FLAGS, *extra, "-c", src, "-o", obj], verbose)
+            return obj
+
+        with ThreadPoolExecutor(max_workers=len(tus)) as pool:
+            objs = list(pool.map(compile_one, tus))
+        run([hipcc, "--offload-arch=gfx950", "-fPIC", "-shared", *objs, "-o", LIB_PATH], verbose)
     return LIB_PATH
 
 
