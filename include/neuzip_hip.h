@@ -44,18 +44,14 @@ extern "C" {
 /* algorithm codes: cuda/algorithms.cuh:8. Only ANS exists here. */
 #define NZ_ALGO_ANS 0
 
-/* The library's own geometry (chunk_size 0, lane_syms 0): tables shared by
-   256 Ki elements, eight wavefronts of 512 symbols per lane each: 1.008 x the
-   order-0 entropy of the exponents, everything counted.  The reference hands
-   nvcomp chunks of 64 Ki (cuda/neuzip.cu:31); that size is honoured when asked
-   for, cut into two segments of 512 symbols per lane. */
-#define NZ_DEFAULT_CHUNK 262144u
-#define NZ_DEFAULT_LANE_SYMS 512u
+/* The library's own geometry (chunk_size 0): tables shared by 128 Ki elements,
+   eight wavefronts of 256 symbols per lane each.  The reference hands nvcomp
+   chunks of 64 Ki (cuda/neuzip.cu:31); that size is honoured when asked for,
+   cut into four segments of 256 symbols per lane. */
+#define NZ_DEFAULT_CHUNK 131072u
+#define NZ_DEFAULT_LANE_SYMS 256u
+#define NZ_LANE_SYMS_64K 256u
 #define NZ_LANE_SYMS_AUTO 0xFFFFFFFFu /* nz_manager_create: choose per tensor */
-/* shortest segments the per-tensor choice makes by itself: 432 symbols per lane
-   keep a tensor of N(0, 0.02) weights under 1.01 x the entropy of its exponents
-   (nz_manager_set_size_budget moves it) */
-#define NZ_AUTO_MIN_LANE_SYMS 432u
 
 typedef struct nz_manager nz_manager;
 

@@ -18,8 +18,9 @@ OK = 0
 ERR_ARG, ERR_DTYPE, ERR_NOT_FOUND, ERR_HIP, ERR_CAPACITY, ERR_CORRUPT, ERR_ALIGN, ERR_ALGO = range(-1, -9, -1)
 DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 ALGO_ANS = 0
-DEFAULT_CHUNK = 262144
-DEFAULT_LANE_SYMS = 512
+DEFAULT_CHUNK = 131072
+DEFAULT_LANE_SYMS = 256
+LANE_SYMS_64K = 256
 LANE_SYMS_AUTO = 0xFFFFFFFF
 DECODE_CHECK, DECODE_STREAM_OUT, DECODE_RESIDENT_OUT = 1, 2, 4  # nz_decode flags
 

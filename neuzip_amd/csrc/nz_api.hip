@@ -46,8 +46,11 @@ uint64_t norm_bytes_of(uint64_t n, uint32_t ns) { return ns ? (n + ns - 1) / ns 
 
 // Device scratch of one encode call.
 struct EncLayout {
-  uint64_t tab_ser, info, carry, slots, seg_body, seg_units, chunk_units, pub, placed, lb_state, bytes;
+  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units, pub, placed, lb_state, bytes;
 };
+
+// segments short enough for the kernel that keeps the exponents in registers
+bool enc_in_registers(const NzGeom& g) { return g.lane_syms <= NZ_ENC_MAX_LANE_SYMS; }
 
 EncLayout enc_layout(const NzGeom& g) {
   EncLayout L;
@@ -57,11 +60,14 @@ EncLayout enc_layout(const NzGeom& g) {
     o = align_up(o + b, 256);
     return at;
   };
+  L.exps = take(enc_in_registers(g) ? 0 : g.n + 16);  // only long segments park their exponents in memory
   L.tab_ser = take(g.n_chunks * NZ_TABLE_MAX_BYTES);
   L.info = take(g.n_chunks * sizeof(NzChunkInfo));
   L.carry = take(g.n_segs * NZ_CARRY_BYTES);
-  L.slots = take(g.n_segs * nz_slot_bytes(g.lane_syms) + 16);  // a record body with every lane stream at its worst case
-  L.seg_body = take(g.n_segs * 4);
+  L.slots = take(g.n_segs * 2 * (uint64_t)g.seg_syms + 16);  // one 2-byte word per symbol: the worst case
+  L.states = take(g.n_segs * NZ_STATE_MAX_BYTES);
+  L.seg_words = take(g.n_segs * 4);
+  L.seg_sbytes = take(g.n_segs * 4);
   L.seg_units = take((g.n_segs + 1) * 4);
   L.chunk_units = take((g.n_chunks + 1) * 4);
   L.pub = take(g.n_chunks * 16);  // size announcements of the chunks (records placed by the encode kernel)
@@ -92,9 +98,8 @@ uint64_t next_nonce() {
 }
 
 // How often a chunk of a direct encode looks for an announcement it waits for
-// (about a microsecond per look) before it gives up: some tens of milliseconds,
-// since a wait that is given up only costs one more kernel.
-std::atomic<uint32_t> g_lookback_spins{1u << 15};
+// (about a microsecond per look) before it gives up.
+std::atomic<uint32_t> g_lookback_spins{1u << 21};
 
 // One tensor of an encode call, as the kernels see it.  `comp`/`comp_cap`: where
 // the container goes (known only after phase 1 when the buffer is sized to fit).
@@ -113,11 +118,14 @@ NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws
   it.d_status = d_status;
   it.nm = NzNorm{ns ? norm : nullptr, log2_of(ns ? ns : 1)};
   it.g = g;
+  it.exps = L.exps;
   it.tab_ser = L.tab_ser;
   it.info = L.info;
   it.carry = L.carry;
   it.slots = L.slots;
-  it.seg_body = L.seg_body;
+  it.states = L.states;
+  it.seg_words = L.seg_words;
+  it.seg_sbytes = L.seg_sbytes;
   it.seg_units = L.seg_units;
   it.chunk_units = L.chunk_units;
   it.pub = L.pub;
@@ -127,7 +135,7 @@ NzEncItem enc_item(const NzGeom& g, const void* in, uint8_t* packed, uint8_t* ws
   it.use_placed = 0;
   it.nonce = next_nonce();
   it.d_gave_up = nullptr;
-  it.direct = (comp != nullptr && g.n_segs != 0) ? 1u : 0u;
+  it.direct = (comp != nullptr && g.n_segs != 0 && enc_in_registers(g)) ? 1u : 0u;
   it.spin_limit = g_lookback_spins.load(std::memory_order_relaxed);
   return it;
 }
@@ -145,80 +153,84 @@ bool enc_batch_close(NzEncBatch* b) {
   return true;
 }
 
-// Kernels may use more than 64 KiB of LDS per workgroup: that has to be allowed
-// once per kernel and device, and is done for all of them before the first
-// launch on a device.
-int allow_lds() {
+// One encode launch for the tensors of `b` whose segments are of class `cls`
+// (0..2: up to 64 / 128 / 256 symbols per lane, coded from registers; 3: longer).
+// The register encode kernels may use more than 64 KiB of LDS per workgroup
+// (word staging): that has to be allowed once per kernel and device, and is
+// done for all of them before the first encode on a device.
+int allow_encode_lds() {
   static std::atomic<uint64_t> allowed{0};  // bit d: done on device d
   int dev = 0;
   NZ_HIP(hipGetDevice(&dev));
   if (dev < 0 || dev >= 64) return fail(NZ_ERR_ARG, "device index out of range");
   if ((allowed.load(std::memory_order_acquire) >> dev) & 1ull) return NZ_OK;
-  NZ_HIP(nz_allow_lds<7>());
-  NZ_HIP(nz_allow_lds<3>());
-  NZ_HIP(nz_allow_lds<1>());
-  NZ_HIP(nz_allow_lds<0>());
+  NZ_HIP(nz_allow_encode_lds<7>());
+  NZ_HIP(nz_allow_encode_lds<3>());
+  NZ_HIP(nz_allow_encode_lds<1>());
+  NZ_HIP(nz_allow_encode_lds<0>());
   allowed.fetch_or(1ull << dev, std::memory_order_release);
   return NZ_OK;
 }
 
-#define NZ_LDS_TOTAL (160u * 1024u)
-
-// groups of 8 symbols per lane the encode kernel keeps in registers: its template argument
-int enc_groups(const NzGeom& g) { return g.lane_syms <= 64 ? 8 : g.lane_syms <= 128 ? 16 : g.lane_syms <= 256 ? 32 : 64; }
-
-// Dwords of LDS per wavefront in which a direct encode of segments with
-// `lane_syms` symbols per lane builds its record body, for workgroups of `waves`
-// wavefronts: room for lane streams of five bits per symbol, or what the
-// compute unit has left next to the kernel's own LDS.
-uint32_t stage_dwords_for(uint32_t lane_syms, uint32_t waves) {
-  const uint32_t fixed = ((uint32_t)sizeof(NzEncLds) + 1023u) & ~511u;  // the kernel's own LDS and slack
-  const uint32_t most = ((NZ_LDS_TOTAL - fixed) / waves / 4u) & ~3u;
-  const uint32_t want = NZ_BODY_HEAD_MAX / 4 + NZ_LANES * (((lane_syms * 5u) >> 5) + 9u);
-  return want < most ? want : most;
+// Words of LDS staging per wavefront for a direct encode of class `cls` with
+// workgroups of `waves` wavefronts: what a workgroup can have without lowering
+// the number of workgroups that the registers allow per compute unit (4, 6, 8
+// wavefronts per SIMD unit for 256, 128, 64 symbols per lane), less the
+// kernel's own LDS.
+uint32_t stage_words_for(int cls, uint32_t waves) {
+  const uint32_t waves_per_cu = cls == 2 ? 16u : cls == 1 ? 24u : 32u;
+  const uint32_t groups = waves_per_cu / waves ? waves_per_cu / waves : 1u;
+  const uint32_t per_group = 160u * 1024u / groups;
+  const uint32_t fixed = ((uint32_t)sizeof(NzEncLds) + 511u) & ~511u;  // the kernel's own LDS
+  if (per_group <= fixed + 1024u) return 0;
+  const uint32_t per_wave = ((per_group - fixed - 512u) / waves) & ~127u;  // bytes (512: the closing slack, rounding)
+  return per_wave / 2;
 }
 
 template <int S>
-int launch_encode_class(NzEncBatch& b, int ng, uint32_t lane_syms, uint32_t chunks, uint32_t max_spc, hipStream_t st) {
+int launch_encode_class(NzEncBatch& b, int cls, uint32_t chunks, uint32_t max_spc, hipStream_t st) {
   const uint32_t waves = max_spc < 4 ? 4 : max_spc;
   const dim3 grid(chunks), block(64 * waves);
   bool direct = false;
   for (uint32_t i = 0; i < b.count; ++i) direct = direct || b.item[i].direct;
-  b.stage_dwords = direct ? stage_dwords_for(lane_syms, waves) : 0u;
-  const uint32_t lds = waves * b.stage_dwords * 4u;
-  nz_launch_encode<S>(b, ng, grid, block, lds, st);
+  b.stage_words = (direct && cls < 3) ? stage_words_for(cls, waves) : 0u;
+  const uint32_t lds = b.stage_words ? waves * b.stage_words * 2u + 16u : 0u;
+  nz_launch_encode<S>(b, cls, grid, block, lds, st);
   return NZ_OK;
+}
+
+int enc_class(const NzGeom& g) {
+  return g.lane_syms <= 64 ? 0 : g.lane_syms <= 128 ? 1 : g.lane_syms <= NZ_ENC_MAX_LANE_SYMS ? 2 : 3;
 }
 
 // Phase 1 for all tensors of the batch: everything up to the directory.  Header
 // + directory land in each item's `hdr`, the container size in its *d_total.
 int encode_phase1(NzEncBatch* b, int precision, uint32_t ns, hipStream_t st) {
   if (!enc_batch_close(b)) return fail(NZ_ERR_ARG, "too many chunks for one launch");
-  if (int rc = allow_lds()) return rc;
+  if (int rc = allow_encode_lds()) return rc;
   for (uint32_t i = 0; i < b->count; ++i)
     if (int rc = launch_absmax(b->item[i].in, b->item[i].g.n, ns, const_cast<uint8_t*>(b->item[i].nm.bytes), st))
       return rc;
   // the tensors of the batch, by segment-length class: one launch per class in use
-  for (int ng = 8; ng <= 64; ng *= 2) {
+  for (int cls = 0; cls < 4; ++cls) {
     NzEncBatch sub{};
-    uint32_t chunks = 0, max_spc = 1, max_lane = 0;
+    uint32_t chunks = 0, max_spc = 1;
     for (uint32_t i = 0; i < b->count; ++i) {
       const NzEncItem& it = b->item[i];
-      if (it.g.n_chunks == 0 || enc_groups(it.g) != ng) continue;
+      if (it.g.n_chunks == 0 || enc_class(it.g) != cls) continue;
       NzEncItem& d = sub.item[sub.count++];
       d = it;
       chunks += (uint32_t)it.g.n_chunks;
       d.chunk_end = chunks;
       if (it.g.spc > max_spc) max_spc = it.g.spc;
-      if (it.g.lane_syms > max_lane) max_lane = it.g.lane_syms;
     }
     if (!sub.count) continue;
     int rc;
     switch (precision) {
-      case 7: rc = launch_encode_class<7>(sub, ng, max_lane, chunks, max_spc, st); break;
-      case 3: rc = launch_encode_class<3>(sub, ng, max_lane, chunks, max_spc, st); break;
-      case 1: rc = launch_encode_class<1>(sub, ng, max_lane, chunks, max_spc, st); break;
-      default: rc = launch_encode_class<0>(sub, ng, max_lane, chunks, max_spc, st); break;
+      case 7: rc = launch_encode_class<7>(sub, cls, chunks, max_spc, st); break;
+      case 3: rc = launch_encode_class<3>(sub, cls, chunks, max_spc, st); break;
+      case 1: rc = launch_encode_class<1>(sub, cls, chunks, max_spc, st); break;
+      default: rc = launch_encode_class<0>(sub, cls, chunks, max_spc, st); break;
     }
     if (rc) return rc;
   }
@@ -269,59 +281,29 @@ int encode_replace(const NzEncItem& item, const uint8_t* placed_in, hipStream_t 
   return encode_phase2(&one, st);
 }
 
-// LDS bytes per wavefront for its record in a decode launch of workgroups of
-// `spc` wavefronts: a quarter more than the container's average record (plus
-// the table and the head of the body), never more than the largest record
-// there can be or than the compute unit has.  A record that is larger still is
-// read from global memory by its wavefront.
-uint32_t rec_lds_for(const NzGeom& g, uint64_t comp_bytes, uint32_t spc) {
-  const uint64_t avg = g.n_segs && comp_bytes > g.rec_off ? (comp_bytes - g.rec_off) / g.n_segs : 0;
-  uint64_t want = avg + avg / 4 + NZ_DEC_REC_LDS_MIN;
-  const uint64_t largest = (uint64_t)g.seg_syms + NZ_CARRY_BYTES + NZ_TABLE_MAX_BYTES + 16;  // a coded chunk is smaller than a raw one
-  if (want > largest) want = largest;
-  const uint64_t most = (NZ_LDS_TOTAL - 8u * NZ_M) / (spc ? spc : 1u);
-  if (want > most) want = most;
-  if (want < NZ_DEC_REC_LDS_MIN) want = NZ_DEC_REC_LDS_MIN;
-  return (uint32_t)(want & ~(uint64_t)15);
-}
-
 // `flags`: NZ_DECODE_STREAM_OUT / NZ_DECODE_RESIDENT_OUT override the output
 // policy that is otherwise chosen by the size of the dense tensor
 int decode_launch(const NzGeom& g, int precision, const void* comp, uint64_t comp_bytes,
                   const void* packed, void* out, uint32_t* d_status, uint32_t ns, const void* norm,
                   int flags, hipStream_t st) {
   if (g.n_chunks == 0) return NZ_OK;
-  if (int rc = allow_lds()) return rc;
   const NzNorm nm{ns ? (const uint8_t*)norm : nullptr, log2_of(ns ? ns : 1)};
   const uint32_t so = (flags & NZ_DECODE_STREAM_OUT) ? 1u : (flags & NZ_DECODE_RESIDENT_OUT) ? 0u
                                                                                               : (nz_stream_output(g.n) ? 1u : 0u);
-  const uint32_t rl = rec_lds_for(g, comp_bytes, g.spc);
   switch (precision) {
-    case 7: nz_launch_decode<7>(g, comp, comp_bytes, packed, out, d_status, nm, so, rl, st); break;
-    case 3: nz_launch_decode<3>(g, comp, comp_bytes, packed, out, d_status, nm, so, rl, st); break;
-    case 1: nz_launch_decode<1>(g, comp, comp_bytes, packed, out, d_status, nm, so, rl, st); break;
-    default: nz_launch_decode<0>(g, comp, comp_bytes, packed, out, d_status, nm, so, rl, st); break;
+    case 7: nz_launch_decode<7>(g, comp, comp_bytes, packed, out, d_status, nm, so, st); break;
+    case 3: nz_launch_decode<3>(g, comp, comp_bytes, packed, out, d_status, nm, so, st); break;
+    case 1: nz_launch_decode<1>(g, comp, comp_bytes, packed, out, d_status, nm, so, st); break;
+    default: nz_launch_decode<0>(g, comp, comp_bytes, packed, out, d_status, nm, so, st); break;
   }
   NZ_HIP(hipGetLastError());
   return NZ_OK;
 }
 
-// LDS bytes per wavefront for the records of a batch: the largest any item wants
-void batch_rec_lds(NzBatch* b, uint32_t max_spc) {
-  uint32_t rl = NZ_DEC_REC_LDS_MIN;
-  for (uint32_t i = 0; i < b->count; ++i) {
-    const uint32_t r = rec_lds_for(b->item[i].g, b->item[i].comp_bytes, max_spc);
-    if (r > rl) rl = r;
-  }
-  b->rec_lds = rl;
-}
-
 // all items of one launch share the output policy (`stream_out`)
-int decode_batch_launch(NzBatch& b, uint32_t grid, uint32_t max_spc, int precision, bool stream_out,
+int decode_batch_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int precision, bool stream_out,
                         uint32_t* d_status, hipStream_t st) {
   if (grid == 0) return NZ_OK;
-  if (int rc = allow_lds()) return rc;
-  batch_rec_lds(&b, max_spc);
   switch (precision) {
     case 7: nz_launch_decode_batch<7>(b, grid, max_spc, stream_out, d_status, st); break;
     case 3: nz_launch_decode_batch<3>(b, grid, max_spc, stream_out, d_status, st); break;
@@ -332,10 +314,8 @@ int decode_batch_launch(NzBatch& b, uint32_t grid, uint32_t max_spc, int precisi
   return NZ_OK;
 }
 
-int gemv_launch(NzBatch& b, uint32_t grid, uint32_t max_spc, int precision, uint32_t* d_status,
+int gemv_launch(const NzBatch& b, uint32_t grid, uint32_t max_spc, int precision, uint32_t* d_status,
                 hipStream_t st) {
-  if (int rc = allow_lds()) return rc;
-  batch_rec_lds(&b, max_spc);
   switch (precision) {
     case 7: nz_launch_gemv<7>(b, grid, max_spc, d_status, st); break;
     case 3: nz_launch_gemv<3>(b, grid, max_spc, d_status, st); break;
@@ -349,8 +329,8 @@ int gemv_launch(NzBatch& b, uint32_t grid, uint32_t max_spc, int precision, uint
 int make_geom(NzGeom* g, uint64_t n, uint32_t chunk, uint32_t lane_syms) {
   if (nz_geom_make(g, n, chunk, lane_syms))
     return fail(NZ_ERR_ARG,
-                "unsupported geometry: lane_syms must be a multiple of 8 from 24 to 512, chunk_size a multiple "
-                "of 512 cut into 1..8 segments of 64*lane_syms, the last one at least 1536 long");
+                "unsupported geometry: lane_syms must be a multiple of 8 (>= 16), chunk_size a multiple "
+                "of 512 cut into 1..8 segments of 64*lane_syms, the last one at least 1024 long");
   if (g->n_chunks > 0x7FFFFFFFull) return fail(NZ_ERR_ARG, "tensor too large");
   return NZ_OK;
 }
@@ -449,9 +429,8 @@ struct nz_manager {
   uint32_t normalizer = 0;  // elements per normalizer group, 0 = none
   uint32_t chunk_syms, lane_syms;
   bool own_chunk = false;   // chunk_size 0 was given: the library's own table scope
-  bool auto_lanes = false;  // pick the segment length per tensor (pick_geometry)
-  uint32_t auto_min_lane = NZ_AUTO_MIN_LANE_SYMS;  // shortest segments auto mode may pick: the size budget
-  uint32_t cus = 256;       // compute units of the device
+  bool auto_lanes = false;  // pick the geometry per tensor so that small tensors still fill the GPU
+  uint32_t slots = 768;     // decode workgroups of eight wavefronts the device holds at once (3 per CU)
   std::unordered_map<std::string, Entry> entries;  // compress_cache + meta_cache
   std::unordered_map<std::string, std::pair<uint32_t, uint32_t>> hints;  // name -> (chunk, lane) for its next writes
   std::mutex mu;
@@ -470,7 +449,7 @@ struct nz_manager {
 
 extern "C" {
 
-int nz_abi_version(void) { return 5; }
+int nz_abi_version(void) { return 4; }
 
 const char* nz_last_error(void) { return g_err.c_str(); }
 
@@ -611,16 +590,19 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
     return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
   const bool auto_lanes = lane_syms == NZ_LANE_SYMS_AUTO;
   const bool own_chunk = chunk_size == 0;
-  if (lane_syms == 0 || auto_lanes) {
-    // the longest segments the chunk allows: every lane and segment costs about nine bits of container
-    lane_syms = NZ_DEFAULT_LANE_SYMS;
-    if (!own_chunk)
-      while (lane_syms > 24 && nz_geom_check(chunk_size, lane_syms)) lane_syms -= 8;
-  }
   if (own_chunk) {
-    // eight segments per table, fewer only for segments too long for that
-    chunk_size = lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK;
-    if (chunk_size > NZ_DEFAULT_CHUNK) chunk_size = NZ_DEFAULT_CHUNK;
+    chunk_size = NZ_DEFAULT_CHUNK;
+    // an explicit segment length too short for eight segments to cover the
+    // default chunk goes with the smaller table scope
+    if (lane_syms != 0 && !auto_lanes && (uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size)
+      chunk_size = 65536;
+  }
+  if (lane_syms == 0 || auto_lanes) {
+    // the best measured segment length for the chunk: 8 segments of 256 per lane
+    // in a 128 Ki chunk, four of them in a 64 Ki chunk
+    lane_syms = chunk_size == NZ_DEFAULT_CHUNK ? NZ_DEFAULT_LANE_SYMS : NZ_LANE_SYMS_64K;
+    while (lane_syms > 8 && (uint64_t)lane_syms * NZ_LANES > chunk_size) lane_syms /= 2;
+    while ((uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size) lane_syms *= 2;
   }
   NzGeom g;
   if (int rc = make_geom(&g, 0, chunk_size, lane_syms)) return rc;
@@ -649,7 +631,7 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   int dev = 0, cus = 0;
   if (e == hipSuccess) e = hipGetDevice(&dev);
   if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-  if (e == hipSuccess && cus > 0) m->cus = (uint32_t)cus;
+  if (e == hipSuccess && cus > 0) m->slots = 3u * (uint32_t)cus;
   if (e != hipSuccess) {
     for (int k = 0; k < 2; ++k)
       if (m->rw[k].ev) (void)hipEventDestroy(m->rw[k].ev);
@@ -704,16 +686,11 @@ void release_entry(Entry& e) {
   e.comp = e.packed = e.norm = nullptr;
 }
 
-// Geometry of a tensor of n elements.  A launch runs one workgroup of eight
-// wavefronts per chunk, one workgroup per compute unit at a time; its time is
-// (rounds of workgroups) x (symbols per lane).  Every lane and segment costs
-// about nine bits of container (the length of the lane's stream, its share of
-// directory, table and padding), so segments are kept long: the default of 512
-// symbols per lane stores 1.008 x the exponents' entropy.  In auto mode a
-// tensor gets the segment length between `auto_min_lane` (what the manager's
-// size budget allows) and 512 that needs the fewest rounds, the longest among
-// equals; tensors too small to fill the device are not cut finer than that
-// (they are what the batch calls are for).
+// Geometry of a tensor of n elements.  Throughput of both codec directions is
+// set by the number of wavefronts in flight (one per 64 * lane_syms elements).
+// In auto mode a tensor too small to give every SIMD two wavefronts at the
+// default gets shorter segments (and, with the library's own chunk, the smaller
+// 64 Ki table scope that allows them), at ~4.5 bits per extra lane.
 int pick_geometry(const nz_manager* m, const char* name, uint64_t n, NzGeom* g, uint32_t* chunk_out,
                   uint32_t* lane_out) {
   uint32_t lane_syms = m->lane_syms, chunk_syms = m->chunk_syms;
@@ -723,19 +700,53 @@ int pick_geometry(const nz_manager* m, const char* name, uint64_t n, NzGeom* g, 
     *lane_out = hint->second.second;
     return make_geom(g, n, *chunk_out, *lane_out);
   }
-  if (m->auto_lanes && m->own_chunk) {
-    const uint64_t cus = m->cus ? m->cus : 256;
-    uint64_t best_cost = ~0ull;
-    for (uint32_t lane = NZ_MAX_LANE_SYMS; lane >= m->auto_min_lane && lane >= 24; lane -= 8) {
-      const uint64_t chunk = (uint64_t)lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK;
-      const uint64_t chunks = n ? (n + chunk - 1) / chunk : 1;
-      const uint64_t cost = ((chunks + cus - 1) / cus) * lane;
-      if (cost < best_cost) {
-        best_cost = cost;
-        lane_syms = lane;
-        chunk_syms = (uint32_t)chunk;
+  if (m->auto_lanes && m->own_chunk && chunk_syms == NZ_DEFAULT_CHUNK && lane_syms == NZ_DEFAULT_LANE_SYMS) {
+    // The device holds `slots` decode workgroups (three per compute unit) at
+    // once, and a launch is fastest when every compute unit has the same number
+    // of them: 378 workgroups on 256 units run as long as 512 would (measured on
+    // a 4096 x 14336 matrix: 51 us with 378 chunks, 38 us with 512).  A tensor
+    // with more default-sized chunks than slots keeps the default geometry.  A
+    // smaller one is cut into one, two or three workgroups per compute unit
+    // (more of them only where the model below promises 10 % or more), with
+    // segments of 64 to 512
+    // symbols per lane (shorter segments cost compression: ~4.5 bits per lane
+    // and segment); a tensor too small for that gets 32 Ki chunks of eight
+    // 4 Ki segments.  Time of a round ~ symbols per lane x time of a step, which
+    // grows with the wavefronts that share a SIMD unit (2, 4, 6 of them: about
+    // 107, 147, 215 ns per step).
+    const uint64_t slots = m->slots, cus = slots / 3;
+    const uint64_t chunks = (n + chunk_syms - 1) / chunk_syms;
+    if (chunks > slots || cus == 0) {
+      // default
+    } else {
+      static const uint32_t step_ns[3] = {107, 147, 215};
+      uint64_t best_t = ~0ull;
+      uint32_t best_lane = 0;
+      for (uint32_t k = 1; k <= 3; ++k) {
+        const uint64_t per_lane = (n + k * cus * 512 - 1) / (k * cus * 512);  // a chunk is 8 x 64 lanes
+        const uint32_t lane = (uint32_t)((per_lane + 7) / 8) * 8;
+        if (lane < 64 || lane > 2 * NZ_DEFAULT_LANE_SYMS) continue;
+        if (nz_geom_check(lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK, lane)) continue;
+        const uint64_t t = (uint64_t)lane * step_ns[k - 1];
+        if (best_lane == 0 || 10 * t < 9 * best_t) {  // more, shorter segments only for a gain above 10 %
+          best_t = t;
+          best_lane = lane;
+        }
+      }
+      if (best_lane) {
+        lane_syms = best_lane;
+        chunk_syms = best_lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK;
+      } else {
+        chunk_syms = 32768;
+        lane_syms = 64;
       }
     }
+  } else if (m->auto_lanes) {
+    // a chunk size given by the caller: shorter segments while that is a valid
+    // geometry and the tensor has fewer than 2048 segments
+    while (lane_syms > 16 && nz_geom_check(chunk_syms, (lane_syms / 2 + 7) & ~7u) == 0 &&
+           n / ((uint64_t)lane_syms * NZ_LANES) < 2048)
+      lane_syms = (lane_syms / 2 + 7) & ~7u;
   }
   *chunk_out = chunk_syms;
   *lane_out = lane_syms;
@@ -1201,14 +1212,12 @@ int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indi
   }
   const NzNorm nm{m->normalizer ? (const uint8_t*)ent.norm : nullptr, log2_of(m->normalizer ? m->normalizer : 1)};
   uint16_t* scratch = (uint16_t*)m->ws;
-  if (int rc = allow_lds()) return rc;
-  const uint32_t rows_rec_lds = rec_lds_for(g, ent.comp_bytes, g.spc);
   for (uint64_t at = 0; at < count; at += per_slice) {
     const uint32_t rows_now = (uint32_t)(count - at < per_slice ? count - at : per_slice);
     const long long* idx = (const long long*)dev_indices + at;
 #define NZ_ROWS_CASE(S)                                                                              \
   nz_launch_rows<S>(g, ent.comp, ent.comp_bytes, ent.packed, scratch, m->d_status, nm, idx,         \
-                    rows_now, row_len, cpr, rows_rec_lds, st)
+                    rows_now, row_len, cpr, st)
     switch (m->precision) {
       case 7: NZ_ROWS_CASE(7); break;
       case 3: NZ_ROWS_CASE(3); break;
@@ -1243,8 +1252,8 @@ int nz_manager_geometry_hint(nz_manager* m, const char* name, uint32_t chunk_siz
   }
   if (nz_geom_check(chunk_size, lane_syms))
     return fail(NZ_ERR_ARG,
-                "unsupported geometry: lane_syms must be a multiple of 8 from 24 to 512, chunk_size a multiple "
-                "of 512 cut into 1..8 segments of 64*lane_syms, the last one at least 1536 long");
+                "unsupported geometry: lane_syms must be a multiple of 8 (>= 16), chunk_size a multiple "
+                "of 512 cut into 1..8 segments of 64*lane_syms, the last one at least 1024 long");
   m->hints[name] = std::make_pair(chunk_size, lane_syms);
   return NZ_OK;
 }

@@ -6,36 +6,30 @@
 //   header (64 B) | directory ((n_segs + 1) x u32) | segment records | 16 zero bytes
 //
 // * chunk   = `chunk_syms` consecutive exponents that share one 12-bit
-//             frequency table and are decoded by one workgroup (the reference
-//             hands nvcomp chunk_size = 65536, cuda/neuzip.cu:31).
+//             frequency table (the reference hands nvcomp the same unit:
+//             chunk_size = 65536, cuda/neuzip.cu:31).
 // * segment = 64 * `lane_syms` consecutive exponents decoded by ONE wavefront:
-//             lane l owns the 8-symbol groups (g * 64 + l) * 8 + j and codes
-//             them with two table-ANS states (A: even j, B: odd j) into one
-//             private bit stream.  A chunk is cut into spc = 1..8 segments,
-//             the last one holding what remains of the chunk (>= 1536
+//             64 interleaved rANS states, lane l owning the 8-symbol groups
+//             (g * 64 + l) * 8 + j.  A chunk is cut into spc = 1..8 segments,
+//             the last one holding what remains of the chunk (>= 1024
 //             symbols); segment c * spc + k is the k-th segment of chunk c.
 // * directory entry k = offset of segment k's record in 4-byte units from
 //             `rec_off`; entry n_segs = end of the last record.
-// * record  = [table, first segment of a chunk only] [states: 64 x 24 bits,
-//             lane l at bytes 3l .. 3l+2, state A in the low 12 bits]
-//             [u32 minlen | w << 24] [64 fields of w bits: len_l - minlen]
-//             [the 64 lane streams back to back, bit-granular, little endian]
-//             padded to 4 bytes; or, for a chunk whose coded form would not be
-//             smaller, [0xFF 0 0 0, first segment only] raw exponent bytes
-//             padded to 4 [+ the carried bytes if full].
-// * coder   = table ANS with T = 4096 states.  Slot i of [0, T) belongs to the
-//             symbol whose cumulative 12-bit frequency range holds i; state X
-//             stands on slot (X % 64) * 64 + X / 64; the k-th state of symbol
-//             s in ascending order stands for x = f_s + k: the decoder reads
-//             n = 12 - floor(log2 x) bits b and moves to (x << n) - T + b.  A
-//             lane's stream is read from its end downwards, A's bits above
-//             B's for each pair of symbols.
-// * carry   = the encoder of a FULL segment starts the two states of lane l
-//             from T | 12 payload bits each: bytes 3l .. 3l+2 of the last
-//             NZ_CARRY_BYTES bytes of the segment's packed sign|mantissa
-//             stream, which are not stored in the packed stream; the decoder
-//             finds them in its final states.  So the 24 bits a lane's start
-//             states cost in the record are paid back.
+// * record  = [table, first segment of a chunk only] [final encoder states:
+//             64 two-bit length codes (lane l at bits 2l, 2l+1; code c = the
+//             state takes 5 + c nibbles) and the states as a little-endian
+//             nibble stream in lane order, padded to 4 bytes] [u16
+//             renormalisation words, front-to-back in decode order] padded to
+//             4 bytes; or, for a chunk whose coded form
+//             would not be smaller, [0xFF 0 0 0, first segment only] raw
+//             exponent bytes padded to 4 [+ 64 x u16 carried bits if full].
+// * carry   = the encoder of a FULL segment starts lane l in state
+//             2^16 | c_l instead of 2^16, where c_l are bytes 2l, 2l+1 of the
+//             last 128 bytes of the segment's packed sign|mantissa stream.
+//             Those 128 bytes are not stored in the packed stream (every full
+//             segment stores NZ_CARRY_BYTES fewer); the decoder finds them in
+//             the low halves of its final states.  This returns 16 of the
+//             ~24 bits that flushing a 32-bit rANS state costs per lane.
 #pragma once
 
 #include <stddef.h>
@@ -48,9 +42,10 @@
 #endif
 
 #define NZ_MAGIC 0x315A4E41u
-#define NZ_FORMAT_VERSION 5u
+#define NZ_FORMAT_VERSION 4u
 #define NZ_PROB_BITS 12
 #define NZ_M (1u << NZ_PROB_BITS)
+#define NZ_L (1u << 16)
 #define NZ_LANES 64
 #define NZ_GROUP 8
 #define NZ_GROUP_SYMS 512
@@ -60,11 +55,8 @@
 #define NZ_MAX_RUNS 15
 #define NZ_TABLE_MAX_BYTES 424 /* 1 + 32 + 384 rounded up to a multiple of 8 */
 #define NZ_MAX_SEGS_PER_CHUNK 8
-#define NZ_CARRY_BYTES 192 /* 64 lanes x 2 states x 12 bits */
-#define NZ_STATES_BYTES 192
-#define NZ_LENS_MAX_BYTES 196 /* u32 header + 64 fields of up to 24 bits */
-#define NZ_BODY_HEAD_MAX (NZ_STATES_BYTES + NZ_LENS_MAX_BYTES)
-#define NZ_MAX_LANE_SYMS 512u
+#define NZ_CARRY_BYTES 128 /* 64 lanes x 16 bits */
+#define NZ_STATE_MAX_BYTES 272 /* 16 bytes of length codes + 64 x 32 bits */
 #define NZ_TAIL_PAD 16     /* zero bytes after the last record: 16-byte loads stay inside */
 
 struct NzGeom {
@@ -88,12 +80,12 @@ struct NzChunkInfo {
 };
 
 static inline int nz_geom_check(uint32_t chunk_syms, uint32_t lane_syms) {
-  if (lane_syms < 24 || (lane_syms % NZ_GROUP) != 0 || lane_syms > NZ_MAX_LANE_SYMS) return -1;
+  if (lane_syms < 16 || (lane_syms % NZ_GROUP) != 0 || lane_syms > (1u << 16)) return -1;
   uint64_t seg = (uint64_t)lane_syms * NZ_LANES;
   if (chunk_syms == 0 || (chunk_syms % NZ_GROUP_SYMS) != 0 || chunk_syms > (1u << 24)) return -1;
   uint64_t spc = (chunk_syms + seg - 1) / seg;
   if (spc < 1 || spc > NZ_MAX_SEGS_PER_CHUNK) return -1;
-  if (chunk_syms - (spc - 1) * seg < 8 * NZ_CARRY_BYTES) return -1;  // the last segment must be able to carry 192 bytes
+  if (chunk_syms - (spc - 1) * seg < 1024) return -1;  // the last segment must be able to carry 128 bytes
   return 0;
 }
 
@@ -126,7 +118,7 @@ NZ_HD static inline uint32_t nz_seg_nominal(uint32_t chunk_syms, uint32_t seg_sy
   return k + 1 < spc ? seg_syms : chunk_syms - (spc - 1) * seg_syms;
 }
 
-// Segments the tensor does not end inside ("full": they carry NZ_CARRY_BYTES packed bytes).
+// Segments the tensor does not end inside ("full": they carry 128 packed bytes).
 static inline uint64_t nz_full_segments(const NzGeom* g) {
   uint64_t rem = g->n % g->chunk_syms, fs = rem / g->seg_syms;
   if (fs > g->spc - 1) fs = g->spc - 1;
@@ -137,12 +129,4 @@ static inline uint64_t nz_full_segments(const NzGeom* g) {
 // carried bytes of every full segment.
 static inline uint64_t nz_packed_stored_bytes_of(const NzGeom* g, int s) {
   return nz_packed_bytes_of(g->n, s) - (uint64_t)NZ_CARRY_BYTES * nz_full_segments(g);
-}
-
-// Bytes of the scratch slot of one segment: the record body (states, lengths,
-// lane streams of up to 12 bits per symbol with one spare dword each) when it
-// is not assembled in LDS, or the raw exponent bytes of a chunk stored raw.
-NZ_HD static inline uint32_t nz_slot_lane_dwords(uint32_t lane_syms) { return (lane_syms * NZ_PROB_BITS + 31) / 32 + 2; }
-NZ_HD static inline uint64_t nz_slot_bytes(uint32_t lane_syms) {
-  return (uint64_t)NZ_BODY_HEAD_MAX + 4ull * NZ_LANES * nz_slot_lane_dwords(lane_syms) + 12;
 }

@@ -2,7 +2,7 @@
 //
 //   nz_split_unpacked_kernel   Manager::split            cuda/high_level.cu:265-321
 //   nz_encode_kernel           kernel_aligned_split      cuda/kernels.cuh:62-156
-//                              + per-chunk exponent histogram, 12-bit frequency
+//   nz_encode_long_kernel      + per-chunk exponent histogram, 12-bit frequency
 //                              table and its serialized form, then
 //                              nvcomp ANS compress       cuda/high_level.cu:103-115
 //   nz_compact_kernel          exact-size compaction     cuda/high_level.cu:117-124
@@ -11,9 +11,8 @@
 //                              cuda/high_level.cu:184-201, cuda/kernels.cuh:167-217
 //
 // The whole path is byte/integer work bound by HBM traffic; there is no dense
-// contraction, hence no MFMA.  One wavefront decodes one segment, every lane
-// with two table-ANS states and a bit stream of its own; the exponent never
-// exists in HBM, on either side.
+// contraction, hence no MFMA.  One wavefront decodes one segment with 64
+// interleaved rANS states; the exponent never exists in HBM on the decode side.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -22,6 +21,8 @@
 
 #define NZ_HIST_COPIES 8u
 #define NZ_HIST_STRIDE 257u
+#define NZ_RING_WORDS 1024u  // per-wave LDS ring of renormalisation words
+#define NZ_RING_DWORDS (NZ_RING_WORDS / 2)
 
 // ----------------------------------------------------------------------------
 // element-wise split / merge arithmetic
@@ -244,19 +245,6 @@ __device__ __forceinline__ uint32_t nz_get12(const uint8_t* p, uint32_t i) {
   return (w >> (bit & 4u)) & 0xFFFu;
 }
 
-// Rank of state X among the states of the symbol that owns slots [c, c + f), in
-// ascending order: the states Y < X whose slot (Y % 64) * 64 + Y / 64 lies in
-// that range.  With q = X / 64, r = X % 64: the states of the rows before q
-// (slots i in range with i % 64 < q), plus those of row q itself before r
-// (slots 64 r' + q >= c with r' < r; they lie below X's own slot, inside the range).
-NZ_HD static inline uint32_t nz_state_rank(uint32_t X, uint32_t c, uint32_t f) {
-  const uint32_t q = X >> 6, r = X & 63u, hi = c + f;
-  const uint32_t hq = (hi & 63u) < q ? (hi & 63u) : q, cq = (c & 63u) < q ? (c & 63u) : q;
-  const uint32_t rows = (hi >> 6) * q + hq - (c >> 6) * q - cq;
-  const uint32_t t = (c + 63u - q) >> 6;
-  return rows + r - (r < t ? r : t);
-}
-
 #ifndef NZ_TEMPLATES_ONLY
 // ----------------------------------------------------------------------------
 // Manager::split: unpacked exponent and sign|mantissa bytes, precision 7 always
@@ -300,9 +288,17 @@ __global__ __launch_bounds__(256) void nz_split_unpacked_kernel(const uint16_t* 
 // encode: one workgroup per chunk
 // ----------------------------------------------------------------------------
 //
-// nz_encode_kernel: wavefront k of the workgroup splits segment k of the chunk,
-// keeps the exponent bytes of its lanes in registers, and codes them from there
-// once the chunk's tables exist: the exponents never reach memory.
+// Two kernels share the pieces below.  nz_encode_kernel (segments of up to
+// NZ_ENC_MAX_LANE_SYMS symbols per lane, which covers every geometry the
+// library picks by itself): wavefront k of the workgroup splits segment k of
+// the chunk, keeps the exponent bytes of its lanes in registers, and codes
+// them from there once the chunk's table exists: the exponents never reach
+// memory.  nz_encode_long_kernel (longer segments): all wavefronts split the
+// chunk and park the exponents in scratch, then one wavefront per segment
+// codes them from there.
+
+#define NZ_ENC_MAX_LANE_SYMS 256u
+#define NZ_ENC_LONG_THREADS 1024u
 
 // f(constant I) for I = FROM, FROM + STEP, ... while I < TO (or, with a negative
 // step, while I >= TO): straight-line code with compile-time indices, so that
@@ -318,16 +314,6 @@ __device__ __forceinline__ void nz_static_for(F&& f) {
     nz_static_for<FROM + STEP, TO, STEP>(f);
   }
 }
-
-// a dword pointer into LDS (ds_ instructions) or into global memory
-template <bool INLDS>
-struct NzU32Ptr {
-  typedef uint32_t* type;
-};
-template <>
-struct NzU32Ptr<true> {
-  typedef __attribute__((address_space(3))) uint32_t* type;
-};
 
 // sums / maxima over the workgroup (at most 16 wavefronts)
 __device__ __forceinline__ uint32_t nz_block_sum(uint32_t v, uint32_t* red) {
@@ -358,30 +344,25 @@ __device__ __forceinline__ uint32_t nz_block_max(uint32_t v, uint32_t* red) {
 // LDS of an encode workgroup.  8 histogram copies (one per lane & 7) at a
 // stride of 257 words: exponents of weights cluster on a few values, so a
 // single copy would serialise most of a wavefront's atomics on one address;
-// the odd stride keeps the copies of a bin in different banks.  The histogram
-// is dead once the frequencies exist; the encoder's state table takes its place.
+// the odd stride keeps the copies of a bin in different banks.
 struct NzEncLds {
-  union {
-    uint32_t hist[NZ_HIST_COPIES * NZ_HIST_STRIDE];
-    uint16_t enc[NZ_M];  // enc[cum[s] + k] = T | the k-th state of symbol s
-  };
+  uint32_t hist[NZ_HIST_COPIES * NZ_HIST_STRIDE];
   uint32_t red[16];
   uint32_t scan_s[4];
   uint64_t mw[4];
-  uint32_t cf[256];  // per live symbol, in symbol order: frequency,
-  uint32_t lc[257];  //   first slot (then 4096 behind the last),
-  uint32_t ls[256];  //   symbol
-  // per symbol: x = (n0 << 16) - (f << n0) with n0 = 12 - floor(log2 f), so that a state x in
-  // [T, 2T) writes (x + that) >> 16 bits; y = LDS byte address of enc[cum - f]
-  uint2 sym[256];
+  uint32_t cf[256];
+  // per symbol: x = freq << 20 (renormalisation threshold), y = freq, z = cum,
+  // w = bits of a float just below 1 / freq (four units in the last place
+  // under the correctly rounded quotient)
+  uint4 tab[256];
+  uint32_t sbuf[NZ_MAX_SEGS_PER_CHUNK][NZ_STATE_MAX_BYTES / 4];
   uint32_t pad_sym, raw;
   // for records that go straight to their place: the chunk's record sizes, the
   // sum over the chunks before it, whether the wait for those was given up
   uint32_t seg_units[NZ_MAX_SEGS_PER_CHUNK];
   uint32_t chunk_total, gave_up;
-  uint32_t redo;   // a lane ran out of staging room: the chunk is coded again, into the slots
-  uint32_t lb[2];  // the two words of the scratch's announcement state, as thread 0 read them
-  uint64_t red64[NZ_MAX_SEGS_PER_CHUNK];
+  uint32_t redo;  // a wavefront ran out of staging room: the chunk is coded again, into the slots
+  uint64_t red64[NZ_ENC_LONG_THREADS / 64];
 };
 
 // Split one element group: 8 bf16 values -> 8 exponent bytes (byte j of `e` =
@@ -449,9 +430,8 @@ __device__ __forceinline__ uint64_t nz_split_tail(const uint16_t* __restrict__ i
 }
 
 // From the chunk's histogram (cn symbols): the 12-bit frequency table (sum
-// exactly 4096), the encoder's per-symbol entries and its state table in LDS,
-// the serialized table and the chunk record.  Run by the whole workgroup (at
-// least 256 threads).
+// exactly 4096), the encoder's per-symbol entries in LDS, the serialized table
+// and the chunk record.  Run by the whole workgroup (at least 256 threads).
 // -> an estimate of the chunk's coded length in bits (sum of count x -log2 of
 // the quantised probability), the same in every thread.
 __device__ __forceinline__ uint32_t nz_build_table(NzEncLds& L, const uint32_t cn, uint8_t* __restrict__ out,
@@ -485,15 +465,11 @@ __device__ __forceinline__ uint32_t nz_build_table(NzEncLds& L, const uint32_t c
   }
   if (own && (tid & 63) == 63) L.scan_s[tid >> 6] = incl;
   __syncthreads();
-  uint32_t cum = 0;
   if (own) {
     uint32_t woff = 0;
     for (uint32_t w = 0; w < (tid >> 6); ++w) woff += L.scan_s[w];
-    cum = woff + incl - f;
-    typedef __attribute__((address_space(3))) uint16_t lds_u16;
-    const uint32_t enc_lds = (uint32_t)(uintptr_t)((lds_u16*)L.enc);
-    const uint32_t n0 = f ? (uint32_t)__clz((int)f) - 19u : 0u;  // 12 - floor(log2 f)
-    L.sym[tid] = make_uint2(f ? (n0 << 16) - (f << n0) : 0u, enc_lds + 2u * (cum - f));
+    const uint32_t cum = woff + incl - f;
+    L.tab[tid] = make_uint4(f << 20, f, cum, f ? __float_as_uint(1.0f / (float)f) - 4u : 0u);
   }
 
   // ---- serialise the table, in parallel ----
@@ -510,10 +486,7 @@ __device__ __forceinline__ uint32_t nz_build_table(NzEncLds& L, const uint32_t c
                            (w > 2 ? (uint32_t)__popcll(m2) : 0u) +
                            (uint32_t)__popcll(bal & ((1ull << (tid & 63)) - 1ull));
     L.cf[below] = f;
-    L.lc[below] = cum;
-    L.ls[below] = tid;
   }
-  if (tid == 0) L.lc[kk] = NZ_M;
   // a run starts at a live symbol whose predecessor is not live
   const uint64_t s0 = m0 & ~(m0 << 1);
   const uint64_t s1 = m1 & ~((m1 << 1) | (m0 >> 63));
@@ -578,20 +551,6 @@ __device__ __forceinline__ uint32_t nz_build_table(NzEncLds& L, const uint32_t c
     *info_c = ci;
     L.pad_sym = imax;
   }
-  // The encoder's state table (the histogram, whose place it takes, was read
-  // long ago).  State X stands on slot (X % 64) * 64 + X / 64; the symbol that
-  // owns the slot is found by bisection over the live symbols' first slots.
-  for (uint32_t X = tid; X < NZ_M; X += blockDim.x) {
-    const uint32_t slot = ((X & 63u) << 6) | (X >> 6);
-    uint32_t lo = 0, hi = kk;  // lc[lo] <= slot < lc[hi]
-    while (hi - lo > 1) {
-      const uint32_t mid = (lo + hi) >> 1;
-      if (L.lc[mid] <= slot) lo = mid;
-      else hi = mid;
-    }
-    const uint32_t c0 = L.lc[lo];
-    L.enc[c0 + nz_state_rank(X, c0, L.cf[lo])] = (uint16_t)(NZ_M | X);
-  }
   __syncthreads();
   return est_bits;
 }
@@ -602,28 +561,31 @@ __device__ __forceinline__ uint32_t nz_build_table(NzEncLds& L, const uint32_t c
 // ----------------------------------------------------------------------------
 __device__ __forceinline__ bool nz_chunk_finalize(uint64_t c, uint64_t n, uint32_t chunk_syms,
                                                   uint32_t seg_syms, uint32_t spc, NzChunkInfo* info,
-                                                  const uint32_t* seg_body, uint32_t* seg_units, uint32_t* chunk_units,
+                                                  const uint32_t* seg_words, const uint32_t* seg_state_bytes,
+                                                  uint32_t* seg_units, uint32_t* chunk_units,
                                                   uint32_t* lds_seg_units, uint32_t* lds_chunk_total) {
   const uint64_t base = c * chunk_syms;
   const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
   const uint32_t nseg = (cn + seg_syms - 1) / seg_syms;
   const uint32_t tab_len = info[c].tab_len;
-  uint64_t coded_total = tab_len, raw_total = 4;
+  uint64_t rans_total = tab_len, raw_total = 4;
   for (uint32_t k = 0; k < nseg; ++k) {
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
-    coded_total += seg_body[c * spc + k];
+    const uint32_t w = seg_words[c * spc + k];
+    rans_total += seg_state_bytes[c * spc + k] + 2 * (uint64_t)((w + 1) & ~1u);
     raw_total += ((sn + 3) & ~3u) + (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
   }
-  const bool raw = coded_total >= raw_total;
+  const bool raw = rans_total >= raw_total;
   info[c].raw = raw ? 1u : 0u;
-  uint32_t chunk_total = 0;  // a record has at most ~2^17 units, a chunk eight records
+  uint32_t chunk_total = 0;  // a record has at most ~2^21 units, a chunk eight records
   for (uint32_t k = 0; k < nseg; ++k) {
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
+    const uint32_t w = seg_words[c * spc + k];
     uint32_t bytes;
     if (raw)
       bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u) +
               (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
-    else bytes = (k == 0 ? tab_len : 0u) + seg_body[c * spc + k];
+    else bytes = (k == 0 ? tab_len : 0u) + seg_state_bytes[c * spc + k] + 2u * ((w + 1) & ~1u);
     seg_units[c * spc + k] = bytes / 4;
     lds_seg_units[k] = bytes / 4;
     chunk_total += bytes / 4;
@@ -634,121 +596,87 @@ __device__ __forceinline__ bool nz_chunk_finalize(uint64_t c, uint64_t n, uint32
 }
 
 // ----------------------------------------------------------------------------
-// table-ANS encode of one segment by one wavefront
+// rANS encode of one segment by one wavefront
 // ----------------------------------------------------------------------------
 //
-// Every lane runs backwards over its symbols with two states (A: even j of a
-// group, B: odd j) and appends what they write to a private bit stream, low
-// bits first: the decoder reads the stream from its end downwards, A's bits
-// above B's in every pair.  The streams grow dword by dword in a staging area
-// (lane l at dwords l * stride ...) and are packed back to back, bit-granular,
-// once their lengths are known.
+// The 64 lanes run backwards over their symbols.  Per symbol: emit the low 16
+// state bits when the state is at or above freq << 20 (ranked into the word
+// slot back to front, so that the decoder reads front to back), then
+// x = (x / f) << 12 | (x % f) + cum.  A segment's slot holds one word per
+// symbol, the most any input can emit, so there is no overflow path; a chunk
+// that codes to more than its raw size is stored raw (decided at the end of the
+// kernel, once all segments of the chunk are coded).
 
-// The 8 symbols of one group (byte j of `sy` = symbol j), last pair first.
-// acc/cnt: the lane's bits that do not fill a dword yet; wp: where its next
-// dword goes.
-template <bool INLDS>
-__device__ __forceinline__ void nz_enc_group(uint32_t& xa, uint32_t& xb, uint64_t& acc, uint32_t& cnt,
-                                             typename NzU32Ptr<INLDS>::type& wp, const uint64_t sy,
-                                             const uint2* __restrict__ symtab) {
-  typedef __attribute__((address_space(3))) const uint16_t lds_cu16;
-  // the per-symbol entries do not depend on the states: fetch them up front
-  uint2 e[8];
+// the 8 symbols of one group (byte j of `sy` = symbol j), last symbol first
+// (words go to the segment's slot in scratch memory, or with LDS to the
+// wavefront's staging area: word p of the slot at LDS byte address lds0 + 2 p)
+template <bool LDS>
+__device__ __forceinline__ void nz_enc_group(uint32_t& x, uint32_t& pos, const uint64_t sy,
+                                             const uint4* __restrict__ tab, uint16_t* __restrict__ slot,
+                                             const uint32_t lds0) {
+  typedef __attribute__((address_space(3))) uint16_t lds_u16;
+  // the table entries do not depend on the state: fetch four at a time, up front
 #pragma unroll
-  for (int j = 0; j < 8; ++j) e[j] = symtab[(uint32_t)(sy >> (8 * j)) & 0xFFu];
+  for (int h = 1; h >= 0; --h) {
+  uint4 e[8];
 #pragma unroll
-  for (int j = 6; j >= 0; j -= 2) {
-    const uint32_t nb = (xb + e[j + 1].x) >> 16;
-    const uint32_t fb = __builtin_amdgcn_ubfe(xb, 0u, nb);
-    xb = *(lds_cu16*)(uintptr_t)(((xb >> nb) << 1) + e[j + 1].y);
-    const uint32_t na = (xa + e[j].x) >> 16;
-    const uint32_t fa = __builtin_amdgcn_ubfe(xa, 0u, na);
-    xa = *(lds_cu16*)(uintptr_t)(((xa >> na) << 1) + e[j].y);
-    acc |= (uint64_t)(fb | (fa << nb)) << cnt;
-    cnt += na + nb;
-    if (cnt >= 32u) {
-      *wp = (uint32_t)acc;
-      ++wp;
-      acc >>= 32;
-      cnt -= 32u;
+  for (int j = 4 * h; j < 4 * h + 4; ++j) e[j] = tab[(uint32_t)(sy >> (8 * j)) & 0xFFu];
+#pragma unroll
+  for (int j = 4 * h + 3; j >= 4 * h; --j) {
+    const uint32_t f = e[j].y;
+    const bool need = x >= e[j].x;
+    const uint64_t m = __ballot(need);
+    pos -= (uint32_t)__popcll(m);
+    if (need) {  // a 32-bit byte offset from the segment's slot: one add-shift for the address
+      if constexpr (LDS)
+        *(lds_u16*)(uintptr_t)(lds0 + ((pos + nz_rank_below(m)) << 1)) = (uint16_t)(x & 0xFFFFu);
+      else
+        *reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(slot) + ((pos + nz_rank_below(m)) << 1)) =
+            (uint16_t)(x & 0xFFFFu);
     }
+    x = need ? (x >> 16) : x;
+    // x < f << 20 here, so the quotient x / f is below 2^20.  The float estimate
+    // x * r with r four units in the last place under 1 / f (itself within half
+    // a unit) never exceeds the quotient - the roundings of x and of the product
+    // add at most one unit each - and falls short of it by less than
+    // 2^20 * 11 * 2^-24 < 1: truncated it is the exact quotient or one less,
+    // and the remainder tells which.  With the exact quotient q the new state
+    // is (q << 12) + (x - q f) + cum = x + q (4096 - f) + cum.
+    uint32_t q = (uint32_t)((float)x * __uint_as_float(e[j].w));
+    q += (x - __umul24(q, f) >= f) ? 1u : 0u;
+    x = __umul24(q, NZ_M - f) + (x + e[j].z);
+  }
   }
 }
 
-// The body of a segment record from what the coding left: the final states, the
-// lengths of the lane streams, and the streams packed back to back (in place:
-// a stream never moves up).  `body`: 97 dwords of head room, then the staging
-// area of `stride` dwords per lane.  -> bytes of the body (uniform).
-template <bool INLDS>
-__device__ __forceinline__ uint32_t nz_enc_body(typename NzU32Ptr<INLDS>::type body, const uint32_t stride,
-                                                const uint32_t len, const uint32_t xa, const uint32_t xb,
-                                                const uint32_t lane) {
-  typedef typename NzU32Ptr<INLDS>::type ptr_t;
-  const auto sync = [&]() {
-    if constexpr (INLDS) {
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-    } else {
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
-      __builtin_amdgcn_wave_barrier();
-    }
-  };
-  // states: 24 bits per lane -> 48 dwords, four lanes per three dwords
-  const uint32_t sv = (xa & (NZ_M - 1u)) | ((xb & (NZ_M - 1u)) << 12);
-  const uint32_t s1 = (uint32_t)__shfl_down((int)sv, 1, 64), s2 = (uint32_t)__shfl_down((int)sv, 2, 64),
-                 s3 = (uint32_t)__shfl_down((int)sv, 3, 64);
-  if ((lane & 3u) == 0u) {
-    ptr_t q = body + (lane >> 2) * 3u;
-    q[0] = sv | (s1 << 24);
-    q[1] = (s1 >> 8) | (s2 << 16);
-    q[2] = (s2 >> 16) | (s3 << 8);
-  }
-  uint32_t mn = len, mx = len;
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    const uint32_t a = (uint32_t)__shfl_xor((int)mn, o, 64), b = (uint32_t)__shfl_xor((int)mx, o, 64);
-    mn = a < mn ? a : mn;
-    mx = b > mx ? b : mx;
-  }
-  const uint32_t lw = (mx - mn) ? 32u - (uint32_t)__clz((int)(mx - mn)) : 0u;  // bits of the largest field
-  if (lane == 0) body[NZ_STATES_BYTES / 4] = mn | (lw << 24);
-  ptr_t fld = body + NZ_STATES_BYTES / 4 + 1;
-  if (lane < 2u * lw) fld[lane] = 0u;
-  sync();
-  if (lw) {
-    const uint32_t v = len - mn, bit = lane * lw, sh = bit & 31u;
-    atomicOr((uint32_t*)(fld + (bit >> 5)), v << sh);
-    if (sh + lw > 32u) atomicOr((uint32_t*)(fld + (bit >> 5) + 1), v >> (32u - sh));
-  }
-  const uint32_t incl = nz_wave_scan(len, lane);
+// Final states, variable length: 64 two-bit codes (code c = 5 + c nibbles),
+// then the states as a little-endian nibble stream in lane order.  A state
+// is >= 2^16, so it takes 20..32 bits; a flat 32 would waste ~4 more per lane.
+__device__ __forceinline__ void nz_enc_finish(const uint32_t x, const uint32_t words, const uint64_t seg,
+                                              uint32_t* __restrict__ sb, const uint32_t lane,
+                                              uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words,
+                                              uint32_t* __restrict__ seg_state_bytes) {
+  const uint32_t code = (x >> 20 ? 1u : 0u) + (x >> 24 ? 1u : 0u) + (x >> 28 ? 1u : 0u);
+  const uint32_t nn = 5u + code;
+  const uint32_t incl = nz_wave_scan(nn, lane);
+  const uint32_t at = incl - nn;  // nibble offset of this lane's field
   const uint32_t total = __builtin_amdgcn_readlane(incl, 63);
-  // pack the streams: lane after lane, all 64 threads on one stream
-  ptr_t dst = fld + 2u * lw;
-  ptr_t stage = body + NZ_BODY_HEAD_MAX / 4;
-  uint32_t pos = 0, carry = 0;
-  for (uint32_t l = 0; l < NZ_LANES; ++l) {
-    const uint32_t ln = __builtin_amdgcn_readlane(len, l);
-    if (ln == 0) continue;
-    const uint32_t nd = (ln + 31u) >> 5, sh = pos & 31u, d0 = pos >> 5;
-    const uint32_t nout = (sh + ln + 31u) >> 5;
-    ptr_t src = stage + l * stride;
-    uint32_t last = 0;
-    for (uint32_t t0 = 0; t0 < nout; t0 += NZ_LANES) {
-      const uint32_t t = t0 + lane;
-      const uint32_t v = t < nd ? src[t] : 0u;
-      const uint32_t vp = (t >= 1u && t - 1u < nd) ? src[t - 1u] : 0u;
-      uint32_t o = sh ? ((v << sh) | (vp >> (32u - sh))) : v;
-      if (t == 0) o |= carry;
-      sync();  // every read of this turn before its writes (a stream never moves up, but it may overlap itself)
-      if (t < nout) dst[d0 + t] = o;
-      if (t0 + NZ_LANES >= nout) last = __builtin_amdgcn_readlane(o, (nout - 1u - t0));
-      sync();
-    }
-    pos += ln;
-    carry = (pos & 31u) ? last : 0u;
+  const uint32_t sbytes = 16u + ((((total + 1u) >> 1) + 3u) & ~3u);
+  for (uint32_t i = lane; i < NZ_STATE_MAX_BYTES / 4; i += 64) sb[i] = 0;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  atomicOr(&sb[lane >> 4], code << (2 * (lane & 15)));
+  const uint64_t field = (uint64_t)x << (4 * (at & 7));
+  atomicOr(&sb[4 + (at >> 3)], (uint32_t)field);
+  if (field >> 32) atomicOr(&sb[5 + (at >> 3)], (uint32_t)(field >> 32));
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  uint32_t* sdst = states + seg * (NZ_STATE_MAX_BYTES / 4);
+  for (uint32_t i = lane; i < sbytes / 4; i += 64) sdst[i] = sb[i];
+  if (lane == 0) {
+    seg_words[seg] = words;
+    seg_state_bytes[seg] = sbytes;
   }
-  sync();
-  return NZ_STATES_BYTES + 4u + 8u * lw + ((((total + 7u) >> 3) + 3u) & ~3u);
 }
 
 // The tensors of one encode call ride in the kernel argument block (as the
@@ -767,14 +695,12 @@ struct NzEncItem {
   uint32_t* d_status;   // bit 0: the container does not fit
   NzNorm nm;            // normalizer bytes (nullptr: none)
   NzGeom g;
-  // slots: nz_slot_bytes() per segment - the record body when it is not assembled in LDS,
-  // the exponent bytes of a chunk stored raw; seg_body: bytes of every segment's record body
-  uint64_t tab_ser, info, carry, slots, seg_body, seg_units, chunk_units;
+  uint64_t exps, tab_ser, info, carry, slots, states, seg_words, seg_sbytes, seg_units, chunk_units;
   uint32_t chunk_end, seg_end;  // running totals over the batch
-  // records straight to their place (`direct` != 0): where the chunks announce
-  // their sizes (two words per chunk, offset into ws), the number that marks
-  // this call's announcements, how often a chunk looks for an announcement
-  // before it gives up, and where it says so (may be null)
+  // records straight to their place (nz_encode_kernel, `direct` != 0): where the
+  // chunks announce their sizes (two words per chunk, offset into ws), the
+  // number that marks this call's announcements, how often a chunk looks for
+  // an announcement before it gives up, and where it says so (may be null)
   uint64_t pub, nonce;
   uint64_t* d_gave_up;
   uint32_t direct, spin_limit;
@@ -788,7 +714,7 @@ struct NzEncItem {
   // before its first use is as good a start as any.
   uint64_t lb_state;
   // `placed`: one byte per segment (offset into ws), left by a direct encode: 1 =
-  // the record is in the container and not in the scratch (its body went there
+  // the record is in the container and not in the scratch (its words went there
   // from LDS).  nz_compact_kernel with `use_placed` takes such records from
   // `old_comp`, where they lie at the offsets they keep.
   uint64_t placed;
@@ -797,7 +723,7 @@ struct NzEncItem {
 };
 struct NzEncBatch {
   uint32_t count;
-  uint32_t stage_dwords;  // nz_encode_kernel: dwords of LDS per wavefront for the record body (dynamic LDS), 0 = none
+  uint32_t stage_words;  // nz_encode_kernel: 16-bit words of LDS staging per wavefront (dynamic LDS), 0 = none
   NzEncItem item[NZ_ENC_BATCH_MAX];
 };
 
@@ -826,22 +752,25 @@ __device__ __forceinline__ void nz_write_header(uint8_t* comp, const NzGeom& g, 
 // ----------------------------------------------------------------------------
 // NT threads (t = 0 .. NT-1) move the record of segment `seg` = segment k of
 // chunk c to o0, counted in 4-byte units from the start of the record area
-// (`mine` = its size in the same units; ci: the chunk's info; `body`: the
-// record body of `body_bytes` bytes, in the segment's slot or in LDS).  With
-// `whole` the record is not assembled from its parts but copied from there (the
-// same record in another container).  They write the segment's directory
-// entry; those of the last segment add the closing entry, the header, the
-// container size and the overflow flag.  -> whether the record fits the
-// container (if not, nothing of it is written).
+// (`mine` = its size in the same units; ci, sbytes, w: the chunk's info, the
+// size of the coder states, the number of words; `words`: where the words are,
+// the end of the segment's slot or a staging area in LDS).  With `whole` the
+// record is not assembled from its parts but copied from there (the same record
+// in another container).  They write the segment's directory entry; those of
+// the last segment add the closing entry, the header, the container size and
+// the overflow flag.  -> whether the record fits the container (if not, nothing
+// of it is written).
 template <uint32_t NT>
 __device__ __forceinline__ bool nz_move_record(const NzEncItem& it, const uint64_t seg, const uint64_t c,
                                                const uint32_t k, const uint64_t o0, const uint32_t mine,
-                                               const NzChunkInfo ci, const uint32_t* body, const uint32_t body_bytes,
-                                               const uint8_t* whole, const uint32_t t) {
+                                               const NzChunkInfo ci, const uint32_t sbytes, const uint32_t w,
+                                               const uint16_t* words, const uint8_t* whole, const uint32_t t) {
   static_assert(NT >= NZ_TAIL_PAD, "too few threads for the closing zeros");
   const NzGeom& g = it.g;
   const uint8_t* __restrict__ tab_ser = it.ws + it.tab_ser;
   const uint8_t* __restrict__ carry = it.ws + it.carry;
+  const uint16_t* __restrict__ slots = reinterpret_cast<const uint16_t*>(it.ws + it.slots);
+  const uint32_t* __restrict__ states = reinterpret_cast<const uint32_t*>(it.ws + it.states);
   uint8_t* __restrict__ comp = it.comp;
   const uint64_t o1 = o0 + mine;
   const bool fits = o1 <= 0xFFFFFFFFull && g.rec_off + 4 * o1 + NZ_TAIL_PAD <= it.comp_cap;
@@ -877,7 +806,7 @@ __device__ __forceinline__ bool nz_move_record(const NzEncItem& it, const uint64
       off = 4;
     }
     const uint32_t padded = (sn + 3) & ~3u;
-    const uint8_t* rawp = it.ws + it.slots + seg * nz_slot_bytes(g.lane_syms);  // left there by the encode kernel
+    const uint8_t* rawp = reinterpret_cast<const uint8_t*>(slots + seg * g.seg_syms);  // left there by the encode kernel
     for (uint32_t i = t; i < padded; i += NT) dst[off + i] = i < sn ? rawp[i] : 0;
     if (sn == nom)
       for (uint32_t i = t; i < NZ_CARRY_BYTES; i += NT) dst[off + padded + i] = carry[seg * NZ_CARRY_BYTES + i];
@@ -889,17 +818,44 @@ __device__ __forceinline__ bool nz_move_record(const NzEncItem& it, const uint64
     for (uint32_t i = t; i < ci.tab_len; i += NT) dst[i] = tb[i];
     off = ci.tab_len;
   }
-  uint32_t* bdst = reinterpret_cast<uint32_t*>(dst + off);
-  const uint32_t nd = body_bytes / 4;
-  for (uint32_t i = t; i < nd; i += NT) bdst[i] = body[i];
+  uint32_t* sdst = reinterpret_cast<uint32_t*>(dst + off);
+  for (uint32_t i = t; i < sbytes / 4; i += NT) sdst[i] = states[seg * (NZ_STATE_MAX_BYTES / 4) + i];
+  // the words are 2-byte aligned; they are moved as dwords (two aligned loads and a
+  // funnel shift when the source is off by one word; the load past the last word
+  // stays inside the scratch buffer or the staging area)
+  const uint16_t* src = words;
+  const uint32_t mis = (uint32_t)((reinterpret_cast<uintptr_t>(src) >> 1) & 1u);
+  const uint32_t* s32 = reinterpret_cast<const uint32_t*>(src - mis);
+  uint32_t* wdst = reinterpret_cast<uint32_t*>(dst + off + sbytes);
+  const uint32_t nd = (w + 1) / 2;
+  const uint32_t nd4 = nd & ~3u;  // four dwords per thread and turn, then the last one to three singly
+  for (uint32_t i = 4 * t; i < nd4; i += 4 * NT) {
+    const uint32_t a0 = s32[i], a1 = s32[i + 1], a2 = s32[i + 2], a3 = s32[i + 3];
+    uint4 v = make_uint4(a0, a1, a2, a3);
+    if (mis) {
+      const uint32_t a4 = s32[i + 4];
+      v = make_uint4(__builtin_amdgcn_alignbit(a1, a0, 16), __builtin_amdgcn_alignbit(a2, a1, 16),
+                     __builtin_amdgcn_alignbit(a3, a2, 16), __builtin_amdgcn_alignbit(a4, a3, 16));
+    }
+    if ((w & 1) && i + 4 == nd) v.w &= 0xFFFFu;  // the padding word of an odd count is zero
+    wdst[i] = v.x;
+    wdst[i + 1] = v.y;
+    wdst[i + 2] = v.z;
+    wdst[i + 3] = v.w;
+  }
+  for (uint32_t i = nd4 + t; i < nd; i += NT) {
+    uint32_t v = mis ? __builtin_amdgcn_alignbit(s32[i + 1], s32[i], 16) : s32[i];
+    if ((w & 1) && i == nd - 1) v &= 0xFFFFu;
+    wdst[i] = v;
+  }
   return true;
 }
 
-// Workgroup = max(4, segments per chunk) wavefronts; wavefront k owns segment k,
-// whose exponents stay in registers (NG groups of 8 symbols per lane).
-extern __shared__ uint32_t nz_enc_stage[];  // record bodies of nz_encode_kernel: stage_dwords per wavefront
+// Segments of up to 8 * NG symbols per lane: the exponents stay in registers.
+// Workgroup = max(4, segments per chunk) wavefronts; wavefront k owns segment k.
+extern __shared__ uint32_t nz_enc_stage[];  // word staging of nz_encode_kernel: stage_words / 2 dwords per wavefront + 4
 template <int S, int NG>
-__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void nz_encode_kernel(const NzEncBatch b) {
+__global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kernel(const NzEncBatch b) {
   __shared__ NzEncLds L;
   uint32_t t = 0, first = 0;
   while (t + 1 < b.count && blockIdx.x >= b.item[t].chunk_end) {
@@ -914,7 +870,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void
   const uint16_t* __restrict__ in = it.in;
   const NzNorm nm = it.nm;
   NzChunkInfo* info = reinterpret_cast<NzChunkInfo*>(it.ws + it.info);
-  uint32_t* seg_body = reinterpret_cast<uint32_t*>(it.ws + it.seg_body);
+  uint32_t* seg_words = reinterpret_cast<uint32_t*>(it.ws + it.seg_words);
+  uint32_t* seg_state_bytes = reinterpret_cast<uint32_t*>(it.ws + it.seg_sbytes);
   uint32_t* seg_units = reinterpret_cast<uint32_t*>(it.ws + it.seg_units);
 
   const uint32_t tid = threadIdx.x;
@@ -930,24 +887,23 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;  // at most NG
   const bool seg_full = has_seg && seg_n == nom;
 
-  // state of the scratch's size announcements (see NzEncItem::lb_state): read
-  // once, by one thread, long before it is needed, so that every thread of the
-  // workgroup acts on the same values
+  // state of the scratch's size announcements (see NzEncItem::lb_state), read
+  // long before it is needed
   uint32_t* lb_state = reinterpret_cast<uint32_t*>(it.ws + it.lb_state);
-  if (tid == 0) {
-    L.lb[0] = it.direct ? __hip_atomic_load(lb_state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-    L.lb[1] = it.direct ? __hip_atomic_load(lb_state + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
-    L.redo = 0;
+  uint32_t lb_gen = 0;
+  bool direct = false;  // this run places its records itself
+  if (it.direct) {
+    lb_gen = __hip_atomic_load(lb_state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    direct = __hip_atomic_load(lb_state + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != NZ_LOOKBACK_ABORT;
   }
   for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += blockDim.x) L.hist[i] = 0;
+  if (tid == 0) L.redo = 0;
   __syncthreads();
-  const uint32_t lb_gen = L.lb[0];
-  const bool direct = it.direct && L.lb[1] != NZ_LOOKBACK_ABORT;  // this run places its records itself
   uint32_t* myhist = L.hist + (lane & (NZ_HIST_COPIES - 1)) * NZ_HIST_STRIDE;
 
   // ---- phase 1: split.  Packed bytes go to the stored layout: segment k of a
   // chunk starts at k * seg_keep, and the last NZ_CARRY_BYTES of a full segment
-  // go to carry[seg] instead (they ride in the coder's start states).
+  // go to carry[seg] instead (they ride in the rANS start states).
   const uint32_t seg_keep = seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES;  // of a segment of nominal length
   const uint64_t chunk_keep = (uint64_t)chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * spc;
   const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
@@ -1025,49 +981,39 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void
   __threadfence_block();  // the carried bytes are read back below
   __syncthreads();
 
-  // ---- the chunk's tables ----
+  // ---- the chunk's table ----
   const uint32_t est_bits = nz_build_table(L, cn, it.ws + it.tab_ser + c * NZ_TABLE_MAX_BYTES, info + c);
 
   // ---- phase 2: code the segment from the registers, last group first ----
-  // The lane streams grow in the wavefront's area of LDS when the records are
-  // placed by this kernel and the estimate says they fit (a quarter more than
-  // the estimate per lane), else in the segment's slot in scratch memory, where
-  // every lane has room for the worst case.  A lane that would still run out of
-  // LDS stops its wavefront; the chunk is then coded again into the slots (the
-  // exponents are still in registers).
+  // The words go to the segment's slot in scratch memory, or, when the records
+  // are placed by this kernel and the estimate says they fit, to the wavefront's
+  // staging area in LDS (the last `stage_w` words of the slot), from where they
+  // are written once, to their final place.  A wavefront that would run out of
+  // staging stops; the chunk is then coded again into the slots (the exponents
+  // are still in registers).
+  const uint32_t cap_words = seg_syms;
+  uint16_t* slot = reinterpret_cast<uint16_t*>(it.ws + it.slots) + seg * cap_words;
+  const uint32_t stage_w = b.stage_words < cap_words ? b.stage_words : cap_words;
+  const uint32_t stage_lo = cap_words - stage_w;  // first word of the slot that has a place in the staging area
+  const uint32_t est_seg_words = (uint32_t)(((uint64_t)est_bits * seg_syms / cn) >> 4);
+  bool staged = direct && stage_w >= 1024 && est_seg_words + (est_seg_words >> 4) + 64 <= stage_w;
   typedef __attribute__((address_space(3))) uint32_t lds_u32;
-  uint32_t* slot = reinterpret_cast<uint32_t*>(it.ws + it.slots + seg * nz_slot_bytes(g.lane_syms));
-  const uint32_t slot_stride = nz_slot_lane_dwords(g.lane_syms);
-  lds_u32* area = (lds_u32*)nz_enc_stage + wave * b.stage_dwords;
-  const uint32_t est_lane = (uint32_t)(((uint64_t)est_bits * g.lane_syms / cn) >> 5);  // dwords of an average lane stream
-  const uint32_t lds_stride = (est_lane + (est_lane >> 2) + 6u) | 1u;  // odd: the lanes' dwords spread over the banks
-  bool staged = direct && b.stage_dwords >= NZ_BODY_HEAD_MAX / 4 + NZ_LANES * lds_stride;
-  uint32_t body_bytes = 0;
+  uint32_t* stage = nz_enc_stage + wave * (b.stage_words / 2);
+  const uint32_t stage_lds = (uint32_t)(uintptr_t)((lds_u32*)stage);
+  uint32_t pos_end = cap_words;  // where the segment's words begin in its slot
   const auto code_segment = [&](auto lds_tag) -> bool {
-    constexpr bool INLDS = decltype(lds_tag)::value != 0;
-    typedef typename NzU32Ptr<INLDS>::type ptr_t;
+    constexpr bool LDS = decltype(lds_tag)::value != 0;
     const uint32_t pad = L.pad_sym;
-    const uint32_t stride = INLDS ? lds_stride : slot_stride;
-    ptr_t body;
-    if constexpr (INLDS) body = area;
-    else body = slot;
-    // a full segment starts from T | 12 carried bits of the packed stream in either state
-    uint32_t pay = 0;
-    if (seg_full)
-      pay = (uint32_t)carry_seg[3 * lane] | ((uint32_t)carry_seg[3 * lane + 1] << 8) | ((uint32_t)carry_seg[3 * lane + 2] << 16);
-    uint32_t xa = NZ_M | (pay & (NZ_M - 1u)), xb = NZ_M | (pay >> 12);
-    uint64_t acc = 0;
-    uint32_t cnt = 0;
-    ptr_t wp0 = body + NZ_BODY_HEAD_MAX / 4 + lane * stride;
-    ptr_t wp = wp0;
+    // a full segment starts from 2^16 | 16 carried bits of the packed stream
+    uint32_t x = NZ_L | (seg_full ? (uint32_t)reinterpret_cast<const uint16_t*>(carry_seg)[lane] : 0u);
+    uint32_t pos = cap_words;
     bool out_of_room = false;
     nz_static_for<NG - 1, 0, -1>([&](auto g8c) {
       constexpr int g8 = decltype(g8c)::value;
       uint32_t gv = (uint32_t)g8;
       asm volatile("" : "+s"(gv));
       if (gv < ngroups && !out_of_room) {
-        // a group writes at most 96 bits: three dwords, and one more for what is left at the end
-        if (INLDS && __ballot((uint32_t)(wp - wp0) + 4u > stride) != 0) {
+        if (LDS && pos - stage_lo < NZ_GROUP * NZ_LANES) {  // a group emits at most 512 words
           out_of_room = true;
         } else {
           uint64_t sy = ex[g8];
@@ -1079,15 +1025,14 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void
               sy = (sy & keepm) | ((0x0101010101010101ull * pad) & ~keepm);
             }
           }
-          nz_enc_group<INLDS>(xa, xb, acc, cnt, wp, sy, L.sym);
+          nz_enc_group<LDS>(x, pos, sy, L.tab, slot, stage_lds - 2u * stage_lo);
         }
       }
     });
     if (out_of_room) return true;
-    if (cnt) *wp = (uint32_t)acc;
-    const uint32_t len = 32u * (uint32_t)(wp - wp0) + cnt;
-    body_bytes = nz_enc_body<INLDS>(body, stride, len, xa, xb, lane);
-    if (lane == 0) seg_body[seg] = body_bytes;
+    nz_enc_finish(x, cap_words - pos, seg, L.sbuf[wave], lane, reinterpret_cast<uint32_t*>(it.ws + it.states),
+                  seg_words, seg_state_bytes);
+    pos_end = pos;
     return false;
   };
 #pragma nounroll
@@ -1099,7 +1044,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void
         code_segment(NzConst<0>{});
       }
     }
-    // every segment of the chunk is coded (or one has run out of room)
+    // every segment of the chunk is coded (or one has run out of staging)
     __threadfence_block();
     __syncthreads();
     if (!(staged && L.redo)) break;
@@ -1107,13 +1052,13 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void
   }
   // decide coded-or-raw and size the records
   if (tid == 0) {
-    L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_body, seg_units,
+    L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
                               reinterpret_cast<uint32_t*>(it.ws + it.chunk_units), L.seg_units, &L.chunk_total);
     L.gave_up = 0;
   }
   __syncthreads();
   if (L.raw && has_seg) {
-    // a chunk that does not compress: its exponent bytes take the place of the body
+    // a chunk that does not compress: its exponent bytes take the place of the words
     uint8_t* rawp = reinterpret_cast<uint8_t*>(slot);
     nz_static_for<0, NG, 1>([&](auto g8c) {
       constexpr int g8 = decltype(g8c)::value;
@@ -1146,14 +1091,13 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void
   // the run's 64-bit mark on top and the size (or its complement) below, so
   // that whatever the scratch memory held before cannot pass for an
   // announcement.  Then it adds up the announcements of the chunks before it,
-  // waiting for those that are not there yet.  Workgroups of one launch are
-  // observed to start in the order of their numbers, so a chunk waited for is
-  // normally running or done, and none of them waits before it has announced;
-  // nothing guarantees that order across the dies of the device or next to
-  // another kernel, so the wait is bounded (`spin_limit` looks per
-  // announcement): a chunk that gives up says so and leaves its records where
-  // they are, for nz_compact_kernel.  Nothing but the announcements passes
-  // between workgroups: relaxed device-scope accesses, no fences.
+  // waiting for those that are not there yet.  Workgroups start in the order of
+  // their numbers, so every chunk waited for is running or done, and none of
+  // them waits before it has announced; the wait is bounded all the same
+  // (`spin_limit` looks per announcement): a chunk that gives up says so and
+  // leaves its records where they are, for nz_compact_kernel.  Nothing but
+  // the announcements passes between workgroups: relaxed device-scope
+  // accesses, no fences.
   typedef unsigned long long nz_u64;
   nz_u64* pub = reinterpret_cast<nz_u64*>(it.ws + it.pub);
   const uint32_t mark_a = (uint32_t)(it.nonce >> 32) ^ lb_gen, mark_b = (uint32_t)it.nonce ^ (lb_gen * 0x9E3779B1u);
@@ -1186,9 +1130,10 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void
   if (lane == 0) L.red64[wave] = part;
   __threadfence_block();  // also: the raw bytes above are read back by the move
   __syncthreads();
-  // a body assembled in LDS to the segment's slot, for the kernel that places records afterwards
+  // staged words of this wavefront to their slot, for the kernel that places records afterwards
   const auto unstage = [&]() {
-    for (uint32_t i = lane; i < body_bytes / 4; i += NZ_LANES) slot[i] = area[i];
+    const uint16_t* sw = reinterpret_cast<const uint16_t*>(stage);
+    for (uint32_t p = pos_end + lane; p < cap_words; p += NZ_LANES) slot[p] = sw[p - stage_lo];
   };
   // the workgroup of the last chunk has seen every other announce (or has given
   // up): all of them have read the count, which can now move on
@@ -1212,11 +1157,127 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, (NG > 32 ? 2 : 4)) void
     for (uint32_t q = 0; q < blockDim.x / 64; ++q) o0 += L.red64[q];
     for (uint32_t q = 0; q < wave; ++q) o0 += L.seg_units[q];
     const bool from_stage = staged && !L.raw;
-    const uint32_t* body = from_stage ? (const uint32_t*)(uint32_t*)area : slot;
-    const bool fits = nz_move_record<64>(it, seg, c, wave, o0, L.seg_units[wave], info[c], body, body_bytes,
-                                         nullptr, lane);
+    const uint16_t* words = from_stage ? reinterpret_cast<const uint16_t*>(stage) + (pos_end - stage_lo) : slot + pos_end;
+    const bool fits = nz_move_record<64>(it, seg, c, wave, o0, L.seg_units[wave], info[c], seg_state_bytes[seg],
+                                         cap_words - pos_end, words, nullptr, lane);
     if (from_stage && !fits) unstage();
     if (lane == 0) placed[seg] = (from_stage && fits) ? 1 : 0;
+  }
+}
+
+// Longer segments: all wavefronts split the chunk into scratch, then one
+// wavefront per segment codes from there.
+template <int S>
+__global__ __launch_bounds__(NZ_ENC_LONG_THREADS) void nz_encode_long_kernel(const NzEncBatch b) {
+  __shared__ NzEncLds L;
+  uint32_t t = 0, first = 0;
+  while (t + 1 < b.count && blockIdx.x >= b.item[t].chunk_end) {
+    first = b.item[t].chunk_end;
+    ++t;
+  }
+  const NzEncItem& it = b.item[t];
+  const NzGeom& g = it.g;
+  const uint64_t c = blockIdx.x - first;
+  const uint64_t n = g.n;
+  const uint32_t chunk_syms = g.chunk_syms, seg_syms = g.seg_syms, spc = g.spc;
+  const uint16_t* __restrict__ in = it.in;
+  const NzNorm nm = it.nm;
+  uint8_t* carry = it.ws + it.carry;
+  uint8_t* exps = it.ws + it.exps;
+  NzChunkInfo* info = reinterpret_cast<NzChunkInfo*>(it.ws + it.info);
+  uint32_t* seg_words = reinterpret_cast<uint32_t*>(it.ws + it.seg_words);
+  uint32_t* seg_state_bytes = reinterpret_cast<uint32_t*>(it.ws + it.seg_sbytes);
+  uint32_t* seg_units = reinterpret_cast<uint32_t*>(it.ws + it.seg_units);
+
+  const uint32_t tid = threadIdx.x;
+  const uint64_t base = c * chunk_syms;
+  const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
+
+  for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += blockDim.x) L.hist[i] = 0;
+  __syncthreads();
+  uint32_t* myhist = L.hist + (tid & (NZ_HIST_COPIES - 1)) * NZ_HIST_STRIDE;
+
+  const uint32_t seg_keep = seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES;     // of a segment of nominal length
+  const uint64_t chunk_keep = (uint64_t)chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * spc;
+  const uint64_t seg0 = c * spc;
+  for (uint32_t i = tid * 8; i < cn; i += blockDim.x * 8) {
+    const uint64_t gi = base + i;
+    const uint32_t sk = i / seg_syms;                       // segment inside the chunk
+    const uint32_t sb = (i - sk * seg_syms) / 8 * (S + 1);  // byte inside the segment
+    const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, sk);
+    const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
+    const bool seg_full = base + (uint64_t)sk * seg_syms + nom <= n;
+    uint8_t* pp = (seg_full && sb >= keep) ? carry + (seg0 + sk) * NZ_CARRY_BYTES + (sb - keep)
+                                           : it.packed + c * chunk_keep + (uint64_t)sk * seg_keep + sb;
+    const uint32_t rem = cn - i;
+    uint64_t e;
+    if (rem >= 8) {
+      uint4 v = *reinterpret_cast<const uint4*>(in + gi);
+      if (nm.bytes) v = nz_scale8<false>(v, nz_norm_load8(nm, gi), nm.log2n >= 3);
+      uint64_t f;
+      nz_split_group<S>(v, e, f);
+      nz_store_packed<S>(pp, f);
+      *reinterpret_cast<uint64_t*>(exps + gi) = e;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) atomicAdd(&myhist[(uint32_t)(e >> (8 * j)) & 0xFFu], 1u);
+    } else {
+      e = nz_split_tail<S>(in, gi, rem, pp, nm);
+      for (uint32_t j = 0; j < rem; ++j) {
+        exps[gi + j] = (uint8_t)(e >> (8 * j));
+        atomicAdd(&myhist[(uint32_t)(e >> (8 * j)) & 0xFFu], 1u);
+      }
+    }
+  }
+  __syncthreads();
+  nz_build_table(L, cn, it.ws + it.tab_ser + c * NZ_TABLE_MAX_BYTES, info + c);
+  // exponents and carried bytes of this chunk are read back below
+  __threadfence_block();
+  __syncthreads();
+
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const uint32_t lane = tid & 63;
+  const uint64_t seg = seg0 + wave;
+  const uint64_t seg_base = base + (uint64_t)wave * seg_syms;
+  const uint32_t cap_words = seg_syms;
+  uint16_t* slot = reinterpret_cast<uint16_t*>(it.ws + it.slots) + seg * cap_words;
+  const bool has_seg = wave < spc && seg_base < n;
+  uint32_t seg_n = 0;
+  if (has_seg) {
+    const uint32_t nom = nz_seg_nominal(chunk_syms, seg_syms, spc, wave);
+    seg_n = (uint32_t)((n - seg_base) < nom ? (n - seg_base) : nom);
+    const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
+    const uint32_t pad = L.pad_sym;
+    const uint8_t* src = exps + seg_base;
+    uint32_t x = NZ_L | (seg_n == nom ? (uint32_t)reinterpret_cast<const uint16_t*>(carry)[seg * NZ_LANES + lane] : 0u);
+    uint32_t pos = cap_words;
+    for (uint32_t gq = ngroups; gq-- > 0;) {
+      const uint32_t idx0 = (gq * NZ_LANES + lane) * NZ_GROUP;
+      uint64_t sy;
+      if (idx0 + 8 <= seg_n) {
+        sy = *reinterpret_cast<const uint64_t*>(src + idx0);
+      } else {
+        sy = 0;
+        for (int j = 0; j < 8; ++j) {
+          uint32_t bb = (idx0 + j < seg_n) ? src[idx0 + j] : pad;
+          sy |= (uint64_t)bb << (8 * j);
+        }
+      }
+      nz_enc_group<false>(x, pos, sy, L.tab, slot, 0u);
+    }
+    nz_enc_finish(x, cap_words - pos, seg, L.sbuf[wave], lane, reinterpret_cast<uint32_t*>(it.ws + it.states),
+                  seg_words, seg_state_bytes);
+  }
+  __threadfence_block();
+  __syncthreads();
+  if (tid == 0) L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
+                                          reinterpret_cast<uint32_t*>(it.ws + it.chunk_units), L.seg_units,
+                                          &L.chunk_total);
+  __syncthreads();
+  if (L.raw && has_seg) {
+    // a chunk that does not compress: its exponent bytes take the place of the words
+    uint8_t* rawp = reinterpret_cast<uint8_t*>(slot);
+    const uint8_t* src = exps + seg_base;
+    for (uint32_t i = lane; i < seg_n; i += 64) rawp[i] = src[i];
   }
 }
 
@@ -1276,7 +1337,8 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   const NzEncItem& it = b.item[t];
   const NzGeom& g = it.g;
   const NzChunkInfo* __restrict__ info = reinterpret_cast<const NzChunkInfo*>(it.ws + it.info);
-  const uint32_t* __restrict__ seg_body = reinterpret_cast<const uint32_t*>(it.ws + it.seg_body);
+  const uint32_t* __restrict__ seg_words = reinterpret_cast<const uint32_t*>(it.ws + it.seg_words);
+  const uint32_t* __restrict__ seg_state_bytes = reinterpret_cast<const uint32_t*>(it.ws + it.seg_sbytes);
   const uint32_t* __restrict__ seg_units = reinterpret_cast<const uint32_t*>(it.ws + it.seg_units);
   const uint32_t* __restrict__ chunk_units = reinterpret_cast<const uint32_t*>(it.ws + it.chunk_units);
   const uint64_t seg = blockIdx.x - first;
@@ -1289,42 +1351,43 @@ __global__ __launch_bounds__(256) void nz_compact_kernel(const NzEncBatch b) {
   if (tid < k) part += seg_units[c * g.spc + tid];
   const uint32_t mine = seg_units[seg];
   const NzChunkInfo ci = info[c];
-  const uint32_t bbytes = seg_body[seg];
+  const uint32_t sbytes = seg_state_bytes[seg];
+  const uint32_t w = seg_words[seg];
   const bool in_old = it.use_placed && (it.ws + it.placed)[seg] != 0;
   const uint64_t o0 = nz_block_sum64(part, red4);
-  const uint32_t* body = reinterpret_cast<const uint32_t*>(it.ws + it.slots + seg * nz_slot_bytes(g.lane_syms));
-  nz_move_record<256>(it, seg, c, k, o0, mine, ci, body, bbytes,
+  const uint16_t* words = reinterpret_cast<const uint16_t*>(it.ws + it.slots) + seg * g.seg_syms + (g.seg_syms - w);
+  nz_move_record<256>(it, seg, c, k, o0, mine, ci, sbytes, w, words,
                       in_old ? it.old_comp + g.rec_off + 4 * o0 : nullptr, tid);
 }
 
 #endif  // NZ_TEMPLATES_ONLY
 
 // ----------------------------------------------------------------------------
-// fused table-ANS decode + merge: one workgroup per chunk, one wavefront per segment
+// fused rANS decode + merge: one workgroup per chunk, one wavefront per segment
 // ----------------------------------------------------------------------------
 //
-// LDS: the state table, 4096 entries of 8 bytes
-//          lo = bits to read | symbol << 24      hi = 8 * (next state before the bits)
-//      (the symbol is a whole byte for v_perm_b32, the bit count sits where
-//      v_bfe_u32 and the shifts look for it, and hi is the byte offset of the
-//      next entry less the bits), then per wavefront `rec_lds` bytes that hold
-//      the segment's whole record: the 64 lanes read their private bit streams
-//      from there.  A record larger than that stays in global memory and is
-//      read from there (slow, and rare: the host sizes rec_lds from the
-//      container's average record).
-// A step of one lane decodes two symbols, one with each of its two states: two
-// independent table reads, one 64-bit window of its stream, two bit-field
-// extracts.  There is no exchange between lanes.
+// LDS: a 4096-entry slot table of 8-byte entries
+//          lo = freq | symbol << 24      hi = slot - cum[symbol]
+//      (so that one v_mad_u32_u24 of lo's low 24 bits gives the next state and
+//      the symbol is a whole byte for v_perm_b32), per wavefront a ring of
+//      1024 16-bit units (2 KiB) that is a sliding window over the segment's
+//      record (it first holds the record's head: table, coder states, first
+//      words), and the 257 cumulative frequencies of the table parse.  Eight
+//      wavefronts per chunk need 49 KiB, so three workgroups share the 160 KiB
+//      of a CU.
+// A rANS step per lane: one table read, one multiply-add, and when the state
+// falls below 2^16 a 16-bit word taken at (words consumed so far by the wave +
+// rank of the lane among the lanes that need one).
 
-// What the table parse leaves for the state-table fill (runs, windows, flags)
-// lies under the last entries of the table itself; those are filled last, from
+#define NZ_RING_ALLOC_DWORDS NZ_RING_DWORDS
+// What the table parse leaves for the slot-table fill (runs, windows, flags)
+// lies in the last slots of the table itself; those are filled last, from
 // registers.
 #define NZ_TMETA_DWORDS (512 + 256 + 4)
-#define NZ_TMETA_SLOT ((uint32_t)(NZ_M - 416))  /* first entry under it; a multiple of 32 */
+#define NZ_TMETA_SLOT ((uint32_t)(NZ_M - 416))  /* first slot under it; a multiple of 32 */
 static_assert(2 * (NZ_M - NZ_TMETA_SLOT) >= NZ_TMETA_DWORDS && NZ_TMETA_SLOT % 32 == 0, "parse results fit under the tail");
 // dynamic LDS of a decode workgroup whose chunks have up to `spc` segments
-#define NZ_DEC_LDS_BYTES(spc, rec_lds) ((size_t)8 * NZ_M + (size_t)(spc) * (size_t)(rec_lds))
-#define NZ_DEC_REC_LDS_MIN 1024u  /* holds table, states and lengths of any record */
+#define NZ_DEC_LDS_BYTES(spc) ((size_t)(2 * NZ_M + (spc) * NZ_RING_ALLOC_DWORDS) * 4)
 
 // S+1 packed bytes of one 8-element group, as a little-endian integer
 template <int S>
@@ -1333,15 +1396,6 @@ __device__ __forceinline__ uint64_t nz_load_sm(const uint8_t* p) {
   else if constexpr (S == 3) return *reinterpret_cast<const uint32_t*>(p);
   else if constexpr (S == 1) return *reinterpret_cast<const uint16_t*>(p);
   else return *p;
-}
-
-// the same from bytes at any alignment (the carried bytes: 192 per segment is not a multiple of every group size)
-template <int S>
-__device__ __forceinline__ uint64_t nz_load_sm_bytes(const uint8_t* p) {
-  uint64_t v = 0;
-#pragma unroll
-  for (int i = 0; i < (S + 1); ++i) v |= (uint64_t)p[i] << (8 * i);
-  return v;
 }
 
 // 8 decoded values to the dense output as a streaming (non-temporal) 16-byte
@@ -1570,76 +1624,142 @@ struct NzGemvWalk {
   }
 };
 
-// Decoder state of one lane.  INLDS: the lane streams are read from the record's
-// copy in LDS (P is an LDS bit address), else from the record in global memory
-// (P counts from the record's first byte).
-template <bool INLDS>
+// Decoder state of one wavefront.
 struct NzWaveDec {
-  uint32_t lut_lds;      // LDS byte address of the state table
-  const uint8_t* rec;    // the record in global memory (uniform)
-  uint32_t P;            // low end of the lane's 32-bit window: the bits above it, up to P + 32, are the next to be read
-                         // (the low 24 bits count; what the sums of table words leave above them is ignored)
-  uint32_t XA, XB;       // 8 * state
+  const uint2* lut;
+  uint32_t* ring32;       // 512 dwords = 1024 words: a window of the record
+  const uint8_t* words;   // start of the record (uniform); word indices count from here
+  uint32_t lim;           // largest byte offset from `words` that may be loaded: container end - 16 (uniform)
+  uint32_t ring_lds;      // LDS byte address of the ring (the same in all lanes, kept in a vector register)
+  uint32_t nwords;        // 16-bit units the record holds, table and states included
+  uint32_t lane;
+  uint32_t x;             // this lane's rANS state
+  uint32_t base;          // words consumed by the wave (the same in all lanes, kept in a vector register)
+  uint32_t filled;        // dwords staged into the ring (multiple of 256; uniform)
+  uint32_t sel_keep, sel_shift;  // byte selectors of the renormalisation (vector registers)
+  uint4 r;                // 8 words per lane fetched during the previous group
 
-  // Decode the next 8 symbols of the lane into byte 3 of ew[0..7], two at a time:
-  // state A's bits are the top of the window, state B's right below.
-  __device__ __forceinline__ void group(uint32_t (&ew)[8]) {
-    typedef uint32_t nz_u32x2 __attribute__((ext_vector_type(2)));
-    typedef __attribute__((address_space(3))) const uint32_t lds_cu32;
-    typedef __attribute__((address_space(3))) const nz_u32x2 lds_cu32x2;
+  // 16 bytes of the word stream at dword index d (multiple of 4 per lane).
+  // Addresses are clamped to the container's closing padding, so every load is
+  // unconditional and in bounds; words past the record are never consumed by
+  // a valid stream.
+  __device__ __forceinline__ uint4 fetch(uint32_t d) const {
+    const uint32_t off = 4u * d < lim ? 4u * d : lim;
+    const uint32_t* q = reinterpret_cast<const uint32_t*>(words + off);
+    return make_uint4(q[0], q[1], q[2], q[3]);
+  }
+
+  __device__ __forceinline__ void commit(uint32_t d, const uint4& v) {
+    *reinterpret_cast<uint4*>(ring32 + (d & (NZ_RING_DWORDS - 1))) = v;
+  }
+
+  // record at comp + pos of a container of comp_bytes (pos + 16 <= comp_bytes)
+  __device__ __forceinline__ void attach(const uint8_t* comp, uint64_t comp_bytes, uint64_t pos, uint32_t* ring) {
+    typedef __attribute__((address_space(3))) uint32_t lds_u32;
+    ring32 = ring;
+    ring_lds = (uint32_t)(uintptr_t)((lds_u32*)ring);
+    words = comp + pos;
+    const uint64_t room = comp_bytes - NZ_TAIL_PAD - pos;
+    lim = room < 0xFFFFFFF0ull ? (uint32_t)room : 0xFFFFFFF0u;
+  }
+
+  // Stage the first 512 dwords of the record (table of a chunk's first record,
+  // coder states, first words) into the ring.
+  __device__ __forceinline__ void stage() {
+    uint4 v[2];
 #pragma unroll
-    for (int j = 0; j < 8; j += 2) {
-      const uint32_t a = (P >> 3) & 0x1FFFFCu;
-      uint32_t w0, w1;
-      if constexpr (INLDS) {
-        w0 = *(lds_cu32*)(uintptr_t)a;
-        w1 = *(lds_cu32*)(uintptr_t)(a + 4u);
-      } else {
-        const uint32_t* q = reinterpret_cast<const uint32_t*>(rec + a);
-        w0 = q[0];
-        w1 = q[1];
-      }
-      const uint32_t D = __builtin_amdgcn_alignbit(w1, w0, P);
-      const nz_u32x2 eA = *(lds_cu32x2*)(uintptr_t)(lut_lds + XA);
-      const nz_u32x2 eB = *(lds_cu32x2*)(uintptr_t)(lut_lds + XB);
-      // offsets and widths are taken from the low five bits of their operands
-      const uint32_t both = eA.x + eB.x;
-      const uint32_t fA = __builtin_amdgcn_ubfe(D, 0u - eA.x, eA.x);
-      const uint32_t fB = __builtin_amdgcn_ubfe(D, 0u - both, eB.x);
-      XA = (fA << 3) + eA.y;
-      XB = (fB << 3) + eB.y;
-      P -= both;
-      ew[j] = eA.x;
-      ew[j + 1] = eB.x;
+    for (uint32_t q = 0; q < 2; ++q) v[q] = fetch(256 * q + 4 * lane);
+#pragma unroll
+    for (uint32_t q = 0; q < 2; ++q) commit(256 * q + 4 * lane, v[q]);
+    filled = 512;
+  }
+
+  // Start decoding from state x0; the words begin `first_word` 16-bit units
+  // into the record (at most 348, so at least 676 words are staged ahead).
+  __device__ __forceinline__ void start(uint32_t x0, uint32_t first_word) {
+    x = x0;
+    base = first_word;
+    filled = __builtin_amdgcn_readfirstlane(filled);
+    r = fetch(filled + 4 * lane);  // the 512 words behind the staged window
+    // keep the three per-lane constants in vector registers of their own (an
+    // instruction can name only one scalar register or literal)
+    sel_keep = 0x07060504u;
+    sel_shift = 0x05040100u;
+    asm volatile("" : "+v"(sel_keep), "+v"(sel_shift), "+v"(ring_lds), "+v"(base));
+  }
+
+  // Decode the next 8 symbols of every lane into byte 3 of ew[0..7].
+  //
+  // Ring upkeep: the 512 words that follow the staged window wait in
+  // registers (`r`, fetched right after the previous commit, addresses clamped
+  // to the container); at the start of a group they are committed to the ring
+  // if no more than 512 words are still ahead of `base`, and the next 512 are
+  // fetched.  A group consumes at most 8 * 64 = 512 words, so at least 512
+  // words are ahead at every group start, the window [base, filled) never
+  // exceeds the 1024 ring words, and a fetch has at least one group (for
+  // exponent data about six) to arrive before its commit.
+  //
+  // A step issues: slot read, multiply-add, compare, the lane's word index
+  // (words consumed by the wave + its rank among the lanes that renormalise:
+  // the two mbcnt instructions add the rank to `base`), the index wrapped into
+  // the ring, the word read, and one byte permute whose selector either keeps
+  // the state or shifts the word in; `base` advances by the ballot's
+  // popcount.  No execution-mask changes and three scalar instructions per
+  // step (popcount and the two waits).
+  __device__ __forceinline__ void group(uint32_t (&ew)[8]) {
+    const uint32_t ahead = __builtin_amdgcn_readfirstlane(base);
+    if ((2 * filled - ahead) <= 512u) {
+      commit(filled + 4 * lane, r);
+      filled += 256;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      r = fetch(filled + 4 * lane);
+    }
+    typedef __attribute__((address_space(3))) const uint16_t lds_cu16;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint2 e = lut[x & (NZ_M - 1)];
+      x = __umul24(e.x, x >> NZ_PROB_BITS) + e.y;
+      ew[j] = e.x;
+      const bool need = x < NZ_L;
+      const uint64_t m = __ballot(need);
+      const uint32_t widx = __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32),
+                                                      __builtin_amdgcn_mbcnt_lo((uint32_t)m, base));
+      uint32_t ring_word = widx & (NZ_RING_WORDS - 1);
+      asm volatile("" : "+v"(ring_word));  // mask, then one shift-add (not shift, mask, add)
+      const uint32_t at = (ring_word << 1) + ring_lds;
+      uint32_t w = *(lds_cu16*)(uintptr_t)at;
+      // keep the word read unconditional: straight-line code, no exec-mask branch
+      asm volatile("" : "+v"(w));
+      const uint32_t sel = need ? sel_shift : sel_keep;
+      x = __builtin_amdgcn_perm(x, w, sel);  // x << 16 | w where the state fell below 2^16
+      base += (uint32_t)__popcll(m);
     }
   }
 };
 
 // One workgroup decodes chunk `c` of one tensor; wavefront k of the workgroup
 // takes segment k of the chunk (wavefronts beyond the chunk's segments only
-// help to build the state table).
+// help to build the slot table).
 // With GEMV the decoded values are not stored: they are multiplied with the
 // activation `gv.x` and summed into `gv.acc` (the tensor is a row-major matrix
 // with rows of gv.in_features elements, a multiple of 512, so that no group is
 // ragged and no group straddles two rows).
 // With NORM every merged value is multiplied by its group's factor (`nm`)
 // before it is stored or used.
-// `rec_lds`: LDS bytes per wavefront for its record (a multiple of 16, at least
-// NZ_DEC_REC_LDS_MIN).
 template <int S, bool GEMV, bool NORM, bool STREAM>
 __device__ __forceinline__ void nz_decode_chunk(
     const uint8_t* __restrict__ comp, const uint64_t comp_bytes, const uint8_t* __restrict__ packed,
     uint16_t* __restrict__ out, const NzGeom& g, uint32_t* __restrict__ d_status, const uint64_t c,
-    const NzGemv& gv, const NzNorm& nm, const uint32_t rec_lds) {
+    const NzGemv& gv, const NzNorm& nm) {
   extern __shared__ uint32_t lds[];
-  typedef __attribute__((address_space(3))) uint32_t lds_u32;
   uint2* lut = reinterpret_cast<uint2*>(lds);                   // 4096 x 8 bytes
-  uint8_t* recs = reinterpret_cast<uint8_t*>(lds + 2 * NZ_M);   // spc record areas of rec_lds bytes
+  uint32_t* rings = lds + 2 * NZ_M;                             // spc rings
   uint32_t* tmeta = lds + 2 * NZ_TMETA_SLOT;                    // what the table parse leaves for the fill:
   uint2* runs = reinterpret_cast<uint2*>(tmeta);                //   per live symbol (freq | symbol << 24, first slot)
   uint2* wins = runs + 256;                                     //   per 32 slots (bitmap of run starts, runs before)
   uint32_t* tflag = reinterpret_cast<uint32_t*>(wins + 128);    //   [0] frequencies sum to 4096, [1] table bytes
-  const uint8_t* tb = recs;                                     // table bytes: start of the chunk's first record
+  const uint8_t* tb = reinterpret_cast<const uint8_t*>(rings);  // table bytes: start of the first record
 
   const uint32_t tid = threadIdx.x;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keep it scalar
@@ -1659,10 +1779,11 @@ __device__ __forceinline__ void nz_decode_chunk(
       atomicOr(d_status, 16u);
   }
 
-  // Two rounds of global loads, then (almost) only LDS: every wavefront reads
-  // the chunk's directory entries itself, then copies its record into its area
-  // of LDS (the chunk's first record begins with the table, which is parsed
-  // from there) and fetches the packed bytes of its first group.
+  // Two rounds of global loads, then only LDS: every wavefront reads the
+  // chunk's directory entries itself, then stages the first 2 KiB of its
+  // record into its ring (for the chunk's first record that window begins with
+  // the table, which all wavefronts parse from there) and fetches the packed
+  // bytes of its first group.
   const uint32_t dv = lane <= nseg ? dir[seg0 + lane] : 0u;
   const uint64_t f0 = __builtin_amdgcn_readlane(dv, 0), f1 = __builtin_amdgcn_readlane(dv, 1);
   if (f1 <= f0 || g.rec_off + 4 * f1 + NZ_TAIL_PAD > comp_bytes) {
@@ -1676,40 +1797,36 @@ __device__ __forceinline__ void nz_decode_chunk(
   const uint32_t seg_n = (uint32_t)((g.n - seg_base) < nom ? (g.n - seg_base) : nom);
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;
   const uint64_t o0 = __builtin_amdgcn_readlane(dv, wk), o1 = __builtin_amdgcn_readlane(dv, wk + 1);
-  const bool bad_rec = o1 < o0 || g.rec_off + 4 * o1 + NZ_TAIL_PAD > comp_bytes || 4 * (o1 - o0) > 0xFFFFF0ull;
+  const bool bad_rec = o1 < o0 || g.rec_off + 4 * o1 + NZ_TAIL_PAD > comp_bytes;
   const uint64_t rec_pos = g.rec_off + 4 * o0;  // uniform: the readlanes above are scalar
-  const uint32_t rec_all = bad_rec ? 0u : (uint32_t)(4 * (o1 - o0));
-  const uint8_t* rec_g = comp + (bad_rec ? g.rec_off : rec_pos);
-  uint8_t* area = recs + (size_t)wk * rec_lds;
-  const bool in_lds = rec_all <= rec_lds;
-  // stored packed layout: every full segment keeps seg_p - NZ_CARRY_BYTES bytes, its
-  // last NZ_CARRY_BYTES bytes ride in the coder states (or behind the symbols of a raw record)
+  const uint32_t rec_all = (uint32_t)(4 * (o1 - o0));
+  // stored packed layout: every full segment keeps seg_p - 128 bytes, its last
+  // 128 bytes ride in the coder states (or behind the symbols of a raw record)
   const bool carry = seg_n == nom;
   const uint32_t keep = nom / 8 * (S + 1) - NZ_CARRY_BYTES;
   const uint64_t chunk_keep = (uint64_t)g.chunk_syms / 8 * (S + 1) - (uint64_t)NZ_CARRY_BYTES * g.spc;
   const uint8_t* pk = packed + c * chunk_keep + (uint64_t)wk * (g.seg_syms / 8 * (S + 1) - NZ_CARRY_BYTES);
   uint16_t* dst = out + seg_base;
   // groups whose packed bytes are (partly) carried are merged after the loop
-  constexpr uint32_t TAILG = (NZ_CARRY_BYTES + 64u * (S + 1) - 1u) / (64u * (S + 1));  // 1, 1, 2, 3 for S = 7, 3, 1, 0
-  const uint32_t tailg = carry ? TAILG : 0u;
+  const uint32_t tailg = carry ? (S == 0 ? 2u : 1u) : 0u;
   const uint32_t body = ngroups - tailg;
   // Groups in which every lane has 8 elements run without any predicate; the
-  // packed bytes are fetched ahead of their use (the address of a fetch past
-  // the last group is clamped, its value unused).
+  // packed bytes are fetched one group ahead of their use (the address of the
+  // fetch past the last group is clamped, its value unused).
   const uint32_t whole = seg_n / NZ_GROUP_SYMS < body ? seg_n / NZ_GROUP_SYMS : body;
   const uint32_t lane_off = lane * (S + 1);
   const uint32_t last_off = whole ? (whole - 1) * NZ_LANES * (S + 1) + lane_off : 0u;
+  NzWaveDec w;
+  w.lut = lut;
+  w.attach(comp, comp_bytes, bad_rec ? 0 : rec_pos, rings + wk * NZ_RING_ALLOC_DWORDS);
+  w.nwords = rec_all / 2;
+  w.lane = lane;
+  w.filled = 0;
   uint64_t sm_next = 0, nb_next = 0;
   uint4 xq_next = make_uint4(0, 0, 0, 0);
   NzGemvWalk walk;
   if (has_seg && !bad_rec) {
-    // the record, or as much of it as the area holds (its head at least), 16 bytes per lane and turn;
-    // the last load may reach up to 12 bytes past the record: the container's closing zeros
-    const uint32_t stage = rec_all < rec_lds ? rec_all : rec_lds;
-    for (uint32_t off = lane * 16u; off < stage; off += 64u * 16u) {
-      const uint32_t* q = reinterpret_cast<const uint32_t*>(rec_g + off);
-      *reinterpret_cast<uint4*>(area + off) = make_uint4(q[0], q[1], q[2], q[3]);
-    }
+    w.stage();
     if constexpr (GEMV) {
       walk.start(gv, g, seg_base, seg_n, wk, lane);
       xq_next = walk.load(walk.col);
@@ -1811,38 +1928,35 @@ __device__ __forceinline__ void nz_decode_chunk(
       }
     }
     __syncthreads();
-    // State table: consecutive threads fill consecutive states.  State X stands
-    // on slot (X % 64) * 64 + X / 64; the symbol of a slot is the run it falls
-    // into (the number of runs that start at or before it, minus one); the
-    // state's rank among the states of its symbol, in ascending order, has a
-    // closed form (nz_state_rank).  (Of a table whose frequencies do not sum to
-    // 4096 nothing was written: the fill then reads zeros and the chunk is
-    // given up right after.)  The last entries lie under the parse results:
-    // they wait in registers until every thread has read what it needs.
+    // slot table: consecutive threads fill consecutive slots.  The run of a
+    // slot is the number of runs that start at or before it, minus one.  (Of a
+    // table whose frequencies do not sum to 4096 nothing was written: the fill
+    // then reads zeros and the chunk is given up right after.)  The last slots
+    // lie under the parse results: their entries wait in registers until every
+    // thread has read what it needs.
     {
-      const auto entry_of = [&](uint32_t X) {
-        const uint32_t slot = ((X & 63u) << 6) | (X >> 6);
+      const uint32_t below = (2u << (tid & 31)) - 1u;  // bits of a window up to this thread's slot
+      const auto entry_of = [&](uint32_t slot) {
         const uint2 wn = wins[slot >> 5];
-        const uint32_t k = wn.y + (uint32_t)__popc(wn.x & ((2u << (slot & 31u)) - 1u)) - 1u;
+        const uint32_t k = wn.y + (uint32_t)__popc(wn.x & below) - 1u;
         const uint2 rn = runs[k & 255u];
-        const uint32_t f = rn.x & 0xFFFFu, xs = f + nz_state_rank(X, rn.y, f);
-        const uint32_t n = (uint32_t)__clz((int)(xs | 1u)) - 19u;  // 12 - floor(log2 xs), xs < 8192
-        return make_uint2(n | (rn.x & 0xFF000000u), (((xs << n) - NZ_M) & (NZ_M - 1u)) << 3);
+        return make_uint2(rn.x, slot - rn.y);
       };
-      for (uint32_t X = tid; X < NZ_TMETA_SLOT; X += blockDim.x) lut[X] = entry_of(X);
+      for (uint32_t slot = tid; slot < NZ_TMETA_SLOT; slot += blockDim.x) lut[slot] = entry_of(slot);
+      // (NZ_TMETA_SLOT is a multiple of 32, so `below` fits these slots as well)
       constexpr uint32_t LAST = (NZ_M - NZ_TMETA_SLOT + 63) / 64;  // per thread, for the smallest workgroup
       uint2 last[LAST];
 #pragma unroll
       for (uint32_t i = 0; i < LAST; ++i) {
-        const uint32_t X = NZ_TMETA_SLOT + tid + i * blockDim.x;
-        last[i] = X < NZ_M ? entry_of(X) : make_uint2(0u, 0u);
+        const uint32_t slot = NZ_TMETA_SLOT + tid + i * blockDim.x;
+        last[i] = slot < NZ_M ? entry_of(slot) : make_uint2(0u, 0u);
       }
       const uint32_t table_ok = tflag[0], table_len = tflag[1];
       __syncthreads();
 #pragma unroll
       for (uint32_t i = 0; i < LAST; ++i) {
-        const uint32_t X = NZ_TMETA_SLOT + tid + i * blockDim.x;
-        if (X < NZ_M) lut[X] = last[i];
+        const uint32_t slot = NZ_TMETA_SLOT + tid + i * blockDim.x;
+        if (slot < NZ_M) lut[slot] = last[i];
       }
       if (!table_ok) {
         if (tid == 0) atomicOr(d_status, 2u);
@@ -1883,7 +1997,7 @@ __device__ __forceinline__ void nz_decode_chunk(
       if (rem >= 8) {
         uint64_t sy = (uint64_t)reinterpret_cast<const uint32_t*>(raw + idx0)[0] |
                       ((uint64_t)reinterpret_cast<const uint32_t*>(raw + idx0)[1] << 32);
-        const uint64_t sm = (carry && b >= keep) ? nz_load_sm_bytes<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
+        const uint64_t sm = (carry && b >= keep) ? nz_load_sm<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
         uint32_t ew[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) ew[j] = (uint32_t)((sy >> (8 * j)) & 0xFFu) << 24;
@@ -1906,157 +2020,136 @@ __device__ __forceinline__ void nz_decode_chunk(
     return;
   }
 
-  // head of the record body, read from the area (it is always staged): the two
-  // start states of every lane, then the lengths of the lane streams
-  if (rec_bytes < NZ_STATES_BYTES + 4u) {
+  if (rec_bytes < 16) {
     if (lane == 0) atomicOr(d_status, 2u);
     return;
   }
-  const uint8_t* bodyp = area + rec_skip;
-  const uint32_t sv = (uint32_t)bodyp[3 * lane] | ((uint32_t)bodyp[3 * lane + 1] << 8) | ((uint32_t)bodyp[3 * lane + 2] << 16);
-  const uint32_t hdr = *reinterpret_cast<const uint32_t*>(bodyp + NZ_STATES_BYTES);
-  const uint32_t minlen = hdr & 0xFFFFFFu, lw = hdr >> 24;
-  if (lw > 24u || rec_bytes < NZ_STATES_BYTES + 4u + 8u * lw) {
+  // final encoder states, read from the staged window: 64 two-bit length
+  // codes, then a nibble stream
+  const uint32_t* rec32 = w.ring32 + rec_skip / 4;
+  const uint32_t nn = 5u + ((rec32[lane >> 4] >> (2 * (lane & 15))) & 3u);
+  const uint32_t incl = nz_wave_scan(nn, lane);
+  const uint32_t at = incl - nn;
+  const uint32_t sbytes = 16u + ((((__builtin_amdgcn_readlane(incl, 63) + 1u) >> 1) + 3u) & ~3u);
+  if (rec_bytes < sbytes) {
     if (lane == 0) atomicOr(d_status, 2u);
     return;
   }
-  const uint32_t fbit = lane * lw;
-  const uint32_t* fwp = reinterpret_cast<const uint32_t*>(bodyp + NZ_STATES_BYTES + 4u) + (fbit >> 5);
-  const uint32_t fld = __builtin_amdgcn_alignbit(fwp[1], fwp[0], fbit) & ((1u << lw) - 1u);  // (the dword past the fields is inside the area)
-  const uint32_t len = minlen + fld;
-  const uint32_t incl = nz_wave_scan(len, lane);
-  const uint32_t total_bits = __builtin_amdgcn_readlane(incl, 63);
-  const uint32_t head = rec_skip + NZ_STATES_BYTES + 4u + 8u * lw;  // first byte of the lane streams, from the record's start
-  if (total_bits > 0xFFFFFFu || (uint64_t)(rec_all - head) * 8u < total_bits) {
-    if (lane == 0) atomicOr(d_status, 2u);
-    return;
-  }
+  // the 8 bytes read here may reach into the words: still inside the window
+  const uint32_t fb = 16u + (at >> 1);
+  const uint64_t win = (uint64_t)rec32[fb >> 2] | ((uint64_t)rec32[(fb >> 2) + 1] << 32);
+  const uint32_t x0 = (uint32_t)(win >> (8 * (fb & 3) + 4 * (at & 1))) & (0xFFFFFFFFu >> (32 - 4 * nn));
+  w.start(x0, (rec_skip + sbytes) / 2);
 
-  const auto run = [&](auto in_lds_tag) {
-    constexpr bool INLDS = decltype(in_lds_tag)::value != 0;
-    NzWaveDec<INLDS> w;
-    w.lut_lds = (uint32_t)(uintptr_t)((lds_u32*)lds);
-    w.rec = rec_g;
-    const uint32_t base_bits = 8u * (head + (INLDS ? (uint32_t)(uintptr_t)((lds_u32*)(uint32_t*)area) : 0u));
-    const uint32_t start_bits = base_bits + incl - len;
-    w.P = base_bits + incl - 32u;
-    w.XA = (sv & 0xFFFu) << 3;
-    w.XB = (sv >> 12) << 3;
-
-    // Groups in which every lane has 8 elements.  Packed bytes (and normalizer
-    // bytes) are fetched TWO groups before their use, alternately into two
-    // registers, so that the wait in front of a merge is for a load issued two
-    // groups earlier and for nothing younger: neither the latency of a load
-    // that misses every cache nor the previous group's store is waited for.
-    const auto sm_at = [&](uint32_t gq) {
-      const uint32_t off = gq * NZ_LANES * (S + 1) + lane_off;
-      return nz_stream_sm<S>(pk + (off < last_off ? off : last_off));
-    };
-    // `wide`: groups of 8 elements or more, one byte per lane and group.  The
-    // walk over the full groups exists once per case, so that the common one has
-    // no branch between the byte's load and its use two groups later (a load
-    // behind a branch is waited for at the join, with every store before it).
-    const auto nb_at = [&](uint32_t gq, auto wide) -> uint64_t {
-      const uint64_t e0 = seg_base + ((gq < whole ? gq : whole - 1) * NZ_LANES + lane) * NZ_GROUP;
-      if constexpr (decltype(wide)::value) return nm.bytes[e0 >> nm.log2n];
-      else return nz_norm_load8(nm, e0);
-    };
-    const auto full_group = [&](uint32_t gq, const uint64_t sm, const uint64_t nb, auto wide) {
-      const uint4 xq = xq_next;
-      if constexpr (GEMV) xq_next = walk.load(walk.next_col());  // always inside x
-      uint32_t ew[8];
-      w.group(ew);
-      // the merge starts only here: its wait for the packed bytes must not be
-      // hoisted in front of the decode steps
-      uint32_t sml = (uint32_t)sm, smh = (uint32_t)(sm >> 32);
-      asm volatile("" : "+v"(sml), "+v"(smh), "+v"(ew[7]));
-      uint4 mv = nz_merge_group<S>(((uint64_t)smh << 32) | sml, ew);
-      if constexpr (NORM) mv = nz_scale8<true>(mv, nb, decltype(wide)::value);
-      if constexpr (GEMV) walk.add(mv, xq, lane);
-      else if constexpr (STREAM) nz_stream_store(dst + (gq * NZ_LANES + lane) * NZ_GROUP, mv);
-      else *reinterpret_cast<uint4*>(dst + (gq * NZ_LANES + lane) * NZ_GROUP) = mv;
-    };
-    const auto full_groups = [&](auto wide) {
-      uint64_t sm_a = sm_next, sm_b = 0, nb_a = nb_next, nb_b = 0;
-      if (whole > 1) {
-        sm_b = sm_at(1);
-        if constexpr (NORM) nb_b = nb_at(1, wide);
-      }
-      uint32_t gq = 0;
-      for (; gq + 1 < whole; gq += 2) {
-        full_group(gq, sm_a, nb_a, wide);
-        sm_a = sm_at(gq + 2);
-        if constexpr (NORM) nb_a = nb_at(gq + 2, wide);
-        full_group(gq + 1, sm_b, nb_b, wide);
-        sm_b = sm_at(gq + 3);
-        if constexpr (NORM) nb_b = nb_at(gq + 3, wide);
-      }
-      if (gq < whole) full_group(gq, sm_a, nb_a, wide);
-    };
-    if (!NORM || nm.log2n >= 3) full_groups(NzConst<1>{});
-    else full_groups(NzConst<0>{});
-    if (!GEMV && whole < body) {  // the ragged last group of the tensor
-      const uint32_t idx0 = (whole * NZ_LANES + lane) * NZ_GROUP;
-      uint32_t ew[8];
-      w.group(ew);
-      if (idx0 < seg_n) {
-        const uint32_t rem = seg_n - idx0 < 8 ? seg_n - idx0 : 8;
-        for (uint32_t j = 0; j < rem; ++j) {
-          const uint32_t bit = (idx0 + j) * (S + 1);
-          const uint32_t rp = ((uint32_t)pk[bit >> 3] >> (7u - S - (bit & 7u))) & ((2u << S) - 1u);
-          uint32_t sym = 0;
-#pragma unroll
-          for (int q = 0; q < 8; ++q) sym = (uint32_t)q == j ? (ew[q] >> 24) : sym;
-          uint32_t h = nz_merge_one<S>(sym, rp);
-          if constexpr (NORM) h = nz_norm_mul(h, nm.bytes[(seg_base + idx0 + j) >> nm.log2n]);
-          dst[idx0 + j] = (uint16_t)h;
-        }
-      }
-    }
-    uint32_t ext[TAILG][8];
-#pragma unroll
-    for (uint32_t t = 0; t < TAILG; ++t)
-      if (t < tailg) w.group(ext[t]);
-
-    // every lane must have read its stream down to its first bit and be back at
-    // the encoder's start states (T | carried bits; zero when nothing is carried)
-    const uint32_t fin = (w.XA >> 3) | ((w.XB >> 3) << 12);
-    const bool bad = (((w.P + 32u) ^ start_bits) & 0xFFFFFFu) != 0u || (!carry && fin != 0u);
-    if (__ballot(bad) != 0 && lane == 0) atomicOr(d_status, 4u);
-
-    if (carry) {
-      // the record's copy is dead now: park the carried bytes at the start of the area
-      area[3 * lane] = (uint8_t)fin;
-      area[3 * lane + 1] = (uint8_t)(fin >> 8);
-      area[3 * lane + 2] = (uint8_t)(fin >> 16);
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      const uint8_t* tailp = area;
-#pragma unroll
-      for (uint32_t t = 0; t < TAILG; ++t) {
-        if (t < tailg) {
-          const uint32_t idx0 = ((body + t) * NZ_LANES + lane) * NZ_GROUP;
-          const uint32_t b = idx0 / 8 * (S + 1);
-          const uint64_t sm = b >= keep ? nz_load_sm_bytes<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
-          uint4 mv = nz_merge_group<S>(sm, ext[t]);
-          if constexpr (NORM) mv = nz_scale8<true>(mv, nz_norm_load8(nm, seg_base + idx0), nm.log2n >= 3);
-          if constexpr (GEMV) walk.add(mv, walk.load(walk.col), lane);
-          else *reinterpret_cast<uint4*>(dst + idx0) = mv;
-        }
-      }
-    }
-    if constexpr (GEMV)
-      if (walk.pending) walk.flush(lane);
+  // Groups in which every lane has 8 elements.  Packed bytes (and normalizer
+  // bytes) are fetched TWO groups before their use, alternately into two
+  // registers, so that the wait in front of a merge is for a load issued two
+  // groups (about two microseconds) earlier and for nothing younger: neither
+  // the latency of a load that misses every cache nor the previous group's
+  // store is waited for.
+  const auto sm_at = [&](uint32_t gq) {
+    const uint32_t off = gq * NZ_LANES * (S + 1) + lane_off;
+    return nz_stream_sm<S>(pk + (off < last_off ? off : last_off));
   };
-  if (in_lds) run(NzConst<1>{});
-  else run(NzConst<0>{});
+  // `wide`: groups of 8 elements or more, one byte per lane and group.  The
+  // walk over the full groups exists once per case, so that the common one has
+  // no branch between the byte's load and its use two groups later (a load
+  // behind a branch is waited for at the join, with every store before it).
+  const auto nb_at = [&](uint32_t gq, auto wide) -> uint64_t {
+    const uint64_t e0 = seg_base + ((gq < whole ? gq : whole - 1) * NZ_LANES + lane) * NZ_GROUP;
+    if constexpr (decltype(wide)::value) return nm.bytes[e0 >> nm.log2n];
+    else return nz_norm_load8(nm, e0);
+  };
+  const auto full_group = [&](uint32_t gq, const uint64_t sm, const uint64_t nb, auto wide) {
+    const uint4 xq = xq_next;
+    if constexpr (GEMV) xq_next = walk.load(walk.next_col());  // always inside x
+    uint32_t ew[8];
+    w.group(ew);
+    // the merge starts only here: its wait for the packed bytes must not be
+    // hoisted in front of the rANS steps
+    uint32_t sml = (uint32_t)sm, smh = (uint32_t)(sm >> 32);
+    asm volatile("" : "+v"(sml), "+v"(smh), "+v"(ew[7]));
+    uint4 mv = nz_merge_group<S>(((uint64_t)smh << 32) | sml, ew);
+    if constexpr (NORM) mv = nz_scale8<true>(mv, nb, decltype(wide)::value);
+    if constexpr (GEMV) walk.add(mv, xq, lane);
+    else if constexpr (STREAM) nz_stream_store(dst + (gq * NZ_LANES + lane) * NZ_GROUP, mv);
+    else *reinterpret_cast<uint4*>(dst + (gq * NZ_LANES + lane) * NZ_GROUP) = mv;
+  };
+  const auto full_groups = [&](auto wide) {
+    uint64_t sm_a = sm_next, sm_b = 0, nb_a = nb_next, nb_b = 0;
+    if (whole > 1) {
+      sm_b = sm_at(1);
+      if constexpr (NORM) nb_b = nb_at(1, wide);
+    }
+    uint32_t gq = 0;
+    for (; gq + 1 < whole; gq += 2) {
+      full_group(gq, sm_a, nb_a, wide);
+      sm_a = sm_at(gq + 2);
+      if constexpr (NORM) nb_a = nb_at(gq + 2, wide);
+      full_group(gq + 1, sm_b, nb_b, wide);
+      sm_b = sm_at(gq + 3);
+      if constexpr (NORM) nb_b = nb_at(gq + 3, wide);
+    }
+    if (gq < whole) full_group(gq, sm_a, nb_a, wide);
+  };
+  if (!NORM || nm.log2n >= 3) full_groups(NzConst<1>{});
+  else full_groups(NzConst<0>{});
+  if (!GEMV && whole < body) {  // the ragged last group of the tensor
+    const uint32_t idx0 = (whole * NZ_LANES + lane) * NZ_GROUP;
+    uint32_t ew[8];
+    w.group(ew);
+    if (idx0 < seg_n) {
+      const uint32_t rem = seg_n - idx0 < 8 ? seg_n - idx0 : 8;
+      for (uint32_t j = 0; j < rem; ++j) {
+        const uint32_t bit = (idx0 + j) * (S + 1);
+        const uint32_t rp = ((uint32_t)pk[bit >> 3] >> (7u - S - (bit & 7u))) & ((2u << S) - 1u);
+        uint32_t sym = 0;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) sym = (uint32_t)q == j ? (ew[q] >> 24) : sym;
+        uint32_t h = nz_merge_one<S>(sym, rp);
+        if constexpr (NORM) h = nz_norm_mul(h, nm.bytes[(seg_base + idx0 + j) >> nm.log2n]);
+        dst[idx0 + j] = (uint16_t)h;
+      }
+    }
+  }
+  uint32_t ext[2][8];
+#pragma unroll
+  for (uint32_t t = 0; t < 2; ++t)
+    if (t < tailg) w.group(ext[t]);
+
+  // every lane must be back at the encoder's start state (2^16 | carried bits)
+  // and the wave must not have read past its record
+  const bool bad = (carry ? (w.x >> 16) != 1u : w.x != NZ_L) || (w.base > w.nwords);
+  if (__ballot(bad) != 0 && lane == 0) atomicOr(d_status, 4u);
+
+  if (carry) {
+    // the ring is dead now: park the 128 carried bytes at its start
+    reinterpret_cast<uint16_t*>(w.ring32)[lane] = (uint16_t)(w.x & 0xFFFFu);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const uint8_t* tailp = reinterpret_cast<const uint8_t*>(w.ring32);
+#pragma unroll
+    for (uint32_t t = 0; t < 2; ++t) {
+      if (t < tailg) {
+        const uint32_t idx0 = ((body + t) * NZ_LANES + lane) * NZ_GROUP;
+        const uint32_t b = idx0 / 8 * (S + 1);
+        const uint64_t sm = b >= keep ? nz_load_sm<S>(tailp + (b - keep)) : nz_load_sm<S>(pk + b);
+        uint4 mv = nz_merge_group<S>(sm, ext[t]);
+        if constexpr (NORM) mv = nz_scale8<true>(mv, nz_norm_load8(nm, seg_base + idx0), nm.log2n >= 3);
+        if constexpr (GEMV) walk.add(mv, walk.load(walk.col), lane);
+        else *reinterpret_cast<uint4*>(dst + idx0) = mv;
+      }
+    }
+  }
+  if constexpr (GEMV)
+    if (walk.pending) walk.flush(lane);
 }
 
 template <int S, bool NORM, bool STREAM>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
-    uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status, const NzNorm nm, uint32_t rec_lds) {
-  nz_decode_chunk<S, false, NORM, STREAM>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x, NzGemv{}, nm, rec_lds);
+    uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status, const NzNorm nm) {
+  nz_decode_chunk<S, false, NORM, STREAM>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x, NzGemv{}, nm);
 }
 
 // Several tensors in one launch: the grid is the concatenation of their
@@ -2081,7 +2174,7 @@ struct NzBatch {
   uint32_t in_features;  // matrix-vector product only
   const uint16_t* x;     // matrix-vector product only
   uint32_t log2n;        // normalized tensors only
-  uint32_t rec_lds;      // LDS bytes per wavefront for its record
+  uint32_t reserved;
   NzBatchItem item[NZ_BATCH_MAX];
 };
 
@@ -2095,7 +2188,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_batch_ke
   }
   const NzBatchItem& it = b.item[t];
   nz_decode_chunk<S, false, NORM, STREAM>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status,
-                                          blockIdx.x - first, NzGemv{}, NzNorm{it.norm, b.log2n}, b.rec_lds);
+                                          blockIdx.x - first, NzGemv{}, NzNorm{it.norm, b.log2n});
 }
 
 // The same walk over several matrices that multiply one activation row.
@@ -2110,7 +2203,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_gemv_ker
   const NzBatchItem& it = b.item[t];
   const NzGemv gv{b.x, it.acc, it.y, it.bias, b.in_features};
   nz_decode_chunk<S, true, NORM, false>(it.comp, it.comp_bytes, it.packed, nullptr, it.g, d_status,
-                                        blockIdx.x - first, gv, NzNorm{it.norm, b.log2n}, b.rec_lds);
+                                        blockIdx.x - first, gv, NzNorm{it.norm, b.log2n});
 }
 
 // ----------------------------------------------------------------------------
@@ -2124,7 +2217,7 @@ template <int S, bool NORM>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_rows_kernel(
     const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
     uint16_t* __restrict__ scratch, NzGeom g, uint32_t* __restrict__ d_status, const NzNorm nm,
-    const long long* __restrict__ indices, uint32_t row_len, uint32_t cpr, uint32_t rec_lds) {
+    const long long* __restrict__ indices, uint32_t row_len, uint32_t cpr) {
   const uint32_t i = blockIdx.x / cpr, k = blockIdx.x - i * cpr;
   const long long idx = indices[i];
   if (idx < 0 || (uint64_t)idx >= g.n / row_len) {
@@ -2138,7 +2231,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_rows_ker
   // that the chunk's first element lands at the start of this workgroup's slot
   uint16_t* out = scratch + ((int64_t)blockIdx.x - (int64_t)c) * (int64_t)g.chunk_syms;
   // (the slots are read back by the copy kernel right away: ordinary stores)
-  nz_decode_chunk<S, false, NORM, false>(comp, comp_bytes, packed, out, g, d_status, c, NzGemv{}, nm, rec_lds);
+  nz_decode_chunk<S, false, NORM, false>(comp, comp_bytes, packed, out, g, d_status, c, NzGemv{}, nm);
 }
 
 #ifndef NZ_TEMPLATES_ONLY

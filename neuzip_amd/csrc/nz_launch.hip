@@ -6,57 +6,37 @@
 #define NZ_TEMPLATES_ONLY
 #include "nz_launch.h"
 
-#define NZ_MAX_LDS (160 * 1024)
-
 template <int S>
-hipError_t nz_allow_lds() {
-  hipError_t e = hipSuccess;
-#define NZ_ALLOW(kernel)                                                                                   \
-  if (e == hipSuccess)                                                                                     \
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&kernel), hipFuncAttributeMaxDynamicSharedMemorySize, \
-                            NZ_MAX_LDS - (int)sizeof(NzEncLds) - 1024)
-  NZ_ALLOW((nz_encode_kernel<S, 8>));
-  NZ_ALLOW((nz_encode_kernel<S, 16>));
-  NZ_ALLOW((nz_encode_kernel<S, 32>));
-  NZ_ALLOW((nz_encode_kernel<S, 64>));
-#undef NZ_ALLOW
-#define NZ_ALLOW(kernel)                                                                                   \
-  if (e == hipSuccess)                                                                                     \
-    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&kernel), hipFuncAttributeMaxDynamicSharedMemorySize, NZ_MAX_LDS)
-  NZ_ALLOW((nz_decode_kernel<S, false, false>));
-  NZ_ALLOW((nz_decode_kernel<S, false, true>));
-  NZ_ALLOW((nz_decode_kernel<S, true, false>));
-  NZ_ALLOW((nz_decode_kernel<S, true, true>));
-  NZ_ALLOW((nz_decode_batch_kernel<S, false, false>));
-  NZ_ALLOW((nz_decode_batch_kernel<S, false, true>));
-  NZ_ALLOW((nz_decode_batch_kernel<S, true, false>));
-  NZ_ALLOW((nz_decode_batch_kernel<S, true, true>));
-  NZ_ALLOW((nz_decode_gemv_kernel<S, false>));
-  NZ_ALLOW((nz_decode_gemv_kernel<S, true>));
-  NZ_ALLOW((nz_decode_rows_kernel<S, false>));
-  NZ_ALLOW((nz_decode_rows_kernel<S, true>));
-#undef NZ_ALLOW
+hipError_t nz_allow_encode_lds() {
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nz_encode_kernel<S, 8>),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nz_encode_kernel<S, 16>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nz_encode_kernel<S, 32>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
   return e;
 }
 
 template <int S>
-void nz_launch_encode(const NzEncBatch& b, int ng, dim3 grid, dim3 block, uint32_t lds, hipStream_t st) {
-  switch (ng) {
-    case 8: hipLaunchKernelGGL((nz_encode_kernel<S, 8>), grid, block, lds, st, b); break;
-    case 16: hipLaunchKernelGGL((nz_encode_kernel<S, 16>), grid, block, lds, st, b); break;
-    case 32: hipLaunchKernelGGL((nz_encode_kernel<S, 32>), grid, block, lds, st, b); break;
-    default: hipLaunchKernelGGL((nz_encode_kernel<S, 64>), grid, block, lds, st, b); break;
+void nz_launch_encode(const NzEncBatch& b, int cls, dim3 grid, dim3 block, uint32_t lds, hipStream_t st) {
+  switch (cls) {
+    case 0: hipLaunchKernelGGL((nz_encode_kernel<S, 8>), grid, block, lds, st, b); break;
+    case 1: hipLaunchKernelGGL((nz_encode_kernel<S, 16>), grid, block, lds, st, b); break;
+    case 2: hipLaunchKernelGGL((nz_encode_kernel<S, 32>), grid, block, lds, st, b); break;
+    default: hipLaunchKernelGGL((nz_encode_long_kernel<S>), grid, dim3(NZ_ENC_LONG_THREADS), 0, st, b); break;
   }
 }
 
 template <int S>
 void nz_launch_decode(const NzGeom& g, const void* comp, uint64_t comp_bytes, const void* packed, void* out,
-                      uint32_t* d_status, const NzNorm& nm, uint32_t stream_out, uint32_t rec_lds, hipStream_t st) {
-  const size_t lds = NZ_DEC_LDS_BYTES(g.spc, rec_lds);
+                      uint32_t* d_status, const NzNorm& nm, uint32_t stream_out, hipStream_t st) {
+  const size_t lds = NZ_DEC_LDS_BYTES(g.spc);
   const dim3 gd((uint32_t)g.n_chunks), bd(64 * g.spc);
 #define NZ_DEC_LAUNCH(NORM, STREAM)                                                                            \
   hipLaunchKernelGGL((nz_decode_kernel<S, NORM, STREAM>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes, \
-                     (const uint8_t*)packed, (uint16_t*)out, g, d_status, nm, rec_lds)
+                     (const uint8_t*)packed, (uint16_t*)out, g, d_status, nm)
   if (nm.bytes) {
     if (stream_out) NZ_DEC_LAUNCH(true, true);
     else NZ_DEC_LAUNCH(true, false);
@@ -70,7 +50,7 @@ void nz_launch_decode(const NzGeom& g, const void* comp, uint64_t comp_bytes, co
 template <int S>
 void nz_launch_decode_batch(const NzBatch& b, uint32_t grid, uint32_t max_spc, bool stream_out, uint32_t* d_status,
                             hipStream_t st) {
-  const size_t lds = NZ_DEC_LDS_BYTES(max_spc, b.rec_lds);
+  const size_t lds = NZ_DEC_LDS_BYTES(max_spc);
   const dim3 gd(grid), bd(64 * max_spc);
 #define NZ_BATCH_LAUNCH(NORM, STREAM) \
   hipLaunchKernelGGL((nz_decode_batch_kernel<S, NORM, STREAM>), gd, bd, lds, st, b, d_status)
@@ -86,7 +66,7 @@ void nz_launch_decode_batch(const NzBatch& b, uint32_t grid, uint32_t max_spc, b
 
 template <int S>
 void nz_launch_gemv(const NzBatch& b, uint32_t grid, uint32_t max_spc, uint32_t* d_status, hipStream_t st) {
-  const size_t lds = NZ_DEC_LDS_BYTES(max_spc, b.rec_lds);
+  const size_t lds = NZ_DEC_LDS_BYTES(max_spc);
   const dim3 gd(grid), bd(64 * max_spc);
   if (b.item[0].norm) hipLaunchKernelGGL((nz_decode_gemv_kernel<S, true>), gd, bd, lds, st, b, d_status);
   else hipLaunchKernelGGL((nz_decode_gemv_kernel<S, false>), gd, bd, lds, st, b, d_status);
@@ -95,22 +75,22 @@ void nz_launch_gemv(const NzBatch& b, uint32_t grid, uint32_t max_spc, uint32_t*
 template <int S>
 void nz_launch_rows(const NzGeom& g, const void* comp, uint64_t comp_bytes, const void* packed, uint16_t* scratch,
                     uint32_t* d_status, const NzNorm& nm, const long long* idx, uint32_t count, uint32_t row_len,
-                    uint32_t cpr, uint32_t rec_lds, hipStream_t st) {
-  const size_t lds = NZ_DEC_LDS_BYTES(g.spc, rec_lds);
+                    uint32_t cpr, hipStream_t st) {
+  const size_t lds = NZ_DEC_LDS_BYTES(g.spc);
   const dim3 gd(count * cpr), bd(64 * g.spc);
   if (nm.bytes)
     hipLaunchKernelGGL((nz_decode_rows_kernel<S, true>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,
-                       (const uint8_t*)packed, scratch, g, d_status, nm, idx, row_len, cpr, rec_lds);
+                       (const uint8_t*)packed, scratch, g, d_status, nm, idx, row_len, cpr);
   else
     hipLaunchKernelGGL((nz_decode_rows_kernel<S, false>), gd, bd, lds, st, (const uint8_t*)comp, comp_bytes,
-                       (const uint8_t*)packed, scratch, g, d_status, nm, idx, row_len, cpr, rec_lds);
+                       (const uint8_t*)packed, scratch, g, d_status, nm, idx, row_len, cpr);
 }
 
-template hipError_t nz_allow_lds<NZ_S>();
+template hipError_t nz_allow_encode_lds<NZ_S>();
 template void nz_launch_encode<NZ_S>(const NzEncBatch&, int, dim3, dim3, uint32_t, hipStream_t);
 template void nz_launch_decode<NZ_S>(const NzGeom&, const void*, uint64_t, const void*, void*, uint32_t*, const NzNorm&,
-                                     uint32_t, uint32_t, hipStream_t);
+                                     uint32_t, hipStream_t);
 template void nz_launch_decode_batch<NZ_S>(const NzBatch&, uint32_t, uint32_t, bool, uint32_t*, hipStream_t);
 template void nz_launch_gemv<NZ_S>(const NzBatch&, uint32_t, uint32_t, uint32_t*, hipStream_t);
 template void nz_launch_rows<NZ_S>(const NzGeom&, const void*, uint64_t, const void*, uint16_t*, uint32_t*,
-                                   const NzNorm&, const long long*, uint32_t, uint32_t, uint32_t, uint32_t, hipStream_t);
+                                   const NzNorm&, const long long*, uint32_t, uint32_t, uint32_t, hipStream_t);

@@ -339,16 +339,15 @@ typedef struct {
 } geom_t;
 
 int nzo_check_geometry(uint32_t chunk_syms, uint32_t lane_syms) {
-  if (lane_syms < 24 || lane_syms % NZO_GROUP) return NZO_ERR_ARG;
-  if (lane_syms > NZO_MAX_LANE_SYMS) return NZO_ERR_ARG;
+  if (lane_syms < 16 || lane_syms % NZO_GROUP) return NZO_ERR_ARG;
+  if (lane_syms > (1u << 16)) return NZO_ERR_ARG;
   uint64_t seg = (uint64_t)lane_syms * NZO_LANES;
   if (chunk_syms == 0 || chunk_syms % NZO_GROUP_SYMS || chunk_syms > (1u << 24)) return NZO_ERR_ARG;
   /* a chunk is cut into spc segments of 64 * lane_syms symbols, the last one
-     holding what remains (at least 1536 symbols, so that it can carry 192 bytes
-     at one bit per element) */
+     holding what remains (at least 1024 symbols, so that it can carry 128 bytes) */
   uint64_t spc = (chunk_syms + seg - 1) / seg;
   if (spc < 1 || spc > 8) return NZO_ERR_ARG;
-  if (chunk_syms - (spc - 1) * seg < 8 * NZO_CARRY_BYTES) return NZO_ERR_ARG;
+  if (chunk_syms - (spc - 1) * seg < 1024) return NZO_ERR_ARG;
   return NZO_OK;
 }
 
@@ -375,18 +374,16 @@ static uint32_t seg_nominal(const geom_t* g, uint32_t k) {
 
 /* worst-case bytes of one segment record holding seg_n symbols */
 static size_t seg_rec_cap(const geom_t* g) {
-  /* table (<= 420) + states (192) + lengths (4 + 8 * 24) + 12 bits per symbol; RAW: 4 + seg_syms + 192 */
-  size_t coded = 420 + 3 * NZO_LANES + 4 + 192 + ((size_t)g->seg_syms * NZO_PROB_BITS + 7) / 8 + 8;
-  size_t raw = 4 + (size_t)g->seg_syms + NZO_CARRY_BYTES + 8;
-  return coded > raw ? coded : raw;
+  /* table (<= 420) + states (<= 272) + words (at most one per symbol) ; RAW: 4 + seg_syms + 128 */
+  return 420 + 272 + 2 * (size_t)g->seg_syms + 8;
 }
 
 size_t nzo_exp_bound(uint64_t n, uint32_t chunk_syms, uint32_t lane_syms) {
   geom_t g;
   if (make_geom(&g, n, chunk_syms, lane_syms)) return 0;
   /* a chunk is never stored larger than its RAW form: 4 per chunk, and per
-     segment pad4(seg_n) symbols + the carried bytes */
-  return g.rec_off + (size_t)n + (4 + NZO_CARRY_BYTES) * (size_t)g.n_segs + 4 * (size_t)g.n_chunks +
+     segment pad4(seg_n) symbols + 128 carried bytes */
+  return g.rec_off + (size_t)n + (4 + 2 * NZO_LANES) * (size_t)g.n_segs + 4 * (size_t)g.n_chunks +
          NZO_TAIL_PAD;
 }
 
@@ -399,235 +396,132 @@ static void put32(uint8_t* p, uint32_t v) {
 static uint32_t get32(const uint8_t* p) {
   return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
 }
-/* ------------------------------------------------------------------------- */
-/* tANS tables of a chunk                                                    */
-/* ------------------------------------------------------------------------- */
-
-/* The coder is a table ANS with T = 4096 states.  Slot i of [0, T) belongs to
-   the symbol whose cumulative frequency range holds i; state X stands on slot
-   (X mod 64) * 64 + X div 64 (the two base-64 digits of X swapped), which
-   spreads every symbol's states evenly over [0, T).  The k-th state of symbol s
-   in ascending order (k = 0 .. f-1) stands for x_s = f + k:
-     decoder, in state X: symbol s, n = 12 - floor(log2 x_s) bits are read,
-                          next state = (x_s << n) - T + those bits;
-     encoder, in state x in [T, 2T) with symbol s: n such that x >> n lies in
-                          [f, 2f), the low n bits of x are written, next state
-                          = T + the (x >> n) - f -th state of s. */
-typedef struct {
-  uint8_t sym[NZO_M];   /* decoder: symbol of state X */
-  uint8_t nbits[NZO_M]; /*          bits it reads */
-  uint16_t base[NZO_M]; /*          next state before the bits are added */
-  uint16_t enc[NZO_M];  /* encoder: enc[cum[s] + k] = k-th state of s */
-  uint32_t dnb[256];    /*          n = (x + dnb[s]) >> 16 */
-  int32_t start[256];   /*          next state = T + enc[(x >> n) + start[s]] */
-} tans_t;
-
-static uint32_t floor_log2(uint32_t v) {
-  uint32_t r = 0;
-  while (v >>= 1) ++r;
-  return r;
+static void put16(uint8_t* p, uint32_t v) {
+  p[0] = (uint8_t)v;
+  p[1] = (uint8_t)(v >> 8);
 }
-
-static void build_tans(const uint16_t freq[256], tans_t* t) {
-  uint8_t slot_sym[NZO_M];
-  uint32_t cum[257], next[256];
-  uint32_t acc = 0;
-  for (int s = 0; s < 256; ++s) {
-    cum[s] = acc;
-    for (uint32_t i = 0; i < freq[s]; ++i) slot_sym[acc + i] = (uint8_t)s;
-    acc += freq[s];
-    next[s] = 0;
-  }
-  for (uint32_t X = 0; X < NZO_M; ++X) {
-    uint32_t slot = (X & 63u) * 64u + (X >> 6);
-    uint32_t s = slot_sym[slot];
-    uint32_t k = next[s]++;
-    uint32_t xs = freq[s] + k;
-    uint32_t n = NZO_PROB_BITS - floor_log2(xs);
-    t->sym[X] = (uint8_t)s;
-    t->nbits[X] = (uint8_t)n;
-    t->base[X] = (uint16_t)((xs << n) - NZO_M);
-    t->enc[cum[s] + k] = (uint16_t)X;
-  }
-  for (int s = 0; s < 256; ++s) {
-    uint32_t f = freq[s];
-    if (!f) {
-      t->dnb[s] = 0;
-      t->start[s] = 0;
-      continue;
-    }
-    uint32_t n0 = NZO_PROB_BITS - floor_log2(f);
-    t->dnb[s] = (n0 << 16) - (f << n0);
-    t->start[s] = (int32_t)cum[s] - (int32_t)f;
-  }
-}
+static uint32_t get16(const uint8_t* p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8); }
 
 /* ------------------------------------------------------------------------- */
 /* segment encode / decode: 64 lanes, lane l owns symbols (g*64+l)*8 + j     */
 /* ------------------------------------------------------------------------- */
 
-/* Body of a coded segment record (after the chunk's table, if any):
-     states   64 x 24 bits, lane l at bytes 3l .. 3l+2 (little endian): state A
-              in the low 12 bits, state B in the high 12 - the decoder's start
-              states.  A codes the lane's symbols with even j, B those with odd j.
-     lengths  u32 = minlen | w << 24, then 64 fields of w bits (field l at bit
-              l * w, little endian): len_l - minlen, the bits of lane l's stream
-     streams  the 64 lane streams back to back, bit-granular, little endian,
-              zero padded to 4 bytes.
-   A lane's stream is read from its END downwards: the n bits of a symbol lie
-   right under the position the reader has reached, so the encoder, which runs
-   over the symbols backwards, simply appends.  The encoder starts both states
-   of a lane from T | 12 payload bits (24 bits per lane: bytes 3l .. 3l+2 of the
-   segment's NZO_CARRY_BYTES carried bytes); the decoder ends on them. */
-#define LANE_BITS_MAX(lane_syms) ((size_t)(lane_syms) * NZO_PROB_BITS)
-
-typedef struct {
-  uint32_t* w; /* bits, little endian dwords */
-  uint32_t len;
-} bits_t;
-
-/* append the low n (<= 32) bits of v; the store has a spare dword */
-static void bits_append(bits_t* b, uint32_t v, uint32_t n) {
-  if (!n) return;
-  uint32_t sh = b->len & 31;
-  uint64_t wide = (uint64_t)(n < 32 ? v & ((1u << n) - 1u) : v) << sh;
-  b->w[b->len >> 5] |= (uint32_t)wide;
-  b->w[(b->len >> 5) + 1] |= (uint32_t)(wide >> 32);
-  b->len += n;
-}
-/* n (<= 24) bits at bit offset `bit` of a little-endian byte string; touches
-   only the bytes that hold them */
-static uint32_t bits_get(const uint8_t* p, uint64_t bit, uint32_t n) {
-  if (!n) return 0;
-  const uint8_t* q = p + (bit >> 3);
-  uint32_t sh = (uint32_t)(bit & 7), nb = (sh + n + 7) / 8;
-  uint32_t v = 0;
-  for (uint32_t i = 0; i < nb; ++i) v |= (uint32_t)q[i] << (8 * i);
-  return (v >> sh) & ((1u << n) - 1u);
-}
-/* OR n (<= 32) bits into a zeroed little-endian byte string */
-static void bits_put(uint8_t* p, uint64_t bit, uint32_t v, uint32_t n) {
-  if (!n) return;
-  uint8_t* q = p + (bit >> 3);
-  uint32_t sh = (uint32_t)(bit & 7), nb = (sh + n + 7) / 8;
-  uint64_t wide = (uint64_t)(n < 32 ? v & ((1u << n) - 1u) : v) << sh;
-  for (uint32_t i = 0; i < nb; ++i) q[i] |= (uint8_t)(wide >> (8 * i));
-}
-
-/* -> bytes of the body written to out (a multiple of 4) */
-static size_t encode_segment(const uint8_t* syms, uint32_t seg_n, uint32_t lane_syms, int pad_sym,
-                             const tans_t* t, const uint8_t* seeds, uint8_t* out) {
-  uint32_t ngroups = (seg_n + NZO_GROUP_SYMS - 1) / NZO_GROUP_SYMS;
-  size_t lane_words = (LANE_BITS_MAX(lane_syms) + 31) / 32 + 1;
-  uint32_t* store = (uint32_t*)calloc(NZO_LANES * lane_words, 4);
-  bits_t lane[NZO_LANES];
-  uint32_t xa[NZO_LANES], xb[NZO_LANES];
+/* Final encoder states, variable length: 64 two-bit length codes (lane l at
+   bits 2l, 2l+1 of a 16-byte little-endian block; code c means the state is
+   stored in 5 + c nibbles), then the states as a little-endian nibble stream in
+   lane order, zero padded to a multiple of 4 bytes.  A state is >= 2^16, so it
+   needs 20..32 bits; storing only the nibbles in use saves about 4 bits per
+   lane over a flat 32. */
+static size_t pack_states(const uint32_t x[NZO_LANES], uint8_t* out) {
+  uint8_t nib[NZO_LANES * 8 + 8];
+  size_t t = 0;
+  memset(out, 0, 16);
   for (int l = 0; l < NZO_LANES; ++l) {
-    lane[l].w = store + (size_t)l * lane_words;
-    lane[l].len = 0;
-    uint32_t pay = seeds ? (uint32_t)seeds[3 * l] | ((uint32_t)seeds[3 * l + 1] << 8) |
-                               ((uint32_t)seeds[3 * l + 2] << 16)
-                         : 0u;
-    xa[l] = NZO_M | (pay & 0xFFFu);
-    xb[l] = NZO_M | (pay >> 12);
+    uint32_t c = 0;
+    while (c < 3 && (x[l] >> (4 * (5 + c))) != 0) ++c;
+    out[(2 * l) >> 3] |= (uint8_t)(c << ((2 * l) & 7));
+    for (uint32_t k = 0; k < 5 + c; ++k) nib[t++] = (x[l] >> (4 * k)) & 0xF;
   }
+  size_t bytes = ((t + 1) / 2 + 3) & ~(size_t)3;
+  memset(out + 16, 0, bytes);
+  for (size_t k = 0; k < t; ++k) out[16 + (k >> 1)] |= (uint8_t)(nib[k] << (4 * (k & 1)));
+  return 16 + bytes;
+}
+
+static int unpack_states(const uint8_t* rec, size_t avail, uint32_t x[NZO_LANES], size_t* used) {
+  if (avail < 16) return NZO_ERR_CORRUPT;
+  size_t t = 0;
+  uint32_t n[NZO_LANES];
+  for (int l = 0; l < NZO_LANES; ++l) {
+    n[l] = 5 + ((rec[(2 * l) >> 3] >> ((2 * l) & 7)) & 3);
+    t += n[l];
+  }
+  size_t bytes = ((t + 1) / 2 + 3) & ~(size_t)3;
+  if (avail < 16 + bytes) return NZO_ERR_CORRUPT;
+  size_t k = 0;
+  for (int l = 0; l < NZO_LANES; ++l) {
+    uint32_t v = 0;
+    for (uint32_t q = 0; q < n[l]; ++q, ++k)
+      v |= (uint32_t)((rec[16 + (k >> 1)] >> (4 * (k & 1))) & 0xF) << (4 * q);
+    x[l] = v;
+  }
+  *used = 16 + bytes;
+  return NZO_OK;
+}
+
+/* Encode one segment.  Words are produced back to front into words[cap_words]
+   so that the decoder reads them front to back.  Returns the number of words,
+   or -1 when more than cap_words would be needed (segment stored RAW). */
+static int64_t encode_segment(const uint8_t* syms, uint32_t seg_n, int pad_sym,
+                              const uint16_t* freq, const uint16_t* cum, const uint16_t* seeds,
+                              uint16_t* words, uint32_t cap_words, uint32_t states[NZO_LANES]) {
+  uint32_t x[NZO_LANES];
+  /* the encoder's start state carries 16 payload bits per lane (see header) */
+  for (int l = 0; l < NZO_LANES; ++l) x[l] = NZO_L | (seeds ? seeds[l] : 0u);
+  uint32_t ngroups = (seg_n + NZO_GROUP_SYMS - 1) / NZO_GROUP_SYMS;
+  uint32_t pos = cap_words;
   for (uint32_t g = ngroups; g-- > 0;) {
     for (int j = NZO_GROUP - 1; j >= 0; --j) {
+      uint8_t sym[NZO_LANES];
+      uint8_t need[NZO_LANES];
+      uint32_t cnt = 0;
       for (int l = 0; l < NZO_LANES; ++l) {
         uint32_t idx = (g * NZO_LANES + (uint32_t)l) * NZO_GROUP + (uint32_t)j;
-        uint32_t s = idx < seg_n ? syms[idx] : (uint32_t)pad_sym;
-        uint32_t* x = (j & 1) ? &xb[l] : &xa[l];
-        uint32_t n = (*x + t->dnb[s]) >> 16;
-        bits_append(&lane[l], *x & ((1u << n) - 1u), n);
-        *x = NZO_M + t->enc[(int32_t)(*x >> n) + t->start[s]];
+        sym[l] = idx < seg_n ? syms[idx] : (uint8_t)pad_sym;
+        need[l] = x[l] >= ((uint32_t)freq[sym[l]] << 20);
+        cnt += need[l];
+      }
+      if (cnt > pos) return -1;
+      pos -= cnt;
+      uint32_t p = 0;
+      for (int l = 0; l < NZO_LANES; ++l) {
+        if (need[l]) {
+          words[pos + p++] = (uint16_t)(x[l] & 0xFFFF);
+          x[l] >>= 16;
+        }
+        uint32_t f = freq[sym[l]];
+        x[l] = ((x[l] / f) << NZO_PROB_BITS) + (x[l] % f) + cum[sym[l]];
       }
     }
   }
-  size_t off = 0;
-  for (int l = 0; l < NZO_LANES; ++l) {
-    uint32_t v = (xa[l] - NZO_M) | ((xb[l] - NZO_M) << 12);
-    out[off++] = (uint8_t)v;
-    out[off++] = (uint8_t)(v >> 8);
-    out[off++] = (uint8_t)(v >> 16);
-  }
-  uint32_t minlen = lane[0].len, maxlen = lane[0].len;
-  uint64_t total = 0;
-  for (int l = 0; l < NZO_LANES; ++l) {
-    if (lane[l].len < minlen) minlen = lane[l].len;
-    if (lane[l].len > maxlen) maxlen = lane[l].len;
-    total += lane[l].len;
-  }
-  uint32_t w = 0;
-  while ((maxlen - minlen) >> w) ++w;
-  put32(out + off, minlen | (w << 24));
-  off += 4;
-  memset(out + off, 0, 8 * (size_t)w);
-  for (int l = 0; l < NZO_LANES; ++l) bits_put(out + off, (uint64_t)l * w, lane[l].len - minlen, w);
-  off += 8 * (size_t)w;
-  size_t sbytes = (size_t)(((total + 7) / 8 + 3) & ~(uint64_t)3);
-  memset(out + off, 0, sbytes);
-  uint64_t at = 0;
-  for (int l = 0; l < NZO_LANES; ++l) {
-    for (uint32_t i = 0; i < lane[l].len; i += 32) {
-      uint32_t n = lane[l].len - i < 32 ? lane[l].len - i : 32;
-      bits_put(out + off, at + i, lane[l].w[i >> 5], n);
-    }
-    at += lane[l].len;
-  }
-  off += sbytes;
-  free(store);
-  return off;
+  for (int l = 0; l < NZO_LANES; ++l) states[l] = x[l];
+  /* move to the front of the buffer */
+  uint32_t count = cap_words - pos;
+  memmove(words, words + pos, (size_t)count * 2);
+  return count;
 }
 
-static int decode_segment(const uint8_t* rec, size_t rec_bytes, uint32_t seg_n, const tans_t* t,
-                          uint8_t* out, uint8_t* seeds) {
-  if (rec_bytes < 3 * NZO_LANES + 4) return NZO_ERR_CORRUPT;
-  uint32_t xa[NZO_LANES], xb[NZO_LANES];
-  for (int l = 0; l < NZO_LANES; ++l) {
-    uint32_t v = (uint32_t)rec[3 * l] | ((uint32_t)rec[3 * l + 1] << 8) | ((uint32_t)rec[3 * l + 2] << 16);
-    xa[l] = v & 0xFFFu;
-    xb[l] = v >> 12;
-  }
-  size_t off = 3 * NZO_LANES;
-  uint32_t hdr = get32(rec + off);
-  off += 4;
-  uint32_t minlen = hdr & 0xFFFFFFu, w = hdr >> 24;
-  if (w > 24 || rec_bytes < off + 8 * (size_t)w) return NZO_ERR_CORRUPT;
-  uint64_t start[NZO_LANES + 1];
-  start[0] = 0;
+static int decode_segment(const uint8_t* rec, size_t rec_bytes, uint32_t seg_n,
+                          const uint32_t* lut, uint8_t* out, uint16_t* seeds) {
+  uint32_t x[NZO_LANES];
+  size_t sbytes;
+  if (unpack_states(rec, rec_bytes, x, &sbytes)) return NZO_ERR_CORRUPT;
   for (int l = 0; l < NZO_LANES; ++l)
-    start[l + 1] = start[l] + minlen + bits_get(rec + off, (uint64_t)l * w, w);
-  off += 8 * (size_t)w;
-  if ((rec_bytes - off) * 8 < start[NZO_LANES]) return NZO_ERR_CORRUPT;
-  const uint8_t* bits = rec + off;
-  uint64_t q[NZO_LANES];
-  for (int l = 0; l < NZO_LANES; ++l) q[l] = start[l + 1];
+    if (x[l] < NZO_L) return NZO_ERR_CORRUPT;
+  const uint8_t* w = rec + sbytes;
+  size_t nwords = (rec_bytes - sbytes) / 2, base = 0;
   uint32_t ngroups = (seg_n + NZO_GROUP_SYMS - 1) / NZO_GROUP_SYMS;
   for (uint32_t g = 0; g < ngroups; ++g) {
     for (int j = 0; j < NZO_GROUP; ++j) {
       for (int l = 0; l < NZO_LANES; ++l) {
-        uint32_t* x = (j & 1) ? &xb[l] : &xa[l];
-        uint32_t n = t->nbits[*x];
+        uint32_t e = lut[x[l] & (NZO_M - 1)];
+        x[l] = (e >> 20) * (x[l] >> NZO_PROB_BITS) + ((e >> 8) & 0xFFF);
         uint32_t idx = (g * NZO_LANES + (uint32_t)l) * NZO_GROUP + (uint32_t)j;
-        if (idx < seg_n) out[idx] = t->sym[*x];
-        if (q[l] < start[l] + n) return NZO_ERR_CORRUPT;
-        q[l] -= n;
-        *x = t->base[*x] + bits_get(bits, q[l], n);
+        if (idx < seg_n) out[idx] = (uint8_t)(e & 0xFF);
+        if (x[l] < NZO_L) {
+          uint32_t word = base < nwords ? get16(w + 2 * base) : 0;
+          ++base;
+          x[l] = (x[l] << 16) | word;
+        }
       }
     }
   }
+  if (base > nwords) return NZO_ERR_CORRUPT;
   for (int l = 0; l < NZO_LANES; ++l) {
-    /* every bit of the lane's stream read, and the states back at the encoder's
-       start states: T | payload (payload 0 when nothing is carried) */
-    if (q[l] != start[l]) return NZO_ERR_CORRUPT;
-    uint32_t v = xa[l] | (xb[l] << 12);
-    if (seeds) {
-      seeds[3 * l] = (uint8_t)v;
-      seeds[3 * l + 1] = (uint8_t)(v >> 8);
-      seeds[3 * l + 2] = (uint8_t)(v >> 16);
-    } else if (v != 0) {
-      return NZO_ERR_CORRUPT;
-    }
+    /* back at the encoder's start state: 2^16 | payload (payload 0 when nothing is carried) */
+    if ((x[l] >> 16) != 1u) return NZO_ERR_CORRUPT;
+    if (seeds) seeds[l] = (uint16_t)(x[l] & 0xFFFFu);
+    else if (x[l] != NZO_L) return NZO_ERR_CORRUPT;
   }
   return NZO_OK;
 }
@@ -639,13 +533,13 @@ static int decode_segment(const uint8_t* rec, size_t rec_bytes, uint32_t seg_n, 
 typedef struct {
   const geom_t* g;
   const uint8_t* syms;
-  const uint8_t* seeds; /* NZO_CARRY_BYTES per segment, or NULL */
-  uint8_t* scratch;     /* n_segs * seg_rec_cap */
-  uint32_t* seg_bytes;  /* n_segs */
-  uint64_t c0, c1;      /* chunk range */
+  const uint16_t* seeds; /* 64 per full segment, or NULL */
+  uint8_t* scratch;      /* n_segs * seg_rec_cap */
+  uint32_t* seg_bytes;   /* n_segs */
+  uint64_t c0, c1;       /* chunk range */
 } enc_job_t;
 
-static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint8_t* seeds, uint64_t c,
+static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint16_t* seeds, uint64_t c,
                          uint8_t* scratch, uint32_t* seg_bytes) {
   uint64_t base = c * g->chunk_syms;
   uint64_t cn64 = g->n - base < g->chunk_syms ? g->n - base : g->chunk_syms;
@@ -654,16 +548,20 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint8_t* se
   uint32_t cnt[256];
   memset(cnt, 0, sizeof cnt);
   for (uint32_t i = 0; i < cn; ++i) cnt[cs[i]]++;
-  uint16_t freq[256];
+  uint16_t freq[256], cum[256];
   int pad = nzo_normalize_freqs(cnt, cn, freq);
-  tans_t* t = (tans_t*)malloc(sizeof(tans_t));
-  build_tans(freq, t);
-  uint8_t table[424];
+  uint32_t acc = 0;
+  for (int i = 0; i < 256; ++i) {
+    cum[i] = (uint16_t)acc;
+    acc += freq[i];
+  }
+  uint8_t table[420];
   size_t tbytes = nzo_table_serialize(freq, table);
   uint32_t nseg = (cn + g->seg_syms - 1) / g->seg_syms;
   uint64_t seg0 = c * g->spc;
   size_t cap = seg_rec_cap(g);
-  size_t coded_total = tbytes, raw_total = 4;
+  size_t rans_total = tbytes, raw_total = 4;
+  int overflow = 0;
   for (uint32_t k = 0; k < nseg; ++k) {
     uint32_t sn = cn - k * g->seg_syms < g->seg_syms ? cn - k * g->seg_syms : g->seg_syms;
     uint8_t* rec = scratch + (seg0 + k) * cap;
@@ -672,15 +570,30 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint8_t* se
       memcpy(rec, table, tbytes);
       off = tbytes;
     }
+    uint32_t states[NZO_LANES];
+    uint16_t* words = (uint16_t*)malloc(2 * (size_t)g->seg_syms + 8);
     /* only full segments carry payload in their start states */
-    const uint8_t* sd = (seeds && sn == seg_nominal(g, k)) ? seeds + (seg0 + k) * NZO_CARRY_BYTES : NULL;
-    off += encode_segment(cs + (size_t)k * g->seg_syms, sn, g->lane_syms, pad, t, sd, rec + off);
+    const uint16_t* sd = (seeds && sn == seg_nominal(g, k)) ? seeds + (seg0 + k) * NZO_LANES : NULL;
+    /* one word per symbol is the most a segment can emit: no overflow */
+    int64_t nw = encode_segment(cs + (size_t)k * g->seg_syms, sn, pad, freq, cum, sd, words,
+                                g->seg_syms, states);
+    if (nw < 0) {
+      overflow = 1;
+      nw = 0;
+    }
+    off += pack_states(states, rec + off);
+    for (int64_t i = 0; i < nw; ++i) put16(rec + off + 2 * i, words[i]);
+    off += 2 * (size_t)nw;
+    if (nw & 1) {
+      put16(rec + off, 0);
+      off += 2;
+    }
+    free(words);
     seg_bytes[seg0 + k] = (uint32_t)off;
-    coded_total += off - (k == 0 ? tbytes : 0);
-    raw_total += (((size_t)sn + 3) & ~(size_t)3) + (sn == seg_nominal(g, k) ? NZO_CARRY_BYTES : 0);
+    rans_total += off - (k == 0 ? tbytes : 0);
+    raw_total += (((size_t)sn + 3) & ~(size_t)3) + (sn == seg_nominal(g, k) ? 2 * NZO_LANES : 0);
   }
-  free(t);
-  if (coded_total >= raw_total) {
+  if (overflow || rans_total >= raw_total) {
     for (uint32_t k = 0; k < nseg; ++k) {
       uint32_t sn = cn - k * g->seg_syms < g->seg_syms ? cn - k * g->seg_syms : g->seg_syms;
       uint8_t* rec = scratch + (seg0 + k) * cap;
@@ -694,10 +607,10 @@ static void encode_chunk(const geom_t* g, const uint8_t* syms, const uint8_t* se
       size_t padded = ((size_t)sn + 3) & ~(size_t)3;
       memset(rec + off + sn, 0, padded - sn);
       off += padded;
-      if (sn == seg_nominal(g, k)) { /* a raw full segment still has to hold its carried bytes */
-        if (seeds) memcpy(rec + off, seeds + (seg0 + k) * NZO_CARRY_BYTES, NZO_CARRY_BYTES);
-        else memset(rec + off, 0, NZO_CARRY_BYTES);
-        off += NZO_CARRY_BYTES;
+      if (sn == seg_nominal(g, k)) { /* a raw full segment still has to hold its 64 x 16 carried bits */
+        for (int l = 0; l < NZO_LANES; ++l)
+          put16(rec + off + 2 * l, seeds ? seeds[(seg0 + k) * NZO_LANES + l] : 0u);
+        off += 2 * NZO_LANES;
       }
       seg_bytes[seg0 + k] = (uint32_t)off;
     }
@@ -728,7 +641,7 @@ static void write_header(uint8_t* out, const geom_t* g, uint64_t total) {
 }
 
 int64_t nzo_exp_encode(const uint8_t* syms, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
-                       const uint8_t* seeds, uint8_t* out, size_t cap, int threads) {
+                       const uint16_t* seeds, uint8_t* out, size_t cap, int threads) {
   geom_t g;
   if (make_geom(&g, n, chunk_syms, lane_syms)) return NZO_ERR_ARG;
   if (cap < g.rec_off) return NZO_ERR_CAP;
@@ -798,41 +711,43 @@ done:
   return ret;
 }
 
+static void build_lut(const uint16_t freq[256], uint32_t* lut) {
+  uint32_t c = 0;
+  for (int s = 0; s < 256; ++s) {
+    uint32_t f = freq[s];
+    for (uint32_t i = 0; i < f; ++i) lut[c + i] = (f << 20) | (i << 8) | (uint32_t)s;
+    c += f;
+  }
+}
+
 typedef struct {
   const geom_t* g;
   const uint8_t* comp;
   size_t comp_bytes;
   uint8_t* out;
-  uint8_t* seeds; /* NZO_CARRY_BYTES per segment, or NULL */
+  uint16_t* seeds; /* 64 per full segment, or NULL */
   uint64_t c0, c1;
   int status;
 } dec_job_t;
 
 static int decode_chunk(const geom_t* g, const uint8_t* comp, size_t comp_bytes, uint64_t c,
-                        uint8_t* out, uint8_t* seeds) {
+                        uint8_t* out, uint16_t* seeds) {
   uint64_t base = c * g->chunk_syms;
   uint32_t cn = (uint32_t)(g->n - base < g->chunk_syms ? g->n - base : g->chunk_syms);
   uint32_t nseg = (cn + g->seg_syms - 1) / g->seg_syms;
   uint64_t seg0 = c * g->spc;
   const uint8_t* dir = comp + g->dir_off;
-  tans_t* t = (tans_t*)malloc(sizeof(tans_t));
-  int rc = NZO_OK;
+  uint32_t lut[NZO_M];
   int raw = 0;
-  for (uint32_t k = 0; k < nseg && rc == NZO_OK; ++k) {
+  for (uint32_t k = 0; k < nseg; ++k) {
     uint64_t o0 = get32(dir + 4 * (seg0 + k)), o1 = get32(dir + 4 * (seg0 + k + 1));
-    if (o1 < o0 || g->rec_off + 4 * o1 > comp_bytes) {
-      rc = NZO_ERR_CORRUPT;
-      break;
-    }
+    if (o1 < o0 || g->rec_off + 4 * o1 > comp_bytes) return NZO_ERR_CORRUPT;
     const uint8_t* rec = comp + g->rec_off + 4 * o0;
     size_t rbytes = 4 * (size_t)(o1 - o0);
     uint32_t sn = cn - k * g->seg_syms < g->seg_syms ? cn - k * g->seg_syms : g->seg_syms;
     uint8_t* dst = out + base + (size_t)k * g->seg_syms;
     if (k == 0) {
-      if (rbytes < 4) {
-        rc = NZO_ERR_CORRUPT;
-        break;
-      }
+      if (rbytes < 4) return NZO_ERR_CORRUPT;
       if (rec[0] == NZO_MODE_RAW) {
         raw = 1;
         rec += 4;
@@ -840,31 +755,26 @@ static int decode_chunk(const geom_t* g, const uint8_t* comp, size_t comp_bytes,
       } else {
         uint16_t freq[256];
         size_t used;
-        if (nzo_table_parse(rec, rbytes, freq, &used)) {
-          rc = NZO_ERR_CORRUPT;
-          break;
-        }
-        build_tans(freq, t);
+        if (nzo_table_parse(rec, rbytes, freq, &used)) return NZO_ERR_CORRUPT;
+        build_lut(freq, lut);
         rec += used;
         rbytes -= used;
       }
     }
-    uint8_t tmp[NZO_CARRY_BYTES];
-    uint8_t* sd = sn == seg_nominal(g, k) ? (seeds ? seeds + (seg0 + k) * NZO_CARRY_BYTES : tmp) : NULL;
+    uint16_t tmp[NZO_LANES];
+    uint16_t* sd = sn == seg_nominal(g, k) ? (seeds ? seeds + (seg0 + k) * NZO_LANES : tmp) : NULL;
     if (raw) {
       size_t padded = ((size_t)sn + 3) & ~(size_t)3;
-      if (rbytes < padded + (sd ? NZO_CARRY_BYTES : 0)) {
-        rc = NZO_ERR_CORRUPT;
-        break;
-      }
+      if (rbytes < padded + (sd ? 2 * NZO_LANES : 0)) return NZO_ERR_CORRUPT;
       memcpy(dst, rec, sn);
-      if (sd) memcpy(sd, rec + padded, NZO_CARRY_BYTES);
+      if (sd)
+        for (int l = 0; l < NZO_LANES; ++l) sd[l] = (uint16_t)get16(rec + padded + 2 * l);
     } else {
-      rc = decode_segment(rec, rbytes, sn, t, dst, sd);
+      int r = decode_segment(rec, rbytes, sn, lut, dst, sd);
+      if (r) return r;
     }
   }
-  free(t);
-  return rc;
+  return NZO_OK;
 }
 
 static void* dec_worker(void* arg) {
@@ -881,7 +791,7 @@ static void* dec_worker(void* arg) {
 }
 
 int nzo_exp_decode(const uint8_t* comp, size_t comp_bytes, uint64_t n, uint8_t* syms_out,
-                   uint8_t* seeds_out, int threads) {
+                   uint16_t* seeds_out, int threads) {
   if (comp_bytes < NZO_HEADER_BYTES) return NZO_ERR_CORRUPT;
   if (get32(comp) != NZO_MAGIC || get32(comp + 4) != NZO_VERSION) return NZO_ERR_CORRUPT;
   uint64_t hn = (uint64_t)get32(comp + 8) | ((uint64_t)get32(comp + 12) << 32);
@@ -977,10 +887,10 @@ static void run_sm(void* (*fn)(void*), const uint16_t* data, uint16_t* out, uint
 }
 
 /* Stored layout of the packed sign|mantissa stream: the reference layout
-   (byte idx*(s+1)/8, MSB first) with the last NZO_CARRY_BYTES bytes of every
-   FULL segment taken out; those 64 x 24 bits ride in the start states of the
-   segment's 64 lanes (lane l carries bytes 3l .. 3l+2).  A segment is full when
-   the tensor does not end inside it. */
+   (byte idx*(s+1)/8, MSB first) with the last 128 bytes of every FULL segment
+   taken out; those 64 x 16 bits ride in the start states of the segment's 64
+   rANS lanes (lane l carries bytes 2l and 2l+1, little endian).  A segment is
+   full when the tensor does not end inside it. */
 static uint64_t full_segments(const geom_t* g) {
   uint64_t rem = g->n % g->chunk_syms, fs = rem / g->seg_syms;
   if (fs > g->spc - 1) fs = g->spc - 1;
@@ -990,12 +900,12 @@ static uint64_t full_segments(const geom_t* g) {
 size_t nzo_packed_stored_bytes(uint64_t n, int s, uint32_t chunk_syms, uint32_t lane_syms) {
   geom_t g;
   if (make_geom(&g, n, chunk_syms, lane_syms)) return 0;
-  return nzo_packed_bytes(n, s) - NZO_CARRY_BYTES * (size_t)full_segments(&g);
+  return nzo_packed_bytes(n, s) - 2 * NZO_LANES * (size_t)full_segments(&g);
 }
 
 /* move the packed bytes between the reference layout (`full`) and the stored
    layout + per-segment carried bytes */
-static void carry_layout(const geom_t* g, int s, uint8_t* full, uint8_t* stored, uint8_t* seeds,
+static void carry_layout(const geom_t* g, int s, uint8_t* full, uint8_t* stored, uint16_t* seeds,
                          int to_stored) {
   size_t total = nzo_packed_bytes(g->n, s), src = 0, dst = 0;
   for (uint64_t c = 0; c < g->n_chunks; ++c) {
@@ -1006,13 +916,15 @@ static void carry_layout(const geom_t* g, int s, uint8_t* full, uint8_t* stored,
       uint32_t sn = cn - k * g->seg_syms < g->seg_syms ? cn - k * g->seg_syms : g->seg_syms;
       int is_full = sn == seg_nominal(g, k);
       size_t bytes = is_full ? (size_t)sn * (size_t)(s + 1) / 8 : total - src;
-      size_t keep = is_full ? bytes - NZO_CARRY_BYTES : bytes;
+      size_t keep = is_full ? bytes - 2 * NZO_LANES : bytes;
       if (to_stored) memcpy(stored + dst, full + src, keep);
       else memcpy(full + src, stored + dst, keep);
       if (is_full) {
-        uint8_t* sd = seeds + (c * g->spc + k) * NZO_CARRY_BYTES;
-        if (to_stored) memcpy(sd, full + src + keep, NZO_CARRY_BYTES);
-        else memcpy(full + src + keep, sd, NZO_CARRY_BYTES);
+        uint16_t* sd = seeds + (c * g->spc + k) * NZO_LANES;
+        for (int l = 0; l < NZO_LANES; ++l) {
+          if (to_stored) sd[l] = (uint16_t)get16(full + src + keep + 2 * l);
+          else put16(full + src + keep + 2 * l, sd[l]);
+        }
       }
       src += bytes;
       dst += keep;
@@ -1028,7 +940,7 @@ int64_t nzo_compress_bf16(const uint16_t* data, uint64_t n, int s, uint32_t chun
   if (make_geom(&g, n, chunk_syms, lane_syms)) return NZO_ERR_ARG;
   uint8_t* exps = (uint8_t*)malloc((size_t)n + 1);
   uint8_t* full = (uint8_t*)malloc(nzo_packed_bytes(n, s) + 1);
-  uint8_t* seeds = (uint8_t*)calloc((size_t)(g.n_segs + 1), NZO_CARRY_BYTES);
+  uint16_t* seeds = (uint16_t*)calloc((size_t)(g.n_segs + 1) * NZO_LANES, 2);
   if (!exps || !full || !seeds) {
     free(exps);
     free(full);
@@ -1052,7 +964,7 @@ int nzo_decompress_bf16(const uint8_t* comp, size_t comp_bytes, const uint8_t* f
   if (make_geom(&g, n, get32(comp + 16), get32(comp + 20))) return NZO_ERR_CORRUPT;
   uint8_t* exps = (uint8_t*)malloc((size_t)n + 1);
   uint8_t* full = (uint8_t*)malloc(nzo_packed_bytes(n, s) + 1);
-  uint8_t* seeds = (uint8_t*)calloc((size_t)(g.n_segs + 1), NZO_CARRY_BYTES);
+  uint16_t* seeds = (uint16_t*)calloc((size_t)(g.n_segs + 1) * NZO_LANES, 2);
   if (!exps || !full || !seeds) {
     free(exps);
     free(full);

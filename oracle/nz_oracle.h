@@ -24,13 +24,13 @@
  *     the invariants in the tests; NaN inputs and the reference's behaviour for
  *     group sizes other than 1024 are PARITY UNPINNED (see the source).
  *
- *  2. nzo_exp_* is the chunked, 64-lane table-ANS container that replaces the
- *     closed-source nvcomp ANS call sites
+ *  2. nzo_exp_* is the chunked, 64-way lane-interleaved rANS container that
+ *     replaces the closed-source nvcomp ANS call sites
  *        cuda/high_level.cu:103-124 (compress) and :184-192 (decompress).
  *     The nvcomp bitstream is opaque, so the byte format here is this
  *     project's own; PARITY UNPINNED for the compressed bytes and exact
  *     compressed size.  What is pinned: lossless identity on arbitrary
- *     bytes, the Shannon bound on the size, and textbook table-ANS state
+ *     bytes, the Shannon bound on the size, and textbook rANS state
  *     invariants (checked in the tests).
  */
 #ifndef NZ_ORACLE_H
@@ -45,9 +45,10 @@ extern "C" {
 
 /* ---- format constants (shared with the HIP implementation by value) ---- */
 #define NZO_MAGIC 0x315A4E41u /* "ANZ1" little endian */
-#define NZO_VERSION 5u
+#define NZO_VERSION 4u
 #define NZO_PROB_BITS 12
 #define NZO_M (1u << NZO_PROB_BITS)
+#define NZO_L (1u << 16)
 #define NZO_LANES 64
 #define NZO_GROUP 8                        /* consecutive symbols per lane per group */
 #define NZO_GROUP_SYMS (NZO_LANES * NZO_GROUP) /* 512 */
@@ -56,8 +57,6 @@ extern "C" {
 #define NZO_MODE_BITMAP 0x00
 #define NZO_MAX_RUNS 15
 #define NZO_TAIL_PAD 16
-#define NZO_CARRY_BYTES 192  /* 64 lanes x 2 states x 12 bits */
-#define NZO_MAX_LANE_SYMS 512
 
 /* ---- split / merge ---- */
 size_t nzo_packed_bytes(uint64_t n, int s);
@@ -83,13 +82,13 @@ int nzo_table_parse(const uint8_t* in, size_t avail, uint16_t freq[256], size_t*
 /* ---- exponent container ---- */
 int nzo_check_geometry(uint32_t chunk_syms, uint32_t lane_syms);
 size_t nzo_exp_bound(uint64_t n, uint32_t chunk_syms, uint32_t lane_syms);
-/* seeds: NZO_CARRY_BYTES per segment (segment c*spc + k at seeds + 192*(c*spc + k);
-   only full segments use theirs), the payload carried in the coder's start
-   states; NULL = all zero / ignored. */
+/* seeds: 64 x u16 per segment (segment c*spc + k at seeds + 64*(c*spc + k); only
+   full segments use theirs), the payload carried in the rANS start states;
+   NULL = all zero / ignored. */
 int64_t nzo_exp_encode(const uint8_t* syms, uint64_t n, uint32_t chunk_syms, uint32_t lane_syms,
-                       const uint8_t* seeds, uint8_t* out, size_t cap, int threads);
+                       const uint16_t* seeds, uint8_t* out, size_t cap, int threads);
 int nzo_exp_decode(const uint8_t* comp, size_t comp_bytes, uint64_t n, uint8_t* syms_out,
-                   uint8_t* seeds_out, int threads);
+                   uint16_t* seeds_out, int threads);
 
 /* ---- whole tensor (split + encode / decode + merge) ---- */
 int64_t nzo_compress_bf16(const uint16_t* data, uint64_t n, int s, uint32_t chunk_syms,

@@ -65,10 +65,10 @@ def lib() -> ctypes.CDLL:
         L.nzo_exp_bound.restype = ctypes.c_size_t
         L.nzo_exp_bound.argtypes = [ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32]
         L.nzo_exp_encode.restype = ctypes.c_int64
-        L.nzo_exp_encode.argtypes = [u8p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32, u8p, u8p,
+        L.nzo_exp_encode.argtypes = [u8p, ctypes.c_uint64, ctypes.c_uint32, ctypes.c_uint32, u16p, u8p,
                                      ctypes.c_size_t, ctypes.c_int]
         L.nzo_exp_decode.restype = ctypes.c_int
-        L.nzo_exp_decode.argtypes = [u8p, ctypes.c_size_t, ctypes.c_uint64, u8p, u8p, ctypes.c_int]
+        L.nzo_exp_decode.argtypes = [u8p, ctypes.c_size_t, ctypes.c_uint64, u8p, u16p, ctypes.c_int]
         L.nzo_packed_stored_bytes.restype = ctypes.c_size_t
         L.nzo_packed_stored_bytes.argtypes = [ctypes.c_uint64, ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32]
         L.nzo_compress_bf16.restype = ctypes.c_int64
@@ -201,12 +201,9 @@ def segment_count(n: int, chunk_syms: int, lane_syms: int) -> int:
     return (n // chunk_syms) * spc + -(-(n % chunk_syms) // seg)
 
 
-CARRY_BYTES = 192  # per full segment: 64 lanes x 2 coder states x 12 bits
-
-
 def exp_encode(syms: np.ndarray, chunk_syms: int = 65536, lane_syms: int = 512, threads: int = 1,
                seeds: np.ndarray | None = None) -> np.ndarray:
-    """Entropy-code a byte stream; `seeds` (uint8, CARRY_BYTES per segment) is the
+    """Entropy-code a byte stream; `seeds` (uint16, 64 per full segment) is the
     payload carried in the coder's start states."""
     syms = _u8(syms)
     cap = exp_bound(syms.size, chunk_syms, lane_syms)
@@ -215,9 +212,9 @@ def exp_encode(syms: np.ndarray, chunk_syms: int = 65536, lane_syms: int = 512, 
     out = np.zeros(cap, np.uint8)
     sp = None
     if seeds is not None:
-        seeds = np.ascontiguousarray(seeds, dtype=np.uint8).reshape(-1)
-        assert seeds.size >= CARRY_BYTES * segment_count(syms.size, chunk_syms, lane_syms)
-        sp = _p(seeds, ctypes.c_uint8)
+        seeds = np.ascontiguousarray(seeds, dtype=np.uint16).reshape(-1)
+        assert seeds.size >= 64 * segment_count(syms.size, chunk_syms, lane_syms)
+        sp = _p(seeds, ctypes.c_uint16)
     r = lib().nzo_exp_encode(_p(syms, ctypes.c_uint8), syms.size, chunk_syms, lane_syms, sp,
                              _p(out, ctypes.c_uint8), cap, threads)
     if r < 0:
@@ -228,17 +225,17 @@ def exp_encode(syms: np.ndarray, chunk_syms: int = 65536, lane_syms: int = 512, 
 def exp_decode(comp: np.ndarray, n: int, threads: int = 1, lane_syms: int | None = None,
                chunk_syms: int = 65536):
     """Returns (rc, symbols) or, with lane_syms given, (rc, symbols, seeds) where
-    seeds holds CARRY_BYTES bytes per segment (meaningful for full segments only)."""
+    seeds holds 64 values per segment (meaningful for full segments only)."""
     comp = _u8(comp)
     out = np.zeros(n, np.uint8)
     if lane_syms is None:
         rc = lib().nzo_exp_decode(_p(comp, ctypes.c_uint8), comp.size, n, _p(out, ctypes.c_uint8), None, threads)
         return int(rc), out
     nseg = segment_count(n, chunk_syms, lane_syms)
-    seeds = np.zeros(CARRY_BYTES * (nseg + 1), np.uint8)
+    seeds = np.zeros(64 * nseg + 64, np.uint16)
     rc = lib().nzo_exp_decode(_p(comp, ctypes.c_uint8), comp.size, n, _p(out, ctypes.c_uint8),
-                              _p(seeds, ctypes.c_uint8), threads)
-    return int(rc), out, seeds[: CARRY_BYTES * nseg]
+                              _p(seeds, ctypes.c_uint16), threads)
+    return int(rc), out, seeds[: 64 * nseg]
 
 
 def compress_bf16(bits: np.ndarray, s: int, chunk_syms: int = 65536, lane_syms: int = 512, threads: int = 1):

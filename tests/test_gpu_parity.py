@@ -21,7 +21,7 @@ def _to_dev(bits: np.ndarray):
     return torch.from_numpy(bits.view(np.int16).copy()).cuda()
 
 
-def gpu_encode(bits, s, chunk=262144, lane=512, norm_size=0):
+def gpu_encode(bits, s, chunk=131072, lane=256, norm_size=0):
     """-> (container, stored packed stream[, normalizer bytes when norm_size > 0]) as device tensors"""
     L, m = _lib()
     n = bits.size
@@ -45,7 +45,7 @@ def gpu_encode(bits, s, chunk=262144, lane=512, norm_size=0):
     return res + (norm[: L.nz_norm_bytes(n, norm_size)].clone(),) if norm_size else res
 
 
-def gpu_decode(comp, packed, n, s, chunk=262144, lane=512, check=True, norm_size=0, norm=None):
+def gpu_decode(comp, packed, n, s, chunk=131072, lane=256, check=True, norm_size=0, norm=None):
     L, m = _lib()
     if norm_size:
         norm = torch.cat([norm, torch.zeros(8, dtype=torch.uint8, device="cuda")])
@@ -71,7 +71,7 @@ def test_roundtrip_matches_oracle(oracle, n, s):
     print(f"case n={n} s={s}", flush=True)
     comp, packed = gpu_encode(bits, s)
     # container and packed stream are byte-identical to the oracle's
-    o_comp, o_packed = oracle.compress_bf16(bits, s, 262144, 512)
+    o_comp, o_packed = oracle.compress_bf16(bits, s, 131072, 256)
     assert np.array_equal(packed.cpu().numpy(), o_packed)
     assert np.array_equal(comp.cpu().numpy(), o_comp)
     rc, out = gpu_decode(comp, packed, n, s)
