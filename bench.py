@@ -633,7 +633,7 @@ def main():
     n = args.rows * args.cols
     chunk = args.chunk_size or lib_mod.DEFAULT_CHUNK
     lane = args.lane_symbols or (lib_mod.DEFAULT_LANE_SYMS if chunk == lib_mod.DEFAULT_CHUNK else
-                                 lib_mod.LANE_SYMS_64K if chunk == 65536 else max(16, chunk // 512))
+                                 344 if chunk == 65536 else max(16, chunk // 512))
     R = max(1, args.rotate)
     dense_bytes = 2 * n
     ws = Workspace(torch, L, lib_mod, max(n, STRESS_ROWS * STRESS_COLS if not args.no_stress else n), chunk, lane)

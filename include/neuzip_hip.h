@@ -50,8 +50,13 @@ extern "C" {
    cut into four segments of 256 symbols per lane. */
 #define NZ_DEFAULT_CHUNK 131072u
 #define NZ_DEFAULT_LANE_SYMS 256u
-#define NZ_LANE_SYMS_64K 256u
 #define NZ_LANE_SYMS_AUTO 0xFFFFFFFFu /* nz_manager_create: choose per tensor */
+/* Size budget of a manager's own geometry choices: stored exponent bytes
+   (container and all) over the order-0 entropy of the exponents, estimated
+   from the geometry for weights of ~2.55 bits per exponent.  The reference's
+   nvcomp cannot be measured here; this is the stand-in for "within 1 % of
+   nvcomp ANS". */
+#define NZ_DEFAULT_SIZE_BUDGET 1.01
 
 typedef struct nz_manager nz_manager;
 
@@ -175,21 +180,45 @@ int nz_decode(const void* dev_comp, uint64_t comp_bytes, const void* dev_packed,
 /* Manager(algorithm, chunk_size) for the class Manager_f{precision}_n{normalizer_size}
    (cuda/neuzip.cu:19-38, neuzip/binding.py:69-70).  precision in {0,1,3,7};
    normalizer_size 0 or a power of two up to 1024 (block normalizers, see above);
-   chunk_size 0 selects NZ_DEFAULT_CHUNK; lane_syms 0 the best segment length
-   for the chunk (NZ_DEFAULT_LANE_SYMS, NZ_LANE_SYMS_64K, or the chunk cut in 1..8);
-   NZ_LANE_SYMS_AUTO picks the geometry per tensor from its size and the
-   number of decode workgroups the device holds at once (three per compute
-   unit): with chunk_size 0, a tensor with fewer default-sized chunks than that
-   is cut into one, two or three chunks per compute unit (eight segments of 64
-   to 512 symbols per lane each), so that every compute unit holds the same
-   number of workgroups, and a tensor too small for that into 32 Ki chunks of
-   eight 4 Ki segments (shorter segments cost ~4.5 bits of container per lane
-   and segment); with a given chunk_size only the segments are shortened.
-   Every entry records the geometry it was written with
-   (nz_manager_geometry). */
+   chunk_size 0 selects the library's own table scope.
+   lane_syms > 0 is used as given.  lane_syms 0 leaves the segment length to
+   the library, which chooses it per tensor: the shortest segments from
+   NZ_DEFAULT_LANE_SYMS up whose estimated stored size is within the manager's
+   size budget (nz_manager_set_size_budget).  With the library's own chunk these
+   are chunks of eight segments: NZ_DEFAULT_CHUNK / NZ_DEFAULT_LANE_SYMS from
+   about six million elements up, 264 to 280 symbols per lane for one to four
+   million; a given chunk_size of 64 Ki: 344 symbols per lane, three segments.
+   NZ_LANE_SYMS_AUTO may, in addition, shorten the segments of a tensor that is
+   too small to fill the device: with the library's own chunk it cuts the
+   tensor into one, two or three decode workgroups per compute unit (chunks of
+   eight segments of 64..512 symbols per lane, in multiples of 8) when that is
+   modelled 10 % faster, and a tensor too small for that into 32 Ki chunks of
+   eight 4 Ki segments; with a given chunk_size only the segments are
+   shortened.  Shorter segments cost ~43 bytes each, so at the default budget
+   of 1.01 none qualifies and small tensors keep their size (serve them with
+   the batch calls); a larger budget buys wavefronts with bytes.  Every entry
+   records the geometry it was written with (nz_manager_geometry). */
 int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_t chunk_size,
                       uint32_t lane_syms, nz_manager** out);
 void nz_manager_destroy(nz_manager* m);
+
+/* No counterpart in the reference (nvcomp's ratio is what it is).  The
+   manager's own geometry choices (lane_syms 0 or NZ_LANE_SYMS_AUTO at creation)
+   keep the estimated stored size of a tensor's exponents within `ratio` x their
+   order-0 entropy.  The estimate, for weights of about 2.55 bits per exponent:
+   1.0008 + (134.4 x segments + 78 x chunks + 600) / elements, a short last
+   segment or chunk counting as a whole one; a geometry is accepted when the
+   estimate plus 0.0003, kept in hand for exponents of lower entropy, is within
+   the budget.  A tensor so small that no geometry reaches the budget keeps
+   the default one.  Default NZ_DEFAULT_SIZE_BUDGET; valid above 1.002 up to 2.
+   Affects the writes that follow. */
+int nz_manager_set_size_budget(nz_manager* m, double ratio);
+double nz_manager_size_budget(const nz_manager* m);
+/* The estimate itself for a tensor of n elements (0 for an invalid geometry),
+   and whether the manager's own choices would accept the geometry for it, for
+   a caller who chooses geometries by hand (nz_manager_geometry_hint). */
+double nz_estimated_size_ratio(uint64_t n, uint32_t chunk_size, uint32_t lane_syms);
+int nz_manager_in_budget(const nz_manager* m, uint64_t n, uint32_t chunk_size, uint32_t lane_syms);
 
 /* Manager::write(name, tensor), cuda/high_level.cu:132-162.  Replaces an
    existing entry of the same name (:137-140).  Synchronises the stream once

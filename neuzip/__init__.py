@@ -6,7 +6,8 @@
 are the objects of :mod:`neuzip_amd`; the reference's module paths
 (``neuzip.utils``, ``neuzip.nn.linear`` ...) resolve to their counterparts.
 ``neuzip.Manager`` keeps the reference's constructor signature,
-``chunk_size=2**16`` included (neuzip/binding.py:56-62).
+``chunk_size=2**16`` included (neuzip/binding.py:56-62); left at that default, every
+tensor gets the geometry the library picks for its size.
 """
 import sys as _sys
 

@@ -20,14 +20,14 @@ DTYPE_BF16, DTYPE_F16, DTYPE_F32 = 0, 1, 2
 ALGO_ANS = 0
 DEFAULT_CHUNK = 131072
 DEFAULT_LANE_SYMS = 256
-LANE_SYMS_64K = 256
+DEFAULT_SIZE_BUDGET = 1.01
 LANE_SYMS_AUTO = 0xFFFFFFFF
 DECODE_CHECK, DECODE_STREAM_OUT, DECODE_RESIDENT_OUT = 1, 2, 4  # nz_decode flags
 
 EXPORTS = [
     "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",
     "nz_encode_workspace_bytes", "nz_norm_bytes", "nz_split", "nz_encode", "nz_encode_static", "nz_decode",
-    "nz_manager_create", "nz_manager_destroy", "nz_manager_write", "nz_manager_write_batch",
+    "nz_manager_create", "nz_manager_destroy", "nz_manager_set_size_budget", "nz_manager_size_budget", "nz_estimated_size_ratio", "nz_manager_in_budget", "nz_manager_write", "nz_manager_write_batch",
     "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
     "nz_manager_meta", "nz_manager_geometry", "nz_manager_size", "nz_manager_size_reference", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
     "nz_manager_norm_bytes", "nz_manager_buffers", "nz_manager_erase", "nz_manager_check",
@@ -76,6 +76,14 @@ def load() -> ctypes.CDLL:
     L.nz_manager_create.argtypes = [i32, i32, i32, u32, u32, ctypes.POINTER(vp)]
     L.nz_manager_destroy.restype = None
     L.nz_manager_destroy.argtypes = [vp]
+    L.nz_manager_set_size_budget.restype = i32
+    L.nz_manager_set_size_budget.argtypes = [vp, ctypes.c_double]
+    L.nz_manager_size_budget.restype = ctypes.c_double
+    L.nz_manager_size_budget.argtypes = [vp]
+    L.nz_manager_in_budget.restype = i32
+    L.nz_manager_in_budget.argtypes = [vp, u64, u32, u32]
+    L.nz_estimated_size_ratio.restype = ctypes.c_double
+    L.nz_estimated_size_ratio.argtypes = [u64, u32, u32]
     L.nz_manager_write.restype = i32
     L.nz_manager_write.argtypes = [vp, ctypes.c_char_p, vp, u64, i32, vp]
     L.nz_manager_write_batch.restype = i32

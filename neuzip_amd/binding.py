@@ -38,7 +38,8 @@ class _HipBackend:
     """Backend object with the method set of the reference's C++ Manager
     (cuda/neuzip.cu:28-37): read / write / size / linear / linear_without_bias / split."""
 
-    def __init__(self, precision: int, normalizer_size: int, chunk_size: int, lane_symbols: int):
+    def __init__(self, precision: int, normalizer_size: int, chunk_size: int, lane_symbols: int,
+                 size_budget: Optional[float] = None):
         self._L = _lib.load()
         self._h = ctypes.c_void_p()
         self.auto_geometry = lane_symbols == "auto" and not chunk_size
@@ -47,9 +48,13 @@ class _HipBackend:
         rc = self._L.nz_manager_create(_lib.ALGO_ANS, precision, normalizer_size, chunk_size,
                                        lane_symbols, ctypes.byref(self._h))
         _lib.raise_for(rc)
+        if size_budget is not None:
+            _lib.raise_for(self._L.nz_manager_set_size_budget(self._h, float(size_budget)))
         self._device = torch.device("cuda", torch.cuda.current_device())
         self._normalizer = int(normalizer_size)
         self._known = {}  # handle -> (encoded name, element count), dropped on write
+        self._names1 = {}  # handle -> one-element ctypes array with its encoded name (fused product of one matrix)
+        self.fused_rows = True  # serve single-row linear() calls with the fused decode-and-multiply kernel
 
     def close(self):
         if getattr(self, "_h", None) is not None and self._h:
@@ -77,8 +82,13 @@ class _HipBackend:
         if flat.data_ptr() % 16:
             flat = flat.clone()
         self._known.pop(handle, None)
+        stream = torch.cuda.current_stream(flat.device)
         rc = self._L.nz_manager_write(self._h, handle.encode(), flat.data_ptr(), flat.numel(), code,
-                                      _stream_ptr(flat.device))
+                                      stream.cuda_stream)
+        # A write into existing buffers returns while the encode kernel is still reading `flat`.
+        # Memory that came from another stream's pool must not go back to it before then.
+        if rc == 0 and flat.numel():
+            flat.record_stream(stream)
         _lib.raise_for(rc)
 
     def write_batch(self, handles, tensors) -> None:
@@ -98,8 +108,11 @@ class _HipBackend:
             names = (ctypes.c_char_p * k)(*[h.encode() for h in hs])
             ptrs = (ctypes.c_void_p * k)(*[f.data_ptr() for f in fs])
             ns = (ctypes.c_uint64 * k)(*[f.numel() for f in fs])
-            rc = self._L.nz_manager_write_batch(self._h, names, ptrs, ns, k, _lib.DTYPE_BF16,
-                                                _stream_ptr(self._device))
+            stream = torch.cuda.current_stream(self._device)
+            rc = self._L.nz_manager_write_batch(self._h, names, ptrs, ns, k, _lib.DTYPE_BF16, stream.cuda_stream)
+            for f in fs:  # see write(): the kernel may still be reading them
+                if rc == 0 and f.numel():
+                    f.record_stream(stream)
             _lib.raise_for(rc)
 
     def read(self, handle: str) -> torch.Tensor:
@@ -126,6 +139,19 @@ class _HipBackend:
         c, l = ctypes.c_uint32(), ctypes.c_uint32()
         _lib.raise_for(self._L.nz_manager_geometry(self._h, handle.encode(), ctypes.byref(c), ctypes.byref(l)))
         return int(c.value), int(l.value)
+
+    @property
+    def size_budget(self) -> float:
+        """stored exponent bytes over their order-0 entropy that the manager's geometry choices keep to"""
+        return float(self._L.nz_manager_size_budget(self._h))
+
+    def estimated_size_ratio(self, numel: int, chunk_size: int, lane_symbols: int) -> float:
+        """the library's estimate of that ratio for a tensor of ``numel`` elements (0 for an invalid geometry)"""
+        return float(self._L.nz_estimated_size_ratio(numel, chunk_size, lane_symbols))
+
+    def in_budget(self, numel: int, chunk_size: int, lane_symbols: int) -> bool:
+        """whether the manager's own choices would accept this geometry for a tensor of ``numel`` elements"""
+        return bool(self._L.nz_manager_in_budget(self._h, numel, chunk_size, lane_symbols))
 
     def geometry_hint(self, handle: str, chunk_size: int, lane_symbols: int) -> None:
         """The next writes under ``handle`` use this geometry; (0, 0) takes the hint back."""
@@ -250,10 +276,36 @@ class _HipBackend:
         prev = getattr(self, "_outside", None)
         self._outside = flag if prev is None else prev | flag
 
+    def _fused_row(self, handle: str, inputs: torch.Tensor, shape, bias):
+        """``x @ W^T (+ b)`` for ONE activation row without writing the dense weight:
+        the product is formed while the weight is decoded (nz_manager_gemv_batch).
+        -> None when the call does not qualify (several rows, a row length that is
+        not a multiple of 512, another dtype, a bias the kernel cannot take)."""
+        if (not self.fused_rows or inputs.dim() == 0 or inputs.numel() != inputs.shape[-1] or len(shape) != 2
+                or inputs.shape[-1] != shape[1] or shape[1] % 512 or inputs.dtype != torch.bfloat16
+                or not inputs.is_cuda or (torch.is_grad_enabled() and inputs.requires_grad)):
+            return None
+        if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_cuda or bias.numel() != shape[0]
+                                 or not bias.is_contiguous() or (torch.is_grad_enabled() and bias.requires_grad)):
+            return None
+        x = inputs if inputs.is_contiguous() else inputs.contiguous()
+        if x.data_ptr() % 16:
+            x = x.clone()
+        names = self._names1.get(handle)
+        if names is None:
+            names = self._names1[handle] = (ctypes.c_char_p * 1)(handle.encode())
+        out = torch.empty(shape[0], dtype=torch.bfloat16, device=x.device)
+        self.gemv_batch(names, x, [bias], [out])
+        return out.view(*inputs.shape[:-1], shape[0])
+
     def linear(self, handle: str, inputs: torch.Tensor, shape, bias: torch.Tensor) -> torch.Tensor:
         # cuda/high_level.cu:252-257: addmm(bias, input, W^T).  The reference only
         # accepts a 2-D input here; inputs with leading batch dimensions take
-        # the equivalent F.linear route.
+        # the equivalent F.linear route.  A single activation row (single-token
+        # inference) is served by the fused decode-and-multiply kernel.
+        fused = self._fused_row(handle, inputs, shape, bias)
+        if fused is not None:
+            return fused
         weight = self.read(handle).view(shape)
         if inputs.dim() == 2:
             return torch.addmm(bias, inputs, weight.t())
@@ -261,6 +313,9 @@ class _HipBackend:
 
     def linear_without_bias(self, handle: str, inputs: torch.Tensor, shape) -> torch.Tensor:
         # cuda/high_level.cu:259-263
+        fused = self._fused_row(handle, inputs, shape, None)
+        if fused is not None:
+            return fused
         weight = self.read(handle).view(shape)
         return torch.matmul(inputs, weight.t())
 
@@ -323,23 +378,27 @@ class Manager:
         normalizer_size=None,
         chunk_size=None,
         lane_symbols: int = 0,
+        size_budget: Optional[float] = None,
     ) -> None:
         """``chunk_size`` is the number of exponents that share one frequency
         table.  The reference passes its value (default ``2**16``) to nvcomp as
         the chunk size; here ``None`` selects the library's own table scope of
         ``2**17`` elements decoded by eight wavefronts, which is both smaller and
         faster on this hardware, and ``2**16`` (or any supported value) is
-        honoured when given.  ``lane_symbols`` (extension; 0 = the best value
-        for the chunk) is the number of exponents each of the 64 rANS lanes of a
-        wavefront codes per segment: smaller values expose more wavefronts per
-        chunk at the price of about 4.5 bits of container per lane and segment.
-        ``"auto"`` picks the geometry per tensor from its size and from how many
-        decode workgroups the device holds at once: small tensors get shorter
-        segments (and smaller chunks) so that they still fill the GPU, mid-sized
-        ones slightly longer segments so that two of them decoded by one launch
-        run as a single round of workgroups (meant for single-token inference
-        and for training, where every weight is decoded three times and encoded
-        once per step)."""
+        honoured when given.  ``lane_symbols`` (extension; 0 = the shortest
+        segments that stay inside the size budget for the chunk) is the number of
+        exponents each of the 64 rANS lanes of a wavefront codes per segment:
+        smaller values expose more wavefronts per chunk at the price of about
+        4.5 bits of container per lane and segment.  ``"auto"`` picks the
+        geometry per tensor from its size and from how many decode workgroups
+        the device holds at once, inside the size budget.  ``size_budget``
+        (extension; default 1.01) bounds what the manager's own geometry choices
+        may store for the exponents, as a multiple of their order-0 entropy
+        (estimated from the geometry): at the default, small tensors keep the
+        default geometry and are best served by the calls that take several
+        tensors per launch (``write_many``, ``DecompressAhead``, ``FusedGemv``);
+        a larger budget lets ``"auto"`` give them shorter segments so that each
+        of them fills the GPU on its own."""
         normalizer_size = 0 if normalizer_size is None else normalizer_size
         self.meta_dict = {}  # handle -> original shape
         self._stamps = {}    # handle -> number of writes: lets caches of decoded weights notice
@@ -356,7 +415,7 @@ class Manager:
             raise AttributeError(
                 f"module 'neuzip._cuda' has no attribute 'Manager_f{precision}_n{normalizer_size}'"
             )
-        self._be = _HipBackend(precision, normalizer_size, int(chunk_size or 0), lane_symbols)
+        self._be = _HipBackend(precision, normalizer_size, int(chunk_size or 0), lane_symbols, size_budget)
         # what a checkpoint must agree on (the chunk geometry travels inside every container)
         self._settings = {"precision": int(precision), "normalizer_size": int(normalizer_size)}
 
@@ -410,10 +469,25 @@ class Manager:
         return self._be.size(handle, reference_accounting)
 
     def linear(self, handle: str, inputs: torch.Tensor, bias=None) -> torch.Tensor:
+        """``inputs @ W^T (+ bias)`` against the stored weight (neuzip/binding.py:97-102).
+        One activation row of a multiple of 512 elements (single-token inference)
+        is multiplied while the weight is decoded, without the dense weight ever
+        being written; its sums are formed in an order of their own, so the
+        result agrees with the decompress-then-GEMM path to rounding, not bit for
+        bit (``manager.fused_rows = False`` keeps every call on that path)."""
         shape = self.meta_dict[handle]
         if bias is None:
             return self._be.linear_without_bias(handle, inputs, shape)
         return self._be.linear(handle, inputs, shape, bias)
+
+    @property
+    def fused_rows(self) -> bool:
+        return bool(getattr(self._be, "fused_rows", False))
+
+    @fused_rows.setter
+    def fused_rows(self, on: bool) -> None:
+        if hasattr(self._be, "fused_rows"):
+            self._be.fused_rows = bool(on)
 
     def gather_rows(self, handle: str, indices: torch.Tensor) -> torch.Tensor:
         """Rows ``indices`` of the stored 2-D table ``handle`` as ``[indices.numel(), row_len]``

@@ -98,8 +98,9 @@ uint64_t next_nonce() {
 }
 
 // How often a chunk of a direct encode looks for an announcement it waits for
-// (about a microsecond per look) before it gives up.
-std::atomic<uint32_t> g_lookback_spins{1u << 21};
+// (about a microsecond per look) before it gives up: some tens of milliseconds,
+// as a wait that is given up costs no more than one compaction kernel.
+std::atomic<uint32_t> g_lookback_spins{1u << 15};
 
 // One tensor of an encode call, as the kernels see it.  `comp`/`comp_cap`: where
 // the container goes (known only after phase 1 when the buffer is sized to fit).
@@ -389,6 +390,76 @@ int static_scratch(uint8_t** out) {
   return NZ_OK;
 }
 
+// Stored exponent bytes (container + what the packed stream saves) of a tensor
+// of n elements over the order-0 entropy of its exponents, as a function of
+// the geometry: every lane and segment costs about 4.5 bits (its coder state
+// less the 16 carried bits) and every segment a directory entry and padding
+// (43 bytes a segment in all, a short last segment as much as a full one),
+// every chunk a table (25 bytes), every tensor a header and a ragged end (up to
+// ~190 bytes).  Fitted to measurements on N(0, 0.02) weights (2.545 bits per
+// exponent: 1 byte of container is 3.14 symbols' worth of entropy), where it is
+// within 0.0003 from a million elements up and within 0.0001 from 16 million:
+//   58.7 M elements  131072/256 1.0096, 135168/264 1.0094, 131072/344 1.0076, 262144/512 1.0053
+//   1 Mi elements    131072/256 1.0099, 139264/272 1.0098, 147456/288 1.0093, 262144/512 1.0056
+//   (earlier fits, large tensors: 65536/256 1.0102, 65536/128 1.0185, 32768/64 1.036).
+double est_ratio(uint64_t n, uint32_t chunk_syms, uint32_t lane_syms) {
+  if (n == 0) return 1.0;
+  const uint64_t seg = (uint64_t)lane_syms * NZ_LANES;
+  const uint64_t full = n / chunk_syms, rest = n % chunk_syms;
+  const uint64_t segs = full * ((chunk_syms + seg - 1) / seg) + (rest + seg - 1) / seg;
+  const uint64_t chunks = full + (rest ? 1 : 0);
+  return 1.0008 + (134.4 * (double)segs + 78.0 * (double)chunks + 600.0) / (double)n;
+}
+
+// The overhead is a fixed number of bytes, so the ratio grows as the entropy
+// shrinks (weights drift while they are trained: a 1024 x 1024 GPT-2 weight
+// gained 0.00015 in 20 AdamW steps): a geometry counts as inside a budget when
+// its estimate leaves 0.0003 in hand.
+bool in_budget(uint64_t n, uint32_t chunk_syms, uint32_t lane_syms, double budget) {
+  return est_ratio(n, chunk_syms, lane_syms) + 0.0003 <= budget;
+}
+
+// The geometry a manager uses for a tensor of n elements when the caller
+// leaves the segment length to the library.  The library's own chunk: eight
+// segments per chunk, from the default 256 symbols per lane up to 512 in steps
+// of 8, the shortest (most wavefronts) that is inside the budget.  A given
+// chunk: the shortest valid segments from 256 symbols per lane up that are
+// inside it.  A tensor too small for any of these to reach the budget (its
+// header alone is above it) keeps the starting point: its bytes do not matter
+// and its decode time does.
+void default_geometry(uint64_t n, bool own_chunk, double budget, uint32_t* chunk_syms, uint32_t* lane_syms) {
+  if (own_chunk) {
+    *chunk_syms = NZ_DEFAULT_CHUNK;
+    *lane_syms = NZ_DEFAULT_LANE_SYMS;
+    for (uint32_t lane = NZ_DEFAULT_LANE_SYMS; lane <= 512; lane += 8) {
+      const uint32_t chunk = lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK;
+      if (!in_budget(n, chunk, lane, budget)) continue;
+      *chunk_syms = chunk;
+      *lane_syms = lane;
+      return;
+    }
+    return;
+  }
+  const uint32_t chunk = *chunk_syms;
+  uint32_t first = 0, shortest = 0;
+  for (uint32_t lane = 16; lane <= 65536; lane += 8) {
+    if (nz_geom_check(chunk, lane)) continue;
+    if (!shortest) shortest = lane;
+    if (lane < NZ_DEFAULT_LANE_SYMS) continue;
+    if (!first) first = lane;
+    if (in_budget(n, chunk, lane, budget)) {
+      *lane_syms = lane;
+      return;
+    }
+  }
+  // nothing fits the budget (a small tensor), or the chunk is too short for 256 symbols per lane
+  *lane_syms = first ? first : (shortest ? shortest : NZ_DEFAULT_LANE_SYMS);
+}
+
+// a tensor large enough for the per-tensor terms of the estimate to vanish: what
+// a manager reports as its nominal geometry before it has seen a tensor
+constexpr uint64_t NZ_NOMINAL_N = 1ull << 28;
+
 struct Entry {
   void* comp = nullptr;
   uint64_t comp_bytes = 0, comp_cap = 0;
@@ -429,7 +500,13 @@ struct nz_manager {
   uint32_t normalizer = 0;  // elements per normalizer group, 0 = none
   uint32_t chunk_syms, lane_syms;
   bool own_chunk = false;   // chunk_size 0 was given: the library's own table scope
+  bool own_lanes = false;   // lane_syms 0 or AUTO was given: the segment length follows the size budget
   bool auto_lanes = false;  // pick the geometry per tensor so that small tensors still fill the GPU
+  double budget = NZ_DEFAULT_SIZE_BUDGET;  // stored exponent bytes over their order-0 entropy the manager's own choices stay within
+  hipStream_t last_stream = nullptr;  // stream of the last call that used the shared scratch (write, product, row gather)
+  bool has_stream = false;
+  hipEvent_t order_ev = nullptr;      // orders such a call on another stream behind it
+  uint32_t given_chunk = 0;  // the caller's chunk_size (0: the library's own)
   uint32_t slots = 768;     // decode workgroups of eight wavefronts the device holds at once (3 per CU)
   std::unordered_map<std::string, Entry> entries;  // compress_cache + meta_cache
   std::unordered_map<std::string, std::pair<uint32_t, uint32_t>> hints;  // name -> (chunk, lane) for its next writes
@@ -590,20 +667,14 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
     return fail(NZ_ERR_ARG, "normalizer_size must be 0 or a power of two up to 1024");
   const bool auto_lanes = lane_syms == NZ_LANE_SYMS_AUTO;
   const bool own_chunk = chunk_size == 0;
+  const bool own_lanes = lane_syms == 0 || auto_lanes;
   if (own_chunk) {
     chunk_size = NZ_DEFAULT_CHUNK;
     // an explicit segment length too short for eight segments to cover the
     // default chunk goes with the smaller table scope
-    if (lane_syms != 0 && !auto_lanes && (uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size)
-      chunk_size = 65536;
+    if (!own_lanes && (uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size) chunk_size = 65536;
   }
-  if (lane_syms == 0 || auto_lanes) {
-    // the best measured segment length for the chunk: 8 segments of 256 per lane
-    // in a 128 Ki chunk, four of them in a 64 Ki chunk
-    lane_syms = chunk_size == NZ_DEFAULT_CHUNK ? NZ_DEFAULT_LANE_SYMS : NZ_LANE_SYMS_64K;
-    while (lane_syms > 8 && (uint64_t)lane_syms * NZ_LANES > chunk_size) lane_syms /= 2;
-    while ((uint64_t)lane_syms * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK < chunk_size) lane_syms *= 2;
-  }
+  if (own_lanes) default_geometry(NZ_NOMINAL_N, own_chunk, NZ_DEFAULT_SIZE_BUDGET, &chunk_size, &lane_syms);
   NzGeom g;
   if (int rc = make_geom(&g, 0, chunk_size, lane_syms)) return rc;
   nz_manager* m = new nz_manager();
@@ -611,6 +682,8 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   m->normalizer = (uint32_t)normalizer_size;
   m->chunk_syms = chunk_size;
   m->own_chunk = own_chunk;
+  m->own_lanes = own_lanes;
+  m->given_chunk = own_chunk ? 0u : chunk_size;
   m->lane_syms = lane_syms;
   m->auto_lanes = auto_lanes;
   // device block and its pinned mirror, 1 KiB each: [0, 256) as described at the members;
@@ -628,6 +701,7 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
     m->rw[k].h_totals = reinterpret_cast<uint64_t*>(reinterpret_cast<uint8_t*>(m->h_pin) + 256 + 256 * k);
     e = hipEventCreateWithFlags(&m->rw[k].ev, hipEventDisableTiming);
   }
+  if (e == hipSuccess) e = hipEventCreateWithFlags(&m->order_ev, hipEventDisableTiming);
   int dev = 0, cus = 0;
   if (e == hipSuccess) e = hipGetDevice(&dev);
   if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
@@ -635,6 +709,7 @@ int nz_manager_create(int algorithm, int precision, int normalizer_size, uint32_
   if (e != hipSuccess) {
     for (int k = 0; k < 2; ++k)
       if (m->rw[k].ev) (void)hipEventDestroy(m->rw[k].ev);
+    if (m->order_ev) (void)hipEventDestroy(m->order_ev);
     if (m->d_status) (void)hipFree(m->d_status);
     if (m->h_pin) (void)hipHostFree(m->h_pin);
     delete m;
@@ -657,9 +732,36 @@ void nz_manager_destroy(nz_manager* m) {
     if (m->rw[k].ev) (void)hipEventDestroy(m->rw[k].ev);
   }
   if (m->gemv_acc) (void)hipFree(m->gemv_acc);
+  if (m->order_ev) (void)hipEventDestroy(m->order_ev);
   if (m->d_status) (void)hipFree(m->d_status);
   if (m->h_pin) (void)hipHostFree(m->h_pin);
   delete m;
+}
+
+double nz_estimated_size_ratio(uint64_t n, uint32_t chunk_size, uint32_t lane_syms) {
+  if (nz_geom_check(chunk_size, lane_syms)) return 0.0;
+  return est_ratio(n, chunk_size, lane_syms);
+}
+
+double nz_manager_size_budget(const nz_manager* m) { return m ? m->budget : 0.0; }
+
+int nz_manager_in_budget(const nz_manager* m, uint64_t n, uint32_t chunk_size, uint32_t lane_syms) {
+  return m && !nz_geom_check(chunk_size, lane_syms) && in_budget(n, chunk_size, lane_syms, m->budget) ? 1 : 0;
+}
+
+int nz_manager_set_size_budget(nz_manager* m, double ratio) {
+  if (!m) return fail(NZ_ERR_ARG, "null manager");
+  if (!(ratio > 1.002 && ratio <= 2.0)) return fail(NZ_ERR_ARG, "size budget must be above 1.002 and at most 2");
+  std::lock_guard<std::mutex> lock(m->mu);
+  m->budget = ratio;
+  if (m->own_lanes) {
+    uint32_t chunk = m->own_chunk ? 0u : m->given_chunk, lane = 0;
+    default_geometry(NZ_NOMINAL_N, m->own_chunk, ratio, &chunk, &lane);
+    if (nz_geom_check(chunk, lane)) return fail(NZ_ERR_ARG, "no valid geometry for this chunk size");
+    m->chunk_syms = chunk;
+    m->lane_syms = lane;
+  }
+  return NZ_OK;
 }
 
 }  // extern "C"
@@ -687,10 +789,18 @@ void release_entry(Entry& e) {
 }
 
 // Geometry of a tensor of n elements.  Throughput of both codec directions is
-// set by the number of wavefronts in flight (one per 64 * lane_syms elements).
-// In auto mode a tensor too small to give every SIMD two wavefronts at the
-// default gets shorter segments (and, with the library's own chunk, the smaller
-// 64 Ki table scope that allows them), at ~4.5 bits per extra lane.
+// set by the number of wavefronts in flight (one per 64 * lane_syms elements),
+// the stored size by the number of segments (est_ratio).  A manager that was
+// given a segment length uses it.  One that was not chooses per tensor: the
+// shortest segments from the default up whose estimated size is inside the
+// manager's budget (default_geometry: at the default budget of 1.01 that is
+// 131072/256 from about six million elements up and 264 to 280 symbols per lane
+// for the one to four million elements of a GPT-2 weight).  In auto mode a
+// tensor too small to give every SIMD two wavefronts may get shorter segments
+// still (and, with the library's own chunk, a table scope to match), but only
+// inside the same budget: at 1.01 nothing shorter qualifies, so a small tensor
+// keeps its size and is served well by the calls that take several tensors
+// per launch; a caller who raises the budget buys wavefronts with bytes.
 int pick_geometry(const nz_manager* m, const char* name, uint64_t n, NzGeom* g, uint32_t* chunk_out,
                   uint32_t* lane_out) {
   uint32_t lane_syms = m->lane_syms, chunk_syms = m->chunk_syms;
@@ -700,51 +810,51 @@ int pick_geometry(const nz_manager* m, const char* name, uint64_t n, NzGeom* g, 
     *lane_out = hint->second.second;
     return make_geom(g, n, *chunk_out, *lane_out);
   }
-  if (m->auto_lanes && m->own_chunk && chunk_syms == NZ_DEFAULT_CHUNK && lane_syms == NZ_DEFAULT_LANE_SYMS) {
+  if (m->own_lanes) default_geometry(n, m->own_chunk, m->budget, &chunk_syms, &lane_syms);
+  if (m->auto_lanes && m->own_chunk) {
     // The device holds `slots` decode workgroups (three per compute unit) at
     // once, and a launch is fastest when every compute unit has the same number
     // of them: 378 workgroups on 256 units run as long as 512 would (measured on
     // a 4096 x 14336 matrix: 51 us with 378 chunks, 38 us with 512).  A tensor
-    // with more default-sized chunks than slots keeps the default geometry.  A
-    // smaller one is cut into one, two or three workgroups per compute unit
-    // (more of them only where the model below promises 10 % or more), with
-    // segments of 64 to 512
-    // symbols per lane (shorter segments cost compression: ~4.5 bits per lane
-    // and segment); a tensor too small for that gets 32 Ki chunks of eight
-    // 4 Ki segments.  Time of a round ~ symbols per lane x time of a step, which
+    // with more chunks than slots keeps the geometry chosen above.  A smaller
+    // one may be cut into one, two or three workgroups per compute unit (eight
+    // segments of 64 to 512 symbols per lane each) when that is inside the size
+    // budget and the model below promises 10 % or more; a tensor too small for
+    // that may get 32 Ki chunks of eight 4 Ki segments (again: only inside the
+    // budget).  Time of a round ~ symbols per lane x time of a step, which
     // grows with the wavefronts that share a SIMD unit (2, 4, 6 of them: about
     // 107, 147, 215 ns per step).
     const uint64_t slots = m->slots, cus = slots / 3;
     const uint64_t chunks = (n + chunk_syms - 1) / chunk_syms;
-    if (chunks > slots || cus == 0) {
-      // default
-    } else {
+    if (chunks <= slots && cus != 0) {
       static const uint32_t step_ns[3] = {107, 147, 215};
-      uint64_t best_t = ~0ull;
-      uint32_t best_lane = 0;
+      const uint64_t per_cu = chunks ? (chunks + cus - 1) / cus : 1;  // 1..3 workgroups per compute unit
+      uint64_t best_t = (uint64_t)lane_syms * step_ns[per_cu - 1];
+      bool found = false;
       for (uint32_t k = 1; k <= 3; ++k) {
         const uint64_t per_lane = (n + k * cus * 512 - 1) / (k * cus * 512);  // a chunk is 8 x 64 lanes
         const uint32_t lane = (uint32_t)((per_lane + 7) / 8) * 8;
-        if (lane < 64 || lane > 2 * NZ_DEFAULT_LANE_SYMS) continue;
-        if (nz_geom_check(lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK, lane)) continue;
+        if (lane < 64 || lane > 512) continue;
+        const uint32_t chunk = lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK;
+        if (nz_geom_check(chunk, lane) || !in_budget(n, chunk, lane, m->budget)) continue;
         const uint64_t t = (uint64_t)lane * step_ns[k - 1];
-        if (best_lane == 0 || 10 * t < 9 * best_t) {  // more, shorter segments only for a gain above 10 %
+        if (10 * t < 9 * best_t) {  // another geometry only for a gain above 10 %
           best_t = t;
-          best_lane = lane;
+          lane_syms = lane;
+          chunk_syms = chunk;
+          found = true;
         }
       }
-      if (best_lane) {
-        lane_syms = best_lane;
-        chunk_syms = best_lane * NZ_LANES * NZ_MAX_SEGS_PER_CHUNK;
-      } else {
+      if (!found && n < (uint64_t)64 * cus * 512 && in_budget(n, 32768, 64, m->budget)) {
         chunk_syms = 32768;
         lane_syms = 64;
       }
     }
   } else if (m->auto_lanes) {
     // a chunk size given by the caller: shorter segments while that is a valid
-    // geometry and the tensor has fewer than 2048 segments
+    // geometry inside the size budget and the tensor has fewer than 2048 segments
     while (lane_syms > 16 && nz_geom_check(chunk_syms, (lane_syms / 2 + 7) & ~7u) == 0 &&
+           in_budget(n, chunk_syms, (lane_syms / 2 + 7) & ~7u, m->budget) &&
            n / ((uint64_t)lane_syms * NZ_LANES) < 2048)
       lane_syms = (lane_syms / 2 + 7) & ~7u;
   }
@@ -841,39 +951,44 @@ int settle_slot(nz_manager* m, int k) {
   RewriteSlot& s = m->rw[k];
   if (!s.busy) return NZ_OK;
   if (hipEventQuery(s.ev) != hipSuccess) NZ_HIP(hipEventSynchronize(s.ev));
-  s.busy = false;
+  // the slot stays busy until every entry of the batch has been handled: a call that fails
+  // half way leaves the others pending, and the next use of the slot or of such an entry tries again
   for (uint32_t j = 0; j < s.count; ++j) {
     auto it = m->entries.find(s.names[j]);
     if (it == m->entries.end() || it->second.pending != k) continue;
     Entry& ent = it->second;
-    ent.pending = -1;
     uint64_t total = s.h_totals[j];
     if (s.h_totals[16 + j] == s.b.item[j].nonce) {
       // a chunk gave up waiting for the sizes before it: the records once more, by the compaction
-      ++m->rewrites_redone;
       if (int rc = encode_replace(s.b.item[j], s.b.item[j].comp, s.stream)) return rc;
       NZ_HIP(hipStreamSynchronize(s.stream));
+      s.h_totals[16 + j] = 0;
+      ++m->rewrites_redone;
       total = s.h_totals[j];
     }
-    if (total <= ent.comp_cap) {
-      ent.comp_bytes = total;
-      continue;
+    if (total > ent.comp_cap) {
+      // outgrown: a buffer that fits, the records moved again
+      void* bigger = nullptr;
+      const uint64_t cap = total + total / 32 + 4096;
+      NZ_HIP(hipMalloc(&bigger, cap));
+      NzEncItem again = s.b.item[j];
+      again.comp = (uint8_t*)bigger;
+      again.comp_cap = cap;
+      int rc = encode_replace(again, s.b.item[j].comp, s.stream);
+      if (rc == NZ_OK && hipStreamSynchronize(s.stream) != hipSuccess) rc = fail(NZ_ERR_HIP, "settle: synchronize failed");
+      if (rc != NZ_OK) {
+        (void)hipFree(bigger);
+        return rc;
+      }
+      (void)hipFree(ent.comp);
+      ent.comp = bigger;
+      ent.comp_cap = cap;
+      ++m->rewrites_replaced;
     }
-    // outgrown: a buffer that fits, the records moved again
-    ++m->rewrites_replaced;
-    void* bigger = nullptr;
-    const uint64_t cap = total + total / 32 + 4096;
-    NZ_HIP(hipMalloc(&bigger, cap));
-    NzEncItem again = s.b.item[j];
-    again.comp = (uint8_t*)bigger;
-    again.comp_cap = cap;
-    if (int rc = encode_replace(again, s.b.item[j].comp, s.stream)) return rc;
-    NZ_HIP(hipStreamSynchronize(s.stream));
-    (void)hipFree(ent.comp);
-    ent.comp = bigger;
-    ent.comp_cap = cap;
     ent.comp_bytes = total;
+    ent.pending = -1;
   }
+  s.busy = false;
   return NZ_OK;
 }
 
@@ -882,6 +997,44 @@ int settle_entry(nz_manager* m, const Entry& ent) { return ent.pending >= 0 ? se
 int settle_all(nz_manager* m) {
   for (int k = 0; k < 2; ++k)
     if (int rc = settle_slot(m, k)) return rc;
+  return NZ_OK;
+}
+
+// Is `st` being captured into a graph?  (An error of the query is taken as "no".)
+bool capturing(hipStream_t st) {
+  hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &cap) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return cap != hipStreamCaptureStatusNone;
+}
+
+// A call that may allocate, wait on the host or look at an event from the host
+// cannot be recorded into a graph: it is refused with a message, before it
+// touches anything (the capture stays valid).
+int refuse_under_capture(hipStream_t st, bool may_block, const char* what) {
+  if (may_block && capturing(st))
+    return fail(NZ_ERR_ARG, std::string(what) + ": the stream is being captured into a graph and this call may "
+                                               "allocate or wait on the host; capture nz_encode / nz_decode, or reads "
+                                               "and products of entries that no write is pending for");
+  return NZ_OK;
+}
+
+// Writes, products and row gathers of one manager share its scratch memory
+// (encode workspace, row accumulators): they are ordered on the device.  When
+// such a call arrives on another stream than the one before it, the new stream
+// is made to wait (an event, no host synchronisation) for what the other has
+// been given so far.  Streams under capture are left alone: what a graph holds
+// is ordered by the graph's owner.
+int order_scratch_use(nz_manager* m, hipStream_t st) {
+  if (capturing(st)) return NZ_OK;
+  if (m->has_stream && m->last_stream != st) {
+    NZ_HIP(hipEventRecord(m->order_ev, m->last_stream));
+    NZ_HIP(hipStreamWaitEvent(st, m->order_ev, 0));
+  }
+  m->last_stream = st;
+  m->has_stream = true;
   return NZ_OK;
 }
 
@@ -907,6 +1060,10 @@ int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* 
   if (dtype != NZ_DTYPE_BF16) return fail(NZ_ERR_DTYPE, "Unsupported data type");
   if (count > NZ_WRITE_BATCH_MAX) return fail(NZ_ERR_ARG, "at most 16 tensors per batch");
   hipStream_t st = (hipStream_t)stream;
+  std::lock_guard<std::mutex> lock(m->mu);  // also guards the geometry hints read below
+  // a write allocates, synchronises or (in place) looks at events from the host
+  if (int rc = refuse_under_capture(st, true, "write")) return rc;
+  if (int rc = order_scratch_use(m, st)) return rc;
   // check everything and size the scratch before anything is touched
   NzGeom g[NZ_WRITE_BATCH_MAX];
   uint32_t chunk[NZ_WRITE_BATCH_MAX], lane[NZ_WRITE_BATCH_MAX];
@@ -921,7 +1078,6 @@ int nz_manager_write_batch(nz_manager* m, const char* const* names, const void* 
     if (int rc = pick_geometry(m, names[i], ns[i], &g[i], &chunk[i], &lane[i])) return rc;
     at[i + 1] = at[i] + enc_layout(g[i]).bytes;
   }
-  std::lock_guard<std::mutex> lock(m->mu);
   // ---- in place: every handle already holds a tensor of this size and geometry.  The new
   // streams go straight into the buffers the entries have (an optimizer step changes the
   // container size by a few bytes; a buffer has ~1.5 % of headroom): no allocation, no free,
@@ -1035,6 +1191,7 @@ int nz_manager_read(nz_manager* m, const char* name, void* dev_out, uint64_t cap
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  if (int rc = refuse_under_capture((hipStream_t)stream, it->second.pending >= 0, "read")) return rc;
   if (int rc = settle_entry(m, it->second)) return rc;
   const Entry& ent = it->second;
   if (cap_elems < ent.n) return fail(NZ_ERR_CAPACITY, "output smaller than the stored tensor");
@@ -1053,10 +1210,18 @@ int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* 
     return fail(NZ_ERR_ARG, "null manager, names, outputs or capacities");
   std::lock_guard<std::mutex> lock(m->mu);
   // validate everything before the first launch: a failed call decodes nothing
+  {
+    bool pending = false;
+    for (uint32_t i = 0; i < count; ++i) {
+      if (!names[i]) return fail(NZ_ERR_ARG, "null name");
+      auto it = m->entries.find(names[i]);
+      if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+      pending = pending || it->second.pending >= 0;
+    }
+    if (int rc = refuse_under_capture((hipStream_t)stream, pending, "read_batch")) return rc;
+  }
   for (uint32_t i = 0; i < count; ++i) {
-    if (!names[i]) return fail(NZ_ERR_ARG, "null name");
     auto it = m->entries.find(names[i]);
-    if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
     if (int rc = settle_entry(m, it->second)) return rc;
     const Entry& ent = it->second;
     if (cap_elems[i] < ent.n) return fail(NZ_ERR_CAPACITY, "output smaller than the stored tensor");
@@ -1120,10 +1285,21 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
   b.log2n = log2_of(m->normalizer ? m->normalizer : 1);
   uint64_t grid = 0, rows = 0;
   uint32_t max_spc = 1;
+  {
+    bool blocks = false;
+    uint64_t want_rows = 0;
+    for (uint32_t i = 0; i < count; ++i) {
+      if (!names[i]) return fail(NZ_ERR_ARG, "null name");
+      auto it = m->entries.find(names[i]);
+      if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+      blocks = blocks || it->second.pending >= 0;
+      want_rows += it->second.n / in_features;
+    }
+    if (int rc = refuse_under_capture(st, blocks || m->gemv_rows < want_rows, "gemv_batch")) return rc;
+    if (int rc = order_scratch_use(m, st)) return rc;
+  }
   for (uint32_t i = 0; i < count; ++i) {
-    if (!names[i]) return fail(NZ_ERR_ARG, "null name");
     auto it = m->entries.find(names[i]);
-    if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
     if (int rc = settle_entry(m, it->second)) return rc;
     const Entry& ent = it->second;
     if (ent.n == 0 || ent.n % in_features)
@@ -1177,6 +1353,8 @@ int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indi
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
+  if (int rc = refuse_under_capture(st, true, "gather_rows")) return rc;
+  if (int rc = order_scratch_use(m, st)) return rc;
   if (int rc = settle_entry(m, it->second)) return rc;
   const Entry& ent = it->second;
   if (row_len == 0 || ent.n == 0 || ent.n % row_len)
@@ -1273,7 +1451,7 @@ uint64_t nz_manager_size(nz_manager* m, const char* name) {
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return 0;  // cuda/high_level.cu:209-211
-  (void)settle_entry(m, it->second);
+  if (settle_entry(m, it->second)) return 0;  // the size is not known: nz_last_error() says why
   return it->second.comp_bytes + it->second.packed_bytes + it->second.norm_bytes;
 }
 
@@ -1282,7 +1460,7 @@ uint64_t nz_manager_size_reference(nz_manager* m, const char* name) {
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return 0;
-  (void)settle_entry(m, it->second);
+  if (settle_entry(m, it->second)) return 0;
   const Entry& e = it->second;
   // cuda/high_level.cu:89-93: without normalizers the reference still allocates
   // (and size() counts, :208-221) one byte per 1024 elements
@@ -1295,7 +1473,7 @@ uint64_t nz_manager_exp_bytes(nz_manager* m, const char* name) {
   std::lock_guard<std::mutex> lock(m->mu);
   auto it = m->entries.find(name);
   if (it == m->entries.end()) return 0;
-  (void)settle_entry(m, it->second);
+  if (settle_entry(m, it->second)) return 0;
   return it->second.comp_bytes;
 }
 

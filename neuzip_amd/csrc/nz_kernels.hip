@@ -362,6 +362,7 @@ struct NzEncLds {
   uint32_t seg_units[NZ_MAX_SEGS_PER_CHUNK];
   uint32_t chunk_total, gave_up;
   uint32_t redo;  // a wavefront ran out of staging room: the chunk is coded again, into the slots
+  uint32_t lb[2];  // the two words of the scratch's announcement state, as thread 0 read them
   uint64_t red64[NZ_ENC_LONG_THREADS / 64];
 };
 
@@ -887,18 +888,20 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   const uint32_t ngroups = (seg_n + NZ_GROUP_SYMS - 1) / NZ_GROUP_SYMS;  // at most NG
   const bool seg_full = has_seg && seg_n == nom;
 
-  // state of the scratch's size announcements (see NzEncItem::lb_state), read
-  // long before it is needed
+  // State of the scratch's size announcements (see NzEncItem::lb_state): read
+  // once, by one thread, long before it is needed, and handed to the others
+  // through LDS, so that every thread of the workgroup acts on the same values
+  // (another workgroup may change the words while this one starts).
   uint32_t* lb_state = reinterpret_cast<uint32_t*>(it.ws + it.lb_state);
-  uint32_t lb_gen = 0;
-  bool direct = false;  // this run places its records itself
-  if (it.direct) {
-    lb_gen = __hip_atomic_load(lb_state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    direct = __hip_atomic_load(lb_state + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != NZ_LOOKBACK_ABORT;
+  if (tid == 0) {
+    L.lb[0] = it.direct ? __hip_atomic_load(lb_state, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    L.lb[1] = it.direct ? __hip_atomic_load(lb_state + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    L.redo = 0;
   }
   for (uint32_t i = tid; i < NZ_HIST_COPIES * NZ_HIST_STRIDE; i += blockDim.x) L.hist[i] = 0;
-  if (tid == 0) L.redo = 0;
   __syncthreads();
+  const uint32_t lb_gen = L.lb[0];
+  const bool direct = it.direct && L.lb[1] != NZ_LOOKBACK_ABORT;  // this run places its records itself
   uint32_t* myhist = L.hist + (lane & (NZ_HIST_COPIES - 1)) * NZ_HIST_STRIDE;
 
   // ---- phase 1: split.  Packed bytes go to the stored layout: segment k of a
@@ -1091,9 +1094,11 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   // the run's 64-bit mark on top and the size (or its complement) below, so
   // that whatever the scratch memory held before cannot pass for an
   // announcement.  Then it adds up the announcements of the chunks before it,
-  // waiting for those that are not there yet.  Workgroups start in the order of
-  // their numbers, so every chunk waited for is running or done, and none of
-  // them waits before it has announced; the wait is bounded all the same
+  // waiting for those that are not there yet.  Workgroups of one launch are
+  // observed to start in the order of their numbers, so a chunk waited for is
+  // normally running or done, and none of them waits before it has announced;
+  // nothing guarantees that order across the dies of the device or next to
+  // another kernel that fills the compute units, so the wait is bounded
   // (`spin_limit` looks per announcement): a chunk that gives up says so and
   // leaves its records where they are, for nz_compact_kernel.  Nothing but
   // the announcements passes between workgroups: relaxed device-scope

@@ -109,7 +109,9 @@ class FusedGemv:
         """Matrices that one launch decodes together are stored again with ONE
         geometry under which their chunks are a whole number of workgroups per
         compute unit (at most three, what a unit holds): chosen per tensor, two
-        512-chunk matrices are a round of 768 workgroups and a poorly filled second."""
+        512-chunk matrices are a round of 768 workgroups and a poorly filled second.
+        Only geometries inside the manager's size budget are considered; a group
+        too small to fill the device with those keeps what it has."""
         be = self.manager._be
         if cus is None:
             cus = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
@@ -119,7 +121,7 @@ class FusedGemv:
             lane = -(-sum(sizes) // (k * cus * 512 * 8)) * 8
             while lane <= 512 and sum(-(-n // (lane * 512)) for n in sizes) > k * cus:
                 lane += 8  # every tensor's last chunk is rounded up
-            if not 64 <= lane <= 512:
+            if not 64 <= lane <= 512 or not all(be.in_budget(n, lane * 512, lane) for n in sizes):
                 continue
             t = lane * self._STEP_NS[k - 1]
             if best is None or t <= best[0]:  # measured on gate/up of an 8B model: 2 x 512 chunks 73-76 us, 2 x 256 71.5, 2 x 378 69.4

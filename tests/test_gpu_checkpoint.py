@@ -27,8 +27,11 @@ def test_state_dict_round_trip(tmp_path, oracle, precision, lane):
     mgr.save(path)
     # what was exported is what the oracle writes for the same input
     sd = mgr.state_dict()
-    geom = {0: (131072, 256), 512: (131072, 512), 128: (65536, 128)}.get(lane)  # "auto" picks per tensor
-    if geom:
+    geom = {512: (131072, 512), 128: (65536, 128)}.get(lane)  # 0 and "auto" pick per tensor
+    if lane == 0:
+        assert mgr._be.geometry(hs[0]) == (172032, 336)  # 300000 elements: the shortest segments inside the size budget
+    if lane != "auto":
+        geom = geom or mgr._be.geometry(hs[0])
         o_comp, o_packed = oracle.compress_bf16(bits[0], precision, *geom)
         assert np.array_equal(sd["entries"][hs[0]]["container"].numpy(), o_comp)
         assert np.array_equal(sd["entries"][hs[0]]["packed"].numpy(), o_packed)

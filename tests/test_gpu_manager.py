@@ -6,7 +6,7 @@ from functools import partial
 import numpy as np
 import pytest
 
-from conftest import bf16_bits_normal, closed_form_recon, stress_bits
+from conftest import chunk_entropy_bytes, bf16_bits_normal, closed_form_recon, stress_bits
 
 pytestmark = pytest.mark.gpu
 
@@ -37,7 +37,8 @@ def test_write_read_size(oracle, precision):
         out = mgr.read(h)
         assert out.shape == torch.Size(shp) and out.dtype == torch.bfloat16 and not out.requires_grad
         assert np.array_equal(bits_of(out), oracle.reconstruct(bits_of(w), precision))
-        o_comp, o_packed = oracle.compress_bf16(bits_of(w), precision, 131072, 256)
+        assert mgr._be.geometry(h) == (_default_geometry(n) if n else (131072, 256))  # per tensor, inside the size budget
+        o_comp, o_packed = oracle.compress_bf16(bits_of(w), precision, *mgr._be.geometry(h))
         assert mgr.size(h) == o_comp.size + o_packed.size  # exponents + packed bytes held
         assert mgr._be.packed_bytes(h) == o_packed.size
     assert mgr.size("nope") == 0  # cuda/high_level.cu:209-211
@@ -448,48 +449,91 @@ def test_read_batch_equals_single_reads(oracle):
         assert all(int(o.view(torch.int16).abs().max()) == 0 for o in outs2)
 
 
-def _auto_geometry(n, cus=256):
+def _est_ratio(n, chunk, lane):
+    """nz_api.hip's estimate of a tensor's stored exponent bytes over their entropy"""
+    seg = 64 * lane
+    full, rest = divmod(n, chunk)
+    segs = full * -(-chunk // seg) + -(-rest // seg)
+    return 1.0008 + (134.4 * segs + 78.0 * (full + (rest > 0)) + 600.0) / n
+
+
+def _in_budget(n, chunk, lane, budget):
+    return _est_ratio(n, chunk, lane) + 0.0003 <= budget
+
+
+def _default_geometry(n, budget=1.01):
+    """eight segments per chunk, the shortest from 256 symbols per lane up inside
+    the budget; a tensor too small for any keeps 131072 / 256"""
+    for lane in range(256, 513, 8):
+        if _in_budget(n, 512 * lane, lane, budget):
+            return 512 * lane, lane
+    return 131072, 256
+
+
+def _auto_geometry(n, cus=256, budget=1.01):
     """The per-tensor rule of nz_manager_create(lane_syms = NZ_LANE_SYMS_AUTO) with
-    the library's own chunk: k = 1, 2 or 3 workgroups per compute unit, segments
-    of 64..512 symbols per lane, more workgroups only for a modelled gain above 10 %."""
-    if -(-n // 131072) > 3 * cus:
-        return 131072, 256
-    best = None
-    for k, step_ns in ((1, 107), (2, 147), (3, 215)):
+    the library's own chunk: the default geometry of the tensor, unless one of
+    k = 1, 2, 3 workgroups per compute unit (eight segments of 64..512 symbols
+    per lane) is inside the size budget and modelled 10 % faster; a tensor too
+    small for that gets 32 Ki chunks if the budget allows those."""
+    dchunk, dlane = _default_geometry(n, budget)
+    chunks = -(-n // dchunk)
+    if chunks > 3 * cus:
+        return dchunk, dlane
+    step = (107, 147, 215)
+    best_t, best = dlane * step[max(1, -(-chunks // cus)) - 1], None
+    for k in (1, 2, 3):
         lane = -(-(-(-n // (k * cus * 512))) // 8) * 8
-        if lane < 64 or lane > 512:
+        if lane < 64 or lane > 512 or not _in_budget(n, 512 * lane, lane, budget):
             continue
-        t = lane * step_ns
-        if best is None or 10 * t < 9 * best[0]:
-            best = (t, lane)
-    return (512 * best[1], best[1]) if best else (32768, 64)
+        t = lane * step[k - 1]
+        if 10 * t < 9 * best_t:
+            best_t, best = t, lane
+    if best:
+        return 512 * best, best
+    if n < 64 * cus * 512 and _in_budget(n, 32768, 64, budget):
+        return 32768, 64
+    return dchunk, dlane
 
 
 def test_auto_lane_symbols(oracle):
-    """Per-tensor geometry: a tensor that does not fill the device's 768
-    workgroup slots at the default geometry is cut into 256, 512 or 768 chunks
-    (the same number of workgroups on every compute unit) of eight segments, a
-    very small one into 32 Ki chunks; the stored bytes are those of the oracle
-    at that geometry, and reads are exact."""
+    """Per-tensor geometry inside the size budget: at the default budget every
+    tensor keeps the default geometry or gets longer segments, and what is
+    stored for the exponents of a tensor of a million elements or more stays
+    within 1.01 x their order-0 entropy; a caller who raises the budget gets
+    the shorter segments that let a small tensor fill the device.  The stored
+    bytes are those of the oracle at the chosen geometry, reads are exact."""
     import neuzip_amd
 
-    assert _auto_geometry(14336 * 4096) == (114688, 224) and _auto_geometry(4096 * 4096) == (32768, 64)
-    assert _auto_geometry(16384 * 4096) == (131072, 256) and _auto_geometry(110_000_000) == (131072, 256)
-    for chunk_arg, cases in (
-        (None, tuple((n,) + _auto_geometry(n) for n in (1000, 40_001, 1 << 20, 25_165_824, 40_000_000, 14336 * 4096,
-                                                        70_000_000, 110_000_000))),
-        (65536, ((1 << 20, 65536, 128), (40_000_000, 65536, 256), (70_000_000, 65536, 256))),
+    assert _default_geometry(14336 * 4096) == (131072, 256) and _default_geometry(4096 * 4096) == (131072, 256)
+    assert _default_geometry(4096 * 1024) == (135168, 264) and _default_geometry(1024 * 1024) == (143360, 280)
+    assert _default_geometry(40_001) == (131072, 256)  # too small for any geometry to reach the budget
+    assert _auto_geometry(14336 * 4096) == (131072, 256) and _auto_geometry(4096 * 4096) == (131072, 256)
+    assert _auto_geometry(14336 * 4096, budget=1.05) == (114688, 224)
+    assert _auto_geometry(4096 * 4096, budget=1.05) == (32768, 64)
+    assert _auto_geometry(16384 * 4096, budget=1.05) == (131072, 256)
+    sizes = (1000, 40_001, 1 << 20, 25_165_824, 40_000_000, 14336 * 4096, 70_000_000, 110_000_000)
+    for kwargs, cases in (
+        (dict(lane_symbols="auto"), tuple((n,) + _auto_geometry(n) for n in sizes)),
+        (dict(lane_symbols="auto", size_budget=1.05), tuple((n,) + _auto_geometry(n, budget=1.05) for n in sizes)),
+        (dict(chunk_size=65536, lane_symbols="auto"), ((1 << 20, 65536, 344), (40_000_000, 65536, 344))),
+        (dict(chunk_size=65536, lane_symbols="auto", size_budget=1.05),
+         ((1 << 20, 65536, 128), (40_000_000, 65536, 256), (70_000_000, 65536, 256))),
     ):
-        mgr = neuzip_amd.Manager(chunk_size=chunk_arg, lane_symbols="auto")
+        mgr = neuzip_amd.Manager(**kwargs)
         for n, chunk, lane in cases:
-            print(f"case auto chunk_arg={chunk_arg} n={n}", flush=True)
+            print(f"case auto {kwargs} n={n}", flush=True)
             w = from_bits(bf16_bits_normal(n, seed=n % 97), (n,))
             h = mgr.write(w)
+            assert mgr._be.geometry(h) == (chunk, lane)
             o_comp, o_packed = oracle.compress_bf16(bits_of(w), 7, chunk, lane, threads=8)
             assert mgr.size(h) == o_comp.size + o_packed.size
             assert torch.equal(mgr.read(h), w)
+            if n >= 1 << 20 and "size_budget" not in kwargs:
+                exps = ((bits_of(w) >> 7) & 0xFF).astype(np.uint8)
+                assert mgr.size(h) - n <= 1.01 * chunk_entropy_bytes(exps), (n, chunk, lane)
             del w
-    mgr._be.check()
+        mgr._be.check()
 
 
 def test_trim_releases_the_write_scratch():
@@ -559,7 +603,7 @@ def test_rewrite_in_place_needs_no_size_round_trip(oracle):
             mgr.write_many(ws, hs)
         for w, h in zip(ws, hs):
             assert torch.equal(mgr.read(h), w)
-            o_comp, o_packed = oracle.compress_bf16(bits_of(w), 7, 131072, 256)
+            o_comp, o_packed = oracle.compress_bf16(bits_of(w), 7, *mgr._be.geometry(h))
             assert mgr.size(h) == o_comp.size + o_packed.size
             comp, packed, _ = mgr._be.export(h)
             assert np.array_equal(comp.numpy(), o_comp) and np.array_equal(packed.numpy(), o_packed)
@@ -602,7 +646,7 @@ def test_records_are_placed_again_when_a_workgroup_gives_up_waiting(oracle):
     n = 40 * 131072 + 777                       # 41 chunks
     bits = bf16_bits_normal(n, seed=21)
     o_comp, o_packed = oracle.compress_bf16(bits, 7, 131072, 256)
-    mgr = neuzip_amd.Manager()
+    mgr = neuzip_amd.Manager(lane_symbols=256)
     w = from_bits(bits, (n,))
     h = mgr.write(w)                            # sized to fit: the two-kernel route
     try:

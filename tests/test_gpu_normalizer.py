@@ -74,7 +74,7 @@ def test_manager_with_normalizers(oracle, tmp_path, norm, precision):
     want = oracle.reconstruct_normalized(bits, precision, norm)
     assert np.array_equal(_bits(mgr.read(h)), want)
     o_norm, o_scaled = oracle.block_normalize(bits, norm)
-    o_comp, o_packed = oracle.compress_bf16(o_scaled, precision, 131072, 256)
+    o_comp, o_packed = oracle.compress_bf16(o_scaled, precision, *mgr._be.geometry(h))
     assert mgr.size(h) == o_comp.size + o_packed.size + o_norm.size  # cuda/high_level.cu:208-221
     # split: exponent and sign|mantissa bytes of the normalized tensor, precision 7 (high_level.cu:289)
     e, f = mgr.split(w)

@@ -223,16 +223,25 @@ def test_reference_package_name_is_importable():
 
 def test_group_geometry_choice_is_one_round_of_workgroups():
     """FusedGemv picks, for matrices that one launch decodes together, a geometry
-    under which their chunks are at most three per compute unit in total, and
-    stores them again only when that differs from what they have (host logic,
-    no GPU: a stand-in backend records the calls)."""
+    under which their chunks are at most three per compute unit in total and
+    the estimated stored size stays inside the manager's budget, and stores
+    them again only when that differs from what they have (host logic, no GPU:
+    a stand-in backend records the calls)."""
     from neuzip_amd.fused import FusedGemv, _Group
 
     class Be:
         auto_geometry = True
 
-        def __init__(self, sizes, geo):
-            self.sizes, self.geo, self.hints = sizes, dict(geo), {}
+        def __init__(self, sizes, geo, size_budget=1.01):
+            self.sizes, self.geo, self.hints, self.size_budget = sizes, dict(geo), {}, size_budget
+
+        def estimated_size_ratio(self, n, chunk, lane):
+            full, rest = divmod(n, chunk)
+            segs = full * -(-chunk // (64 * lane)) + -(-rest // (64 * lane))
+            return 1.0008 + (134.4 * segs + 78.0 * (full + (rest > 0)) + 600.0) / n
+
+        def in_budget(self, n, chunk, lane):
+            return self.estimated_size_ratio(n, chunk, lane) + 0.0003 <= self.size_budget
 
         def numel(self, h):
             return self.sizes[h]
@@ -260,10 +269,10 @@ def test_group_geometry_choice_is_one_round_of_workgroups():
         return g
 
     cus = 256
-    for sizes in ({"gate": 14336 * 4096, "up": 14336 * 4096},            # 8B-shaped gate / up
-                  {"q": 4096 * 4096, "k": 1024 * 4096, "v": 1024 * 4096},  # q / k / v
-                  {"a": 3_000_000, "b": 5_000_001}):
-        be = Be(sizes, {h: (131072, 256) for h in sizes})
+    for sizes, budget in (({"gate": 14336 * 4096, "up": 14336 * 4096}, 1.01),            # 8B-shaped gate / up
+                          ({"q": 4096 * 4096, "k": 1024 * 4096, "v": 1024 * 4096}, 1.05),  # q / k / v
+                          ({"a": 3_000_000, "b": 5_000_001}, 1.05)):
+        be = Be(sizes, {h: (131072, 256) for h in sizes}, budget)
         f = FusedGemv.__new__(FusedGemv)
         f.manager = Mgr(be)
         f._fit_geometry(group_of(list(sizes)), cus=cus)
@@ -271,6 +280,7 @@ def test_group_geometry_choice_is_one_round_of_workgroups():
         assert len(geos) == 1
         chunk, lane = geos.pop()
         assert chunk == 512 * lane and 64 <= lane <= 512 and lane % 8 == 0
+        assert all(be.in_budget(n, chunk, lane) for n in sizes.values())
         chunks = sum(-(-n // chunk) for n in sizes.values())
         assert chunks <= 3 * cus
         assert sorted(f.manager.written) == sorted(sizes)
@@ -282,3 +292,10 @@ def test_group_geometry_choice_is_one_round_of_workgroups():
     f.manager = Mgr(be)
     f._fit_geometry(group_of(["gate", "up"]), cus=cus)
     assert be.geo["gate"] == (304 * 512, 304)
+    # groups too small to fill the device inside the default budget keep what they have
+    for sizes in ({"q": 4096 * 4096, "k": 1024 * 4096, "v": 1024 * 4096}, {"a": 3_000_000, "b": 5_000_001}):
+        be = Be(sizes, {h: (131072, 256) for h in sizes})
+        f = FusedGemv.__new__(FusedGemv)
+        f.manager = Mgr(be)
+        f._fit_geometry(group_of(list(sizes)), cus=cus)
+        assert f.manager.written == [] and all(g == (131072, 256) for g in be.geo.values())
