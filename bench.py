@@ -18,7 +18,11 @@ Prints ONE JSON line:
   stress_8192x28672  BASELINE config 5 (448 MiB dense), precision 7 and 3
   sweep          decode/encode throughput and stored size for 7/3/1/0 kept bits
   cpu_baseline   the CPU oracle (same container format) timed on the host cores
-  llama8b_shape  tokens/s of the 8B-shaped decoder with compressed weights
+  llama8b_shape  tokens/s of the 8B-shaped decoder with compressed weights: the
+                 unchanged caller (import neuzip; Manager(precision=7).convert)
+                 first, the package's extensions beside it
+  gpt2m_shape    BASELINE config 4: 20 timed AdamW steps of a GPT-2-medium-shaped
+                 model with its weights kept compressed, against dense
 """
 from __future__ import annotations
 
@@ -155,6 +159,8 @@ def parse_args():
     ap.add_argument("--seq-len", type=int, default=1024)
     ap.add_argument("--verify-steps", type=int, default=10,
                     help="gpt2m: steps of the side-by-side dense / compressed weight comparison")
+    ap.add_argument("--no-gpt2m", action="store_true",
+                    help="skip the GPT-2-medium-shaped training block (BASELINE config 4) of the default line")
     ap.add_argument("--no-llama", action="store_true",
                     help="skip the 8B-shaped decoder that the default run appends to the codec line")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -241,12 +247,85 @@ def time_launches(torch, fn, steps, warmup):
     return wall, e0.elapsed_time(e1) * 1e-3 / steps
 
 
+def settled_launches(torch, fn, steps, warmup, settle_s):
+    """time_launches after `settle_s` seconds of the same launches, untimed: every
+    measured point of a run gets the settled clocks the headline gets.
+    -> wall seconds, event seconds per launch, untimed launches"""
+    n = 0
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < settle_s:
+        fn()
+        torch.cuda.synchronize()
+        n += 1
+    wall, per = time_launches(torch, fn, steps, warmup)
+    return wall, per, n + warmup
+
+
 def _timed(torch, fn):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     out = fn()
     torch.cuda.synchronize()
     return time.perf_counter() - t0, out
+
+
+def entropy_bound_bytes(torch, exps, chunk=65536):
+    """order-0 entropy of the exponent bytes `exps` (int32 on the device), per 64 Ki of them, in bytes"""
+    n = exps.numel()
+    nch = (n + chunk - 1) // chunk
+    idx = torch.arange(n, device=exps.device, dtype=torch.int64) // chunk
+    cnt = torch.bincount(idx * 256 + exps.to(torch.int64), minlength=256 * nch).view(nch, 256).double()
+    p = cnt / cnt.sum(1, keepdim=True).clamp_min(1.0)
+    h = -(torch.where(cnt > 0, cnt * torch.log2(p.clamp_min(1e-300)), torch.zeros_like(cnt))).sum()
+    return float(h) / 8.0
+
+
+def size_over_entropy(torch, mgr, precision, handles=None):
+    """Bytes stored for the exponents of every entry (all that is held, less what
+    the reference's packed sign|mantissa stream takes: the container keeps some
+    of those bytes in its coder states) over the order-0 entropy bound of the
+    stored exponents: over all entries together, and the largest single ratio
+    with the shape and geometry it belongs to."""
+    from neuzip_amd import _lib
+
+    L = _lib.load()
+    be = mgr._be
+    exp_total, bound_total, worst = 0, 0.0, None
+    geoms = {}
+    for h in (handles or list(mgr.meta_dict)):
+        w = mgr.read(h)
+        exps = (w.view(torch.int16).reshape(-1).to(torch.int32) >> 7) & 0xFF
+        bound = entropy_bound_bytes(torch, exps)
+        n = int(w.numel())
+        del w, exps
+        eb = mgr.size(h) - int(L.nz_packed_bytes(n, precision))
+        exp_total += eb
+        bound_total += bound
+        g = be.geometry(h)
+        geoms[g] = geoms.get(g, 0) + 1
+        if bound > 0 and (worst is None or eb / bound > worst[0]):
+            worst = (eb / bound, list(mgr.meta_dict[h]), list(g))
+    return {
+        "all_entries": round(exp_total / bound_total, 5) if bound_total else None,
+        "largest": None if worst is None else {"ratio": round(worst[0], 5), "shape": worst[1], "chunk_lane": worst[2]},
+        "size_budget": round(be.size_budget, 4),
+        "geometries_chunk_lane_count": sorted([list(g) + [c] for g, c in geoms.items()]),
+    }
+
+
+def make_manager(args, precision):
+    """The manager of a model workload: with no geometry flags it is built exactly
+    as a user of the reference builds it (``import neuzip;
+    neuzip.Manager(precision=...)``); flags go through the package's own class."""
+    if not args.chunk_size and args.lane_symbols in (-1, None):
+        import neuzip
+
+        return neuzip.Manager(precision=precision), "import neuzip; neuzip.Manager(precision=%d)" % precision
+    import neuzip_amd
+
+    lane = "auto" if args.lane_symbols < 0 else args.lane_symbols
+    return (neuzip_amd.Manager(precision=precision, chunk_size=args.chunk_size or None, lane_symbols=lane),
+            f"neuzip_amd.Manager(precision={precision}, chunk_size={args.chunk_size or None}, lane_symbols={lane!r})")
 
 
 def llama8b_measure(args, torch, full):
@@ -256,9 +335,11 @@ def llama8b_measure(args, torch, full):
     or as a replayed HIP graph; compressed weights are decoded per Linear (the
     reference's granularity), or per transformer block with one launch, with or
     without decoding the next block ahead on a side stream, or not at all as a
-    dense tensor (decode fused into the matrix-vector product).  `full` adds
-    the per-block modes; the lane setting -1 (auto) shortens the segments of
-    the smaller matrices."""
+    dense tensor (decode fused into the matrix-vector product).  The first
+    compressed mode is the unchanged caller: the model converted with
+    ``import neuzip; neuzip.Manager(precision=...).convert(model)`` and run as
+    it is (its single-token Linears go through the fused product one by one).
+    `full` adds the per-block modes."""
     import neuzip_amd
     from bench_models import LlamaShaped
 
@@ -340,13 +421,20 @@ def llama8b_measure(args, torch, full):
     measure("dense_graph", capture())
     dense_param_bytes = sum(p.numel() * p.element_size() for p in model.parameters())
 
-    mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size or None,
-                             lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
+    mgr, how = make_manager(args, args.precision)
     t_conv, _ = sync_time(lambda: mgr.convert(model))
     torch.cuda.empty_cache()
     comp_bytes = sum(mgr.size(h) for h in mgr.meta_dict)
     comp_dense_bytes = sum(2 * int(np.prod(shp)) for shp in mgr.meta_dict.values())
+    over_entropy = size_over_entropy(torch, mgr, args.precision)
+    torch.cuda.empty_cache()
 
+    # the unchanged caller: nothing but the reference's calls; Manager.linear itself sends a
+    # single activation row through the fused decode-and-multiply kernel
+    measure("unchanged_caller_eager")
+    measure("unchanged_caller_graph", capture())
+    # decompress-then-GEMM for every call, the reference's own route (bit-equal to dense)
+    mgr.fused_rows = False
     measure("per_linear_eager")
     measure("per_linear_graph", capture())
     for ahead in ((False, True) if full else ()):
@@ -360,8 +448,9 @@ def llama8b_measure(args, torch, full):
             measure(tag + "_graph", capture(finish=da.join))
         del da
         torch.cuda.empty_cache()
-    # decode fused into the matrix-vector product (single-token steps only; the
-    # prefill keeps the decompress-then-GEMM path)
+    # decode fused into the matrix-vector product, Linears that share an input in one launch
+    # (single-token steps only; the prefill keeps the decompress-then-GEMM path)
+    mgr.fused_rows = True
     fused = neuzip_amd.FusedGemv(mgr, model)
     with torch.no_grad():
         model.prefill_static(prompt, kcs, vcs)
@@ -373,9 +462,12 @@ def llama8b_measure(args, torch, full):
     mgr._be.check()
 
     modes = [k[:-9] for k in res if k.endswith("_decode_s")]
-    same = all(bool(torch.equal(toks["dense_eager"], toks[m])) for m in modes if not m.startswith("fused"))
+    rounds_its_own_way = ("fused", "unchanged_caller")  # the fused product sums in an order of its own
+    same = all(bool(torch.equal(toks["dense_eager"], toks[m])) for m in modes if not m.startswith(rounds_its_own_way))
     fused_same = bool(torch.equal(toks["fused_eager"], toks["fused_graph"]))
     fused_prefix = int((toks["fused_eager"] != toks["dense_eager"]).int().cumsum(1).eq(0).sum())
+    plain_same = bool(torch.equal(toks["unchanged_caller_eager"], toks["unchanged_caller_graph"]))
+    plain_prefix = int((toks["unchanged_caller_eager"] != toks["dense_eager"]).int().cumsum(1).eq(0).sum())
     comp_modes = [m for m in modes if not m.startswith("dense")]
     tok_s = {m: round((steps - 1) / res[m + "_decode_s"], 2) for m in modes}
     total = {m: res[m + "_prefill_s"] + res[m + "_decode_s"] for m in modes}
@@ -392,7 +484,18 @@ def llama8b_measure(args, torch, full):
         "config": {
             "workload": f"Llama-3-8B-shaped random-init decoder, {layers} layers, batch 1, {T}-token "
                         f"prompt + {steps} greedy steps, Linear weights compressed (precision {args.precision})",
+            "manager": how,
             "best_mode": best,
+            "unchanged_caller": {
+                "decode_tok_s_eager": tok_s["unchanged_caller_eager"],
+                "decode_tok_s_graph": tok_s["unchanged_caller_graph"],
+                "per_token_over_dense_eager": round(tok_s["dense_eager"] / tok_s["unchanged_caller_eager"], 3),
+                "per_token_over_dense_graph": round(tok_s["dense_graph"] / tok_s["unchanged_caller_graph"], 3),
+                "total_over_dense_eager": round(total["unchanged_caller_eager"] / total["dense_eager"], 3),
+                "total_over_dense_graph": round(total["unchanged_caller_graph"] / total["dense_graph"], 3),
+                "graph_tokens_equal_eager": plain_same,
+                "leading_tokens_equal_to_dense": plain_prefix,
+            },
             "tokens_identical_in_all_decompress_modes": same,
             "fused_graph_tokens_equal_fused_eager": fused_same,
             "fused_leading_tokens_equal_to_dense": fused_prefix,
@@ -410,6 +513,7 @@ def llama8b_measure(args, torch, full):
             "compressed_weight_bytes": comp_bytes,
             "dense_bytes_of_compressed_weights": comp_dense_bytes,
             "stored_over_dense": round(comp_bytes / comp_dense_bytes, 5),
+            "exponent_bytes_over_entropy_bound": over_entropy,
             "dense_model_bytes": dense_param_bytes,
         },
     }
@@ -424,6 +528,11 @@ def run_llama8b(args, torch):
 
 
 def run_gpt2m(args, torch):
+    print(json.dumps(gpt2m_measure(args, torch)))
+    return 0
+
+
+def gpt2m_measure(args, torch):
     """BASELINE config 4: GPT-2-medium-shaped model, weights kept compressed and
     re-compressed after every AdamW step; reports the codec share of the step."""
     import neuzip_amd
@@ -465,8 +574,7 @@ def run_gpt2m(args, torch):
     del state0
     torch.cuda.empty_cache()
 
-    mgr = neuzip_amd.Manager(precision=args.precision, chunk_size=args.chunk_size or None,
-                             lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
+    mgr, how = make_manager(args, args.precision)
     mgr.convert(model)
     comp_params = [p for p in model.parameters() if isinstance(p, neuzip_amd.nn.Parameter)]
     rest = [p for p in model.parameters() if not isinstance(p, neuzip_amd.nn.Parameter)]
@@ -539,6 +647,7 @@ def run_gpt2m(args, torch):
     n_comp = len(comp_params)
     stored_ratio = round(sum(mgr.size(p._handle) for p in comp_params) /
                          sum(2 * int(np.prod(p._shape)) for p in comp_params), 5)
+    over_entropy = size_over_entropy(torch, mgr, args.precision, [p._handle for p in comp_params])  # the weights as trained
     del mgr, model, comp_params, rest
     torch.cuda.empty_cache()
 
@@ -561,8 +670,7 @@ def run_gpt2m(args, torch):
                     torch.set_default_dtype(torch.float32)
 
         dense_twin, comp_twin = twin(), twin()
-        mgr2 = neuzip_amd.Manager(precision=7, chunk_size=args.chunk_size or None,
-                                  lane_symbols="auto" if args.lane_symbols < 0 else args.lane_symbols)
+        mgr2, _ = make_manager(args, 7)
         mgr2.convert(comp_twin)
         g = torch.Generator(device="cuda").manual_seed(args.seed + 2)
         with neuzip_amd.DecompressAhead(mgr2, comp_twin, ahead=False):
@@ -588,12 +696,12 @@ def run_gpt2m(args, torch):
             "lockstep_check_lossless": lockstep,
             "rewrites": rewrites,
             "compressed_tensors": n_comp,
-            "lane_symbols": "auto" if args.lane_symbols < 0 else (args.lane_symbols or "default"),
+            "manager": how,
             "stored_over_dense": stored_ratio,
+            "exponent_bytes_over_entropy_bound": over_entropy,
         },
     }
-    print(json.dumps(out))
-    return 0
+    return out
 
 
 def main():
@@ -772,13 +880,13 @@ def main():
         s_out = torch.empty_like(stress)
         cfg5 = {"workload": f"{STRESS_ROWS}x{STRESS_COLS} bf16, Student-t(3) x 0.02, 1 % zeros, 0.1 % subnormals, "
                             "16 outlier columns x 50"}
-        k5 = max(5, args.steps)
+        k5 = max(100, args.steps)
         for s in (7, 3):
             st = ws.encode(stress, s)
             ws.decode(st, s_out, check=True)
             ok = bool(torch.equal(s_out.view(torch.int16), closed_form_torch(torch, stress, s)))
-            _, m_d = time_launches(torch, lambda: ws.decode(st, s_out), k5, 3)
-            _, m_e = time_launches(torch, lambda: ws.encode_into(stress, s, st), k5, 2)
+            _, m_d, _ = settled_launches(torch, lambda: ws.decode(st, s_out), k5, 3, args.settle_s / 2)
+            _, m_e, _ = settled_launches(torch, lambda: ws.encode_into(stress, s, st), k5, 2, args.settle_s / 2)
             ab = st.total + st.packed_bytes + 2 * stress.numel()
             cfg5[f"precision_{s}"] = {
                 "bit_exact": ok,
@@ -792,10 +900,14 @@ def main():
         del stress, s_out
         torch.cuda.empty_cache()
 
-    # ---- encode throughput and the precision sweep (reported, not `value`); rotating like the headline ----
+    # ---- encode throughput and the precision sweep (reported, not `value`); rotating like the headline.
+    # Every point gets the headline's protocol: its own settle phase of the very launches it times
+    # (a point that starts right after allocations, host-synchronised encodes or another kernel
+    # otherwise runs its first launches at clocks that are still moving) and 100 launches or more
+    # between the two events; wall time over event time of the timed region is reported beside it.
     if not args.no_sweep:
         sweep = {}
-        k = max(5, args.steps // 2)
+        k = max(-(-100 // R), args.steps // 2)
         for s in (7, 3, 1, 0):
             ss = sets if s == args.precision else [ws.encode(d, s) for d in denses]
 
@@ -807,14 +919,20 @@ def main():
                 for d, st in zip(denses, ss):
                     ws.encode_into(d, s, st)
 
-            _, m_d = time_launches(torch, dec, k, 2)
-            _, m_e = time_launches(torch, enc, k, 2)
+            w_d, m_d, u_d = settled_launches(torch, dec, k, 2, args.settle_s / 2)
+            w_e, m_e, u_e = settled_launches(torch, enc, k, 2, args.settle_s / 2)
             ab = sum(st.total + st.packed_bytes + dense_bytes for st in ss) / R
             sweep[str(s)] = {
                 "decode_GBps": round(dense_bytes / (m_d / R) / 1e9, 1),
                 "decode_hbm_frac": round(ab / (m_d / R) / 1e9 / HBM_PEAK_GBPS, 4),
+                "decode_launch_us": round(m_d / R * 1e6, 2),
+                "decode_wall_over_event": round(w_d / (m_d * k), 3),
                 "encode_GBps": round(dense_bytes / (m_e / R) / 1e9, 1),
                 "encode_hbm_frac": round(ab / (m_e / R) / 1e9 / HBM_PEAK_GBPS, 4),
+                "encode_launch_us": round(m_e / R * 1e6, 2),
+                "encode_wall_over_event": round(w_e / (m_e * k), 3),
+                "launches_timed": k * R,
+                "untimed_launches_before": [u_d * R, u_e * R],
                 "stored_over_dense": round((ss[0].total + ss[0].packed_bytes) / dense_bytes, 5),
             }
             if ss is not sets:
@@ -850,10 +968,11 @@ def main():
             "matches_gpu_output": cpu_ok,
         }
 
+    del sets, denses, outs, ws
+    torch.cuda.empty_cache()
+
     # ---- the second half of the metric: tokens/s of an 8B-shaped compressed decoder ----
     if not args.no_llama:
-        del sets, denses, outs, ws
-        torch.cuda.empty_cache()
         import copy
 
         largs = copy.copy(args)
@@ -862,16 +981,50 @@ def main():
             lm = llama8b_measure(largs, torch, full=False)
             cfg = lm["config"]
             result["llama8b_shape"] = {
-                "workload": cfg["workload"] + ", lane symbols chosen per tensor",
+                "workload": cfg["workload"],
+                "manager": cfg["manager"],
+                "unchanged_caller": cfg["unchanged_caller"],
                 "decode_tok_s": cfg["decode_tok_s"],
                 "latency_ratio_eager": cfg["latency_ratio_eager"],
                 "latency_ratio_graph": cfg["latency_ratio_graph"],
                 "tokens_identical_in_all_decompress_modes": cfg["tokens_identical_in_all_decompress_modes"],
                 "fused_graph_tokens_equal_fused_eager": cfg["fused_graph_tokens_equal_fused_eager"],
                 "stored_over_dense": cfg["stored_over_dense"],
+                "exponent_bytes_over_entropy_bound": cfg["exponent_bytes_over_entropy_bound"],
             }
         except Exception as e:  # the codec line above stands on its own
             result["llama8b_shape"] = {"error": f"{type(e).__name__}: {e}"}
+        torch.cuda.empty_cache()
+
+    # ---- BASELINE config 4: a GPT-2-medium-shaped model trained with its weights kept compressed ----
+    if not args.no_gpt2m:
+        import copy
+
+        gargs = copy.copy(args)
+        gargs.precision, gargs.lane_symbols, gargs.chunk_size = 7, -1, 0
+        gargs.steps, gargs.warmup, gargs.verify_steps = 20, 3, 5
+        try:
+            gm = gpt2m_measure(gargs, torch)
+            cfg = gm["config"]
+            pb = cfg["decode_per_block"]
+            result["gpt2m_shape"] = {
+                "workload": cfg["workload"],
+                "manager": cfg["manager"],
+                "timed_steps": gargs.steps,
+                "tokens_per_s": gm["value"],
+                "ms_per_step_dense_bf16_adamw": cfg["dense_bf16_torch_adamw_ms_per_step"],
+                "ms_per_step_compressed_decode_per_block": pb["ms_per_step"],
+                "ms_per_step_compressed_decode_per_linear": cfg["decode_per_linear"]["ms_per_step"],
+                "codec_share_of_step_per_block": pb["codec_share_of_step"],
+                "codec_share_of_step_per_linear": cfg["decode_per_linear"]["codec_share_of_step"],
+                "steps_with_the_dense_runs_loss": pb["steps_with_the_dense_runs_loss"],
+                "rewrites": cfg["rewrites"],
+                "lockstep_check_lossless": cfg["lockstep_check_lossless"],
+                "stored_over_dense": cfg["stored_over_dense"],
+                "exponent_bytes_over_entropy_bound": cfg["exponent_bytes_over_entropy_bound"],
+            }
+        except Exception as e:
+            result["gpt2m_shape"] = {"error": f"{type(e).__name__}: {e}"}
 
     print(json.dumps(result))
     return 0

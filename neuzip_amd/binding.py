@@ -55,6 +55,12 @@ class _HipBackend:
         self._known = {}  # handle -> (encoded name, element count), dropped on write
         self._names1 = {}  # handle -> one-element ctypes array with its encoded name (fused product of one matrix)
         self.fused_rows = True  # serve single-row linear() calls with the fused decode-and-multiply kernel
+        self.group_rows = True  # ... and runs of them that share their activation with one launch
+        self._runs = {}         # first handle of a learned run -> (handles, names, rows, biases)
+        self._member_of = {}    # the other handles of learned runs -> their first handle
+        self._no_run = set()    # first handles whose run did not repeat itself
+        self._parked = {}       # handle -> (activation, its version, result, first handle, bias) computed ahead
+        self._cur = None        # the run being observed: (activation, its version, [(handle, rows, bias)])
 
     def close(self):
         if getattr(self, "_h", None) is not None and self._h:
@@ -82,6 +88,7 @@ class _HipBackend:
         if flat.data_ptr() % 16:
             flat = flat.clone()
         self._known.pop(handle, None)
+        self._parked.clear()  # products computed ahead from the weights as they were
         stream = torch.cuda.current_stream(flat.device)
         rc = self._L.nz_manager_write(self._h, handle.encode(), flat.data_ptr(), flat.numel(), code,
                                       stream.cuda_stream)
@@ -105,6 +112,7 @@ class _HipBackend:
             k = len(hs)
             for h in hs:
                 self._known.pop(h, None)
+            self._parked.clear()
             names = (ctypes.c_char_p * k)(*[h.encode() for h in hs])
             ptrs = (ctypes.c_void_p * k)(*[f.data_ptr() for f in fs])
             ns = (ctypes.c_uint64 * k)(*[f.numel() for f in fs])
@@ -276,26 +284,102 @@ class _HipBackend:
         prev = getattr(self, "_outside", None)
         self._outside = flag if prev is None else prev | flag
 
+    # -- single activation rows: decode fused into the product ------------------
+    #
+    # Linears that are called back to back with the very same activation (q/k/v,
+    # gate/up) are served by ONE launch, without the caller saying so: the first
+    # time such a run of calls is seen it is executed call by call and remembered
+    # under its first handle; from then on a call of that handle computes the
+    # whole run and parks the other results, which the calls that follow pick up
+    # if - and only if - they come with the same tensor object, unmodified, and
+    # the same bias.  A run that does not repeat itself is forgotten for good.
+
+    _MAX_RUN = 8
+
+    def _fused_ok(self, inputs: torch.Tensor, shape, bias) -> bool:
+        if (not self.fused_rows or inputs.dim() == 0 or inputs.numel() != inputs.shape[-1] or len(shape) != 2
+                or inputs.shape[-1] != shape[1] or shape[1] % 512 or inputs.dtype != torch.bfloat16
+                or not inputs.is_cuda or (torch.is_grad_enabled() and inputs.requires_grad)):
+            return False
+        if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_cuda or bias.numel() != shape[0]
+                                 or not bias.is_contiguous() or (torch.is_grad_enabled() and bias.requires_grad)):
+            return False
+        return True
+
+    def _forget_run(self, leader: str) -> None:
+        self._runs.pop(leader, None)
+        self._no_run.add(leader)
+        for h in [h for h, first in self._member_of.items() if first == leader]:
+            del self._member_of[h]
+        for h in [h for h, hit in self._parked.items() if hit[3] == leader]:
+            del self._parked[h]
+
+    def _observe(self, handle: str, inputs: torch.Tensor, rows: int, bias) -> None:
+        """one more call that was served on its own: does it continue the current run?"""
+        cur = self._cur
+        if (cur is not None and cur[0] is inputs and cur[1] == inputs._version and len(cur[2]) < self._MAX_RUN
+                and all(h != handle for h, _, _ in cur[2])):
+            cur[2].append((handle, rows, bias))
+            return
+        self._close_run()
+        self._cur = (inputs, inputs._version, [(handle, rows, bias)])
+
+    def _close_run(self) -> None:
+        cur, self._cur = self._cur, None
+        if cur is None or len(cur[2]) < 2:
+            return
+        leader = cur[2][0][0]
+        if leader in self._no_run or any(h in self._runs or h in self._member_of for h, _, _ in cur[2]):
+            return
+        handles = [h for h, _, _ in cur[2]]
+        self._runs[leader] = (handles, (ctypes.c_char_p * len(handles))(*[h.encode() for h in handles]),
+                              [r for _, r, _ in cur[2]], [b for _, _, b in cur[2]])
+        for h in handles[1:]:
+            self._member_of[h] = leader
+
     def _fused_row(self, handle: str, inputs: torch.Tensor, shape, bias):
         """``x @ W^T (+ b)`` for ONE activation row without writing the dense weight:
         the product is formed while the weight is decoded (nz_manager_gemv_batch).
         -> None when the call does not qualify (several rows, a row length that is
         not a multiple of 512, another dtype, a bias the kernel cannot take)."""
-        if (not self.fused_rows or inputs.dim() == 0 or inputs.numel() != inputs.shape[-1] or len(shape) != 2
-                or inputs.shape[-1] != shape[1] or shape[1] % 512 or inputs.dtype != torch.bfloat16
-                or not inputs.is_cuda or (torch.is_grad_enabled() and inputs.requires_grad)):
+        if not self._fused_ok(inputs, shape, bias):
             return None
-        if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_cuda or bias.numel() != shape[0]
-                                 or not bias.is_contiguous() or (torch.is_grad_enabled() and bias.requires_grad)):
-            return None
+        parked = self._parked.pop(handle, None)
+        if parked is not None:
+            x0, version, out, leader, b0 = parked
+            if x0 is inputs and version == inputs._version and b0 is bias:
+                return out.view(*inputs.shape[:-1], shape[0])
+            self._forget_run(leader)  # the run did not repeat itself
         x = inputs if inputs.is_contiguous() else inputs.contiguous()
         if x.data_ptr() % 16:
             x = x.clone()
+        run = self._runs.get(handle) if self.group_rows else None
+        if run is not None:
+            handles, names, rows, biases = run
+            if biases[0] is bias:
+                self._close_run()
+                flat = torch.empty(sum(rows), dtype=torch.bfloat16, device=x.device)
+                outs, at = [], 0
+                for r in rows:
+                    outs.append(flat[at:at + r])
+                    at += r
+                try:
+                    self.gemv_batch(names, x, biases, outs)
+                except (ValueError, RuntimeError):
+                    self._forget_run(handle)  # e.g. scratch that cannot grow while a graph is captured
+                else:
+                    for h, o, b in zip(handles[1:], outs[1:], biases[1:]):
+                        self._parked[h] = (inputs, inputs._version, o, handle, b)
+                    return outs[0].view(*inputs.shape[:-1], shape[0])
+            else:
+                self._forget_run(handle)
         names = self._names1.get(handle)
         if names is None:
             names = self._names1[handle] = (ctypes.c_char_p * 1)(handle.encode())
         out = torch.empty(shape[0], dtype=torch.bfloat16, device=x.device)
         self.gemv_batch(names, x, [bias], [out])
+        if self.group_rows and handle not in self._member_of:
+            self._observe(handle, inputs, shape[0], bias)
         return out.view(*inputs.shape[:-1], shape[0])
 
     def linear(self, handle: str, inputs: torch.Tensor, shape, bias: torch.Tensor) -> torch.Tensor:
@@ -474,7 +558,11 @@ class Manager:
         is multiplied while the weight is decoded, without the dense weight ever
         being written; its sums are formed in an order of their own, so the
         result agrees with the decompress-then-GEMM path to rounding, not bit for
-        bit (``manager.fused_rows = False`` keeps every call on that path)."""
+        bit (``manager.fused_rows = False`` keeps every call on that path).
+        Such calls that come back to back with the same activation tensor (q/k/v,
+        gate/up) are recognised when they first occur and share one launch from
+        then on (``manager.group_rows = False`` turns that off); the numbers are
+        those of the single launches."""
         shape = self.meta_dict[handle]
         if bias is None:
             return self._be.linear_without_bias(handle, inputs, shape)
@@ -488,6 +576,17 @@ class Manager:
     def fused_rows(self, on: bool) -> None:
         if hasattr(self._be, "fused_rows"):
             self._be.fused_rows = bool(on)
+
+    @property
+    def group_rows(self) -> bool:
+        """Whether single-row calls that arrive back to back with the very same
+        activation (q/k/v, gate/up) are learned and served by one launch."""
+        return bool(getattr(self._be, "group_rows", False))
+
+    @group_rows.setter
+    def group_rows(self, on: bool) -> None:
+        if hasattr(self._be, "group_rows"):
+            self._be.group_rows = bool(on)
 
     def gather_rows(self, handle: str, indices: torch.Tensor) -> torch.Tensor:
         """Rows ``indices`` of the stored 2-D table ``handle`` as ``[indices.numel(), row_len]``

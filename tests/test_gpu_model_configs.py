@@ -142,6 +142,13 @@ def test_llama_shaped_decoder_all_modes(oracle):
         assert rel < 0.02, rel
     for a, b in zip(plain, plain_graph):
         assert torch.equal(a, b)
+    # q/k/v and gate/up were recognised as runs that share their activation: one launch each
+    runs = sorted(len(r[0]) for r in mgr._be._runs.values())
+    assert runs == [2, 2, 3, 3], runs
+    mgr.group_rows = False  # every Linear a launch of its own: the same numbers
+    for a, b in zip(plain, run()):
+        assert torch.equal(a, b)
+    mgr.group_rows = True
 
     mgr.fused_rows = False  # every call by decompress-then-GEMM: the dense model's logits exactly
     print("case llama per_linear eager", flush=True)
