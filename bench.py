@@ -163,6 +163,10 @@ def parse_args():
                     help="skip the GPT-2-medium-shaped training block (BASELINE config 4) of the default line")
     ap.add_argument("--no-llama", action="store_true",
                     help="skip the 8B-shaped decoder that the default run appends to the codec line")
+    ap.add_argument("--encode-phases", action="store_true",
+                    help="only print the encode kernel's time per phase (library built with -DNZ_PROBE_PHASES)")
+    ap.add_argument("--protocol-probe", action="store_true",
+                    help="only compare the timing protocols of a sweep point (see protocol_probe)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run five plain 256 MiB device copies (to scale FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
@@ -259,6 +263,93 @@ def settled_launches(torch, fn, steps, warmup, settle_s):
         n += 1
     wall, per = time_launches(torch, fn, steps, warmup)
     return wall, per, n + warmup
+
+
+def protocol_probe(args, torch, L, lib_mod):
+    """Why a sweep point needs the headline's protocol.  For every precision,
+    three times over: five weights encoded into fresh buffers (host-synchronised,
+    as the sweep does), then their decode timed (a) the way the sweep used to -
+    two warm-up steps, ten steps between the events - (b) the same after 0.2 s
+    without work, (c) settled, twenty steps.  One JSON line per measurement;
+    (a) once more per precision with an event after every step."""
+    n, R = args.rows * args.cols, max(1, args.rotate)
+    ws = Workspace(torch, L, lib_mod, n, lib_mod.DEFAULT_CHUNK, lib_mod.DEFAULT_LANE_SYMS)
+    denses = [normal_weight(torch, args.rows, args.cols, args.seed + i) for i in range(R)]
+    outs = [torch.empty_like(d) for d in denses]
+
+    def point(s, k, settle_s, idle_s, per_step=False):
+        ss = [ws.encode(d, s) for d in denses]
+
+        def dec():
+            for st, o in zip(ss, outs):
+                ws.decode(st, o)
+
+        torch.cuda.synchronize()
+        if idle_s:
+            time.sleep(idle_s)
+        if per_step:
+            evs = [torch.cuda.Event(enable_timing=True) for _ in range(k + 1)]
+            for _ in range(2):
+                dec()
+            evs[0].record()
+            for i in range(k):
+                dec()
+                evs[i + 1].record()
+            torch.cuda.synchronize()
+            print(json.dumps({"precision": s, "protocol": "two warm-up steps, an event after every step",
+                              "launch_us_per_step": [round(evs[i].elapsed_time(evs[i + 1]) * 1e3 / R, 1)
+                                                     for i in range(k)]}), flush=True)
+            return
+        if settle_s:
+            w, m, _ = settled_launches(torch, dec, k, 2, settle_s)
+        else:
+            w, m = time_launches(torch, dec, k, 2)
+        print(json.dumps({"precision": s, "steps": k, "settle_s": settle_s, "idle_s_before": idle_s,
+                          "launch_us": round(m / R * 1e6, 2), "decode_GBps": round(2 * n / (m / R) / 1e9, 1),
+                          "wall_over_event": round(w / (m * k), 3)}), flush=True)
+
+    for _ in range(3):
+        for s in (7, 3, 1, 0):
+            point(s, 10, 0, 0)
+            point(s, 10, 0, 0.2)
+            point(s, 20, args.settle_s / 2, 0)
+    for s in (7, 3, 1, 0):
+        point(s, 10, 0, 0, per_step=True)
+    return 0
+
+
+def encode_phases(args, torch, L, lib_mod):
+    """Where the time of nz_encode_kernel goes, phase by phase.  Needs a library
+    built with NZ_HIPCC_EXTRA=-DNZ_PROBE_PHASES (thread 0 of every workgroup then
+    adds the shader-clock cycles between the phase boundaries to six counters)."""
+    if not hasattr(L, "nz_probe_read") or args.precision != 7:
+        print("needs a library built with -DNZ_PROBE_PHASES, and precision 7 (the counters sit in that "
+              "precision's translation unit)", file=sys.stderr)
+        return 2
+    L.nz_probe_read.argtypes = [ctypes.POINTER(ctypes.c_ulonglong), ctypes.c_int]
+    n = args.rows * args.cols
+    chunk, lane = args.chunk_size or lib_mod.DEFAULT_CHUNK, args.lane_symbols or lib_mod.DEFAULT_LANE_SYMS
+    ws = Workspace(torch, L, lib_mod, n, chunk, lane)
+    dense = normal_weight(torch, args.rows, args.cols, args.seed)
+    st = ws.encode(dense, args.precision)
+    for _ in range(50):
+        ws.encode_into(dense, args.precision, st)
+    torch.cuda.synchronize()
+    acc = (ctypes.c_ulonglong * 8)()
+    L.nz_probe_read(acc, 1)
+    k = max(100, args.steps)
+    _, per = time_launches(torch, lambda: ws.encode_into(dense, args.precision, st), k, 0)
+    L.nz_probe_read(acc, 0)
+    names = ("split + histogram", "table", "coding", "finalize + announce", "wait for the chunks before", "record move")
+    groups = k * (-(-n // chunk))
+    total = float(sum(acc[i] for i in range(6)))
+    print(json.dumps({
+        "kernel": f"nz_encode_kernel<{args.precision}, *>", "rows": args.rows, "cols": args.cols, "chunk_size": chunk,
+        "lane_symbols": lane, "launches": k, "launch_us": round(per * 1e6, 2),
+        "cycles_per_workgroup": {nm: round(acc[i] / groups) for i, nm in enumerate(names)},
+        "share": {nm: round(acc[i] / total, 4) for i, nm in enumerate(names)},
+    }))
+    return 0
 
 
 def _timed(torch, fn):
@@ -733,6 +824,10 @@ def main():
                           "bytes_written_per_copy": 256 << 20}))
         return 0
 
+    if args.protocol_probe:
+        return protocol_probe(args, torch, L, lib_mod)
+    if args.encode_phases:
+        return encode_phases(args, torch, L, lib_mod)
     if args.workload == "llama8b":
         return run_llama8b(args, torch)
     if args.workload == "gpt2m":

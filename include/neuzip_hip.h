@@ -118,7 +118,11 @@ int nz_split(const void* dev_bf16, uint64_t n, void* dev_exponents, void* dev_fr
    workspace keeps a count of the runs that have used it.  If `host_total` is not
    NULL the call synchronises the stream, returns the size and status on the
    host (the reference's get_compressed_output_size sync, :114-115) and deals
-   with bit 2 itself. */
+   with bit 2 itself.  With host_total NULL (and in nz_encode_static, and in
+   every replay of a captured call) nobody does: the caller has to look at
+   *dev_status before the container is used, and encode again when bit 2 is
+   set.  dev_bf16 is read until the stream has passed the call: it must stay
+   valid and unmodified until then. */
 int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
               uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
               void* dev_workspace, uint64_t workspace_bytes, uint64_t* dev_total,
@@ -136,7 +140,10 @@ int nz_encode(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_si
    NZ_STATIC_SCRATCH_BYTES is refused with NZ_ERR_CAPACITY (at the default
    geometry: more than about 5.5 million elements).  All calls on one GPU share
    that GPU's array: calls that overlap in time on one GPU (two streams, two
-   threads) race; order them on one stream or with events. */
+   threads) race; order them on one stream or with events.  *dev_status has to
+   be checked before the container is used: bit 0 (it did not fit) and bit 2 (a
+   workgroup gave up waiting, see nz_set_lookback_spins) both leave it
+   incomplete, and this call cannot repair either. */
 #define NZ_STATIC_SCRATCH_BYTES (16u << 20)
 int nz_encode_static(const void* dev_bf16, uint64_t n, int precision, uint32_t chunk_size,
                      uint32_t lane_syms, void* dev_packed, void* dev_comp, uint64_t comp_cap,
@@ -146,12 +153,19 @@ int nz_encode_static(const void* dev_bf16, uint64_t n, int precision, uint32_t c
 /* No counterpart in the reference.  The encode kernel of the calls above (and
    of the manager's writes into existing buffers) places its records itself:
    every workgroup waits until the workgroups of the chunks before its own have
-   announced their record sizes.  The wait is bounded: after `spins` looks at an
-   announcement (about a microsecond each; default 2^21) a workgroup gives up,
-   and the records are placed by a second kernel once the host has seen that
-   (at once in nz_encode with host_total; when the entry is used next in a
-   manager).  For tests and tuning; 0 makes every workgroup give up whose
-   predecessors are not done at its first look. */
+   announced their record sizes.  That the workgroups of a launch start in the
+   order of their numbers, so that everything waited for is running or done,
+   is what has been observed on this device, not something the hardware
+   promises: the eight dies dispatch independently, and two encode launches
+   that are resident at once (two managers on two streams) can each hold
+   compute units while waiting for a predecessor that has not been given one.
+   So the wait is bounded: after `spins` looks at an announcement (about a
+   microsecond each; default 2^15, some tens of milliseconds - a launch takes
+   ~0.1 ms) a workgroup gives up, and the records are placed by a second kernel
+   once the host has seen that (at once in nz_encode with host_total; when the
+   entry is used next in a manager): a wait that was cut short costs one
+   compaction launch, never a wrong container.  For tests and tuning; 0 makes
+   every workgroup give up whose predecessors are not done at its first look. */
 void nz_set_lookback_spins(uint32_t spins);
 
 /* Manager::_decompress_and_merge, cuda/high_level.cu:169-206: entropy decode
@@ -224,7 +238,23 @@ int nz_manager_in_budget(const nz_manager* m, uint64_t n, uint32_t chunk_size, u
    existing entry of the same name (:137-140).  Synchronises the stream once
    to learn the compressed size (as the reference does, :114-115), unless the
    handle already holds a tensor of the same element count (see
-   nz_manager_rewrite_stats). */
+   nz_manager_rewrite_stats): such a write goes into the entry's buffers and
+   returns while the encode kernel is still reading dev_data.  Since a caller
+   cannot tell the two cases apart beforehand: dev_data must stay valid and
+   unmodified until `stream` has passed the write (free or overwrite it in
+   stream order, or after an event / synchronisation; memory from a
+   stream-ordered allocator that belongs to another stream has to be told, as
+   torch's record_stream does).
+   Streams and graphs: writes, products and row gathers of one manager share
+   its scratch memory; a call that arrives on another stream than the one
+   before it is ordered behind that one on the device (an event, no host
+   wait).  A call that may allocate or wait on the host - every write, a read
+   or product of an entry whose in-place rewrite has not been looked at yet, a
+   product that needs larger accumulators, a row gather - is refused with
+   NZ_ERR_ARG while its stream is being captured into a graph, before it
+   touches anything (the capture stays valid); reads and products of settled
+   entries are captured and replay.  Calls on one manager from several host
+   threads are serialised by the manager. */
 int nz_manager_write(nz_manager* m, const char* name, const void* dev_data, uint64_t n,
                      int dtype, void* stream);
 

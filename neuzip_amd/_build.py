@@ -7,6 +7,7 @@ precisions share); they compile side by side and are linked into one library.
 from __future__ import annotations
 
 import os
+import shlex
 import subprocess
 import tempfile
 from concurrent.futures import ThreadPoolExecutor
@@ -66,7 +67,9 @@ def build(verbose: bool = False) -> str:
 
         def compile_one(tu):
             src, extra, obj = tu
-            run([hipcc, *HIPCC_FLAGS, *extra, "-c", src, "-o", obj], verbose)
+            # NZ_HIPCC_EXTRA: more flags for a measurement build (e.g. -DNZ_PROBE_EXTRA_SLOTS)
+            more = shlex.split(os.environ.get("NZ_HIPCC_EXTRA", ""))
+            run([hipcc, *HIPCC_FLAGS, *extra, *more, "-c", src, "-o", obj], verbose)
             return obj
 
         with ThreadPoolExecutor(max_workers=len(tus)) as pool:

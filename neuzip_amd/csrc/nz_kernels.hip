@@ -19,7 +19,9 @@
 
 #include "nz_format.h"
 
+#ifndef NZ_HIST_COPIES
 #define NZ_HIST_COPIES 8u
+#endif
 #define NZ_HIST_STRIDE 257u
 #define NZ_RING_WORDS 1024u  // per-wave LDS ring of renormalisation words
 #define NZ_RING_DWORDS (NZ_RING_WORDS / 2)
@@ -855,9 +857,26 @@ __device__ __forceinline__ bool nz_move_record(const NzEncItem& it, const uint64
 // Segments of up to 8 * NG symbols per lane: the exponents stay in registers.
 // Workgroup = max(4, segments per chunk) wavefronts; wavefront k owns segment k.
 extern __shared__ uint32_t nz_enc_stage[];  // word staging of nz_encode_kernel: stage_words / 2 dwords per wavefront + 4
+#ifdef NZ_PROBE_PHASES
+__device__ unsigned long long nz_probe_acc[8];
+#define NZ_PROBE_MARK(k)                                        \
+  do {                                                          \
+    if (threadIdx.x == 0) {                                     \
+      const unsigned long long now = __builtin_readcyclecounter(); \
+      atomicAdd(&nz_probe_acc[k], now - probe_t);               \
+      probe_t = now;                                            \
+    }                                                           \
+  } while (0)
+#else
+#define NZ_PROBE_MARK(k)
+#endif
+
 template <int S, int NG>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kernel(const NzEncBatch b) {
   __shared__ NzEncLds L;
+#ifdef NZ_PROBE_PHASES
+  unsigned long long probe_t = __builtin_readcyclecounter();
+#endif
   uint32_t t = 0, first = 0;
   while (t + 1 < b.count && blockIdx.x >= b.item[t].chunk_end) {
     first = b.item[t].chunk_end;
@@ -983,9 +1002,11 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   });
   __threadfence_block();  // the carried bytes are read back below
   __syncthreads();
+  NZ_PROBE_MARK(0);
 
   // ---- the chunk's table ----
   const uint32_t est_bits = nz_build_table(L, cn, it.ws + it.tab_ser + c * NZ_TABLE_MAX_BYTES, info + c);
+  NZ_PROBE_MARK(1);
 
   // ---- phase 2: code the segment from the registers, last group first ----
   // The words go to the segment's slot in scratch memory, or, when the records
@@ -1053,6 +1074,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     if (!(staged && L.redo)) break;
     staged = false;
   }
+  NZ_PROBE_MARK(2);
   // decide coded-or-raw and size the records
   if (tid == 0) {
     L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
@@ -1112,6 +1134,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     __hip_atomic_store(pub + 2 * c + 1, ((nz_u64)mark_b << 32) | (uint32_t)~u, __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
   }
+  NZ_PROBE_MARK(3);
   uint64_t part = 0;
   bool lost = false;
   for (uint64_t i = tid; i < c && !lost; i += blockDim.x) {
@@ -1135,6 +1158,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   if (lane == 0) L.red64[wave] = part;
   __threadfence_block();  // also: the raw bytes above are read back by the move
   __syncthreads();
+  NZ_PROBE_MARK(4);
   // staged words of this wavefront to their slot, for the kernel that places records afterwards
   const auto unstage = [&]() {
     const uint16_t* sw = reinterpret_cast<const uint16_t*>(stage);
@@ -1168,6 +1192,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     if (from_stage && !fits) unstage();
     if (lane == 0) placed[seg] = (from_stage && fits) ? 1 : 0;
   }
+  NZ_PROBE_MARK(5);
 }
 
 // Longer segments: all wavefronts split the chunk into scratch, then one

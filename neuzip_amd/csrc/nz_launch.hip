@@ -94,3 +94,15 @@ template void nz_launch_decode_batch<NZ_S>(const NzBatch&, uint32_t, uint32_t, b
 template void nz_launch_gemv<NZ_S>(const NzBatch&, uint32_t, uint32_t, uint32_t*, hipStream_t);
 template void nz_launch_rows<NZ_S>(const NzGeom&, const void*, uint64_t, const void*, uint16_t*, uint32_t*,
                                    const NzNorm&, const long long*, uint32_t, uint32_t, uint32_t, hipStream_t);
+
+#if defined(NZ_PROBE_PHASES) && NZ_S == 7
+// measurement build only: cycles spent per phase of nz_encode_kernel<7, *>, summed over workgroups
+extern "C" int nz_probe_read(unsigned long long* out, int reset) {
+  if (hipMemcpyFromSymbol(out, HIP_SYMBOL(nz_probe_acc), sizeof(unsigned long long) * 8) != hipSuccess) return 1;
+  if (reset) {
+    unsigned long long z[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (hipMemcpyToSymbol(HIP_SYMBOL(nz_probe_acc), z, sizeof(z)) != hipSuccess) return 1;
+  }
+  return 0;
+}
+#endif
