@@ -137,6 +137,9 @@ def parse_args():
                     help="elements per frequency table; 0 = library default (131072), 65536 = the reference's nvcomp chunk")
     ap.add_argument("--lane-symbols", type=int, default=None,
                     help="0 = library default; -1 = chosen per tensor (the default of the model workloads)")
+    ap.add_argument("--size-budget", type=float, default=0.0,
+                    help="model workloads: stored exponent bytes over their entropy that the per-tensor geometry "
+                         "may spend (default: the library's 1.01; e.g. 1.04 buys wavefronts for small matrices)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--rotate", type=int, default=5,
                     help="independent stored copies of the workload a step decodes one after the other "
@@ -408,15 +411,17 @@ def make_manager(args, precision):
     """The manager of a model workload: with no geometry flags it is built exactly
     as a user of the reference builds it (``import neuzip;
     neuzip.Manager(precision=...)``); flags go through the package's own class."""
-    if not args.chunk_size and args.lane_symbols in (-1, None):
+    if not args.chunk_size and args.lane_symbols in (-1, None) and not args.size_budget:
         import neuzip
 
         return neuzip.Manager(precision=precision), "import neuzip; neuzip.Manager(precision=%d)" % precision
     import neuzip_amd
 
-    lane = "auto" if args.lane_symbols < 0 else args.lane_symbols
-    return (neuzip_amd.Manager(precision=precision, chunk_size=args.chunk_size or None, lane_symbols=lane),
-            f"neuzip_amd.Manager(precision={precision}, chunk_size={args.chunk_size or None}, lane_symbols={lane!r})")
+    lane = "auto" if args.lane_symbols in (-1, None) else args.lane_symbols
+    return (neuzip_amd.Manager(precision=precision, chunk_size=args.chunk_size or None, lane_symbols=lane,
+                               size_budget=args.size_budget or None),
+            f"neuzip_amd.Manager(precision={precision}, chunk_size={args.chunk_size or None}, lane_symbols={lane!r}, "
+            f"size_budget={args.size_budget or None})")
 
 
 def llama8b_measure(args, torch, full):

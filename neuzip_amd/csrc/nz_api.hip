@@ -155,7 +155,7 @@ bool enc_batch_close(NzEncBatch* b) {
 }
 
 // One encode launch for the tensors of `b` whose segments are of class `cls`
-// (0..2: up to 64 / 128 / 256 symbols per lane, coded from registers; 3: longer).
+// (0..3: up to 64 / 128 / 256 / 288 symbols per lane, coded from registers; 4: longer).
 // The register encode kernels may use more than 64 KiB of LDS per workgroup
 // (word staging): that has to be allowed once per kernel and device, and is
 // done for all of them before the first encode on a device.
@@ -176,10 +176,10 @@ int allow_encode_lds() {
 // Words of LDS staging per wavefront for a direct encode of class `cls` with
 // workgroups of `waves` wavefronts: what a workgroup can have without lowering
 // the number of workgroups that the registers allow per compute unit (4, 6, 8
-// wavefronts per SIMD unit for 256, 128, 64 symbols per lane), less the
+// wavefronts per SIMD unit for 256 and more, 128, 64 symbols per lane), less the
 // kernel's own LDS.
 uint32_t stage_words_for(int cls, uint32_t waves) {
-  const uint32_t waves_per_cu = cls == 2 ? 16u : cls == 1 ? 24u : 32u;
+  const uint32_t waves_per_cu = cls >= 2 ? 16u : cls == 1 ? 24u : 32u;
   const uint32_t groups = waves_per_cu / waves ? waves_per_cu / waves : 1u;
   const uint32_t per_group = 160u * 1024u / groups;
   const uint32_t fixed = ((uint32_t)sizeof(NzEncLds) + 511u) & ~511u;  // the kernel's own LDS
@@ -194,14 +194,14 @@ int launch_encode_class(NzEncBatch& b, int cls, uint32_t chunks, uint32_t max_sp
   const dim3 grid(chunks), block(64 * waves);
   bool direct = false;
   for (uint32_t i = 0; i < b.count; ++i) direct = direct || b.item[i].direct;
-  b.stage_words = (direct && cls < 3) ? stage_words_for(cls, waves) : 0u;
+  b.stage_words = (direct && cls < 4) ? stage_words_for(cls, waves) : 0u;
   const uint32_t lds = b.stage_words ? waves * b.stage_words * 2u + 16u : 0u;
   nz_launch_encode<S>(b, cls, grid, block, lds, st);
   return NZ_OK;
 }
 
 int enc_class(const NzGeom& g) {
-  return g.lane_syms <= 64 ? 0 : g.lane_syms <= 128 ? 1 : g.lane_syms <= NZ_ENC_MAX_LANE_SYMS ? 2 : 3;
+  return g.lane_syms <= 64 ? 0 : g.lane_syms <= 128 ? 1 : g.lane_syms <= 256 ? 2 : g.lane_syms <= NZ_ENC_MAX_LANE_SYMS ? 3 : 4;
 }
 
 // Phase 1 for all tensors of the batch: everything up to the directory.  Header
@@ -213,7 +213,7 @@ int encode_phase1(NzEncBatch* b, int precision, uint32_t ns, hipStream_t st) {
     if (int rc = launch_absmax(b->item[i].in, b->item[i].g.n, ns, const_cast<uint8_t*>(b->item[i].nm.bytes), st))
       return rc;
   // the tensors of the batch, by segment-length class: one launch per class in use
-  for (int cls = 0; cls < 4; ++cls) {
+  for (int cls = 0; cls < 5; ++cls) {
     NzEncBatch sub{};
     uint32_t chunks = 0, max_spc = 1;
     for (uint32_t i = 0; i < b->count; ++i) {

@@ -299,7 +299,7 @@ __global__ __launch_bounds__(256) void nz_split_unpacked_kernel(const uint16_t* 
 // chunk and park the exponents in scratch, then one wavefront per segment
 // codes them from there.
 
-#define NZ_ENC_MAX_LANE_SYMS 256u
+#define NZ_ENC_MAX_LANE_SYMS 288u  // 36 groups of 8 symbols per lane: what fits the registers of four wavefronts per SIMD
 #define NZ_ENC_LONG_THREADS 1024u
 
 // f(constant I) for I = FROM, FROM + STEP, ... while I < TO (or, with a negative

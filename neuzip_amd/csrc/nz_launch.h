@@ -13,8 +13,8 @@
 template <int S>
 hipError_t nz_allow_encode_lds();
 
-// cls 0..2: nz_encode_kernel<S, 8 | 16 | 32> (segments of up to 64 / 128 / 256
-// symbols per lane, coded from registers); 3: nz_encode_long_kernel<S>
+// cls 0..3: nz_encode_kernel<S, 8 | 16 | 32 | 36> (segments of up to 64 / 128 / 256 /
+// 288 symbols per lane, coded from registers); 4: nz_encode_long_kernel<S>
 template <int S>
 void nz_launch_encode(const NzEncBatch& b, int cls, dim3 grid, dim3 block, uint32_t lds, hipStream_t st);
 

@@ -16,6 +16,9 @@ hipError_t nz_allow_encode_lds() {
   if (e == hipSuccess)
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nz_encode_kernel<S, 32>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(&nz_encode_kernel<S, 36>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
   return e;
 }
 
@@ -25,6 +28,7 @@ void nz_launch_encode(const NzEncBatch& b, int cls, dim3 grid, dim3 block, uint3
     case 0: hipLaunchKernelGGL((nz_encode_kernel<S, 8>), grid, block, lds, st, b); break;
     case 1: hipLaunchKernelGGL((nz_encode_kernel<S, 16>), grid, block, lds, st, b); break;
     case 2: hipLaunchKernelGGL((nz_encode_kernel<S, 32>), grid, block, lds, st, b); break;
+    case 3: hipLaunchKernelGGL((nz_encode_kernel<S, 36>), grid, block, lds, st, b); break;
     default: hipLaunchKernelGGL((nz_encode_long_kernel<S>), grid, dim3(NZ_ENC_LONG_THREADS), 0, st, b); break;
   }
 }

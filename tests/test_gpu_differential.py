@@ -46,3 +46,23 @@ def test_random_cases_match_the_oracle(oracle, seed):
         rc, out = gpu_decode(comp, packed, n, s, chunk, lane)
         assert rc == 0
         assert np.array_equal(out, oracle.reconstruct(bits, s))
+
+
+@pytest.mark.parametrize("chunk,lane", [(135168, 264), (143360, 280), (147456, 288), (151552, 296)])
+def test_segments_between_256_and_288_symbols_per_lane(oracle, chunk, lane):
+    """The geometries a manager picks for tensors of one to a few million elements
+    under its size budget: up to 288 symbols per lane are coded from registers
+    (nz_encode_kernel<S, 36>), 296 by the kernel for longer segments; both give
+    the oracle's bytes, for every precision and kind of data, ragged ends included."""
+    rng = np.random.default_rng(chunk)
+    for s in (7, 3, 1, 0):
+        for kind, n in ((0, 3 * chunk + 12345), (1, chunk + 7), (2, 2 * chunk), (3, chunk - 1), (4, 1_000_003)):
+            bits = _data(rng, n, kind)
+            print(f"case chunk={chunk} lane={lane} s={s} kind={kind} n={n}", flush=True)
+            comp, packed = gpu_encode(bits, s, chunk, lane)
+            o_comp, o_packed = oracle.compress_bf16(bits, s, chunk, lane, threads=8)
+            assert np.array_equal(comp.cpu().numpy(), o_comp)
+            assert np.array_equal(packed.cpu().numpy(), o_packed)
+            rc, out = gpu_decode(comp, packed, n, s, chunk, lane)
+            assert rc == 0
+            assert np.array_equal(out, oracle.reconstruct(bits, s))
