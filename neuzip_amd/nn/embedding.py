@@ -26,14 +26,16 @@ class Embedding(torch.nn.Module):
         self.sparse = embedding.sparse
         self._p = Parameter(self.manager, embedding.weight.data)
         # A lookup decodes whole chunks.  With a manager that chooses the geometry
-        # per tensor, the table is stored with the shortest segments there are
-        # (32 Ki chunks of eight 4 Ki segments): one row of a 128256 x 4096 table
-        # then takes 18 us instead of 39, 512 rows 27 us instead of 55, for 0.6 %
-        # more stored bytes and a slower read of the whole table (424 against 344 us).
+        # per tensor and whose size budget allows them (they store 1.036 x the
+        # exponents' entropy, the default budget is 1.01), the table is stored with
+        # the shortest segments there are (32 Ki chunks of eight 4 Ki segments): one
+        # row of a 128256 x 4096 table then takes 18 us instead of 39, 512 rows 27 us
+        # instead of 55, for 0.6 % more stored bytes and a slower read of the whole
+        # table (424 against 344 us).
         be = getattr(self.manager, "_be", None)
         if getattr(be, "auto_geometry", False):
             h = self._p._handle
-            if be.geometry(h) != (32768, 64):
+            if be.geometry(h) != (32768, 64) and be.in_budget(self._p._shape.numel(), 32768, 64):
                 dense = self.manager.read(h)
                 be.geometry_hint(h, 32768, 64)
                 self.manager.write(dense, h)

@@ -144,21 +144,23 @@ def test_large_lookups_are_bounded(oracle):
 
 
 def test_embedding_table_gets_short_segments_under_per_tensor_geometry(oracle):
-    """With a manager that chooses the geometry per tensor, a converted Embedding
-    stores its table in 32 Ki chunks of eight 4 Ki segments (a lookup decodes whole
-    chunks); the rows are the oracle's."""
+    """With a manager that chooses the geometry per tensor and whose size budget
+    allows it, a converted Embedding stores its table in 32 Ki chunks of eight
+    4 Ki segments (a lookup decodes whole chunks); at the default budget the table
+    keeps the geometry of its size.  The rows are the oracle's either way."""
     import neuzip_amd
 
     rows, dim = 5000, 1024          # 5.1 M elements: on its own the table would get longer segments
     bits = _table_bits(rows, dim, seed=9)
     emb = torch.nn.Embedding(rows, dim).to(torch.bfloat16)
     emb.weight.data = _dev(bits, rows, dim).cpu()
-    mgr = neuzip_amd.Manager(lane_symbols="auto")
-    conv = neuzip_amd.nn.Embedding(mgr, emb)
-    h = conv.weight._handle
-    assert mgr._be.geometry(h) == (32768, 64)
     full = _dev(oracle.reconstruct(bits, 7), rows, dim)
     idx = torch.randint(0, rows, (3, 17), generator=torch.Generator().manual_seed(2)).cuda()
-    assert torch.equal(conv(idx), full[idx])
-    assert torch.equal(mgr.read(h).view(rows, dim), full)
-    mgr._be.check()
+    for budget, geometry in ((1.04, (32768, 64)), (None, (135168, 264))):
+        mgr = neuzip_amd.Manager(lane_symbols="auto", size_budget=budget)
+        conv = neuzip_amd.nn.Embedding(mgr, emb)
+        h = conv.weight._handle
+        assert mgr._be.geometry(h) == geometry
+        assert torch.equal(conv(idx), full[idx])
+        assert torch.equal(mgr.read(h).view(rows, dim), full)
+        mgr._be.check()
