@@ -316,6 +316,19 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
                           uint32_t in_features, const void* const* dev_bias, void* const* dev_y,
                           void* stream);
 
+/* The same for up to NZ_GEMV_MAX_ROWS activation rows (a small batch, or the
+   tokens of a speculative step): dev_x holds x_rows rows of in_features values,
+   dev_y[i] receives x_rows rows of one value per row of matrix i; every weight
+   is decoded once and multiplied with all rows before it is dropped, so the
+   call costs little more than the one-row call (Manager::linear for 2-D
+   inputs, cuda/high_level.cu:252-263, decodes the weight into memory and runs
+   a GEMM over it).  Each output row is, bit for bit, what the one-row call
+   gives for that activation row.  Not built for managers with normalizers. */
+#define NZ_GEMV_MAX_ROWS 8u
+int nz_manager_gemv_rows_batch(nz_manager* m, const char* const* names, uint32_t count,
+                               const void* dev_x, uint32_t x_rows, uint32_t in_features,
+                               const void* const* dev_bias, void* const* dev_y, void* stream);
+
 /* Embedding lookup on a stored table (neuzip/nn/embedding.py:30-39 decompresses
    the WHOLE table for every forward): row dev_indices[i] (int64) of the table
    `name`, read as rows of row_len elements, goes to dev_out[i * row_len ...];

@@ -28,7 +28,7 @@ EXPORTS = [
     "nz_abi_version", "nz_last_error", "nz_packed_bytes", "nz_packed_stored_bytes", "nz_exp_bound_bytes",
     "nz_encode_workspace_bytes", "nz_norm_bytes", "nz_split", "nz_encode", "nz_encode_static", "nz_decode",
     "nz_manager_create", "nz_manager_destroy", "nz_manager_set_size_budget", "nz_manager_size_budget", "nz_estimated_size_ratio", "nz_manager_in_budget", "nz_manager_write", "nz_manager_write_batch",
-    "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gather_rows",
+    "nz_manager_read", "nz_manager_read_batch", "nz_manager_gemv_batch", "nz_manager_gemv_rows_batch", "nz_manager_gather_rows",
     "nz_manager_meta", "nz_manager_geometry", "nz_manager_size", "nz_manager_size_reference", "nz_manager_exp_bytes", "nz_manager_packed_bytes",
     "nz_manager_norm_bytes", "nz_manager_buffers", "nz_manager_erase", "nz_manager_check",
     "nz_manager_export", "nz_manager_import", "nz_manager_trim", "nz_manager_rewrite_stats", "nz_set_lookback_spins", "nz_manager_geometry_hint",
@@ -108,6 +108,9 @@ def load() -> ctypes.CDLL:
     L.nz_manager_gemv_batch.restype = i32
     L.nz_manager_gemv_batch.argtypes = [vp, ctypes.POINTER(ctypes.c_char_p), u32, vp, u32, ctypes.POINTER(vp),
                                         ctypes.POINTER(vp), vp]
+    L.nz_manager_gemv_rows_batch.restype = i32
+    L.nz_manager_gemv_rows_batch.argtypes = [vp, ctypes.POINTER(ctypes.c_char_p), u32, vp, u32, u32,
+                                             ctypes.POINTER(vp), ctypes.POINTER(vp), vp]
     L.nz_manager_read_batch.restype = i32
     L.nz_manager_read_batch.argtypes = [vp, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(vp),
                                         ctypes.POINTER(u64), u32, vp]

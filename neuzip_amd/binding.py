@@ -206,19 +206,21 @@ class _HipBackend:
         _lib.raise_for(rc)
         return out
 
-    def gemv_batch(self, names, x: torch.Tensor, biases, outs) -> None:
-        """``outs[i] = W_i @ x (+ biases[i])`` for the stored matrices ``names``
-        (a ctypes array of encoded handles) and ONE activation row ``x``; the
-        weights are decoded inside the kernel and never written out."""
+    def gemv_batch(self, names, x: torch.Tensor, biases, outs, rows: int = 1) -> None:
+        """``outs[i] = x @ W_i^T (+ biases[i])`` for the stored matrices ``names``
+        (a ctypes array of encoded handles) and ``rows`` (1..8) activation rows
+        ``x`` (contiguous, ``rows * in_features`` values; ``outs[i]`` holds
+        ``rows`` contiguous rows of ``out_features_i``); the weights are decoded
+        inside the kernel, once, and never written out."""
         k = len(names)
-        if x.dtype != torch.bfloat16 or not x.is_contiguous():
-            raise ValueError("gemv_batch needs a contiguous bfloat16 activation row")
+        if x.dtype != torch.bfloat16 or not x.is_contiguous() or rows < 1 or x.numel() % rows:
+            raise ValueError("gemv_batch needs contiguous bfloat16 activation rows")
         ys = (ctypes.c_void_p * k)(*[o.data_ptr() for o in outs])
         bs = None
         if biases is not None and any(b is not None for b in biases):
             bs = (ctypes.c_void_p * k)(*[None if b is None else b.data_ptr() for b in biases])
-        rc = self._L.nz_manager_gemv_batch(self._h, names, k, x.data_ptr(), x.numel(), bs, ys,
-                                           _stream_ptr(x.device))
+        rc = self._L.nz_manager_gemv_rows_batch(self._h, names, k, x.data_ptr(), rows, x.numel() // rows, bs, ys,
+                                                _stream_ptr(x.device))
         _lib.raise_for(rc)
 
     def export(self, handle: str):
@@ -284,7 +286,7 @@ class _HipBackend:
         prev = getattr(self, "_outside", None)
         self._outside = flag if prev is None else prev | flag
 
-    # -- single activation rows: decode fused into the product ------------------
+    # -- one to eight activation rows: decode fused into the product -------------
     #
     # Linears that are called back to back with the very same activation (q/k/v,
     # gate/up) are served by ONE launch, without the caller saying so: the first
@@ -295,12 +297,16 @@ class _HipBackend:
     # the same bias.  A run that does not repeat itself is forgotten for good.
 
     _MAX_RUN = 8
+    _MAX_ROWS = 8  # activation rows one launch multiplies with (NZ_GEMV_MAX_ROWS)
 
     def _fused_ok(self, inputs: torch.Tensor, shape, bias) -> bool:
-        if (not self.fused_rows or inputs.dim() == 0 or inputs.numel() != inputs.shape[-1] or len(shape) != 2
-                or inputs.shape[-1] != shape[1] or shape[1] % 512 or inputs.dtype != torch.bfloat16
-                or not inputs.is_cuda or (torch.is_grad_enabled() and inputs.requires_grad)):
+        if (not self.fused_rows or inputs.dim() == 0 or len(shape) != 2 or inputs.shape[-1] != shape[1]
+                or shape[1] % 512 or not 1 <= inputs.numel() // shape[1] <= self._MAX_ROWS
+                or inputs.dtype != torch.bfloat16 or not inputs.is_cuda
+                or (torch.is_grad_enabled() and inputs.requires_grad)):
             return False
+        if inputs.numel() != shape[1] and self._normalizer:
+            return False  # several rows per launch are not built for normalized tensors
         if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_cuda or bias.numel() != shape[0]
                                  or not bias.is_contiguous() or (torch.is_grad_enabled() and bias.requires_grad)):
             return False
@@ -338,10 +344,11 @@ class _HipBackend:
             self._member_of[h] = leader
 
     def _fused_row(self, handle: str, inputs: torch.Tensor, shape, bias):
-        """``x @ W^T (+ b)`` for ONE activation row without writing the dense weight:
-        the product is formed while the weight is decoded (nz_manager_gemv_batch).
-        -> None when the call does not qualify (several rows, a row length that is
-        not a multiple of 512, another dtype, a bias the kernel cannot take)."""
+        """``x @ W^T (+ b)`` for one to eight activation rows without writing the
+        dense weight: the product is formed while the weight is decoded
+        (nz_manager_gemv_rows_batch).  -> None when the call does not qualify (more
+        rows, a row length that is not a multiple of 512, another dtype, a bias the
+        kernel cannot take)."""
         if not self._fused_ok(inputs, shape, bias):
             return None
         parked = self._parked.pop(handle, None)
@@ -353,18 +360,19 @@ class _HipBackend:
         x = inputs if inputs.is_contiguous() else inputs.contiguous()
         if x.data_ptr() % 16:
             x = x.clone()
+        m_rows = x.numel() // shape[1]
         run = self._runs.get(handle) if self.group_rows else None
         if run is not None:
             handles, names, rows, biases = run
             if biases[0] is bias:
                 self._close_run()
-                flat = torch.empty(sum(rows), dtype=torch.bfloat16, device=x.device)
+                flat = torch.empty(m_rows * sum(rows), dtype=torch.bfloat16, device=x.device)
                 outs, at = [], 0
                 for r in rows:
-                    outs.append(flat[at:at + r])
-                    at += r
+                    outs.append(flat[at:at + m_rows * r])
+                    at += m_rows * r
                 try:
-                    self.gemv_batch(names, x, biases, outs)
+                    self.gemv_batch(names, x, biases, outs, m_rows)
                 except (ValueError, RuntimeError):
                     self._forget_run(handle)  # e.g. scratch that cannot grow while a graph is captured
                 else:
@@ -376,8 +384,8 @@ class _HipBackend:
         names = self._names1.get(handle)
         if names is None:
             names = self._names1[handle] = (ctypes.c_char_p * 1)(handle.encode())
-        out = torch.empty(shape[0], dtype=torch.bfloat16, device=x.device)
-        self.gemv_batch(names, x, [bias], [out])
+        out = torch.empty(m_rows * shape[0], dtype=torch.bfloat16, device=x.device)
+        self.gemv_batch(names, x, [bias], [out], m_rows)
         if self.group_rows and handle not in self._member_of:
             self._observe(handle, inputs, shape[0], bias)
         return out.view(*inputs.shape[:-1], shape[0])
@@ -554,9 +562,9 @@ class Manager:
 
     def linear(self, handle: str, inputs: torch.Tensor, bias=None) -> torch.Tensor:
         """``inputs @ W^T (+ bias)`` against the stored weight (neuzip/binding.py:97-102).
-        One activation row of a multiple of 512 elements (single-token inference)
-        is multiplied while the weight is decoded, without the dense weight ever
-        being written; its sums are formed in an order of their own, so the
+        One to eight activation rows of a multiple of 512 elements (single-token
+        inference, a small batch, a speculative step) are multiplied while the
+        weight is decoded, without the dense weight ever being written; its sums are formed in an order of their own, so the
         result agrees with the decompress-then-GEMM path to rounding, not bit for
         bit (``manager.fused_rows = False`` keeps every call on that path).
         Such calls that come back to back with the same activation tensor (q/k/v,

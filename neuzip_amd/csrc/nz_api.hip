@@ -1268,21 +1268,27 @@ int nz_manager_read_batch(nz_manager* m, const char* const* names, void* const* 
   return NZ_OK;
 }
 
-int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t count, const void* dev_x,
-                          uint32_t in_features, const void* const* dev_bias, void* const* dev_y,
-                          void* stream) {
+int nz_manager_gemv_rows_batch(nz_manager* m, const char* const* names, uint32_t count, const void* dev_x,
+                               uint32_t x_rows, uint32_t in_features, const void* const* dev_bias,
+                               void* const* dev_y, void* stream) {
   if (!m || !names || !dev_y || !dev_x) return fail(NZ_ERR_ARG, "null manager, names, input or outputs");
   if (count == 0 || count > NZ_BATCH_MAX) return fail(NZ_ERR_ARG, "between 1 and 16 matrices per call");
+  if (x_rows == 0 || x_rows > NZ_GEMV_MAX_ROWS) return fail(NZ_ERR_ARG, "between 1 and 8 activation rows per call");
   if (in_features == 0 || in_features % NZ_GROUP_SYMS)
     return fail(NZ_ERR_ARG, "in_features must be a multiple of 512");
   if ((uintptr_t)dev_x & 15) return fail(NZ_ERR_ALIGN, "activation must be 16-byte aligned");
+  if (x_rows > 1 && m->normalizer)
+    return fail(NZ_ERR_ARG, "several activation rows per call are not built for managers with normalizers");
   hipStream_t st = (hipStream_t)stream;
   std::lock_guard<std::mutex> lock(m->mu);
   NzBatch b;
   std::memset(&b, 0, sizeof(b));
   b.x = (const uint16_t*)dev_x;
   b.in_features = in_features;
+  b.x_rows = x_rows;
   b.log2n = log2_of(m->normalizer ? m->normalizer : 1);
+  // accumulator pairs per row of a matrix: as many as the kernel that serves x_rows holds per lane
+  const uint32_t mr = x_rows <= 1 ? 1u : x_rows <= 2 ? 2u : x_rows <= 4 ? 4u : 8u;
   uint64_t grid = 0, rows = 0;
   uint32_t max_spc = 1;
   {
@@ -1293,7 +1299,7 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
       auto it = m->entries.find(names[i]);
       if (it == m->entries.end()) return fail(NZ_ERR_NOT_FOUND, "Data not found");
       blocks = blocks || it->second.pending >= 0;
-      want_rows += it->second.n / in_features;
+      want_rows += it->second.n / in_features * mr;
     }
     if (int rc = refuse_under_capture(st, blocks || m->gemv_rows < want_rows, "gemv_batch")) return rc;
     if (int rc = order_scratch_use(m, st)) return rc;
@@ -1319,8 +1325,8 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
     if (g.spc > max_spc) max_spc = g.spc;
     bi.bias = dev_bias ? (const uint16_t*)dev_bias[i] : nullptr;
     bi.y = (uint16_t*)dev_y[i];
-    bi.reserved = (uint32_t)rows;  // first row, turned into a pointer below
-    rows += ent.n / in_features;
+    bi.reserved = (uint32_t)rows;  // first accumulator pair, turned into a pointer below
+    rows += ent.n / in_features * mr;
     if (grid > 0x7FFFFFFFull || rows > 0x7FFFFFFFull) return fail(NZ_ERR_ARG, "batch too large");
   }
   if (m->gemv_rows < rows) {
@@ -1340,6 +1346,12 @@ int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t coun
   }
   b.count = count;
   return gemv_launch(b, (uint32_t)grid, max_spc, m->precision, m->d_status, st);
+}
+
+int nz_manager_gemv_batch(nz_manager* m, const char* const* names, uint32_t count, const void* dev_x,
+                          uint32_t in_features, const void* const* dev_bias, void* const* dev_y,
+                          void* stream) {
+  return nz_manager_gemv_rows_batch(m, names, count, dev_x, 1, in_features, dev_bias, dev_y, stream);
 }
 
 int nz_manager_gather_rows(nz_manager* m, const char* name, const void* dev_indices, uint64_t count,

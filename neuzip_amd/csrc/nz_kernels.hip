@@ -1529,11 +1529,18 @@ __device__ __forceinline__ uint4 nz_merge_group(uint64_t sm, const uint32_t (&ew
 #define NZ_GEMV_PART_MAX 262144.0f /* 2^18 */
 
 struct NzGemv {
-  const uint16_t* x;      // in_features bf16 values, 16-byte aligned
-  long long* acc;         // two words per row of this tensor (sum | count and flag), all zero between calls
-  uint16_t* y;            // one bf16 per row
-  const uint16_t* bias;   // one bf16 per row, or null
+  const uint16_t* x;      // x_rows activation rows of in_features bf16 values each, 16-byte aligned
+  long long* acc;         // two words per row of this tensor and activation row (sum | count and flag), all zero between calls
+  uint16_t* y;            // x_rows rows of one bf16 per row of the tensor
+  const uint16_t* bias;   // one bf16 per row of the tensor, or null
   uint32_t in_features;   // multiple of 512
+  uint32_t x_rows;        // activation rows that exist (1 .. the kernel's MR); the others are neither read nor written
+};
+
+// what a lane holds of the activation rows for one group of 8 weights
+template <int MR>
+struct NzXq {
+  uint4 v[MR];
 };
 
 typedef __attribute__((ext_vector_type(2))) __bf16 nz_bf16x2;
@@ -1556,6 +1563,7 @@ __device__ __forceinline__ float nz_dot8(const uint4 w, const uint4 x, float acc
 // row comes out as NaN), and a counter of contributions; the wave that brings
 // the count to the number of segments the row touches converts, stores and
 // returns both words to zero.
+template <int MR>
 struct NzGemvWalk {
   const uint4* xq;     // x as 8-element blocks, already offset by the lane
   NzGemv gv;
@@ -1564,12 +1572,16 @@ struct NzGemvWalk {
   uint32_t col;        // column of the current group's first element (uniform)
   uint32_t pending;    // groups added since the last flush (uniform)
   uint32_t seg_syms, last_syms, spc, k;  // segment lengths of a chunk, this wave's segment inside it
-  float sum;
+  uint32_t xstride;    // 16-byte blocks between two activation rows
+  uint64_t w_rows;     // rows of the tensor (= elements between two output rows)
+  float sum[MR];
 
   __device__ __forceinline__ void start(const NzGemv& g, const NzGeom& geom, uint64_t first_elem,
                                         uint32_t seg_n, uint32_t wave_in_chunk, uint32_t lane) {
     gv = g;
     xq = reinterpret_cast<const uint4*>(g.x) + lane;
+    xstride = g.in_features / NZ_GROUP;
+    w_rows = geom.n / g.in_features;
     row = first_elem / g.in_features;
     col = (uint32_t)(first_elem - row * g.in_features);
     seg_first = first_elem;
@@ -1579,12 +1591,23 @@ struct NzGemvWalk {
     last_syms = geom.chunk_syms - (geom.spc - 1) * geom.seg_syms;  // the chunk's (shorter) last segment
     k = wave_in_chunk;
     pending = 0;
-    sum = 0.f;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) sum[m] = 0.f;
   }
   __device__ __forceinline__ uint32_t next_col() const {
     return col + NZ_GROUP_SYMS == gv.in_features ? 0u : col + NZ_GROUP_SYMS;
   }
-  __device__ __forceinline__ uint4 load(uint32_t c) const { return xq[c / NZ_GROUP]; }
+  // the lane's 8 activations of every row for the group at column c (a row that
+  // does not exist reads the last one that does)
+  __device__ __forceinline__ NzXq<MR> load(uint32_t c) const {
+    NzXq<MR> r;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+      const uint32_t mm = (uint32_t)m < gv.x_rows ? (uint32_t)m : gv.x_rows - 1u;
+      r.v[m] = xq[(uint64_t)mm * xstride + c / NZ_GROUP];
+    }
+    return r;
+  }
   // Segments the row [first, last] touches, this wave's included: walk over the
   // segment boundaries to the left and to the right (a row rarely spans more
   // than two or three segments; no division).
@@ -1606,45 +1629,56 @@ struct NzGemvWalk {
     }
     return count;
   }
-  __device__ __forceinline__ void store_row(float v) const {
+  __device__ __forceinline__ void store_row(float v, uint32_t m) const {
     if (gv.bias) v += nz_bf16_to_f32(gv.bias[row]);
-    gv.y[row] = (uint16_t)nz_f32_to_bf16(v);
+    gv.y[(uint64_t)m * w_rows + row] = (uint16_t)nz_f32_to_bf16(v);
   }
   __device__ __forceinline__ void flush(uint32_t lane) {
-    const float t = nz_wave_sum(sum);
+    float t[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) t[m] = nz_wave_sum(sum[m]);
     if (lane == 0) {
       const uint64_t first = row * gv.in_features, last = first + gv.in_features - 1;
       if (first >= seg_first && last < seg_end) {
-        store_row(t);
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+          if ((uint32_t)m < gv.x_rows) store_row(t[m], (uint32_t)m);
       } else {
         // Device-scope atomics execute at the L2 in the order they are issued by
         // this lane when each one waits for the value the previous returned, so
         // no cache flush is needed: the count is issued only after the sum's old
         // value has come back, the exchanges only after the count's.
-        unsigned long long* slot = reinterpret_cast<unsigned long long*>(gv.acc + 2 * row);
-        unsigned long long r0;
-        if (fabsf(t) < NZ_GEMV_PART_MAX)  // false for NaN as well
-          r0 = atomicAdd(slot, (unsigned long long)__float2ll_rn(t * (float)(1ull << NZ_GEMV_FRAC_BITS)));
-        else
-          r0 = atomicOr(slot + 1, 1ull << 32);
-        uint32_t zero;  // 0, but only the hardware knows: ties the next atomic to the returned value
-        asm volatile("v_and_b32 %0, 0, %1" : "=v"(zero) : "v"((uint32_t)r0));
         const uint32_t expected = segments_of_row(first, last);
-        const unsigned long long before = atomicAdd(slot + 1, 1ull + zero);
-        if ((uint32_t)before + 1u == expected) {
-          const long long a = (long long)atomicExch(slot, 0ull);
-          const unsigned long long f = atomicExch(slot + 1, 0ull);
-          store_row((f >> 32) ? __uint_as_float(0x7FC00000u)
-                              : (float)((double)a * (1.0 / (double)(1ull << NZ_GEMV_FRAC_BITS))));
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+          if ((uint32_t)m >= gv.x_rows) continue;
+          unsigned long long* slot = reinterpret_cast<unsigned long long*>(gv.acc + 2 * (row * MR + m));
+          unsigned long long r0;
+          if (fabsf(t[m]) < NZ_GEMV_PART_MAX)  // false for NaN as well
+            r0 = atomicAdd(slot, (unsigned long long)__float2ll_rn(t[m] * (float)(1ull << NZ_GEMV_FRAC_BITS)));
+          else
+            r0 = atomicOr(slot + 1, 1ull << 32);
+          uint32_t zero;  // 0, but only the hardware knows: ties the next atomic to the returned value
+          asm volatile("v_and_b32 %0, 0, %1" : "=v"(zero) : "v"((uint32_t)r0));
+          const unsigned long long before = atomicAdd(slot + 1, 1ull + zero);
+          if ((uint32_t)before + 1u == expected) {
+            const long long a = (long long)atomicExch(slot, 0ull);
+            const unsigned long long f = atomicExch(slot + 1, 0ull);
+            store_row((f >> 32) ? __uint_as_float(0x7FC00000u)
+                                : (float)((double)a * (1.0 / (double)(1ull << NZ_GEMV_FRAC_BITS))),
+                      (uint32_t)m);
+          }
         }
       }
     }
-    sum = 0.f;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) sum[m] = 0.f;
     pending = 0;
   }
-  // add the dot product of the current group, then step to the next group
-  __device__ __forceinline__ void add(const uint4 w, const uint4 x, uint32_t lane) {
-    sum = nz_dot8(w, x, sum);
+  // add the dot products of the current group, then step to the next group
+  __device__ __forceinline__ void add(const uint4 w, const NzXq<MR>& x, uint32_t lane) {
+#pragma unroll
+    for (int m = 0; m < MR; ++m) sum[m] = nz_dot8(w, x.v[m], sum[m]);
     ++pending;
     col = next_col();
     if (col == 0) {
@@ -1777,7 +1811,7 @@ struct NzWaveDec {
 // ragged and no group straddles two rows).
 // With NORM every merged value is multiplied by its group's factor (`nm`)
 // before it is stored or used.
-template <int S, bool GEMV, bool NORM, bool STREAM>
+template <int S, int GEMV, bool NORM, bool STREAM>
 __device__ __forceinline__ void nz_decode_chunk(
     const uint8_t* __restrict__ comp, const uint64_t comp_bytes, const uint8_t* __restrict__ packed,
     uint16_t* __restrict__ out, const NzGeom& g, uint32_t* __restrict__ d_status, const uint64_t c,
@@ -1853,13 +1887,17 @@ __device__ __forceinline__ void nz_decode_chunk(
   w.lane = lane;
   w.filled = 0;
   uint64_t sm_next = 0, nb_next = 0;
-  uint4 xq_next = make_uint4(0, 0, 0, 0);
-  NzGemvWalk walk;
+  constexpr int MR = GEMV ? GEMV : 1;  // activation rows a lane multiplies with (GEMV: 0 = plain decode)
+  // the activations of the next group are fetched a group ahead, unless that would cost the
+  // registers of a whole workgroup per compute unit (eight rows: 32 registers)
+  constexpr bool X_AHEAD = MR < 8;
+  NzXq<X_AHEAD ? MR : 1> xq_next{};
+  NzGemvWalk<MR> walk;
   if (has_seg && !bad_rec) {
     w.stage();
     if constexpr (GEMV) {
       walk.start(gv, g, seg_base, seg_n, wk, lane);
-      xq_next = walk.load(walk.col);
+      if constexpr (X_AHEAD) xq_next = walk.load(walk.col);
     }
     if (whole) {
       sm_next = nz_stream_sm<S>(pk + lane_off);
@@ -2091,8 +2129,13 @@ __device__ __forceinline__ void nz_decode_chunk(
     else return nz_norm_load8(nm, e0);
   };
   const auto full_group = [&](uint32_t gq, const uint64_t sm, const uint64_t nb, auto wide) {
-    const uint4 xq = xq_next;
-    if constexpr (GEMV) xq_next = walk.load(walk.next_col());  // always inside x
+    NzXq<MR> xq;
+    if constexpr (GEMV && X_AHEAD) {
+      xq = xq_next;
+      xq_next = walk.load(walk.next_col());  // always inside x
+    } else if constexpr (GEMV) {
+      xq = walk.load(walk.col);
+    }
     uint32_t ew[8];
     w.group(ew);
     // the merge starts only here: its wait for the packed bytes must not be
@@ -2179,7 +2222,7 @@ template <int S, bool NORM, bool STREAM>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_kernel(
     const uint8_t* __restrict__ comp, uint64_t comp_bytes, const uint8_t* __restrict__ packed,
     uint16_t* __restrict__ out, NzGeom g, uint32_t* __restrict__ d_status, const NzNorm nm) {
-  nz_decode_chunk<S, false, NORM, STREAM>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x, NzGemv{}, nm);
+  nz_decode_chunk<S, 0, NORM, STREAM>(comp, comp_bytes, packed, out, g, d_status, blockIdx.x, NzGemv{}, nm);
 }
 
 // Several tensors in one launch: the grid is the concatenation of their
@@ -2204,7 +2247,7 @@ struct NzBatch {
   uint32_t in_features;  // matrix-vector product only
   const uint16_t* x;     // matrix-vector product only
   uint32_t log2n;        // normalized tensors only
-  uint32_t reserved;
+  uint32_t x_rows;       // matrix-vector product only: activation rows (1..8)
   NzBatchItem item[NZ_BATCH_MAX];
 };
 
@@ -2217,12 +2260,13 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_batch_ke
     ++t;
   }
   const NzBatchItem& it = b.item[t];
-  nz_decode_chunk<S, false, NORM, STREAM>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status,
+  nz_decode_chunk<S, 0, NORM, STREAM>(it.comp, it.comp_bytes, it.packed, it.out, it.g, d_status,
                                           blockIdx.x - first, NzGemv{}, NzNorm{it.norm, b.log2n});
 }
 
-// The same walk over several matrices that multiply one activation row.
-template <int S, bool NORM>
+// The same walk over several matrices that multiply one activation row, or up
+// to MR of them (each decoded weight is then used MR times before it is dropped).
+template <int S, bool NORM, int MR>
 __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_gemv_kernel(
     const NzBatch b, uint32_t* __restrict__ d_status) {
   uint32_t t = 0, first = 0;
@@ -2231,8 +2275,8 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_gemv_ker
     ++t;
   }
   const NzBatchItem& it = b.item[t];
-  const NzGemv gv{b.x, it.acc, it.y, it.bias, b.in_features};
-  nz_decode_chunk<S, true, NORM, false>(it.comp, it.comp_bytes, it.packed, nullptr, it.g, d_status,
+  const NzGemv gv{b.x, it.acc, it.y, it.bias, b.in_features, b.x_rows};
+  nz_decode_chunk<S, MR, NORM, false>(it.comp, it.comp_bytes, it.packed, nullptr, it.g, d_status,
                                         blockIdx.x - first, gv, NzNorm{it.norm, b.log2n});
 }
 
@@ -2261,7 +2305,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK) void nz_decode_rows_ker
   // that the chunk's first element lands at the start of this workgroup's slot
   uint16_t* out = scratch + ((int64_t)blockIdx.x - (int64_t)c) * (int64_t)g.chunk_syms;
   // (the slots are read back by the copy kernel right away: ordinary stores)
-  nz_decode_chunk<S, false, NORM, false>(comp, comp_bytes, packed, out, g, d_status, c, NzGemv{}, nm);
+  nz_decode_chunk<S, 0, NORM, false>(comp, comp_bytes, packed, out, g, d_status, c, NzGemv{}, nm);
 }
 
 #ifndef NZ_TEMPLATES_ONLY

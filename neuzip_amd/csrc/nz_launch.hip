@@ -72,8 +72,13 @@ template <int S>
 void nz_launch_gemv(const NzBatch& b, uint32_t grid, uint32_t max_spc, uint32_t* d_status, hipStream_t st) {
   const size_t lds = NZ_DEC_LDS_BYTES(max_spc);
   const dim3 gd(grid), bd(64 * max_spc);
-  if (b.item[0].norm) hipLaunchKernelGGL((nz_decode_gemv_kernel<S, true>), gd, bd, lds, st, b, d_status);
-  else hipLaunchKernelGGL((nz_decode_gemv_kernel<S, false>), gd, bd, lds, st, b, d_status);
+  // one activation row, or kernels that hold 2, 4 or 8 of them per lane (tensors with
+  // normalizers: one row only, the caller has checked)
+  if (b.item[0].norm) hipLaunchKernelGGL((nz_decode_gemv_kernel<S, true, 1>), gd, bd, lds, st, b, d_status);
+  else if (b.x_rows <= 1) hipLaunchKernelGGL((nz_decode_gemv_kernel<S, false, 1>), gd, bd, lds, st, b, d_status);
+  else if (b.x_rows <= 2) hipLaunchKernelGGL((nz_decode_gemv_kernel<S, false, 2>), gd, bd, lds, st, b, d_status);
+  else if (b.x_rows <= 4) hipLaunchKernelGGL((nz_decode_gemv_kernel<S, false, 4>), gd, bd, lds, st, b, d_status);
+  else hipLaunchKernelGGL((nz_decode_gemv_kernel<S, false, 8>), gd, bd, lds, st, b, d_status);
 }
 
 template <int S>

@@ -275,3 +275,78 @@ def test_group_geometry_is_refitted_and_results_stay_the_same():
         mgr.write(wa * 2, ha)                      # a later write keeps the group's geometry
         assert mgr._be.geometry(ha) == after and torch.equal(mgr.read(ha), wa * 2)
     mgr._be.check()
+
+
+@pytest.mark.parametrize("s", [7, 3])
+@pytest.mark.parametrize("m_rows", [2, 3, 4, 5, 8])
+def test_several_activation_rows_equal_the_one_row_calls(m_rows, s):
+    """nz_manager_gemv_rows_batch: every weight is decoded once and multiplied with
+    up to eight activation rows.  Each output row is, bit for bit, what the one-row
+    call gives for that activation row (same order of additions per row), so it is
+    within the same tolerance of the fp64 product; matrices whose rows lie inside
+    a segment, straddle segments, and a group of matrices in one launch."""
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=s)
+    be = mgr._be
+    cols = 4096
+    shapes = [(4096, cols), (96, cols), (1030, cols)]
+    bits = [_weight(r, c, "normal" if i != 1 else "stress", seed=70 + i + s) for i, (r, c) in enumerate(shapes)]
+    hs = [mgr.write(torch.from_numpy(b.view(np.int16).copy()).cuda().view(torch.bfloat16).view(r, c))
+          for b, (r, c) in zip(bits, shapes)]
+    g = torch.Generator(device="cuda").manual_seed(m_rows)
+    x = torch.randn(m_rows, cols, device="cuda", generator=g).to(torch.bfloat16)
+    biases = [None, torch.randn(96, device="cuda", generator=g).to(torch.bfloat16), None]
+    names = (ctypes.c_char_p * len(hs))(*[h.encode() for h in hs])
+    print(f"case rows={m_rows} s={s}", flush=True)
+    outs = [torch.full((m_rows, r), 7.0, dtype=torch.bfloat16, device="cuda") for r, _ in shapes]
+    be.gemv_batch(names, x, biases, outs, m_rows)
+    torch.cuda.synchronize()
+    for i, (h, b) in enumerate(zip(hs, biases)):
+        for m in range(m_rows):
+            (one,) = _gemv(mgr, [h], x[m].contiguous(), [b])
+            assert torch.equal(one.view(torch.int16), outs[i][m].view(torch.int16)), (i, m)
+            _check(outs[i][m], bits[i], x[m], b, s)
+    # again, with the matrices one by one: the accumulators were left clean
+    for i, h in enumerate(hs):
+        out = torch.full((m_rows, shapes[i][0]), 7.0, dtype=torch.bfloat16, device="cuda")
+        be.gemv_batch((ctypes.c_char_p * 1)(h.encode()), x, [biases[i]], [out], m_rows)
+        assert torch.equal(out.view(torch.int16), outs[i].view(torch.int16))
+    # more than eight rows, or rows with a manager that has normalizers: refused, nothing written
+    xbig = torch.zeros(9, cols, dtype=torch.bfloat16, device="cuda")
+    sink = torch.full((9, 4096), 7.0, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="activation rows"):
+        be.gemv_batch((ctypes.c_char_p * 1)(hs[0].encode()), xbig, None, [sink], 9)
+    assert bool((sink == 7.0).all())
+    be.check()
+
+
+def test_linear_with_a_few_rows_takes_the_fused_product(oracle):
+    """Manager.linear with a 2-D (or batched) input of two to eight rows: served by
+    the fused product (equal to the one-row calls), nine rows and more by
+    decompress-then-GEMM (equal to torch's linear on the decoded weight); Linears
+    that share their input are still recognised and launched together."""
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager(precision=7)
+    cols = 2048
+    ws = [(torch.randn(r, cols, device="cuda") * 0.02).to(torch.bfloat16) for r in (1536, 512, 512)]
+    bias = torch.randn(1536, device="cuda").to(torch.bfloat16)
+    hs = [mgr.write(w) for w in ws]
+    with torch.no_grad():
+        for shape in ((4, cols), (2, 3, cols), (1, 8, cols)):
+            x = torch.randn(*shape, device="cuda").to(torch.bfloat16)
+            for rep in range(3):  # the second pass has learned that the three share their input
+                got = [mgr.linear(hs[0], x, bias), mgr.linear(hs[1], x), mgr.linear(hs[2], x)]
+                flat = x.reshape(-1, cols)
+                for k, (h, w, b) in enumerate(zip(hs, ws, (bias, None, None))):
+                    assert got[k].shape == x.shape[:-1] + (w.shape[0],)
+                    for m in range(flat.shape[0]):
+                        mgr.group_rows = False
+                        one = mgr.linear(h, flat[m].contiguous(), b)
+                        mgr.group_rows = True
+                        assert torch.equal(one, got[k].reshape(-1, w.shape[0])[m]), (shape, rep, k, m)
+        assert sorted(len(r[0]) for r in mgr._be._runs.values()) == [3]
+        x9 = torch.randn(9, cols, device="cuda").to(torch.bfloat16)
+        assert torch.equal(mgr.linear(hs[0], x9, bias), torch.nn.functional.linear(x9, ws[0], bias))
+    mgr._be.check()
