@@ -350,3 +350,92 @@ def test_linear_with_a_few_rows_takes_the_fused_product(oracle):
         x9 = torch.randn(9, cols, device="cuda").to(torch.bfloat16)
         assert torch.equal(mgr.linear(hs[0], x9, bias), torch.nn.functional.linear(x9, ws[0], bias))
     mgr._be.check()
+
+
+def test_runs_of_calls_that_share_their_activation_are_learned_and_checked():
+    """Manager.linear recognises Linears called back to back with the same
+    activation tensor and serves them with one launch from the second time on.
+    A result computed ahead is handed out only for the very same tensor object,
+    unmodified, and the same bias; anything else falls back to a launch of its
+    own and the run is forgotten.  Every result equals the single launch's."""
+    import neuzip_amd
+
+    cols = 1024
+    ws = [(torch.randn(r, cols, device="cuda") * 0.02).to(torch.bfloat16) for r in (768, 256, 256, 512)]
+    bias = torch.randn(256, device="cuda").to(torch.bfloat16)
+
+    def fresh():
+        mgr = neuzip_amd.Manager(precision=7)
+        return mgr, [mgr.write(w) for w in ws]
+
+    def alone(mgr, h, x, b=None):
+        was = mgr.group_rows
+        mgr.group_rows = False
+        try:
+            return mgr.linear(h, x, b)
+        finally:
+            mgr.group_rows = was
+
+    with torch.no_grad():
+        # learned on the first pass, grouped from the second: same numbers, one run of three
+        mgr, hs = fresh()
+        for rep in range(3):
+            x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+            y = [mgr.linear(hs[0], x), mgr.linear(hs[1], x, bias), mgr.linear(hs[2], x)]
+            mgr.linear(hs[3], torch.randn(cols, device="cuda").to(torch.bfloat16))  # another input: not part of the run
+            for k, b in ((0, None), (1, bias), (2, None)):
+                assert torch.equal(y[k], alone(mgr, hs[k], x, b)), (rep, k)
+        assert [r[0] for r in mgr._be._runs.values()] == [hs[:3]]
+        assert not mgr._be._parked
+
+        # the activation is modified in place between two calls of a learned run
+        x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+        y0 = mgr.linear(hs[0], x)          # computes all three ahead
+        x.mul_(2)
+        y1 = mgr.linear(hs[1], x, bias)    # must see the new values
+        assert torch.equal(y1, alone(mgr, hs[1], x, bias))
+        assert hs[0] not in mgr._be._runs and not mgr._be._parked  # forgotten for good
+        for rep in range(2):                # ... and not learned again
+            x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+            mgr.linear(hs[0], x), mgr.linear(hs[1], x, bias), mgr.linear(hs[2], x)
+        assert not mgr._be._runs
+
+        # an equal but different tensor object, and another bias, are not taken for the learned ones
+        mgr, hs = fresh()
+        for rep in range(2):
+            x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+            mgr.linear(hs[0], x), mgr.linear(hs[1], x, bias), mgr.linear(hs[2], x)
+        x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+        mgr.linear(hs[0], x)
+        other = torch.randn(cols, device="cuda").to(torch.bfloat16)
+        assert torch.equal(mgr.linear(hs[1], other, bias), alone(mgr, hs[1], other, bias))
+        mgr, hs = fresh()
+        for rep in range(2):
+            x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+            mgr.linear(hs[0], x), mgr.linear(hs[1], x, bias), mgr.linear(hs[2], x)
+        x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+        mgr.linear(hs[0], x)
+        bias2 = bias.clone().add_(1)
+        assert torch.equal(mgr.linear(hs[1], x, bias2), alone(mgr, hs[1], x, bias2))
+
+        # a weight of the run is rewritten between two calls: nothing computed ahead survives the write
+        mgr, hs = fresh()
+        for rep in range(2):
+            x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+            mgr.linear(hs[0], x), mgr.linear(hs[1], x, bias), mgr.linear(hs[2], x)
+        x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+        mgr.linear(hs[0], x)
+        w_new = (ws[1].float() * 1.5).to(torch.bfloat16)
+        mgr.write(w_new, hs[1])
+        got = mgr.linear(hs[1], x, bias)
+        assert torch.equal(got, alone(mgr, hs[1], x, bias))
+        assert not torch.equal(got, torch.zeros_like(got))
+        # ... and the learned run goes on with the new weight
+        x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+        y = [mgr.linear(hs[0], x), mgr.linear(hs[1], x, bias), mgr.linear(hs[2], x)]
+        assert torch.equal(y[1], alone(mgr, hs[1], x, bias))
+
+        # a member called out of order, without the first one: a launch of its own
+        x = torch.randn(cols, device="cuda").to(torch.bfloat16)
+        assert torch.equal(mgr.linear(hs[2], x), alone(mgr, hs[2], x))
+        mgr._be.check()
