@@ -728,8 +728,11 @@ def gpt2m_measure(args, torch):
     # started from, so with a lossless manager its losses must be the dense run's, bit for bit
     per_block_linears = len(comp_params) // max(1, layers)
     torch.manual_seed(args.seed + 1)
-    with neuzip_amd.DecompressAhead(mgr, model, ahead=False):
-        per_block, wall, comp_losses = run(per_block_linears)
+    da = neuzip_amd.DecompressAhead(mgr, model, ahead=False)  # small blocks share a launch (up to 16 tensors)
+    per_launch = max(da.tensors_per_launch)
+    with da:
+        per_block, wall, comp_losses = run(per_launch)
+    del da
     same = sum(1 for a, b in zip(dense_losses, comp_losses) if torch.equal(a, b))
     per_block["steps_with_the_dense_runs_loss"] = f"{same} of {len(dense_losses)}"
     per_block["dense_first_loss"] = round(float(dense_losses[args.warmup]), 4)
@@ -769,11 +772,13 @@ def gpt2m_measure(args, torch):
         mgr2, _ = make_manager(args, 7)
         mgr2.convert(comp_twin)
         g = torch.Generator(device="cuda").manual_seed(args.seed + 2)
-        with neuzip_amd.DecompressAhead(mgr2, comp_twin, ahead=False):
+        da2 = neuzip_amd.DecompressAhead(mgr2, comp_twin, ahead=False)
+        with da2:
             lockstep = lockstep_adamw(
                 dense_twin, comp_twin, mgr2,
                 lambda i: torch.randint(0, 50257, (args.batch, args.seq_len), device="cuda", generator=g),
-                steps=args.verify_steps, group=per_block_linears)
+                steps=args.verify_steps, group=max(da2.tensors_per_launch))
+        del da2
         mgr2._be.check()
     tokens = args.batch * (args.seq_len - 1) * args.steps
     out = {
@@ -787,6 +792,7 @@ def gpt2m_measure(args, torch):
             "workload": f"GPT-2-medium-shaped random-init model, {layers} layers, batch {args.batch} x seq {args.seq_len}, "
                         f"bf16 weights compressed (precision {args.precision}), re-compressed after each AdamW step",
             "dense_bf16_torch_adamw_ms_per_step": round(dense_ms, 3),
+            "tensors_per_decode_and_write_launch": per_launch,
             "decode_per_block": per_block,
             "decode_per_linear": per_linear,
             "lockstep_check_lossless": lockstep,

@@ -55,22 +55,47 @@ class _Slot:
         self.stamps = []   # per tensor of that block: the handle's write count when it was decoded
 
 
+_MAX_TENSORS = 16  # tensors one decode launch takes (NZ_BATCH_MAX)
+
+
+def _merge_small(groups, numel, fill: int):
+    """Consecutive blocks whose weights are too few to fill the device share a
+    launch: blocks are added to a group until it holds ``fill`` elements (or 16
+    tensors).  A launch takes as long as its longest segment however few of them
+    there are, so the four weights of a GPT-2-medium block (12.6 M elements, 92
+    chunks on 256 compute units) cost as much alone as three such blocks together."""
+    out = []
+    for g in groups:
+        if out and len(out[-1]) + len(g) <= _MAX_TENSORS and sum(numel(m) for m in out[-1]) < fill:
+            out[-1] = out[-1] + g
+        else:
+            out.append(list(g))
+    return out
+
+
 class DecompressAhead:
-    def __init__(self, manager, model: torch.nn.Module, blocks=None, ahead: bool = True, wrap: bool = True):
+    def __init__(self, manager, model: torch.nn.Module, blocks=None, ahead: bool = True, wrap: bool = True,
+                 merge_small: bool = True):
         """``blocks``: modules whose compressed Linears are decoded together
-        (default: the elements of the model's ModuleLists); ``ahead``: decode
-        block k+1 on a side stream while block k computes; ``wrap``: after the
-        last block, already decode the first one for the next forward pass."""
+        (default: the elements of the model's ModuleLists, small ones merged
+        until a launch gives every SIMD unit of the device two wavefronts,
+        unless ``merge_small`` is off); ``ahead``: decode block k+1 on a side
+        stream while block k computes; ``wrap``: after the last block, already
+        decode the first one for the next forward pass."""
         self.manager = manager
         self.wrap = bool(wrap)
         be = manager._be
         groups = _default_blocks(model) if blocks is None else [
             [m for m in b.modules() if isinstance(m, Linear)] for b in blocks]
+        if blocks is None and merge_small:
+            cus = torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+            groups = _merge_small([g for g in groups if g], lambda m: be.numel(m._p._handle), 2 * 4 * cus * 64 * 256)
         self._handles = [[m._p._handle for m in g] for g in groups if g]
         self._where = {}
         for bi, hs in enumerate(self._handles):
             for k, h in enumerate(hs):
                 self._where[h] = (bi, k)
+        self.tensors_per_launch = [len(hs) for hs in self._handles]
         self._plans = [be.batch_plan(hs) for hs in self._handles]
         self._single = {}  # (block, k) -> plan that decodes that one tensor again after a write
         # element offsets of the block's tensors in a slot buffer, 16-byte aligned

@@ -307,7 +307,8 @@ def test_decompress_ahead_decodes_only_the_rewritten_tensor_again():
 
     mgr._be.read_batch = counting
     try:
-        with torch.no_grad(), neuzip_amd.DecompressAhead(mgr, model) as da:
+        # (blocks this small would share one launch: keep them apart, the test is about blocks)
+        with torch.no_grad(), neuzip_amd.DecompressAhead(mgr, model, merge_small=False) as da:
             model(x)
             calls.clear()
             model(x)

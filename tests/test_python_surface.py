@@ -299,3 +299,18 @@ def test_group_geometry_choice_is_one_round_of_workgroups():
         f.manager = Mgr(be)
         f._fit_geometry(group_of(list(sizes)), cus=cus)
         assert f.manager.written == [] and all(g == (131072, 256) for g in be.geo.values())
+
+
+def test_small_blocks_share_a_decode_launch():
+    """DecompressAhead merges consecutive blocks until a launch holds enough
+    elements to fill the device or 16 tensors (host logic, no GPU)."""
+    from neuzip_amd.prefetch import _merge_small
+
+    blocks = [[f"b{i}.{k}" for k in range(4)] for i in range(24)]          # GPT-2-medium: 4 weights, 12.6 M per block
+    size = lambda name: {"0": 3145728, "1": 1048576, "2": 4194304, "3": 4194304}[name[-1]]
+    merged = _merge_small(blocks, size, 2 * 4 * 256 * 64 * 256)
+    assert [len(g) for g in merged] == [12] * 8 and merged[0][:5] == ["b0.0", "b0.1", "b0.2", "b0.3", "b1.0"]
+    big = [[f"l{i}.{k}" for k in range(7)] for i in range(4)]               # an 8B block fills the device by itself
+    assert _merge_small(big, lambda name: 30_000_000, 2 * 4 * 256 * 64 * 256) == big
+    tiny = [[f"t{i}"] for i in range(40)]                                    # never more than 16 tensors per launch
+    assert [len(g) for g in _merge_small(tiny, lambda name: 1000, 10 ** 9)] == [16, 16, 8]
