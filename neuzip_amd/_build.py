@@ -39,8 +39,11 @@ HIPCC_FLAGS = [
 def units(objdir: str):
     """(source, extra flags, object file) of every translation unit."""
     out = [(os.path.join(CSRC, "nz_api.hip"), [], os.path.join(objdir, "nz_api.o"))]
+    # the lossless precision first: its halves take longest, the pool starts them first
     for s in PRECISIONS:
-        out.append((os.path.join(CSRC, "nz_launch.hip"), [f"-DNZ_S={s}"], os.path.join(objdir, f"nz_launch_s{s}.o")))
+        for part, tag in ((0, "enc"), (12, "dec")):
+            out.append((os.path.join(CSRC, "nz_launch.hip"), [f"-DNZ_S={s}", f"-DNZ_PART={part}"],
+                        os.path.join(objdir, f"nz_launch_s{s}_{tag}.o")))
     return out
 
 
@@ -72,7 +75,7 @@ def build(verbose: bool = False) -> str:
             run([hipcc, *HIPCC_FLAGS, *extra, *more, "-c", src, "-o", obj], verbose)
             return obj
 
-        with ThreadPoolExecutor(max_workers=len(tus)) as pool:
+        with ThreadPoolExecutor(max_workers=min(len(tus), os.cpu_count() or 4)) as pool:
             objs = list(pool.map(compile_one, tus))
         run([hipcc, "--offload-arch=gfx950", "-fPIC", "-shared", *objs, "-o", LIB_PATH], verbose)
     return LIB_PATH

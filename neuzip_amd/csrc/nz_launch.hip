@@ -95,16 +95,29 @@ void nz_launch_rows(const NzGeom& g, const void* comp, uint64_t comp_bytes, cons
                        (const uint8_t*)packed, scratch, g, d_status, nm, idx, row_len, cpr);
 }
 
+// NZ_PART (optional) cuts the unit into parts that a build can compile side by side:
+// 0 = the encode kernels, 1 = decode, batch decode and row gather, 2 = the fused products,
+// 12 = both of the latter; undefined = everything.  (Every part parses all of the kernels'
+// source again: on eight cores two parts per precision build fastest, 68 s against 80 s
+// with three and 91 s with one.)
+#if !defined(NZ_PART) || NZ_PART == 0
 template hipError_t nz_allow_encode_lds<NZ_S>();
 template void nz_launch_encode<NZ_S>(const NzEncBatch&, int, dim3, dim3, uint32_t, hipStream_t);
+#endif
+#if !defined(NZ_PART) || NZ_PART == 1 || NZ_PART == 12
 template void nz_launch_decode<NZ_S>(const NzGeom&, const void*, uint64_t, const void*, void*, uint32_t*, const NzNorm&,
                                      uint32_t, hipStream_t);
 template void nz_launch_decode_batch<NZ_S>(const NzBatch&, uint32_t, uint32_t, bool, uint32_t*, hipStream_t);
+#endif
+#if !defined(NZ_PART) || NZ_PART == 2 || NZ_PART == 12
 template void nz_launch_gemv<NZ_S>(const NzBatch&, uint32_t, uint32_t, uint32_t*, hipStream_t);
+#endif
+#if !defined(NZ_PART) || NZ_PART == 1 || NZ_PART == 12
 template void nz_launch_rows<NZ_S>(const NzGeom&, const void*, uint64_t, const void*, uint16_t*, uint32_t*,
                                    const NzNorm&, const long long*, uint32_t, uint32_t, uint32_t, hipStream_t);
+#endif
 
-#if defined(NZ_PROBE_PHASES) && NZ_S == 7
+#if defined(NZ_PROBE_PHASES) && NZ_S == 7 && (!defined(NZ_PART) || NZ_PART == 0)
 // measurement build only: cycles spent per phase of nz_encode_kernel<7, *>, summed over workgroups
 extern "C" int nz_probe_read(unsigned long long* out, int reset) {
   if (hipMemcpyFromSymbol(out, HIP_SYMBOL(nz_probe_acc), sizeof(unsigned long long) * 8) != hipSuccess) return 1;

@@ -30,5 +30,6 @@ def test_device_code_has_no_packed_fp32_forms(tmp_path, source, extra, kernel):
 
 def test_every_precision_has_a_translation_unit(tmp_path):
     units = _build.units(str(tmp_path))
-    assert [u[1] for u in units[1:]] == [[f"-DNZ_S={s}"] for s in (7, 3, 1, 0)]
+    # every precision in two parts (encode; decode family and fused products), compiled side by side
+    assert [u[1] for u in units[1:]] == [[f"-DNZ_S={s}", f"-DNZ_PART={p}"] for s in (7, 3, 1, 0) for p in (0, 12)]
     assert all(os.path.exists(u[0]) for u in units)
