@@ -1117,6 +1117,7 @@ def main():
                 "workload": cfg["workload"],
                 "manager": cfg["manager"],
                 "timed_steps": gargs.steps,
+                "tensors_per_decode_and_write_launch": cfg["tensors_per_decode_and_write_launch"],
                 "tokens_per_s": gm["value"],
                 "ms_per_step_dense_bf16_adamw": cfg["dense_bf16_torch_adamw_ms_per_step"],
                 "ms_per_step_compressed_decode_per_block": pb["ms_per_step"],
