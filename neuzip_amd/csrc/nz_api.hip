@@ -70,7 +70,7 @@ EncLayout enc_layout(const NzGeom& g) {
   L.seg_sbytes = take(g.n_segs * 4);
   L.seg_units = take((g.n_segs + 1) * 4);
   L.chunk_units = take((g.n_chunks + 1) * 4);
-  L.pub = take(g.n_chunks * 16);  // size announcements of the chunks (records placed by the encode kernel)
+  L.pub = take(g.n_chunks * 32);  // size and running-total announcements of the chunks (records placed by the encode kernel)
   L.placed = take(g.n_segs);      // per segment: its record is in the container only
   L.lb_state = take(8);           // run count and abort mark of the announcements
   L.bytes = o;
@@ -1607,6 +1607,8 @@ int nz_manager_import(nz_manager* m, const char* name, const void* host_comp, ui
   if (it != m->entries.end()) {
     // kernels reading the old buffers may still be in flight
     (void)hipDeviceSynchronize();
+    // the outcome of a rewrite that was still pending no longer matters: the entry is replaced
+    // whole (a slot that could not be settled skips entries that are gone)
     (void)settle_entry(m, it->second);
     release_entry(it->second);
     m->entries.erase(it);

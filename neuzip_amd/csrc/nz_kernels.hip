@@ -1126,31 +1126,79 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   // the announcements passes between workgroups: relaxed device-scope
   // accesses, no fences.
   typedef unsigned long long nz_u64;
-  nz_u64* pub = reinterpret_cast<nz_u64*>(it.ws + it.pub);
+  nz_u64* pub = reinterpret_cast<nz_u64*>(it.ws + it.pub);  // four words per chunk: size pair, running-total pair
   const uint32_t mark_a = (uint32_t)(it.nonce >> 32) ^ lb_gen, mark_b = (uint32_t)it.nonce ^ (lb_gen * 0x9E3779B1u);
+  const uint32_t mark_pa = mark_a ^ 0xA5A5A5A5u, mark_pb = mark_b ^ 0x3C3C3C3Cu;  // a size can never pass for a total
   if (tid == 0) {
     const uint32_t u = L.chunk_total;
-    __hip_atomic_store(pub + 2 * c, ((nz_u64)mark_a << 32) | u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(pub + 2 * c + 1, ((nz_u64)mark_b << 32) | (uint32_t)~u, __ATOMIC_RELAXED,
+    __hip_atomic_store(pub + 4 * c, ((nz_u64)mark_a << 32) | u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(pub + 4 * c + 1, ((nz_u64)mark_b << 32) | (uint32_t)~u, __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
   }
   NZ_PROBE_MARK(3);
+  // The chunks before this one, a window of one per thread at a time, nearest first.  A chunk
+  // that has already placed its records has also announced the running total up to and
+  // including itself (below); the nearest such chunk ends the walk, so a workgroup reads the
+  // announcements of the chunks that ran beside it and one total, not those of every chunk
+  // of the tensor.
   uint64_t part = 0;
   bool lost = false;
-  for (uint64_t i = tid; i < c && !lost; i += blockDim.x) {
-    for (uint32_t tries = 0;; ++tries) {
-      const nz_u64 a = __hip_atomic_load(pub + 2 * i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const nz_u64 q = __hip_atomic_load(pub + 2 * i + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if ((uint32_t)(a >> 32) == mark_a && (uint32_t)(q >> 32) == mark_b && (uint32_t)a == (uint32_t)~(uint32_t)q) {
-        part += (uint32_t)a;
-        break;
+  if (c <= blockDim.x) {
+    // every chunk before this one has a thread of its own: their sizes, nothing else
+    if (tid < c) {
+      for (uint32_t tries = 0;; ++tries) {
+        const nz_u64 a = __hip_atomic_load(pub + 4 * tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const nz_u64 q = __hip_atomic_load(pub + 4 * tid + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((uint32_t)(a >> 32) == mark_a && (uint32_t)(q >> 32) == mark_b && (uint32_t)a == (uint32_t)~(uint32_t)q) {
+          part = (uint32_t)a;
+          break;
+        }
+        if (tries >= it.spin_limit) {
+          lost = true;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(8);
       }
-      if (tries >= it.spin_limit) {
-        lost = true;
-        break;
-      }
-      __builtin_amdgcn_s_sleep(8);
     }
+  } else
+  for (uint64_t hi = c; hi > 0;) {
+    const uint64_t lo = hi > blockDim.x ? hi - blockDim.x : 0;
+    const uint64_t i = lo + tid;
+    uint32_t val = 0, key = 0;  // key: position in the window + 1 of an entry that carries a running total
+    if (i < hi) {
+      for (uint32_t tries = 0;; ++tries) {
+        // all four words in flight at once: one round trip per look
+        const nz_u64 a = __hip_atomic_load(pub + 4 * i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const nz_u64 q = __hip_atomic_load(pub + 4 * i + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const nz_u64 pa = __hip_atomic_load(pub + 4 * i + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const nz_u64 pq = __hip_atomic_load(pub + 4 * i + 3, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((uint32_t)(pa >> 32) == mark_pa && (uint32_t)(pq >> 32) == mark_pb &&
+            (uint32_t)pa == (uint32_t)~(uint32_t)pq) {
+          val = (uint32_t)pa;
+          key = (uint32_t)(i - lo) + 1u;
+          break;
+        }
+        if ((uint32_t)(a >> 32) == mark_a && (uint32_t)(q >> 32) == mark_b && (uint32_t)a == (uint32_t)~(uint32_t)q) {
+          val = (uint32_t)a;
+          break;
+        }
+        if (tries >= it.spin_limit) {
+          lost = true;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(8);
+      }
+    }
+    // the same verdict for every thread: did anybody give up, and where is the nearest total
+    const uint32_t verdict = nz_block_max(lost ? 0x80000000u : key, L.red);
+    if (verdict & 0x80000000u) {
+      lost = true;
+      break;
+    }
+    const uint32_t at = (uint32_t)(i - lo) + 1u;  // sizes of the entries after the total, and the total itself
+    if (i < hi && (key ? key == verdict : at > verdict)) part += val;
+    if (verdict) break;
+    hi = lo;
   }
   if (lost) L.gave_up = 1;
 #pragma unroll
@@ -1181,6 +1229,18 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   }
   if (last_chunk && tid == 0)
     __hip_atomic_store(lb_state, lb_gen + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (tid == 0) {
+    // the running total up to and including this chunk, for the chunks that come later (32 bits
+    // of 4-byte units: a container beyond 16 GiB announces none, and its chunks walk on)
+    uint64_t upto = L.chunk_total;
+    for (uint32_t q = 0; q < blockDim.x / 64; ++q) upto += L.red64[q];
+    if (upto <= 0xFFFFFFFFull) {
+      const uint32_t p32 = (uint32_t)upto;
+      __hip_atomic_store(pub + 4 * c + 2, ((nz_u64)mark_pa << 32) | p32, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(pub + 4 * c + 3, ((nz_u64)mark_pb << 32) | (uint32_t)~p32, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
   if (has_seg) {
     uint64_t o0 = 0;
     for (uint32_t q = 0; q < blockDim.x / 64; ++q) o0 += L.red64[q];

@@ -300,3 +300,19 @@ def test_encode_replayed_from_a_graph(oracle):
         assert total == o_comp.size
         assert np.array_equal(comp[:total].cpu().numpy(), o_comp)
         assert np.array_equal(packed.cpu().numpy(), o_packed)
+
+
+@pytest.mark.parametrize("chunk,lane,n", [(8192, 16, 12_000_017), (65536, 256, 80_000_000), (32768, 64, 60_000_001)])
+def test_records_are_placed_across_many_windows_of_chunks(oracle, chunk, lane, n):
+    """More chunks than a workgroup has threads (1465, 1221 and 1832 of them, workgroups
+    of 512 and 256 threads): a chunk finds the records before it from the running
+    total of an earlier chunk plus the sizes of the chunks after that one, over
+    several windows if need be; the container is the oracle's, twice in a row
+    (the second run meets the first run's announcements in the same scratch)."""
+    bits = bf16_bits_normal(n, seed=chunk % 89)
+    o_comp, o_packed = oracle.compress_bf16(bits, 7, chunk, lane, threads=8)
+    for rep in range(2):
+        print(f"case chunk={chunk} lane={lane} n={n} run {rep}", flush=True)
+        comp, packed = gpu_encode(bits, 7, chunk, lane)
+        assert np.array_equal(comp.cpu().numpy(), o_comp)
+        assert np.array_equal(packed.cpu().numpy(), o_packed)
