@@ -362,6 +362,9 @@ struct NzEncLds {
   // for records that go straight to their place: the chunk's record sizes, the
   // sum over the chunks before it, whether the wait for those was given up
   uint32_t seg_units[NZ_MAX_SEGS_PER_CHUNK];
+  // what the wavefronts found for their segments (words, state bytes) and the table's length, for
+  // the thread that sizes the records: the copies in scratch memory are for the kernels that follow
+  uint32_t seg_w[NZ_MAX_SEGS_PER_CHUNK], seg_sb[NZ_MAX_SEGS_PER_CHUNK], tab_len;
   uint32_t chunk_total, gave_up;
   uint32_t redo;  // a wavefront ran out of staging room: the chunk is coded again, into the slots
   uint32_t lb[2];  // the two words of the scratch's announcement state, as thread 0 read them
@@ -553,6 +556,7 @@ __device__ __forceinline__ uint32_t nz_build_table(NzEncLds& L, const uint32_t c
     ci.reserved = 0;
     *info_c = ci;
     L.pad_sym = imax;
+    L.tab_len = padded;
   }
   __syncthreads();
   return est_bits;
@@ -564,18 +568,17 @@ __device__ __forceinline__ uint32_t nz_build_table(NzEncLds& L, const uint32_t c
 // ----------------------------------------------------------------------------
 __device__ __forceinline__ bool nz_chunk_finalize(uint64_t c, uint64_t n, uint32_t chunk_syms,
                                                   uint32_t seg_syms, uint32_t spc, NzChunkInfo* info,
-                                                  const uint32_t* seg_words, const uint32_t* seg_state_bytes,
-                                                  uint32_t* seg_units, uint32_t* chunk_units,
+                                                  const uint32_t* lds_words, const uint32_t* lds_state_bytes,
+                                                  uint32_t tab_len, uint32_t* seg_units, uint32_t* chunk_units,
                                                   uint32_t* lds_seg_units, uint32_t* lds_chunk_total) {
   const uint64_t base = c * chunk_syms;
   const uint32_t cn = (uint32_t)((n - base) < chunk_syms ? (n - base) : chunk_syms);
   const uint32_t nseg = (cn + seg_syms - 1) / seg_syms;
-  const uint32_t tab_len = info[c].tab_len;
   uint64_t rans_total = tab_len, raw_total = 4;
   for (uint32_t k = 0; k < nseg; ++k) {
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
-    const uint32_t w = seg_words[c * spc + k];
-    rans_total += seg_state_bytes[c * spc + k] + 2 * (uint64_t)((w + 1) & ~1u);
+    const uint32_t w = lds_words[k];
+    rans_total += lds_state_bytes[k] + 2 * (uint64_t)((w + 1) & ~1u);
     raw_total += ((sn + 3) & ~3u) + (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
   }
   const bool raw = rans_total >= raw_total;
@@ -583,12 +586,12 @@ __device__ __forceinline__ bool nz_chunk_finalize(uint64_t c, uint64_t n, uint32
   uint32_t chunk_total = 0;  // a record has at most ~2^21 units, a chunk eight records
   for (uint32_t k = 0; k < nseg; ++k) {
     const uint32_t sn = (cn - k * seg_syms) < seg_syms ? (cn - k * seg_syms) : seg_syms;
-    const uint32_t w = seg_words[c * spc + k];
+    const uint32_t w = lds_words[k];
     uint32_t bytes;
     if (raw)
       bytes = (k == 0 ? 4u : 0u) + ((sn + 3) & ~3u) +
               (sn == nz_seg_nominal(chunk_syms, seg_syms, spc, k) ? NZ_CARRY_BYTES : 0u);
-    else bytes = (k == 0 ? tab_len : 0u) + seg_state_bytes[c * spc + k] + 2u * ((w + 1) & ~1u);
+    else bytes = (k == 0 ? tab_len : 0u) + lds_state_bytes[k] + 2u * ((w + 1) & ~1u);
     seg_units[c * spc + k] = bytes / 4;
     lds_seg_units[k] = bytes / 4;
     chunk_total += bytes / 4;
@@ -658,7 +661,8 @@ __device__ __forceinline__ void nz_enc_group(uint32_t& x, uint32_t& pos, const u
 __device__ __forceinline__ void nz_enc_finish(const uint32_t x, const uint32_t words, const uint64_t seg,
                                               uint32_t* __restrict__ sb, const uint32_t lane,
                                               uint32_t* __restrict__ states, uint32_t* __restrict__ seg_words,
-                                              uint32_t* __restrict__ seg_state_bytes) {
+                                              uint32_t* __restrict__ seg_state_bytes, uint32_t* lds_words,
+                                              uint32_t* lds_state_bytes) {
   const uint32_t code = (x >> 20 ? 1u : 0u) + (x >> 24 ? 1u : 0u) + (x >> 28 ? 1u : 0u);
   const uint32_t nn = 5u + code;
   const uint32_t incl = nz_wave_scan(nn, lane);
@@ -679,6 +683,8 @@ __device__ __forceinline__ void nz_enc_finish(const uint32_t x, const uint32_t w
   if (lane == 0) {
     seg_words[seg] = words;
     seg_state_bytes[seg] = sbytes;
+    *lds_words = words;
+    *lds_state_bytes = sbytes;
   }
 }
 
@@ -1055,7 +1061,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     });
     if (out_of_room) return true;
     nz_enc_finish(x, cap_words - pos, seg, L.sbuf[wave], lane, reinterpret_cast<uint32_t*>(it.ws + it.states),
-                  seg_words, seg_state_bytes);
+                  seg_words, seg_state_bytes, &L.seg_w[wave], &L.seg_sb[wave]);
     pos_end = pos;
     return false;
   };
@@ -1077,7 +1083,7 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   NZ_PROBE_MARK(2);
   // decide coded-or-raw and size the records
   if (tid == 0) {
-    L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
+    L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, L.seg_w, L.seg_sb, L.tab_len, seg_units,
                               reinterpret_cast<uint32_t*>(it.ws + it.chunk_units), L.seg_units, &L.chunk_total);
     L.gave_up = 0;
   }
@@ -1247,7 +1253,12 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     for (uint32_t q = 0; q < wave; ++q) o0 += L.seg_units[q];
     const bool from_stage = staged && !L.raw;
     const uint16_t* words = from_stage ? reinterpret_cast<const uint16_t*>(stage) + (pos_end - stage_lo) : slot + pos_end;
-    const bool fits = nz_move_record<64>(it, seg, c, wave, o0, L.seg_units[wave], info[c], seg_state_bytes[seg],
+    NzChunkInfo ci;  // as nz_build_table and nz_chunk_finalize left it in scratch memory, from LDS
+    ci.tab_len = L.tab_len;
+    ci.pad_sym = L.pad_sym;
+    ci.raw = L.raw ? 1u : 0u;
+    ci.reserved = 0;
+    const bool fits = nz_move_record<64>(it, seg, c, wave, o0, L.seg_units[wave], ci, L.seg_sb[wave],
                                          cap_words - pos_end, words, nullptr, lane);
     if (from_stage && !fits) unstage();
     if (lane == 0) placed[seg] = (from_stage && fits) ? 1 : 0;
@@ -1355,11 +1366,11 @@ __global__ __launch_bounds__(NZ_ENC_LONG_THREADS) void nz_encode_long_kernel(con
       nz_enc_group<false>(x, pos, sy, L.tab, slot, 0u);
     }
     nz_enc_finish(x, cap_words - pos, seg, L.sbuf[wave], lane, reinterpret_cast<uint32_t*>(it.ws + it.states),
-                  seg_words, seg_state_bytes);
+                  seg_words, seg_state_bytes, &L.seg_w[wave], &L.seg_sb[wave]);
   }
   __threadfence_block();
   __syncthreads();
-  if (tid == 0) L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, seg_words, seg_state_bytes, seg_units,
+  if (tid == 0) L.raw = nz_chunk_finalize(c, n, chunk_syms, seg_syms, spc, info, L.seg_w, L.seg_sb, L.tab_len, seg_units,
                                           reinterpret_cast<uint32_t*>(it.ws + it.chunk_units), L.seg_units,
                                           &L.chunk_total);
   __syncthreads();
