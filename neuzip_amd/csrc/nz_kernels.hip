@@ -453,7 +453,11 @@ __device__ __forceinline__ uint32_t nz_build_table(NzEncLds& L, const uint32_t c
   }
   const uint32_t live = cnt > 0;
   const uint32_t k = nz_block_sum(live, L.red);
-  uint32_t f = live ? 1u + (uint32_t)(((uint64_t)cnt * (NZ_M - k)) / cn) : 0u;
+  // cnt * (4096 - k) fits 32 bits for chunks of up to 2^19 symbols (every geometry the library
+  // chooses itself): a 32-bit division then, a fraction of the 64-bit one's instructions
+  uint32_t f = 0;
+  if (cn <= (1u << 19)) f = live ? 1u + (cnt * (NZ_M - k)) / cn : 0u;
+  else f = live ? 1u + (uint32_t)(((uint64_t)cnt * (NZ_M - k)) / cn) : 0u;
   const uint32_t sum = nz_block_sum(f, L.red);
   // most frequent symbol, lowest index on ties (cnt <= 2^24 fits above the index byte)
   const uint32_t key = nz_block_max(own ? ((cnt << 8) | (255u - tid)) : 0u, L.red);
