@@ -1029,9 +1029,17 @@ int refuse_under_capture(hipStream_t st, bool may_block, const char* what) {
 // is ordered by the graph's owner.
 int order_scratch_use(nz_manager* m, hipStream_t st) {
   if (capturing(st)) return NZ_OK;
-  if (m->has_stream && m->last_stream != st) {
-    NZ_HIP(hipEventRecord(m->order_ev, m->last_stream));
-    NZ_HIP(hipStreamWaitEvent(st, m->order_ev, 0));
+  if (m->has_stream && m->last_stream != st && !capturing(m->last_stream)) {
+    // (a stream that has gone into capture since its last call here is left alone: an event
+    // recorded on it now would become part of its graph)
+    if (hipEventRecord(m->order_ev, m->last_stream) == hipSuccess) {
+      NZ_HIP(hipStreamWaitEvent(st, m->order_ev, 0));
+    } else {
+      // the stream of the call before is gone (destroyed by its owner): whatever it was given
+      // has to be finished the slow way
+      (void)hipGetLastError();
+      NZ_HIP(hipDeviceSynchronize());
+    }
   }
   m->last_stream = st;
   m->has_stream = true;
