@@ -61,6 +61,8 @@ class _HipBackend:
         self._no_run = set()    # first handles whose run did not repeat itself
         self._parked = {}       # handle -> (activation, its version, result, first handle, bias) computed ahead
         self._cur = None        # the run being observed: (activation, its version, [(handle, rows, bias)])
+        self._parked_w = {}     # handle -> (activation, its version, decoded weight, first handle): decoded ahead
+        self._plans = {}        # first handle of a run -> read_batch plan of its handles
 
     def close(self):
         if getattr(self, "_h", None) is not None and self._h:
@@ -88,7 +90,9 @@ class _HipBackend:
         if flat.data_ptr() % 16:
             flat = flat.clone()
         self._known.pop(handle, None)
-        self._parked.clear()  # products computed ahead from the weights as they were
+        self._parked.clear()  # products and weights computed ahead from the weights as they were
+        self._parked_w.clear()
+        self._plans.clear()   # (a plan holds the element counts of its tensors)
         stream = torch.cuda.current_stream(flat.device)
         rc = self._L.nz_manager_write(self._h, handle.encode(), flat.data_ptr(), flat.numel(), code,
                                       stream.cuda_stream)
@@ -113,6 +117,8 @@ class _HipBackend:
             for h in hs:
                 self._known.pop(h, None)
             self._parked.clear()
+            self._parked_w.clear()
+            self._plans.clear()
             names = (ctypes.c_char_p * k)(*[h.encode() for h in hs])
             ptrs = (ctypes.c_void_p * k)(*[f.data_ptr() for f in fs])
             ns = (ctypes.c_uint64 * k)(*[f.numel() for f in fs])
@@ -319,6 +325,9 @@ class _HipBackend:
             del self._member_of[h]
         for h in [h for h, hit in self._parked.items() if hit[3] == leader]:
             del self._parked[h]
+        for h in [h for h, hit in self._parked_w.items() if hit[3] == leader]:
+            del self._parked_w[h]
+        self._plans.pop(leader, None)
 
     def _observe(self, handle: str, inputs: torch.Tensor, rows: int, bias) -> None:
         """one more call that was served on its own: does it continue the current run?"""
@@ -390,15 +399,59 @@ class _HipBackend:
             self._observe(handle, inputs, shape[0], bias)
         return out.view(*inputs.shape[:-1], shape[0])
 
+    def _weight_for_gemm(self, handle: str, inputs: torch.Tensor, shape, bias) -> torch.Tensor:
+        """The dense weight of ``handle`` for a call with more rows than the fused
+        product takes.  The runs of Linears that share their activation are learned
+        here as well, and the first call of a learned run decodes the weights of
+        the whole run with ONE launch (matrices of a few million elements cannot
+        fill the device on their own); the others wait, keyed on the activation
+        tensor, for the calls that follow."""
+        hit = self._parked_w.pop(handle, None)
+        if hit is not None:
+            x0, version, w, leader = hit
+            if x0 is inputs and version == inputs._version:
+                return w
+            self._forget_run(leader)
+        elif self._parked_w:
+            # a call that no decoded weight is waiting for: what waits belongs to a run that did not repeat itself
+            for _, _, _, leader in list(self._parked_w.values()):
+                self._forget_run(leader)
+        eligible = (self.group_rows and self.fused_rows and inputs.is_cuda and len(shape) == 2
+                    and not (torch.is_grad_enabled() and inputs.requires_grad))
+        run = self._runs.get(handle) if eligible else None
+        if run is not None:
+            handles, _, rows, _ = run
+            self._close_run()
+            plan = self._plans.get(handle)
+            if plan is None:
+                plan = self._plans[handle] = self.batch_plan(handles)
+            sizes = [int(c) for c in plan[1]]
+            flat = torch.empty(sum((n + 7) & ~7 for n in sizes), dtype=torch.bfloat16, device=self._device)
+            outs, at = [], 0
+            for n in sizes:
+                outs.append(flat[at:at + n])
+                at += (n + 7) & ~7
+            try:
+                self.read_batch(plan, outs)
+            except (ValueError, RuntimeError):
+                self._forget_run(handle)
+            else:
+                for h, o, r in zip(handles[1:], outs[1:], rows[1:]):
+                    self._parked_w[h] = (inputs, inputs._version, o.view(r, -1), handle)
+                return outs[0].view(shape)
+        if eligible and handle not in self._member_of:
+            self._observe(handle, inputs, shape[0], bias)
+        return self.read(handle).view(shape)
+
     def linear(self, handle: str, inputs: torch.Tensor, shape, bias: torch.Tensor) -> torch.Tensor:
         # cuda/high_level.cu:252-257: addmm(bias, input, W^T).  The reference only
         # accepts a 2-D input here; inputs with leading batch dimensions take
-        # the equivalent F.linear route.  A single activation row (single-token
-        # inference) is served by the fused decode-and-multiply kernel.
+        # the equivalent F.linear route.  One to eight activation rows (single-token
+        # inference, a small batch) are served by the fused decode-and-multiply kernel.
         fused = self._fused_row(handle, inputs, shape, bias)
         if fused is not None:
             return fused
-        weight = self.read(handle).view(shape)
+        weight = self._weight_for_gemm(handle, inputs, shape, bias)
         if inputs.dim() == 2:
             return torch.addmm(bias, inputs, weight.t())
         return torch.nn.functional.linear(inputs, weight, bias)
@@ -408,7 +461,7 @@ class _HipBackend:
         fused = self._fused_row(handle, inputs, shape, None)
         if fused is not None:
             return fused
-        weight = self.read(handle).view(shape)
+        weight = self._weight_for_gemm(handle, inputs, shape, None)
         return torch.matmul(inputs, weight.t())
 
     def split(self, tensor: torch.Tensor):

@@ -439,3 +439,63 @@ def test_runs_of_calls_that_share_their_activation_are_learned_and_checked():
         x = torch.randn(cols, device="cuda").to(torch.bfloat16)
         assert torch.equal(mgr.linear(hs[2], x), alone(mgr, hs[2], x))
         mgr._be.check()
+
+
+def test_runs_share_a_decode_launch_when_there_are_many_rows():
+    """More rows than the fused product takes: decompress-then-GEMM, and Linears
+    that share their activation have their weights decoded by one launch from the
+    second time on.  Results equal torch's linear on the stored weights bit for
+    bit; a decoded weight computed ahead is used only for the same activation."""
+    import neuzip_amd
+
+    cols = 1024
+    ws = [(torch.randn(r, cols, device="cuda") * 0.02).to(torch.bfloat16) for r in (768, 256, 256, 512)]
+    bias = torch.randn(256, device="cuda").to(torch.bfloat16)
+    mgr = neuzip_amd.Manager(precision=7)
+    hs = [mgr.write(w) for w in ws]
+    calls = []
+    real = mgr._be.read_batch
+
+    def counting(plan, outs):
+        calls.append(plan[2])
+        return real(plan, outs)
+
+    mgr._be.read_batch = counting
+    try:
+        with torch.no_grad():
+            for rep in range(3):
+                x = torch.randn(3, 16, cols, device="cuda").to(torch.bfloat16)
+                y = [mgr.linear(hs[0], x), mgr.linear(hs[1], x, bias), mgr.linear(hs[2], x)]
+                z = mgr.linear(hs[3], torch.randn(40, cols, device="cuda").to(torch.bfloat16))
+                for k, b in ((0, None), (1, bias), (2, None)):
+                    assert torch.equal(y[k], torch.nn.functional.linear(x, ws[k], b)), (rep, k)
+                assert z.shape == (40, 512)
+            assert calls == [3, 3]                      # passes two and three: one launch for the run of three
+            assert [r[0] for r in mgr._be._runs.values()] == [hs[:3]] and not mgr._be._parked_w
+            # the same run serves single rows as well (learned once, whatever the number of rows)
+            x1 = torch.randn(cols, device="cuda").to(torch.bfloat16)
+            y1 = [mgr.linear(hs[0], x1), mgr.linear(hs[1], x1, bias), mgr.linear(hs[2], x1)]
+            mgr.group_rows = False
+            assert all(torch.equal(a, mgr.linear(h, x1, b)) for a, h, b in zip(y1, hs, (None, bias, None)))
+            mgr.group_rows = True
+            # a weight decoded ahead is not used for another activation; the run is forgotten
+            x = torch.randn(20, cols, device="cuda").to(torch.bfloat16)
+            mgr.linear(hs[0], x)
+            other = torch.randn(20, cols, device="cuda").to(torch.bfloat16)
+            assert torch.equal(mgr.linear(hs[1], other, bias), torch.nn.functional.linear(other, ws[1], bias))
+            assert not mgr._be._runs and not mgr._be._parked_w
+            # a rewrite between two calls of a run: the new weight is what the next call sees
+            mgr2 = neuzip_amd.Manager(precision=7)
+            h2 = [mgr2.write(w) for w in ws]
+            for rep in range(2):
+                x = torch.randn(12, cols, device="cuda").to(torch.bfloat16)
+                mgr2.linear(h2[0], x), mgr2.linear(h2[1], x, bias), mgr2.linear(h2[2], x)
+            x = torch.randn(12, cols, device="cuda").to(torch.bfloat16)
+            mgr2.linear(h2[0], x)
+            w_new = (ws[1].float() * 0.5).to(torch.bfloat16)
+            mgr2.write(w_new, h2[1])
+            assert torch.equal(mgr2.linear(h2[1], x, bias), torch.nn.functional.linear(x, w_new, bias))
+            mgr2._be.check()
+    finally:
+        del mgr._be.read_batch
+    mgr._be.check()
