@@ -948,8 +948,12 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
     return (seg_full && sb >= keep) ? carry_seg + (sb - keep) : pk + sb;
   };
   const auto count8 = [&](uint64_t e) {
+#ifndef NZ_PROBE_NO_HIST
 #pragma unroll
     for (int j = 0; j < 8; ++j) atomicAdd(&myhist[(uint32_t)(e >> (8 * j)) & 0xFFu], 1u);
+#else  // measurement build: the split phase without its histogram (the kernel ends after the phase)
+    asm volatile("" ::"v"((uint32_t)e), "v"((uint32_t)(e >> 32)));
+#endif
   };
   typedef uint32_t nz_u32x4 __attribute__((ext_vector_type(4)));
   // Four groups at a time, and the loads of the next four are issued before the
@@ -1013,6 +1017,9 @@ __global__ __launch_bounds__(64 * NZ_MAX_SEGS_PER_CHUNK, 4) void nz_encode_kerne
   __threadfence_block();  // the carried bytes are read back below
   __syncthreads();
   NZ_PROBE_MARK(0);
+#ifdef NZ_PROBE_NO_HIST
+  return;
+#endif
 
   // ---- the chunk's table ----
   const uint32_t est_bits = nz_build_table(L, cn, it.ws + it.tab_ser + c * NZ_TABLE_MAX_BYTES, info + c);
