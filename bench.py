@@ -531,6 +531,7 @@ def llama8b_measure(args, torch, full):
     measure("unchanged_caller_graph", capture())
     # decompress-then-GEMM for every call, the reference's own route (bit-equal to dense)
     mgr.fused_rows = False
+    mgr.decode_ahead = False
     measure("per_linear_eager")
     measure("per_linear_graph", capture())
     for ahead in ((False, True) if full else ()):
@@ -547,6 +548,7 @@ def llama8b_measure(args, torch, full):
     # decode fused into the matrix-vector product, Linears that share an input in one launch
     # (single-token steps only; the prefill keeps the decompress-then-GEMM path)
     mgr.fused_rows = True
+    mgr.decode_ahead = True
     fused = neuzip_amd.FusedGemv(mgr, model)
     with torch.no_grad():
         model.prefill_static(prompt, kcs, vcs)
@@ -737,7 +739,15 @@ def gpt2m_measure(args, torch):
     per_block["steps_with_the_dense_runs_loss"] = f"{same} of {len(dense_losses)}"
     per_block["dense_first_loss"] = round(float(dense_losses[args.warmup]), 4)
     per_block["dense_last_loss"] = round(float(dense_losses[-1]), 4)
+    mgr.decode_ahead = False  # the reference's granularity: every request decodes its own tensor
     per_linear, _, _ = run(1)
+    # the same loop, nothing but the reference's calls, with the manager's default: a request
+    # decodes the weights it has learned to expect next in the same launch
+    mgr.decode_ahead = True
+    per_linear_learned, _, _ = run(1)
+    hits, waste = mgr._be.ahead_stats()
+    per_linear_learned["weights_decoded_ahead_used"] = hits
+    per_linear_learned["weights_decoded_ahead_dropped"] = waste
     mgr._be.check()
     # writes that went into the entries' existing buffers (no allocation, no wait for the size)
     in_place, outgrown = be.rewrite_stats()
@@ -795,6 +805,7 @@ def gpt2m_measure(args, torch):
             "tensors_per_decode_and_write_launch": per_launch,
             "decode_per_block": per_block,
             "decode_per_linear": per_linear,
+            "decode_per_linear_order_learned": per_linear_learned,
             "lockstep_check_lossless": lockstep,
             "rewrites": rewrites,
             "compressed_tensors": n_comp,
@@ -1122,8 +1133,10 @@ def main():
                 "ms_per_step_dense_bf16_adamw": cfg["dense_bf16_torch_adamw_ms_per_step"],
                 "ms_per_step_compressed_decode_per_block": pb["ms_per_step"],
                 "ms_per_step_compressed_decode_per_linear": cfg["decode_per_linear"]["ms_per_step"],
+                "ms_per_step_compressed_unchanged_caller": cfg["decode_per_linear_order_learned"]["ms_per_step"],
                 "codec_share_of_step_per_block": pb["codec_share_of_step"],
                 "codec_share_of_step_per_linear": cfg["decode_per_linear"]["codec_share_of_step"],
+                "codec_share_of_step_unchanged_caller": cfg["decode_per_linear_order_learned"]["codec_share_of_step"],
                 "steps_with_the_dense_runs_loss": pb["steps_with_the_dense_runs_loss"],
                 "rewrites": cfg["rewrites"],
                 "lockstep_check_lossless": cfg["lockstep_check_lossless"],

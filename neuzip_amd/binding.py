@@ -61,8 +61,14 @@ class _HipBackend:
         self._no_run = set()    # first handles whose run did not repeat itself
         self._parked = {}       # handle -> (activation, its version, result, first handle, bias) computed ahead
         self._cur = None        # the run being observed: (activation, its version, [(handle, rows, bias)])
-        self._parked_w = {}     # handle -> (activation, its version, decoded weight, first handle): decoded ahead
-        self._plans = {}        # first handle of a run -> read_batch plan of its handles
+        self.decode_ahead = True  # dense weights: decode the handles that are asked for next in the same launch
+        self._next = {}         # (handle asked for before, handle) -> the handle that was asked for after them
+        self._last2 = (None, None)  # the two handles whose dense weight was asked for last
+        self._ahead = {}        # handle -> (decoded weight, stream it was decoded on), waiting to be asked for
+        self._plans = {}        # tuple of handles -> read_batch plan
+        self._ahead_hits = self._ahead_waste = 0
+        cus = torch.cuda.get_device_properties(self._device).multi_processor_count
+        self.ahead_fill = 2 * 4 * cus * 64 * 256  # elements that give every SIMD unit two wavefronts
 
     def close(self):
         if getattr(self, "_h", None) is not None and self._h:
@@ -89,10 +95,7 @@ class _HipBackend:
         flat = tensor.detach().contiguous().view(-1)
         if flat.data_ptr() % 16:
             flat = flat.clone()
-        self._known.pop(handle, None)
-        self._parked.clear()  # products and weights computed ahead from the weights as they were
-        self._parked_w.clear()
-        self._plans.clear()   # (a plan holds the element counts of its tensors)
+        self._stored_anew(handle)
         stream = torch.cuda.current_stream(flat.device)
         rc = self._L.nz_manager_write(self._h, handle.encode(), flat.data_ptr(), flat.numel(), code,
                                       stream.cuda_stream)
@@ -115,10 +118,7 @@ class _HipBackend:
             hs, fs = handles[at:at + 16], flats[at:at + 16]
             k = len(hs)
             for h in hs:
-                self._known.pop(h, None)
-            self._parked.clear()
-            self._parked_w.clear()
-            self._plans.clear()
+                self._stored_anew(h)
             names = (ctypes.c_char_p * k)(*[h.encode() for h in hs])
             ptrs = (ctypes.c_void_p * k)(*[f.data_ptr() for f in fs])
             ns = (ctypes.c_uint64 * k)(*[f.numel() for f in fs])
@@ -129,7 +129,16 @@ class _HipBackend:
                     f.record_stream(stream)
             _lib.raise_for(rc)
 
-    def read(self, handle: str) -> torch.Tensor:
+    def _stored_anew(self, handle: str) -> None:
+        """``handle`` is about to hold other values: nothing derived from the old ones survives"""
+        self._known.pop(handle, None)
+        self._parked.clear()  # products computed ahead from the weights as they were
+        self._ahead.pop(handle, None)
+        if any(handle in key for key in self._plans):  # a plan holds the element counts of its tensors
+            self._plans = {key: plan for key, plan in self._plans.items() if handle not in key}
+
+    def _meta(self, handle: str):
+        """(encoded name, element count) of a stored handle"""
         known = self._known.get(handle)
         if known is None:
             n = ctypes.c_uint64()
@@ -137,7 +146,10 @@ class _HipBackend:
             name = handle.encode()
             _lib.raise_for(self._L.nz_manager_meta(self._h, name, ctypes.byref(n), ctypes.byref(dt)))
             known = self._known[handle] = (name, int(n.value))
-        name, numel = known
+        return known
+
+    def read(self, handle: str) -> torch.Tensor:
+        name, numel = self._meta(handle)
         out = torch.empty(numel, dtype=torch.bfloat16, device=self._device)
         rc = self._L.nz_manager_read(self._h, name, out.data_ptr(), numel, _stream_ptr(self._device))
         _lib.raise_for(rc)
@@ -248,7 +260,7 @@ class _HipBackend:
         comp = comp.detach().to("cpu", torch.uint8).contiguous()
         packed = packed.detach().to("cpu", torch.uint8).contiguous()
         norm = torch.empty(0, dtype=torch.uint8) if norm is None else norm.detach().to("cpu", torch.uint8).contiguous()
-        self._known.pop(handle, None)
+        self._stored_anew(handle)
         rc = self._L.nz_manager_import(self._h, handle.encode(), comp.data_ptr(), comp.numel(),
                                        packed.data_ptr() if packed.numel() else None, packed.numel(),
                                        norm.data_ptr() if norm.numel() else None, norm.numel(),
@@ -266,6 +278,7 @@ class _HipBackend:
         return int(self._L.nz_manager_packed_bytes(self._h, handle.encode()))
 
     def trim(self) -> None:
+        self._ahead.clear()
         _lib.raise_for(self._L.nz_manager_trim(self._h))
 
     def rewrite_stats(self):
@@ -325,9 +338,6 @@ class _HipBackend:
             del self._member_of[h]
         for h in [h for h, hit in self._parked.items() if hit[3] == leader]:
             del self._parked[h]
-        for h in [h for h, hit in self._parked_w.items() if hit[3] == leader]:
-            del self._parked_w[h]
-        self._plans.pop(leader, None)
 
     def _observe(self, handle: str, inputs: torch.Tensor, rows: int, bias) -> None:
         """one more call that was served on its own: does it continue the current run?"""
@@ -399,49 +409,103 @@ class _HipBackend:
             self._observe(handle, inputs, shape[0], bias)
         return out.view(*inputs.shape[:-1], shape[0])
 
+    # -- dense weights: the handles that are asked for next share the launch -----
+    #
+    # A model asks for its weights in the same order pass after pass (forwards
+    # through the blocks, backwards through them in training).  The order is
+    # learned as "after handles a, b came c"; a request that finds nothing
+    # waiting follows those links and decodes the handles it expects next with
+    # the same launch, until the launch would fill the device (matrices of a few
+    # million elements cannot on their own).  The others wait for their requests.
+    # A weight that waits is dropped when its handle is written, so what is handed
+    # out always equals a decode at the time of the request; a request that was
+    # not foreseen drops everything that waits, and a manager whose requests keep
+    # coming in another order than learned stops decoding ahead.  Requests made
+    # while a stream is being captured take no part in any of this.
+
+    _MAX_AHEAD = 16  # tensors one decode launch takes (NZ_BATCH_MAX)
+
+    def _dense_weight(self, handle: str) -> torch.Tensor:
+        """the decoded weight of ``handle`` (flat), possibly a view of a buffer it shares with its neighbours"""
+        if torch.cuda.is_current_stream_capturing():
+            # a weight that waits across the end of a capture would be memory of the graph's
+            # pool that no kernel has filled yet, and one decoded before the capture would be
+            # baked into the graph by address: a captured request decodes its own tensor
+            self._ahead.clear()
+            self._last2 = (None, None)
+            return self.read(handle)
+        before, last = self._last2
+        if last is not None:
+            self._next[(before, last)] = handle
+        self._last2 = (last, handle)
+        hit = self._ahead.pop(handle, None)
+        if hit is not None:
+            w, decoded_on = hit
+            self._ahead_hits += 1
+            now = torch.cuda.current_stream(self._device)
+            if now != decoded_on:
+                now.wait_stream(decoded_on)
+                w.record_stream(now)
+            return w
+        if self._ahead:  # not what was expected next
+            self._ahead_waste += len(self._ahead)
+            self._ahead.clear()
+            if self._ahead_waste > 64 and self._ahead_waste > self._ahead_hits:
+                self.decode_ahead = False
+        if not self.decode_ahead:
+            return self.read(handle)
+        chain, total, a, b = [handle], self._meta(handle)[1], last, handle
+        while len(chain) < self._MAX_AHEAD and total < self.ahead_fill:
+            nxt = self._next.get((a, b))
+            if nxt is None or nxt in chain:
+                break
+            try:
+                total += self._meta(nxt)[1]
+            except RuntimeError:
+                break  # no longer stored
+            chain.append(nxt)
+            a, b = b, nxt
+        if len(chain) == 1:
+            return self.read(handle)
+        key = tuple(chain)
+        plan = self._plans.get(key)
+        if plan is None:
+            plan = self._plans[key] = self.batch_plan(chain)
+        sizes = [int(c) for c in plan[1]]
+        flat = torch.empty(sum((n + 7) & ~7 for n in sizes), dtype=torch.bfloat16, device=self._device)
+        outs, at = [], 0
+        for n in sizes:
+            outs.append(flat[at:at + n])
+            at += (n + 7) & ~7
+        try:
+            self.read_batch(plan, outs)
+        except (ValueError, RuntimeError):  # e.g. scratch that cannot grow while a graph is captured
+            self._plans.pop(key, None)
+            return self.read(handle)
+        stream = torch.cuda.current_stream(self._device)
+        for h, o in zip(chain[1:], outs[1:]):
+            self._ahead[h] = (o, stream)
+        return outs[0]
+
+    def read_shared(self, handle: str) -> torch.Tensor:
+        """The decoded weight for a caller that only reads it and drops it at once."""
+        return self._dense_weight(handle)
+
+    def ahead_stats(self):
+        """(weights decoded ahead that were asked for, weights decoded ahead and dropped unused)"""
+        return self._ahead_hits, self._ahead_waste
+
     def _weight_for_gemm(self, handle: str, inputs: torch.Tensor, shape, bias) -> torch.Tensor:
         """The dense weight of ``handle`` for a call with more rows than the fused
         product takes.  The runs of Linears that share their activation are learned
-        here as well, and the first call of a learned run decodes the weights of
-        the whole run with ONE launch (matrices of a few million elements cannot
-        fill the device on their own); the others wait, keyed on the activation
-        tensor, for the calls that follow."""
-        hit = self._parked_w.pop(handle, None)
-        if hit is not None:
-            x0, version, w, leader = hit
-            if x0 is inputs and version == inputs._version:
-                return w
-            self._forget_run(leader)
-        elif self._parked_w:
-            # a call that no decoded weight is waiting for: what waits belongs to a run that did not repeat itself
-            for _, _, _, leader in list(self._parked_w.values()):
-                self._forget_run(leader)
-        eligible = (self.group_rows and self.fused_rows and inputs.is_cuda and len(shape) == 2
-                    and not (torch.is_grad_enabled() and inputs.requires_grad))
-        run = self._runs.get(handle) if eligible else None
-        if run is not None:
-            handles, _, rows, _ = run
-            self._close_run()
-            plan = self._plans.get(handle)
-            if plan is None:
-                plan = self._plans[handle] = self.batch_plan(handles)
-            sizes = [int(c) for c in plan[1]]
-            flat = torch.empty(sum((n + 7) & ~7 for n in sizes), dtype=torch.bfloat16, device=self._device)
-            outs, at = [], 0
-            for n in sizes:
-                outs.append(flat[at:at + n])
-                at += (n + 7) & ~7
-            try:
-                self.read_batch(plan, outs)
-            except (ValueError, RuntimeError):
-                self._forget_run(handle)
-            else:
-                for h, o, r in zip(handles[1:], outs[1:], rows[1:]):
-                    self._parked_w[h] = (inputs, inputs._version, o.view(r, -1), handle)
-                return outs[0].view(shape)
-        if eligible and handle not in self._member_of:
-            self._observe(handle, inputs, shape[0], bias)
-        return self.read(handle).view(shape)
+        here as well (for the calls with few rows that may follow)."""
+        if (self.group_rows and self.fused_rows and inputs.is_cuda and len(shape) == 2
+                and not (torch.is_grad_enabled() and inputs.requires_grad)):
+            if handle in self._runs:
+                self._close_run()
+            elif handle not in self._member_of:
+                self._observe(handle, inputs, shape[0], bias)
+        return self._dense_weight(handle).view(shape)
 
     def linear(self, handle: str, inputs: torch.Tensor, shape, bias: torch.Tensor) -> torch.Tensor:
         # cuda/high_level.cu:252-257: addmm(bias, input, W^T).  The reference only
@@ -602,6 +666,8 @@ class Manager:
         """Like ``read``, but the result may be a view of a buffer that the next
         call on this manager reuses: for callers that only read the weight and
         drop it at once (the backward pass of a compressed Linear)."""
+        if hasattr(self._be, "read_shared"):
+            return self._be.read_shared(handle).requires_grad_(False).reshape(self.meta_dict[handle])
         return self.read(handle)
 
     def size(self, handle: str, reference_accounting: bool = False) -> int:
@@ -648,6 +714,23 @@ class Manager:
     def group_rows(self, on: bool) -> None:
         if hasattr(self._be, "group_rows"):
             self._be.group_rows = bool(on)
+
+    @property
+    def decode_ahead(self) -> bool:
+        """Whether a request for a dense weight (a ``linear`` call with many rows,
+        the backward pass of a compressed Linear) also decodes, in the same launch,
+        the weights that were asked for next the last time round, until the launch
+        fills the device.  What is handed out always equals a decode at the time
+        of the request: a write drops the weight that waits for its handle.  Turns
+        itself off on a manager whose requests do not repeat their order."""
+        return bool(getattr(self._be, "decode_ahead", False))
+
+    @decode_ahead.setter
+    def decode_ahead(self, on: bool) -> None:
+        if hasattr(self._be, "decode_ahead"):
+            self._be.decode_ahead = bool(on)
+            if not on:
+                self._be._ahead.clear()
 
     def gather_rows(self, handle: str, indices: torch.Tensor) -> torch.Tensor:
         """Rows ``indices`` of the stored 2-D table ``handle`` as ``[indices.numel(), row_len]``

@@ -441,11 +441,13 @@ def test_runs_of_calls_that_share_their_activation_are_learned_and_checked():
         mgr._be.check()
 
 
-def test_runs_share_a_decode_launch_when_there_are_many_rows():
-    """More rows than the fused product takes: decompress-then-GEMM, and Linears
-    that share their activation have their weights decoded by one launch from the
-    second time on.  Results equal torch's linear on the stored weights bit for
-    bit; a decoded weight computed ahead is used only for the same activation."""
+def test_dense_weights_asked_for_in_a_repeating_order_share_decode_launches():
+    """More rows than the fused product takes: decompress-then-GEMM.  The order in
+    which dense weights are asked for is learned, and a request that finds nothing
+    waiting decodes the handles expected next in the same launch.  Results equal
+    torch's linear on the stored weights bit for bit, whatever was decoded ahead:
+    a write drops the weight that waits for its handle, an unforeseen request
+    drops all that wait, and a manager whose order does not repeat stops."""
     import neuzip_amd
 
     cols = 1024
@@ -460,42 +462,129 @@ def test_runs_share_a_decode_launch_when_there_are_many_rows():
         calls.append(plan[2])
         return real(plan, outs)
 
+    def lin(x, k, b=None, w=None):
+        got = mgr.linear(hs[k], x, b)
+        assert torch.equal(got, torch.nn.functional.linear(x, ws[k] if w is None else w, b)), k
+        return got
+
     mgr._be.read_batch = counting
     try:
         with torch.no_grad():
             for rep in range(3):
                 x = torch.randn(3, 16, cols, device="cuda").to(torch.bfloat16)
-                y = [mgr.linear(hs[0], x), mgr.linear(hs[1], x, bias), mgr.linear(hs[2], x)]
-                z = mgr.linear(hs[3], torch.randn(40, cols, device="cuda").to(torch.bfloat16))
-                for k, b in ((0, None), (1, bias), (2, None)):
-                    assert torch.equal(y[k], torch.nn.functional.linear(x, ws[k], b)), (rep, k)
-                assert z.shape == (40, 512)
-            assert calls == [3, 3]                      # passes two and three: one launch for the run of three
-            assert [r[0] for r in mgr._be._runs.values()] == [hs[:3]] and not mgr._be._parked_w
-            # the same run serves single rows as well (learned once, whatever the number of rows)
+                lin(x, 0), lin(x, 1, bias), lin(x, 2)
+                lin(torch.randn(40, cols, device="cuda").to(torch.bfloat16), 3)
+            # pass one learns; in pass two the second request knows what follows (the four tensors
+            # are far too small to fill the device, so the launch takes all of them, the first
+            # weight of the next pass included); pass three finds that one waiting
+            assert calls == [4, 4]
+            assert mgr._be.ahead_stats() == (5, 0)
+            # the runs of calls that share their activation were learned on the way, for single rows
+            assert [r[0] for r in mgr._be._runs.values()] == [hs[:3]]
             x1 = torch.randn(cols, device="cuda").to(torch.bfloat16)
             y1 = [mgr.linear(hs[0], x1), mgr.linear(hs[1], x1, bias), mgr.linear(hs[2], x1)]
             mgr.group_rows = False
             assert all(torch.equal(a, mgr.linear(h, x1, b)) for a, h, b in zip(y1, hs, (None, bias, None)))
             mgr.group_rows = True
-            # a weight decoded ahead is not used for another activation; the run is forgotten
-            x = torch.randn(20, cols, device="cuda").to(torch.bfloat16)
-            mgr.linear(hs[0], x)
-            other = torch.randn(20, cols, device="cuda").to(torch.bfloat16)
-            assert torch.equal(mgr.linear(hs[1], other, bias), torch.nn.functional.linear(other, ws[1], bias))
-            assert not mgr._be._runs and not mgr._be._parked_w
-            # a rewrite between two calls of a run: the new weight is what the next call sees
+
+            # a rewrite while the old weight waits: the next request sees the new one
+            x = torch.randn(12, cols, device="cuda").to(torch.bfloat16)
+            waiting = lambda: set(mgr._be._ahead)
+            assert waiting() == {hs[0]}
+            lin(x, 0), lin(x, 1, bias)
+            assert waiting() == {hs[2], hs[3], hs[0]}
+            w_new = (ws[2].float() * 0.5).to(torch.bfloat16)
+            mgr.write(w_new, hs[2])
+            assert waiting() == {hs[3], hs[0]}
+            lin(x, 2, w=w_new)                      # decoded again, with what follows it
+            ws[2] = w_new
+            assert waiting() == {hs[3], hs[0], hs[1]}
+            lin(x, 3), lin(x, 0), lin(x, 1, bias)
+            assert not waiting()
+            lin(x, 2)
+            assert waiting() == {hs[3], hs[0], hs[1]}
+            # a request that was not foreseen: served by a decode of its own, what waited is dropped
+            w4 = (torch.randn(128, cols, device="cuda") * 0.02).to(torch.bfloat16)
+            h4 = mgr.write(w4)
+            wasted = mgr._be.ahead_stats()[1]
+            assert torch.equal(mgr.linear(h4, x), torch.nn.functional.linear(x, w4))
+            assert not waiting() and mgr._be.ahead_stats()[1] == wasted + 3
+            # decoded on one stream, asked for on another
+            lin(x, 3), lin(x, 0)
+            assert waiting() == {hs[1], hs[2], hs[3], h4}  # the new handle has joined the learned order
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                y = mgr.linear(hs[1], x, bias)
+            side.synchronize()
+            assert torch.equal(y, torch.nn.functional.linear(x, ws[1], bias))
+            torch.cuda.current_stream().wait_stream(side)
+            # switched off: every request decodes its own tensor
+            mgr.decode_ahead = False
+            assert not mgr._be._ahead
+            n = len(calls)
+            for rep in range(2):
+                lin(x, 0), lin(x, 1, bias), lin(x, 2), lin(x, 3)
+            assert len(calls) == n
+            mgr._be.check()
+
+            # an order that does not repeat: still the right numbers, and the manager gives up
             mgr2 = neuzip_amd.Manager(precision=7)
             h2 = [mgr2.write(w) for w in ws]
-            for rep in range(2):
-                x = torch.randn(12, cols, device="cuda").to(torch.bfloat16)
-                mgr2.linear(h2[0], x), mgr2.linear(h2[1], x, bias), mgr2.linear(h2[2], x)
-            x = torch.randn(12, cols, device="cuda").to(torch.bfloat16)
-            mgr2.linear(h2[0], x)
-            w_new = (ws[1].float() * 0.5).to(torch.bfloat16)
-            mgr2.write(w_new, h2[1])
-            assert torch.equal(mgr2.linear(h2[1], x, bias), torch.nn.functional.linear(x, w_new, bias))
+            gen = torch.Generator().manual_seed(5)
+            for rep in range(80):
+                for k in torch.randperm(4, generator=gen).tolist():
+                    got = mgr2.linear(h2[k], x)
+                    assert torch.equal(got, torch.nn.functional.linear(x, ws[k])), (rep, k)
+            hits, waste = mgr2._be.ahead_stats()
+            assert mgr2.decode_ahead == (not (waste > 64 and waste > hits))
+            assert not mgr2.decode_ahead
             mgr2._be.check()
     finally:
         del mgr._be.read_batch
     mgr._be.check()
+
+
+def test_backward_of_compressed_linears_takes_weights_decoded_ahead():
+    """Training through converted Linears with nothing but the reference's calls:
+    the backward pass asks for the weights in reverse and finds them decoded
+    ahead from its second step on.  Outputs and gradients equal, bit for bit,
+    those of a manager that decodes every weight on its own, and the dense
+    model's to rounding."""
+    import copy
+
+    import neuzip_amd
+
+    torch.manual_seed(3)
+    dense = torch.nn.Sequential(*[torch.nn.Linear(512, 512, bias=(k % 2 == 0)) for k in range(6)]).cuda().bfloat16()
+    mgr_a, mgr_b = neuzip_amd.Manager(precision=7), neuzip_amd.Manager(precision=7)
+    mgr_b.decode_ahead = False
+    comp_a, comp_b = mgr_a.convert(copy.deepcopy(dense)), mgr_b.convert(copy.deepcopy(dense))
+    packed_a = [m._p for m in comp_a.modules() if isinstance(m, neuzip_amd.nn.Linear)]
+    packed_b = [m._p for m in comp_b.modules() if isinstance(m, neuzip_amd.nn.Linear)]
+    assert len(packed_a) == 6
+    for step in range(4):
+        x = torch.randn(24, 512, device="cuda").to(torch.bfloat16)
+        xd, xa, xb = (x.clone().requires_grad_(True) for _ in range(3))
+        yd, ya, yb = dense(xd), comp_a(xa), comp_b(xb)
+        assert torch.equal(ya, yb), step
+        for y in (yd, ya, yb):
+            y.float().square().mean().backward()
+        assert torch.equal(xa.grad, xb.grad), step
+        torch.testing.assert_close(xa.grad.float(), xd.grad.float(), rtol=2e-2, atol=1e-6)
+        for lin_d, pa, pb in zip(dense, packed_a, packed_b):
+            assert torch.equal(pa._gradient, pb._gradient), step
+            torch.testing.assert_close(pa._gradient.view_as(lin_d.weight.grad).float(), lin_d.weight.grad.float(),
+                                       rtol=2e-2, atol=1e-6)
+            lin_d.weight.grad = None
+            pa._gradient = pb._gradient = None
+        if step == 2:  # a weight changes between two steps: every model takes the new one
+            with torch.no_grad():
+                w = dense[3].weight.mul_(0.5)
+                mgr_a.write(w, packed_a[3]._handle)
+                mgr_b.write(w, packed_b[3]._handle)
+    hits, waste = mgr_a._be.ahead_stats()
+    assert hits >= 20 and waste == 0, (hits, waste)
+    assert mgr_b._be.ahead_stats() == (0, 0)
+    mgr_a._be.check()
+    mgr_b._be.check()
