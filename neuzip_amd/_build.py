@@ -1,8 +1,9 @@
 """Compile libneuzip_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
 
-Five translation units: nz_launch.hip once per precision (the kernels that
-exist per kept-mantissa setting) and nz_api.hip (the C ABI and the kernels all
-precisions share); they compile side by side and are linked into one library.
+Nine translation units: nz_launch.hip twice per precision (the encode kernels
+and the decode kernels of one kept-mantissa setting) and nz_api.hip (the C ABI
+and the kernels all precisions share); they compile side by side and are linked
+into one library.
 """
 from __future__ import annotations
 
