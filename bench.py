@@ -681,12 +681,20 @@ def gpt2m_measure(args, torch):
     spans = []
     n_calls = {"decode": 0, "encode": 0}
 
+    depth = [0]
+
     def timed(fn, kind):
         def wrapper(*a, **k):
             n_calls[kind] += 1
+            if depth[0]:  # inside another codec call (held writes stored by it): that one's span covers this
+                return fn(*a, **k)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            r = fn(*a, **k)
+            depth[0] += 1
+            try:
+                r = fn(*a, **k)
+            finally:
+                depth[0] -= 1
             e1.record()
             spans.append((kind, e0, e1))
             return r
@@ -709,10 +717,12 @@ def gpt2m_measure(args, torch):
         warm = [step() for _ in range(args.warmup)]
         torch.cuda.synchronize()
         spans.clear()
+        launched = be.rewrite_stats()[0]
         t0 = time.perf_counter()
         losses = [step() for _ in range(args.steps)]
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
+        launched = be.rewrite_stats()[0] - launched  # every write here goes into the buffers its entry has
         dec = sum(a.elapsed_time(b) for k, a, b in spans if k == "decode") * 1e-3
         enc = sum(a.elapsed_time(b) for k, a, b in spans if k == "encode") * 1e-3
         return {
@@ -722,6 +732,7 @@ def gpt2m_measure(args, torch):
             "encode_s_per_step": round(enc / args.steps, 5),
             "decode_launches_per_step": sum(1 for k, _, _ in spans if k == "decode") / args.steps,
             "encodes_per_step": sum(1 for k, _, _ in spans if k == "encode") / args.steps,
+            "encode_launches_per_step": launched / args.steps,
             "first_loss": round(float(losses[0]), 4),
             "last_loss": round(float(losses[-1]), 4),
         }, wall, warm + losses
@@ -739,11 +750,14 @@ def gpt2m_measure(args, torch):
     per_block["steps_with_the_dense_runs_loss"] = f"{same} of {len(dense_losses)}"
     per_block["dense_first_loss"] = round(float(dense_losses[args.warmup]), 4)
     per_block["dense_last_loss"] = round(float(dense_losses[-1]), 4)
-    mgr.decode_ahead = False  # the reference's granularity: every request decodes its own tensor
+    mgr.decode_ahead = False  # the reference's granularity: every request decodes its own tensor,
+    mgr.write_behind = False  # every write is an encode launch of its own
     per_linear, _, _ = run(1)
     # the same loop, nothing but the reference's calls, with the manager's default: a request
-    # decodes the weights it has learned to expect next in the same launch
+    # decodes the weights it has learned to expect next in the same launch, and small writes
+    # wait (as copies) until 16 of them share a launch
     mgr.decode_ahead = True
+    mgr.write_behind = True
     per_linear_learned, _, _ = run(1)
     hits, waste = mgr._be.ahead_stats()
     per_linear_learned["weights_decoded_ahead_used"] = hits

@@ -34,13 +34,42 @@ def _stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+class _AfterHeldWrites:
+    """The library's functions as a manager's backend calls them: every
+    ``nz_manager_*`` call first stores the writes the backend still holds back,
+    so that no call can observe the store as it was before them."""
+
+    def __init__(self, lib, owner):
+        self._lib, self._owner, self._made = lib, owner, {}
+
+    def __getattr__(self, name):
+        fn = self._made.get(name)
+        if fn is None:
+            raw = getattr(self._lib, name)
+            if name.startswith("nz_manager_"):
+                owner = self._owner
+
+                def fn(*args, _raw=raw):
+                    if owner._held:
+                        owner.flush()
+                    return _raw(*args)
+            else:
+                fn = raw
+            self._made[name] = fn
+        return fn
+
+
 class _HipBackend:
     """Backend object with the method set of the reference's C++ Manager
     (cuda/neuzip.cu:28-37): read / write / size / linear / linear_without_bias / split."""
 
     def __init__(self, precision: int, normalizer_size: int, chunk_size: int, lane_symbols: int,
                  size_budget: Optional[float] = None):
-        self._L = _lib.load()
+        self._raw = _lib.load()
+        self._L = _AfterHeldWrites(self._raw, self)
+        self._held = []  # writes held back: (handle, copy of the tensor, stream the copy was made on)
+        self._held_elems = 0
+        self.write_behind = True  # hold small writes back until 16 of them share a launch
         self._h = ctypes.c_void_p()
         self.auto_geometry = lane_symbols == "auto" and not chunk_size
         if lane_symbols == "auto":
@@ -71,8 +100,9 @@ class _HipBackend:
         self.ahead_fill = 2 * 4 * cus * 64 * 256  # elements that give every SIMD unit two wavefronts
 
     def close(self):
+        self._held = []
         if getattr(self, "_h", None) is not None and self._h:
-            self._L.nz_manager_destroy(self._h)
+            self._raw.nz_manager_destroy(self._h)
             self._h = None
 
     def __del__(self):
@@ -93,10 +123,23 @@ class _HipBackend:
             tensor = tensor.to(self._device)
         code = self._dtype_code(tensor)
         flat = tensor.detach().contiguous().view(-1)
-        if flat.data_ptr() % 16:
+        copied = flat.data_ptr() % 16 != 0
+        if copied:
             flat = flat.clone()
         self._stored_anew(handle)
         stream = torch.cuda.current_stream(flat.device)
+        if (self.write_behind and 0 < flat.numel() <= self.ahead_fill // 4 and flat.device == self._device
+                and not torch.cuda.is_current_stream_capturing()):
+            # A tensor this small is a few dozen workgroups and its encode takes as long as
+            # that of one sixteen times its size: keep a copy (the caller may change or free
+            # the tensor as soon as this call returns) and store it together with the writes
+            # that follow, at the latest before the next call that looks at the store.
+            self._held = [w for w in self._held if w[0] != handle]
+            self._held.append((handle, flat if copied else flat.clone(), stream))
+            self._held_elems = sum(w[1].numel() for w in self._held)
+            if len(self._held) >= 16 or self._held_elems >= self.ahead_fill:
+                self.flush()
+            return
         rc = self._L.nz_manager_write(self._h, handle.encode(), flat.data_ptr(), flat.numel(), code,
                                       stream.cuda_stream)
         # A write into existing buffers returns while the encode kernel is still reading `flat`.
@@ -104,6 +147,27 @@ class _HipBackend:
         if rc == 0 and flat.numel():
             flat.record_stream(stream)
         _lib.raise_for(rc)
+
+    def flush(self) -> None:
+        """Store the writes that are held back (one launch), on the current stream."""
+        if not self._held:
+            return
+        if torch.cuda.is_current_stream_capturing():
+            # the call that asks for this is refused as a whole; the writes stay held
+            raise ValueError("writes are held back and cannot be stored while the stream is being captured")
+        held, self._held, self._held_elems = self._held, [], 0
+        now = torch.cuda.current_stream(self._device)
+        for _, t, made_on in held:
+            if made_on != now:
+                now.wait_stream(made_on)
+                t.record_stream(now)
+        try:
+            self.write_batch([h for h, _, _ in held], [t for _, t, _ in held])
+        except Exception:
+            # nothing is lost: they are stored again (writing one twice is harmless) with the next call
+            self._held = held + self._held
+            self._held_elems = sum(w[1].numel() for w in self._held)
+            raise
 
     def write_batch(self, handles, tensors) -> None:
         """Several writes with one host synchronisation (16 per native call)."""
@@ -659,7 +723,10 @@ class Manager:
 
     def read(self, handle: str) -> torch.Tensor:
         shape = self.meta_dict[handle]  # KeyError for an unknown handle, as in the reference
-        flat = self._be.read(handle)
+        be = self._be
+        # with decode_ahead the tensor may be a view of a buffer it shares with the weights
+        # that are expected to be asked for next (its own part of it: free to be changed)
+        flat = be.read_shared(handle) if getattr(be, "decode_ahead", False) else be.read(handle)
         return flat.requires_grad_(False).reshape(shape)
 
     def read_shared(self, handle: str) -> torch.Tensor:
@@ -714,6 +781,27 @@ class Manager:
     def group_rows(self, on: bool) -> None:
         if hasattr(self._be, "group_rows"):
             self._be.group_rows = bool(on)
+
+    @property
+    def write_behind(self) -> bool:
+        """Whether writes of small tensors (up to 8 M elements, a few dozen
+        workgroups each) are held back, as a copy made at the time of the call,
+        until 16 of them or 33.5 M elements share one encode launch.  Every other
+        call on the manager stores them first, so no call can tell the difference;
+        ``flush()`` stores them at once."""
+        return bool(getattr(self._be, "write_behind", False))
+
+    @write_behind.setter
+    def write_behind(self, on: bool) -> None:
+        if hasattr(self._be, "write_behind"):
+            if not on:
+                self._be.flush()
+            self._be.write_behind = bool(on)
+
+    def flush(self) -> None:
+        """Store the writes that are held back (see ``write_behind``)."""
+        if hasattr(self._be, "flush"):
+            self._be.flush()
 
     @property
     def decode_ahead(self) -> bool:

@@ -582,7 +582,8 @@ def test_write_many_equals_single_writes(oracle):
         many._be.check()
 
 
-def test_rewrite_in_place_needs_no_size_round_trip(oracle):
+@pytest.mark.parametrize("behind", [True, False])
+def test_rewrite_in_place_needs_no_size_round_trip(oracle, behind):
     """Writing again under handles that hold tensors of the same size (the
     re-compress after an optimizer step, neuzip/__init__.py:25-35) goes straight
     into the entries' buffers; the stored bytes are still the oracle's, and an
@@ -590,6 +591,7 @@ def test_rewrite_in_place_needs_no_size_round_trip(oracle):
     import neuzip_amd
 
     mgr = neuzip_amd.Manager()
+    mgr.write_behind = behind  # single writes of small tensors wait for each other and share a launch, or do not
     shapes = [(300, 1000), (257, 513), (64, 4096)]
     ws = [from_bits(bf16_bits_normal(int(np.prod(s)), seed=i), s) for i, s in enumerate(shapes)]
     hs = [mgr.write(w) for w in ws]
@@ -609,7 +611,7 @@ def test_rewrite_in_place_needs_no_size_round_trip(oracle):
             comp, packed, _ = mgr._be.export(h)
             assert np.array_equal(comp.numpy(), o_comp) and np.array_equal(packed.numpy(), o_packed)
     batches, outgrown = mgr._be.rewrite_stats()
-    assert batches == 2 + len(hs) and outgrown == 0
+    assert batches == (3 if behind else 2 + len(hs)) and outgrown == 0
     # a handle whose new content compresses far worse than the old: the container
     # outgrows the buffer it has and moves to a larger one
     n = 1 << 20
@@ -706,3 +708,115 @@ def test_in_place_rewrites_of_two_managers_on_two_streams(oracle):
         assert torch.equal(got.view(torch.int16), want.view(torch.int16))
         assert mgrs[i]._be.placed_again() == 0
         mgrs[i]._be.check()
+
+
+def test_small_writes_are_held_back_and_no_call_can_tell(oracle):
+    """Writes of small tensors wait, as copies made at the time of the call, until
+    16 of them (or enough elements to fill the device) share one encode launch;
+    every other call on the manager stores them first.  What is stored is what
+    the tensor held when ``write`` was called, byte for byte the oracle's."""
+    import neuzip_amd
+
+    mgr = neuzip_amd.Manager()
+    be = mgr._be
+    n = 200_000
+    ws = [from_bits(bf16_bits_normal(n, seed=40 + i), (n,)) for i in range(20)]
+
+    # the value at the time of the call counts, whatever happens to the tensor afterwards
+    src = ws[0].clone()
+    h = mgr.write(src)
+    assert [w[0] for w in be._held] == [h]
+    src.zero_()
+    del src
+    assert torch.equal(mgr.read(h), ws[0]) and not be._held
+    # two writes under one handle before anything is stored: the later one is what is kept
+    mgr.write(ws[1], h)
+    mgr.write(ws[2], h)
+    assert [w[0] for w in be._held] == [h] and torch.equal(be._held[0][1], ws[2])
+    assert mgr.size(h) > 0 and not be._held  # size() looks at the store: stored first
+    o_comp, o_packed = oracle.compress_bf16(bits_of(ws[2]), 7, *be.geometry(h))
+    comp, packed, _ = be.export(h)
+    assert np.array_equal(comp.numpy(), o_comp) and np.array_equal(packed.numpy(), o_packed)
+    # the sixteenth write stores all sixteen with one launch
+    before = be.rewrite_stats()
+    hs = []
+    for i in range(15):
+        hs.append(mgr.write(ws[i]))
+        assert len(be._held) == i + 1
+    hs.append(mgr.write(ws[15]))
+    assert not be._held
+    for i, hh in enumerate(hs):
+        assert torch.equal(mgr.read(hh), ws[i]), i
+    # ... and again into the buffers the entries have: one batch in place
+    for i, hh in enumerate(hs):
+        mgr.write(ws[i + 4], hh)
+    assert not be._held
+    assert be.rewrite_stats()[0] == before[0] + 1
+    for i, hh in enumerate(hs):
+        assert torch.equal(mgr.read(hh), ws[i + 4]), i
+    # explicit flush; a tensor too large to be worth a copy is stored at once
+    mgr.write(ws[0], hs[0])
+    assert be._held
+    mgr.flush()
+    assert not be._held and torch.equal(mgr.read(hs[0]), ws[0])
+    big = from_bits(bf16_bits_normal(be.ahead_fill // 4 + 8, seed=3), (be.ahead_fill // 4 + 8,))
+    hb = mgr.write(big)
+    assert not be._held and torch.equal(mgr.read(hb), big)
+    # written on one stream, stored by a call on another
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fresh = (ws[5].float() * 1.25).to(torch.bfloat16)
+        mgr.write(fresh, hs[1])
+        del fresh
+    assert be._held
+    got = mgr.read(hs[1])
+    assert torch.equal(got, (ws[5].float() * 1.25).to(torch.bfloat16))
+    torch.cuda.current_stream().wait_stream(side)
+    # a call that cannot store them (its stream is being captured) is refused and nothing is lost
+    mgr.write(ws[7], hs[2])
+    out = torch.empty(ws[7].numel(), dtype=torch.bfloat16, device="cuda")
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        with pytest.raises(ValueError, match="being captured"):
+            be.read_into(hs[2], out)
+        out.add_(0)
+    assert [w[0] for w in be._held] == [hs[2]]
+    assert torch.equal(mgr.read(hs[2]), ws[7]) and not be._held
+    # switched off: every write is stored by its own call
+    mgr.write(ws[8], hs[3])
+    mgr.write_behind = False
+    assert not be._held and torch.equal(mgr.read(hs[3]), ws[8])
+    mgr.write(ws[9], hs[3])
+    assert not be._held and torch.equal(mgr.read(hs[3]), ws[9])
+    be.check()
+
+
+def test_the_references_update_loop_reads_ahead_and_writes_behind():
+    """The reference's training example updates every compressed parameter with
+    ``write(read(handle).add_(gradient, alpha=-lr), handle)`` (examples/training/
+    train_clm.py:822-833).  Served with weights decoded ahead and writes held
+    back, the loop leaves exactly the weights that plain dense SGD leaves."""
+    import neuzip_amd
+
+    torch.manual_seed(11)
+    shapes = [(256, 512), (512, 512), (128, 1024), (1024, 256)] * 5
+    dense = [(torch.randn(s, device="cuda") * 0.02).to(torch.bfloat16) for s in shapes]
+    mgr = neuzip_amd.Manager(precision=7)
+    hs = [mgr.write(w) for w in dense]
+    lr = 1e-2
+    for step in range(4):
+        grads = [(torch.randn(s, device="cuda") * 0.01).to(torch.bfloat16) for s in shapes]
+        for h, g in zip(hs, grads):
+            mgr.write(mgr.read(h).add_(g, alpha=-lr), h)
+        for w, g in zip(dense, grads):
+            w.add_(g, alpha=-lr)
+        if step % 2:  # looked at after some steps only: the next step may start with writes still held
+            for h, w in zip(hs, dense):
+                assert torch.equal(mgr.read(h), w), step
+    hits, waste = mgr._be.ahead_stats()
+    assert hits > 40, (hits, waste)
+    for h, w in zip(hs, dense):
+        assert torch.equal(mgr.read(h), w)
+    mgr._be.check()
