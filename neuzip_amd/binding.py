@@ -14,6 +14,7 @@ from typing import Optional
 import torch
 
 from neuzip_amd import _lib
+from neuzip_amd._ahead import RequestOrder
 from neuzip_amd.utils import _convert
 
 _lib.load()  # hard failure when the extension is not built (reference: binding.py:15-20)
@@ -90,14 +91,12 @@ class _HipBackend:
         self._no_run = set()    # first handles whose run did not repeat itself
         self._parked = {}       # handle -> (activation, its version, result, first handle, bias) computed ahead
         self._cur = None        # the run being observed: (activation, its version, [(handle, rows, bias)])
-        self.decode_ahead = True  # dense weights: decode the handles that are asked for next in the same launch
-        self._next = {}         # (handle asked for before, handle) -> the handle that was asked for after them
-        self._last2 = (None, None)  # the two handles whose dense weight was asked for last
-        self._ahead = {}        # handle -> (decoded weight, stream it was decoded on), waiting to be asked for
         self._plans = {}        # tuple of handles -> read_batch plan
-        self._ahead_hits = self._ahead_waste = 0
         cus = torch.cuda.get_device_properties(self._device).multi_processor_count
         self.ahead_fill = 2 * 4 * cus * 64 * 256  # elements that give every SIMD unit two wavefronts
+        # dense weights: which handles to decode in the same launch, and the decoded ones that wait
+        self._order = RequestOrder(self._decode_one, self._decode_many, lambda h: self._meta(h)[1],
+                                   self.ahead_fill, self._MAX_AHEAD)
 
     def close(self):
         self._held = []
@@ -162,15 +161,16 @@ class _HipBackend:
                 now.wait_stream(made_on)
                 t.record_stream(now)
         try:
-            self.write_batch([h for h, _, _ in held], [t for _, t, _ in held])
+            self.write_batch([h for h, _, _ in held], [t for _, t, _ in held], _told=True)
         except Exception:
             # nothing is lost: they are stored again (writing one twice is harmless) with the next call
             self._held = held + self._held
             self._held_elems = sum(w[1].numel() for w in self._held)
             raise
 
-    def write_batch(self, handles, tensors) -> None:
-        """Several writes with one host synchronisation (16 per native call)."""
+    def write_batch(self, handles, tensors, _told: bool = False) -> None:
+        """Several writes with one host synchronisation (16 per native call).
+        (``_told``: the caches have heard of these writes when they were made.)"""
         flats = []
         for t in tensors:
             if not t.is_cuda:
@@ -181,8 +181,9 @@ class _HipBackend:
         for at in range(0, len(handles), 16):
             hs, fs = handles[at:at + 16], flats[at:at + 16]
             k = len(hs)
-            for h in hs:
-                self._stored_anew(h)
+            if not _told:
+                for h in hs:
+                    self._stored_anew(h)
             names = (ctypes.c_char_p * k)(*[h.encode() for h in hs])
             ptrs = (ctypes.c_void_p * k)(*[f.data_ptr() for f in fs])
             ns = (ctypes.c_uint64 * k)(*[f.numel() for f in fs])
@@ -197,7 +198,7 @@ class _HipBackend:
         """``handle`` is about to hold other values: nothing derived from the old ones survives"""
         self._known.pop(handle, None)
         self._parked.clear()  # products computed ahead from the weights as they were
-        self._ahead.pop(handle, None)
+        self._order.written(handle)
         if any(handle in key for key in self._plans):  # a plan holds the element counts of its tensors
             self._plans = {key: plan for key, plan in self._plans.items() if handle not in key}
 
@@ -342,7 +343,7 @@ class _HipBackend:
         return int(self._L.nz_manager_packed_bytes(self._h, handle.encode()))
 
     def trim(self) -> None:
-        self._ahead.clear()
+        self._order.clear()
         _lib.raise_for(self._L.nz_manager_trim(self._h))
 
     def rewrite_stats(self):
@@ -475,66 +476,35 @@ class _HipBackend:
 
     # -- dense weights: the handles that are asked for next share the launch -----
     #
-    # A model asks for its weights in the same order pass after pass (forwards
-    # through the blocks, backwards through them in training).  The order is
-    # learned as "after handles a, b came c"; a request that finds nothing
-    # waiting follows those links and decodes the handles it expects next with
-    # the same launch, until the launch would fill the device (matrices of a few
-    # million elements cannot on their own).  The others wait for their requests.
-    # A weight that waits is dropped when its handle is written, so what is handed
-    # out always equals a decode at the time of the request; a request that was
-    # not foreseen drops everything that waits, and a manager whose requests keep
-    # coming in another order than learned stops decoding ahead.  Requests made
-    # while a stream is being captured take no part in any of this.
+    # A model asks for its weights in the same order pass after pass, and matrices
+    # of a few million elements cannot fill the device on their own: a request
+    # that finds nothing waiting decodes, in the same launch, the handles that the
+    # learned order (neuzip_amd/_ahead.py) expects next, and those wait for their
+    # requests.  A weight that waits is dropped when its handle is written, so what
+    # is handed out always equals a decode at the time of the request.  Requests
+    # made while a stream is being captured take no part in any of this.
 
     _MAX_AHEAD = 16  # tensors one decode launch takes (NZ_BATCH_MAX)
 
-    def _dense_weight(self, handle: str) -> torch.Tensor:
-        """the decoded weight of ``handle`` (flat), possibly a view of a buffer it shares with its neighbours"""
-        if torch.cuda.is_current_stream_capturing():
-            # a weight that waits across the end of a capture would be memory of the graph's
-            # pool that no kernel has filled yet, and one decoded before the capture would be
-            # baked into the graph by address: a captured request decodes its own tensor
-            self._ahead.clear()
-            self._last2 = (None, None)
-            return self.read(handle)
-        before, last = self._last2
-        if last is not None:
-            self._next[(before, last)] = handle
-        self._last2 = (last, handle)
-        hit = self._ahead.pop(handle, None)
-        if hit is not None:
-            w, decoded_on = hit
-            self._ahead_hits += 1
-            now = torch.cuda.current_stream(self._device)
-            if now != decoded_on:
-                now.wait_stream(decoded_on)
-                w.record_stream(now)
-            return w
-        if self._ahead:  # not what was expected next
-            self._ahead_waste += len(self._ahead)
-            self._ahead.clear()
-            if self._ahead_waste > 64 and self._ahead_waste > self._ahead_hits:
-                self.decode_ahead = False
-        if not self.decode_ahead:
-            return self.read(handle)
-        chain, total, a, b = [handle], self._meta(handle)[1], last, handle
-        while len(chain) < self._MAX_AHEAD and total < self.ahead_fill:
-            nxt = self._next.get((a, b))
-            if nxt is None or nxt in chain:
-                break
-            try:
-                total += self._meta(nxt)[1]
-            except RuntimeError:
-                break  # no longer stored
-            chain.append(nxt)
-            a, b = b, nxt
-        if len(chain) == 1:
-            return self.read(handle)
-        key = tuple(chain)
+    @property
+    def decode_ahead(self) -> bool:
+        return self._order.enabled
+
+    @decode_ahead.setter
+    def decode_ahead(self, on: bool) -> None:
+        self._order.enabled = bool(on)
+        if not on:
+            self._order.clear()
+
+    def _decode_one(self, handle: str):
+        return self.read(handle), torch.cuda.current_stream(self._device)
+
+    def _decode_many(self, handles):
+        """one launch for ``handles`` (a handle may appear twice) -> [(flat weight, stream)], or None"""
+        key = tuple(handles)
         plan = self._plans.get(key)
         if plan is None:
-            plan = self._plans[key] = self.batch_plan(chain)
+            plan = self._plans[key] = self.batch_plan(handles)
         sizes = [int(c) for c in plan[1]]
         flat = torch.empty(sum((n + 7) & ~7 for n in sizes), dtype=torch.bfloat16, device=self._device)
         outs, at = [], 0
@@ -543,13 +513,28 @@ class _HipBackend:
             at += (n + 7) & ~7
         try:
             self.read_batch(plan, outs)
-        except (ValueError, RuntimeError):  # e.g. scratch that cannot grow while a graph is captured
+        except (ValueError, RuntimeError):  # e.g. scratch that cannot grow
             self._plans.pop(key, None)
-            return self.read(handle)
+            return None
         stream = torch.cuda.current_stream(self._device)
-        for h, o in zip(chain[1:], outs[1:]):
-            self._ahead[h] = (o, stream)
-        return outs[0]
+        return [(o, stream) for o in outs]
+
+    def _dense_weight(self, handle: str) -> torch.Tensor:
+        """the decoded weight of ``handle`` (flat), possibly a view of a buffer it shares with its neighbours"""
+        if torch.cuda.is_current_stream_capturing():
+            # a weight that waits across the end of a capture would be memory of the graph's
+            # pool that no kernel has filled yet, and one decoded before the capture would be
+            # baked into the graph by address: a captured request decodes its own tensor
+            self._order.clear()
+            self._order.forget_position()
+            return self.read(handle)
+        (w, decoded_on), ahead = self._order.request(handle)
+        if ahead:
+            now = torch.cuda.current_stream(self._device)
+            if now != decoded_on:
+                now.wait_stream(decoded_on)
+                w.record_stream(now)
+        return w
 
     def read_shared(self, handle: str) -> torch.Tensor:
         """The decoded weight for a caller that only reads it and drops it at once."""
@@ -557,7 +542,7 @@ class _HipBackend:
 
     def ahead_stats(self):
         """(weights decoded ahead that were asked for, weights decoded ahead and dropped unused)"""
-        return self._ahead_hits, self._ahead_waste
+        return self._order.hits, self._order.waste
 
     def _weight_for_gemm(self, handle: str, inputs: torch.Tensor, shape, bias) -> torch.Tensor:
         """The dense weight of ``handle`` for a call with more rows than the fused
@@ -817,8 +802,6 @@ class Manager:
     def decode_ahead(self, on: bool) -> None:
         if hasattr(self._be, "decode_ahead"):
             self._be.decode_ahead = bool(on)
-            if not on:
-                self._be._ahead.clear()
 
     def gather_rows(self, handle: str, indices: torch.Tensor) -> torch.Tensor:
         """Rows ``indices`` of the stored 2-D table ``handle`` as ``[indices.numel(), row_len]``

@@ -489,18 +489,20 @@ def test_dense_weights_asked_for_in_a_repeating_order_share_decode_launches():
 
             # a rewrite while the old weight waits: the next request sees the new one
             x = torch.randn(12, cols, device="cuda").to(torch.bfloat16)
-            waiting = lambda: set(mgr._be._ahead)
+            waiting = lambda: mgr._be._order.waiting()
             assert waiting() == {hs[0]}
             lin(x, 0), lin(x, 1, bias)
             assert waiting() == {hs[2], hs[3], hs[0]}
             w_new = (ws[2].float() * 0.5).to(torch.bfloat16)
             mgr.write(w_new, hs[2])
             assert waiting() == {hs[3], hs[0]}
-            lin(x, 2, w=w_new)                      # decoded again, with what follows it
+            lin(x, 2, w=w_new)                      # decoded again, on its own: the others go on waiting
             ws[2] = w_new
-            assert waiting() == {hs[3], hs[0], hs[1]}
-            lin(x, 3), lin(x, 0), lin(x, 1, bias)
+            assert waiting() == {hs[3], hs[0]}
+            lin(x, 3), lin(x, 0)
             assert not waiting()
+            lin(x, 1, bias)                         # the walk that lost a weight to the write ends in front of
+            assert not waiting()                    # that place the next time (and grows again from there)
             lin(x, 2)
             assert waiting() == {hs[3], hs[0], hs[1]}
             # a request that was not foreseen: served by a decode of its own, what waited is dropped
@@ -511,7 +513,7 @@ def test_dense_weights_asked_for_in_a_repeating_order_share_decode_launches():
             assert not waiting() and mgr._be.ahead_stats()[1] == wasted + 3
             # decoded on one stream, asked for on another
             lin(x, 3), lin(x, 0)
-            assert waiting() == {hs[1], hs[2], hs[3], h4}  # the new handle has joined the learned order
+            assert waiting() == {hs[1], hs[2], h4, hs[3]}  # the new handle has taken its place in the learned order
             side = torch.cuda.Stream()
             side.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(side):
@@ -521,7 +523,7 @@ def test_dense_weights_asked_for_in_a_repeating_order_share_decode_launches():
             torch.cuda.current_stream().wait_stream(side)
             # switched off: every request decodes its own tensor
             mgr.decode_ahead = False
-            assert not mgr._be._ahead
+            assert not mgr._be._order.waiting()
             n = len(calls)
             for rep in range(2):
                 lin(x, 0), lin(x, 1, bias), lin(x, 2), lin(x, 3)

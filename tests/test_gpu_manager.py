@@ -820,3 +820,58 @@ def test_the_references_update_loop_reads_ahead_and_writes_behind():
     for h, w in zip(hs, dense):
         assert torch.equal(mgr.read(h), w)
     mgr._be.check()
+
+
+def test_lomo_hooks_with_weights_decoded_ahead_and_writes_held_back():
+    """The reference's memory-efficient training (neuzip/__init__.py:25-35): every
+    compressed parameter is updated and written back from a hook in the middle
+    of the backward pass, so a weight is asked for twice in a row (backward, then
+    update) and written while the weights of the layers before it wait decoded.
+    Equal, step after step, to the dense run and to a manager that decodes and
+    stores every tensor on its own."""
+    import neuzip_amd
+
+    def deep(seed):
+        torch.manual_seed(seed)
+        layers = []
+        for k in range(8):
+            layers += [torch.nn.Linear(256, 256, bias=(k % 3 == 0)), torch.nn.GELU()]
+        m = torch.nn.Sequential(*layers[:-1]).to(torch.bfloat16)
+        for p in m.parameters():
+            p.data.normal_(0, 0.05)
+        return m
+
+    sched = _Sched()
+    dense = deep(5).cuda()
+    models, mgrs = [], []
+    for plain in (False, True):
+        m = deep(5)
+        mgr = neuzip_amd.Manager(precision=7)
+        if plain:
+            mgr.decode_ahead = False
+            mgr.write_behind = False
+        mgr.convert(m)
+        models.append(m.cuda())
+        mgrs.append(mgr)
+    for p in dense.parameters():
+        p.register_post_accumulate_grad_hook(partial(neuzip_amd.lomo_hook, sched))
+    for m in models:
+        for p in m.parameters():
+            hook = neuzip_amd.compressed_lomo_hook if isinstance(p, neuzip_amd.nn.Parameter) else neuzip_amd.lomo_hook
+            p.register_post_accumulate_grad_hook(partial(hook, sched))
+    torch.manual_seed(9)
+    for step in range(6):
+        x = torch.randn(32, 256, device="cuda", dtype=torch.bfloat16)
+        losses = [m(x).float().pow(2).mean() for m in [dense] + models]
+        assert torch.equal(losses[0], losses[1]) and torch.equal(losses[1], losses[2]), step
+        for l in losses:
+            l.backward()
+        if step % 2:
+            for k in range(0, 15, 2):
+                assert torch.equal(models[0][k].weight(), dense[k].weight.data), (step, k)
+                assert torch.equal(models[1][k].weight(), dense[k].weight.data), (step, k)
+    hits, waste = mgrs[0]._be.ahead_stats()
+    assert hits > 30 and waste < hits // 2, (hits, waste)
+    assert mgrs[1]._be.ahead_stats() == (0, 0)
+    for mgr in mgrs:
+        mgr._be.check()
