@@ -634,7 +634,7 @@ def gpt2m_measure(args, torch):
     """BASELINE config 4: GPT-2-medium-shaped model, weights kept compressed and
     re-compressed after every AdamW step; reports the codec share of the step."""
     import neuzip_amd
-    from bench_models import CompressedAdamW, GPT2Shaped
+    from bench_models import CompressedAdamW, GPT2Shaped, ReferenceLoopSGD
 
     layers = args.layers or 24
     torch.manual_seed(args.seed)
@@ -704,9 +704,9 @@ def gpt2m_measure(args, torch):
     be.read_batch = timed(be.read_batch, "decode")
     be.write_batch = timed(be.write_batch, "encode")
 
-    def run(group):
+    def run(group, sgd_loop=False):
         """-> per-step figures with the Linears decoded one by one (group 1) or per block"""
-        opt_c = CompressedAdamW(comp_params, lr=1e-4, group=group)
+        opt_c = ReferenceLoopSGD(comp_params, lr=1e-4) if sgd_loop else CompressedAdamW(comp_params, lr=1e-4, group=group)
         opt_d = torch.optim.AdamW(rest, lr=1e-4)
 
         def step():
@@ -762,6 +762,12 @@ def gpt2m_measure(args, torch):
     hits, waste = mgr._be.ahead_stats()
     per_linear_learned["weights_decoded_ahead_used"] = hits
     per_linear_learned["weights_decoded_ahead_dropped"] = waste
+    # the reference's own update statement (plain SGD through read and write, train_clm.py:822-833)
+    # in place of AdamW: first at the reference's granularity, then with the manager's defaults
+    mgr.decode_ahead = mgr.write_behind = False
+    sgd_loop_plain, _, _ = run(1, sgd_loop=True)
+    mgr.decode_ahead = mgr.write_behind = True
+    sgd_loop, _, _ = run(1, sgd_loop=True)
     mgr._be.check()
     # writes that went into the entries' existing buffers (no allocation, no wait for the size)
     in_place, outgrown = be.rewrite_stats()
@@ -820,6 +826,8 @@ def gpt2m_measure(args, torch):
             "decode_per_block": per_block,
             "decode_per_linear": per_linear,
             "decode_per_linear_order_learned": per_linear_learned,
+            "reference_sgd_loop_per_linear": sgd_loop_plain,
+            "reference_sgd_loop_order_learned": sgd_loop,
             "lockstep_check_lossless": lockstep,
             "rewrites": rewrites,
             "compressed_tensors": n_comp,
@@ -1148,6 +1156,8 @@ def main():
                 "ms_per_step_compressed_decode_per_block": pb["ms_per_step"],
                 "ms_per_step_compressed_decode_per_linear": cfg["decode_per_linear"]["ms_per_step"],
                 "ms_per_step_compressed_unchanged_caller": cfg["decode_per_linear_order_learned"]["ms_per_step"],
+                "ms_per_step_reference_sgd_loop": cfg["reference_sgd_loop_order_learned"]["ms_per_step"],
+                "ms_per_step_reference_sgd_loop_per_linear": cfg["reference_sgd_loop_per_linear"]["ms_per_step"],
                 "codec_share_of_step_per_block": pb["codec_share_of_step"],
                 "codec_share_of_step_per_linear": cfg["decode_per_linear"]["codec_share_of_step"],
                 "codec_share_of_step_unchanged_caller": cfg["decode_per_linear_order_learned"]["codec_share_of_step"],

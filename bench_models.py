@@ -251,6 +251,25 @@ class CompressedAdamW:
                 p.grad = None
 
 
+class ReferenceLoopSGD:
+    """The update the reference's training example applies to compressed
+    parameters, statement for statement (examples/training/train_clm.py:822-833):
+    ``write(read(handle).add_(gradient, alpha=-lr), handle)``, one parameter
+    after the other."""
+
+    def __init__(self, params, lr=1e-4):
+        self.params = list(params)
+        self.lr = lr
+
+    @torch.no_grad()
+    def step(self):
+        for p in self.params:
+            if getattr(p, "_gradient", None) is not None:
+                p._manager.write(p._manager.read(p._handle).add_(p._gradient, alpha=-self.lr), p._handle)
+                p._gradient = None
+                p.grad = None
+
+
 def paired_parameters(dense: torch.nn.Module, comp: torch.nn.Module):
     """``[(name, dense parameter, its counterpart in the converted twin)]``: for a
     compressed Linear the counterpart of ``weight`` is the ``neuzip_amd.nn.Parameter``."""
