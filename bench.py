@@ -506,18 +506,23 @@ def llama8b_measure(args, torch, full):
         return g, logits
 
     res, toks = {}, {}
+    mgr_box = []  # the manager, once the model is converted
 
     def measure(name, graph=None):
         run_mode(graph, 4)  # warm-up
         res[name + "_prefill_s"], res[name + "_decode_s"], toks[name] = run_mode(graph)
+        ahead = ""
+        if mgr_box and hasattr(mgr_box[0]._be, "ahead_stats"):
+            ahead = ", weights decoded ahead used / dropped so far %d / %d" % mgr_box[0]._be.ahead_stats()
         print(f"[llama8b] {name}: prefill {res[name + '_prefill_s']:.3f} s, "
-              f"{(steps - 1) / res[name + '_decode_s']:.1f} tok/s", file=sys.stderr, flush=True)
+              f"{(steps - 1) / res[name + '_decode_s']:.1f} tok/s{ahead}", file=sys.stderr, flush=True)
 
     measure("dense_eager")
     measure("dense_graph", capture())
     dense_param_bytes = sum(p.numel() * p.element_size() for p in model.parameters())
 
     mgr, how = make_manager(args, args.precision)
+    mgr_box.append(mgr)
     t_conv, _ = sync_time(lambda: mgr.convert(model))
     torch.cuda.empty_cache()
     comp_bytes = sum(mgr.size(h) for h in mgr.meta_dict)

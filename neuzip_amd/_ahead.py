@@ -32,7 +32,10 @@ class RequestOrder:
         self.decode_one, self.decode_many, self.size_of = decode_one, decode_many, size_of
         self.fill, self.most = int(fill), int(most)
         self.enabled = True
-        self.hits = self.waste = 0
+        self.hits = self.waste = 0          # objects decoded ahead that were asked for / dropped unused, ever
+        self._recent = [0, 0]               # the same two over the last thousand or so
+        self._pause = 0                     # requests still to be served one by one: the order did not repeat itself
+        self._pause_next = 256              # ... and for how many the next time it does not
         self._next: Dict[tuple, tuple] = {}     # place -> (the handle that was asked for next, after a write?)
         self._at: tuple = (None, None, 0, False)  # the place of the last request
         self._wrote = False                     # has anything been written since that request?
@@ -55,6 +58,7 @@ class RequestOrder:
             self._cut[start] = min(at, self._cut.get(start, at))
             self._rewritten.add(handle)
             self.waste += 1
+            self._recent[1] += 1
 
     def clear(self) -> None:
         """drop everything that waits (nothing is counted)"""
@@ -64,6 +68,11 @@ class RequestOrder:
     def forget_position(self) -> None:
         """the next request is not taken as the successor of the last ones"""
         self._at = (None, None, 0, False)
+
+    @property
+    def paused(self) -> bool:
+        """no walks at the moment: the order of the requests has not been repeating itself"""
+        return self._pause > 0
 
     def waiting(self):
         """the handles something waits for"""
@@ -82,6 +91,9 @@ class RequestOrder:
             if not queue:
                 del self._waiting[handle]
             self.hits += 1
+            self._recent[0] += 1
+            if self._recent[0] + self._recent[1] > 1024:
+                self._recent = [self._recent[0] // 2, self._recent[1] // 2]
             return obj, True
         if self._waiting:
             if handle in self._rewritten:
@@ -89,11 +101,19 @@ class RequestOrder:
                 self._rewritten.discard(handle)
                 return self._decode_walk(start, self._walk(start, self._waiting)), False
             # not what was expected next
-            self.waste += sum(len(q) for q in self._waiting.values())
+            lost = sum(len(q) for q in self._waiting.values())
+            self.waste += lost
+            self._recent[1] += lost
             self._waiting.clear()
-            if self.waste > 64 and self.waste > self.hits:
-                self.enabled = False  # the requests of this owner do not repeat their order
+            if self._recent[1] > 64 and self._recent[1] > self._recent[0]:
+                # the requests do not come in the order they came in before: no walks for a
+                # while (the order is still being learned), twice as long every time it happens
+                self._pause, self._pause_next = self._pause_next, min(2 * self._pause_next, 1 << 16)
+                self._recent = [0, 0]
         self._rewritten.clear()
+        if self._pause:
+            self._pause -= 1
+            return self.decode_one(handle), False
         if not self.enabled:
             return self.decode_one(handle), False
         return self._decode_walk(start, self._walk(start)), False

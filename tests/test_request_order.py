@@ -151,19 +151,32 @@ def test_an_unforeseen_request_drops_everything_that_waits():
     assert s.order.waste == wasted + n - 1 and not s.order.waiting()
 
 
-def test_requests_without_a_repeating_order_switch_it_off():
+def test_requests_without_a_repeating_order_are_served_one_by_one_for_a_while():
     rng = random.Random(4)
     s = Store({k: 100 for k in range(6)})
-    for rep in range(200):
+    pauses = 0
+    for rep in range(400):
         order = list(range(6))
         rng.shuffle(order)
+        was = s.order.paused
         for k in order:
             s.request(k)
-    assert not s.order.enabled and s.order.waste > s.order.hits
+        pauses += s.order.paused and not was
+    assert pauses >= 2 and s.order.paused     # again and again, each pause twice as long as the one before
     s.launches.clear()
     for k in range(6):
         s.request(k)
     assert s.launches == [[k] for k in range(6)]
+    # the order settles: once the pause is over the walks are back
+    for rep in range(2000):
+        for k in range(6):
+            s.request(k)
+    assert not s.order.paused
+    s.launches.clear()
+    for rep in range(4):
+        for k in range(6):
+            s.request(k)
+    assert len(s.launches) <= 5
 
 
 @pytest.mark.parametrize("seed", range(12))
