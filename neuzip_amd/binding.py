@@ -707,10 +707,13 @@ class Manager:
                 self._be.write(h, t)
 
     def read(self, handle: str) -> torch.Tensor:
+        """The stored tensor, decompressed (neuzip/binding.py:88-92).  With
+        ``decode_ahead`` the result may be a view into a buffer it shares with the
+        weights that are expected to be asked for next: its own part of it, free to
+        be changed in place, but ``clone()`` it before serialising it or keeping it
+        for long (the view keeps the whole buffer alive)."""
         shape = self.meta_dict[handle]  # KeyError for an unknown handle, as in the reference
         be = self._be
-        # with decode_ahead the tensor may be a view of a buffer it shares with the weights
-        # that are expected to be asked for next (its own part of it: free to be changed)
         flat = be.read_shared(handle) if getattr(be, "decode_ahead", False) else be.read(handle)
         return flat.requires_grad_(False).reshape(shape)
 
