@@ -709,12 +709,14 @@ def gpt2m_measure(args, torch):
     be.read_batch = timed(be.read_batch, "decode")
     be.write_batch = timed(be.write_batch, "encode")
 
-    def run(group, sgd_loop=False):
+    def run(group, sgd_loop=False, hooks_only=False):
         """-> per-step figures with the Linears decoded one by one (group 1) or per block"""
         opt_c = ReferenceLoopSGD(comp_params, lr=1e-4) if sgd_loop else CompressedAdamW(comp_params, lr=1e-4, group=group)
         opt_d = torch.optim.AdamW(rest, lr=1e-4)
 
         def step():
+            if hooks_only:  # the hooks registered on the parameters do all the updating
+                return train_step([])
             loss = train_step([opt_c, opt_d])
             opt_d.zero_grad(set_to_none=True)
             return loss
@@ -773,6 +775,26 @@ def gpt2m_measure(args, torch):
     sgd_loop_plain, _, _ = run(1, sgd_loop=True)
     mgr.decode_ahead = mgr.write_behind = True
     sgd_loop, _, _ = run(1, sgd_loop=True)
+
+    # the reference's update hooks (neuzip/__init__.py:16-35): every parameter is updated, and a
+    # compressed one written back, from a post-accumulate-grad hook in the middle of the backward pass
+    class _FixedLR:
+        def get_last_lr(self):
+            return [1e-4]
+
+    from functools import partial
+
+    def with_hooks(params_and_hooks):
+        return [p.register_post_accumulate_grad_hook(partial(h, _FixedLR())) for p, h in params_and_hooks]
+
+    hooked = [(p, neuzip_amd.compressed_lomo_hook) for p in comp_params] + [(p, neuzip_amd.lomo_hook) for p in rest]
+    mgr.decode_ahead = mgr.write_behind = False
+    handles = with_hooks(hooked)
+    lomo_plain, _, _ = run(1, hooks_only=True)
+    mgr.decode_ahead = mgr.write_behind = True
+    lomo, _, _ = run(1, hooks_only=True)
+    for hd in handles:
+        hd.remove()
     mgr._be.check()
     # writes that went into the entries' existing buffers (no allocation, no wait for the size)
     in_place, outgrown = be.rewrite_stats()
@@ -833,6 +855,8 @@ def gpt2m_measure(args, torch):
             "decode_per_linear_order_learned": per_linear_learned,
             "reference_sgd_loop_per_linear": sgd_loop_plain,
             "reference_sgd_loop_order_learned": sgd_loop,
+            "reference_update_hooks_per_linear": lomo_plain,
+            "reference_update_hooks_order_learned": lomo,
             "lockstep_check_lossless": lockstep,
             "rewrites": rewrites,
             "compressed_tensors": n_comp,
@@ -1163,6 +1187,8 @@ def main():
                 "ms_per_step_compressed_unchanged_caller": cfg["decode_per_linear_order_learned"]["ms_per_step"],
                 "ms_per_step_reference_sgd_loop": cfg["reference_sgd_loop_order_learned"]["ms_per_step"],
                 "ms_per_step_reference_sgd_loop_per_linear": cfg["reference_sgd_loop_per_linear"]["ms_per_step"],
+                "ms_per_step_reference_update_hooks": cfg["reference_update_hooks_order_learned"]["ms_per_step"],
+                "ms_per_step_reference_update_hooks_per_linear": cfg["reference_update_hooks_per_linear"]["ms_per_step"],
                 "codec_share_of_step_per_block": pb["codec_share_of_step"],
                 "codec_share_of_step_per_linear": cfg["decode_per_linear"]["codec_share_of_step"],
                 "codec_share_of_step_unchanged_caller": cfg["decode_per_linear_order_learned"]["codec_share_of_step"],
