@@ -673,6 +673,25 @@ def gpt2m_measure(args, torch):
     torch.cuda.synchronize()
     dense_ms = (time.perf_counter() - t0) / args.steps * 1e3
     del opt
+    # ... and with the reference's update hooks on every parameter (plain SGD inside the backward pass)
+    import neuzip_amd as _nz
+    from functools import partial as _partial
+
+    class _LR:
+        def get_last_lr(self):
+            return [1e-4]
+
+    dense_hooks = [p.register_post_accumulate_grad_hook(_partial(_nz.lomo_hook, _LR())) for p in model.parameters()]
+    for _ in range(args.warmup):
+        train_step([])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        train_step([])
+    torch.cuda.synchronize()
+    dense_hooks_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    for hd in dense_hooks:
+        hd.remove()
     model.load_state_dict(state0)
     del state0
     torch.cuda.empty_cache()
@@ -849,6 +868,7 @@ def gpt2m_measure(args, torch):
             "workload": f"GPT-2-medium-shaped random-init model, {layers} layers, batch {args.batch} x seq {args.seq_len}, "
                         f"bf16 weights compressed (precision {args.precision}), re-compressed after each AdamW step",
             "dense_bf16_torch_adamw_ms_per_step": round(dense_ms, 3),
+            "dense_bf16_update_hooks_ms_per_step": round(dense_hooks_ms, 3),
             "tensors_per_decode_and_write_launch": per_launch,
             "decode_per_block": per_block,
             "decode_per_linear": per_linear,
@@ -1182,6 +1202,7 @@ def main():
                 "tensors_per_decode_and_write_launch": cfg["tensors_per_decode_and_write_launch"],
                 "tokens_per_s": gm["value"],
                 "ms_per_step_dense_bf16_adamw": cfg["dense_bf16_torch_adamw_ms_per_step"],
+                "ms_per_step_dense_bf16_update_hooks": cfg["dense_bf16_update_hooks_ms_per_step"],
                 "ms_per_step_compressed_decode_per_block": pb["ms_per_step"],
                 "ms_per_step_compressed_decode_per_linear": cfg["decode_per_linear"]["ms_per_step"],
                 "ms_per_step_compressed_unchanged_caller": cfg["decode_per_linear_order_learned"]["ms_per_step"],
